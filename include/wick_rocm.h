@@ -1,0 +1,185 @@
+/*
+ * wick_rocm.h -- C ABI of the MI355X (gfx950) backend for wick's block-quantized
+ * matmul path: Q8_0 activation quantization, decode GEMV, batched prefill GEMM
+ * over GGUF Q4_0 / Q8_0 weight blocks.
+ *
+ * The reference has no C ABI for this path; its boundary is Rust-internal.  Each
+ * entry point below names the reference interface it stands in for (paths are
+ * relative to the reference checkout).  A Rust host (`backend/rocm.rs`) binds
+ * these with a plain `extern "C"` block and links `libwick_rocm.a`.
+ *
+ * Conventions
+ *   - Every function returns a wick_rocm_status (0 = ok, negative = error) and
+ *     never throws or aborts across the boundary.  `wick_rocm_last_error` gives
+ *     the message of the last failure on that context (thread-safe copy-out).
+ *   - Pointers named d_* are device pointers (HBM); all others are host pointers.
+ *   - The caller owns activation / output buffers; the library owns the context,
+ *     its stream and uploaded weights.
+ *   - All hot-path calls only ENQUEUE work on the context's stream (like encoding
+ *     into a Metal command encoder, wick/src/model/metal_lfm2.rs:1-4); nothing
+ *     synchronises except wick_rocm_sync / wick_rocm_download / event queries.
+ *   - Calls on one context serialise on an internal mutex, the counterpart of the
+ *     GPU models' `infer_lock` (wick/src/model/metal_lfm2.rs:254-267).
+ *   - Weight bytes keep the GGUF block layout verbatim (wick/src/quant.rs:13-34):
+ *     row-major, m rows of k/32 blocks; Q4_0 block = {f16 d; u8 qs[16]} (18 B),
+ *     Q8_0 block = {f16 d; i8 qs[32]} (34 B).  Nothing is repacked.
+ *   - Quantized activations use the reference's split layout
+ *     (wick/src/kv_cache.rs:103-106, wick/src/backend/simd.rs:683-685):
+ *     scales f32 [n][k/32] (values are f16-representable), quants i8 [n][k].
+ */
+#ifndef WICK_ROCM_H
+#define WICK_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum wick_rocm_status {
+    WICK_ROCM_OK = 0,
+    WICK_ROCM_ERR_INVALID_ARG = -1, /* null pointer, zero size, bad stride or alignment */
+    WICK_ROCM_ERR_UNSUPPORTED_DTYPE = -2, /* ggml type other than Q4_0 (2) / Q8_0 (8) */
+    WICK_ROCM_ERR_BAD_SHAPE = -3,   /* k % 32 != 0, byte count != m * (k/32) * block bytes */
+    WICK_ROCM_ERR_HIP = -4,         /* a HIP runtime call failed (message has the HIP error) */
+    WICK_ROCM_ERR_NO_DEVICE = -5,   /* no gfx950 device with that index */
+    WICK_ROCM_ERR_STATE = -6        /* capture begun twice, graph launched while capturing, ... */
+} wick_rocm_status;
+
+/* ggml tensor type ids, wick/src/gguf.rs:36-51 */
+enum { WICK_ROCM_TYPE_Q4_0 = 2, WICK_ROCM_TYPE_Q8_0 = 8 };
+
+/* Output layouts of the batched GEMM. */
+enum {
+    /* Y[col * y_stride + row]: the GPU call-site convention of encode_gemm,
+     * wick/src/model/metal_lfm2.rs:770-776, 881-992. */
+    WICK_ROCM_LAYOUT_TOKEN_MAJOR = 0,
+    /* out[row * y_stride + col] (y_stride >= n): the CPU kernels' convention,
+     * wick/src/backend/simd.rs:685, 696-704. */
+    WICK_ROCM_LAYOUT_ROW_MAJOR = 1
+};
+
+typedef struct wick_rocm_ctx wick_rocm_ctx;
+typedef struct wick_rocm_weight wick_rocm_weight;
+typedef struct wick_rocm_graph wick_rocm_graph;
+typedef struct wick_rocm_event wick_rocm_event;
+
+/* ---- context ------------------------------------------------------------
+ * Stands in for MetalContext::new / GpuContext::new
+ * (wick/src/backend/metal.rs:21-191, wick/src/backend/wgpu.rs:15-580): one
+ * device, one in-order queue (HIP stream at default priority). */
+int wick_rocm_device_count(int *count);
+int wick_rocm_ctx_create(int device_id, wick_rocm_ctx **out);
+void wick_rocm_ctx_destroy(wick_rocm_ctx *ctx);
+/* Copies the last error message of this context into buf (NUL-terminated). */
+int wick_rocm_last_error(wick_rocm_ctx *ctx, char *buf, size_t buf_len);
+/* "gfx950 ..." device name and CU count, for logs (wick-cli prints the backend label,
+ * wick-cli/src/main.rs:869-878). */
+int wick_rocm_device_info(wick_rocm_ctx *ctx, char *name_buf, size_t name_len, int *compute_units,
+                          size_t *hbm_bytes);
+/* The context's hipStream_t, as an opaque pointer, for interop with other HIP code. */
+void *wick_rocm_ctx_stream(wick_rocm_ctx *ctx);
+
+/* ---- device buffers (activation / output storage the caller owns) ---------
+ * Counterpart of MetalContext::create_buffer / read_f32 (wick/src/backend/metal.rs). */
+int wick_rocm_buffer_alloc(wick_rocm_ctx *ctx, size_t nbytes, void **d_ptr);
+int wick_rocm_buffer_free(wick_rocm_ctx *ctx, void *d_ptr);
+int wick_rocm_upload(wick_rocm_ctx *ctx, void *d_dst, const void *src, size_t nbytes);   /* H2D, ordered on the stream */
+int wick_rocm_download(wick_rocm_ctx *ctx, void *dst, const void *d_src, size_t nbytes); /* D2H, waits for the stream */
+int wick_rocm_sync(wick_rocm_ctx *ctx);
+
+/* ---- weights ----------------------------------------------------------------
+ * Stands in for MetalWeight {mmap_offset, dtype, m, k} (wick/src/model/metal_lfm2.rs:28-36,
+ * 409-421).  A discrete GPU cannot wrap the GGUF mmap in place, so the block
+ * bytes are copied once, verbatim, into HBM.  `nbytes` must equal
+ * m * (k/32) * block_bytes(ggml_type).  The handle stays valid until
+ * wick_rocm_weight_free or context destruction. */
+int wick_rocm_weight_upload(wick_rocm_ctx *ctx, const void *host_blocks, size_t nbytes, int ggml_type,
+                            uint32_t m, uint32_t k, wick_rocm_weight **out);
+int wick_rocm_weight_free(wick_rocm_ctx *ctx, wick_rocm_weight *w);
+int wick_rocm_weight_info(const wick_rocm_weight *w, int *ggml_type, uint32_t *m, uint32_t *k, size_t *nbytes);
+const void *wick_rocm_weight_device_ptr(const wick_rocm_weight *w);
+
+/* ---- Q8_0 activation quantizer ------------------------------------------
+ * quantize_f32_to_q8_0_neon (wick/src/backend/simd.rs:255-323; wrapper
+ * wick/src/backend/cpu.rs:315-328) applied to n columns, as quantize_to_scratch /
+ * quantize_columns do (wick/src/model/lfm2.rs:571-612).  Column j is read from
+ * d_x[j * x_stride + 0..k) (token-major f32, x_stride >= k).  Writes
+ * d_scales[j * (k/32) + b] and d_quants[j * k + i].  Bit-exact with the
+ * reference: d = amax/127, id = 1/d from the unrounded d, stored scale =
+ * f32(f16(d)), q = (i8) round-ties-even(x * id). */
+int wick_rocm_quantize_q8_0(wick_rocm_ctx *ctx, const float *d_x, uint32_t n, uint32_t k, uint32_t x_stride,
+                            int8_t *d_quants, float *d_scales);
+
+/* ---- decode GEMV (n = 1) ----------------------------------------------------
+ * gemv_with_preq (wick/src/backend/cpu.rs:334-354) -> gemv_q4_0_q8_0_neon /
+ * gemv_q8_0_q8_0_neon (wick/src/backend/simd.rs:328-415, 440-524):
+ *   y[i] (+)= sum_b f32(isum_{i,b}) * (f32(d_w[i,b]) * x_scales[b]).
+ * `accumulate` != 0 gives y += W x, the residual form of
+ * encode_gemv_weight_accumulate (wick/src/model/metal_lfm2.rs:702-710). */
+int wick_rocm_gemv_q8(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_t *d_quants, const float *d_scales,
+                      float *d_y, int accumulate);
+
+/* Several weights against ONE quantized activation in a single launch: the
+ * shared-quantization groups of the decode step ({Q,K,V}, {gate,up};
+ * wick/src/model/lfm2.rs:752-775, 1053-1067; fused Metal forms
+ * wick/src/model/metal_lfm2.rs:1043-1119).  All weights must share k and dtype. */
+int wick_rocm_gemv_q8_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *ws, float *const *d_ys, uint32_t count,
+                            const int8_t *d_quants, const float *d_scales, int accumulate);
+
+/* ---- batched prefill GEMM -----------------------------------------------
+ * gemm_q4_0_q8_0_neon / gemm_q8_0_q8_0_neon (wick/src/backend/simd.rs:696-925,
+ * 937-1019; caller gemm_preq, wick/src/model/lfm2.rs:539-565):
+ *   C[i,j] (+)= sum_b f32(isum_{i,j,b}) * (f32(d_w[i,b]) * scales[j*nb + b]).
+ * Written as Y[j * y_stride + i] (TOKEN_MAJOR, y_stride >= m) or
+ * out[i * y_stride + j] (ROW_MAJOR, y_stride >= n).  Any n >= 1; small n takes the
+ * bandwidth-bound multi-token GEMV, larger n the int8-MFMA kernel (the hand-off
+ * mirrors GEMM_MIN_N, wick/src/model/metal_lfm2.rs:18-21, 899-927). */
+int wick_rocm_gemm_q8(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_t *d_quants, const float *d_scales,
+                      uint32_t n, float *d_y, uint32_t y_stride, int y_layout, int accumulate);
+
+/* ---- the literal call-site shape ---------------------------------------
+ * encode_gemm(w, x, x_off_bytes, y, y_off_bytes, n, x_stride, y_stride, accumulate)
+ * and, with n = 1, encode_gemv_impl(w, input, input_off, output, output_off, accumulate)
+ * (wick/src/model/metal_lfm2.rs:881-992, 1231-1335): X[col*x_stride + i] f32 in,
+ * Y[col*y_stride + row] f32 out.  Quantizes the n columns into context-owned
+ * scratch (grown on demand, never inside a graph capture) and runs GEMV or GEMM.
+ * Offsets are in bytes like the reference's. */
+int wick_rocm_matmul_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const float *d_x, size_t x_off_bytes, uint32_t n,
+                         uint32_t x_stride, float *d_y, size_t y_off_bytes, uint32_t y_stride, int accumulate);
+/* Pre-sizes the scratch used by wick_rocm_matmul_f32 for up to max_n columns of
+ * up to max_k elements (call before capturing a graph). */
+int wick_rocm_reserve_scratch(wick_rocm_ctx *ctx, uint32_t max_n, uint32_t max_k);
+
+/* ---- parity hook ----------------------------------------------------------
+ * The exact per-block i32 dots the kernels scale and accumulate
+ * (wick/src/backend/simd.rs:369-383, 478-492): d_out[(j*m + i)*(k/32) + b]. */
+int wick_rocm_block_dots_i32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_t *d_quants, uint32_t n,
+                             int32_t *d_out);
+
+/* ---- one submission per token -------------------------------------------
+ * The reference's GPU backends encode a whole token into one command buffer and
+ * commit once (wick/src/model/metal_lfm2.rs:1-4).  The HIP counterpart is stream
+ * capture into a graph: begin, enqueue any hot-path calls, end, then launch the
+ * graph as often as needed. */
+int wick_rocm_graph_begin(wick_rocm_ctx *ctx);
+int wick_rocm_graph_end(wick_rocm_ctx *ctx, wick_rocm_graph **out);
+int wick_rocm_graph_launch(wick_rocm_ctx *ctx, wick_rocm_graph *g);
+int wick_rocm_graph_destroy(wick_rocm_ctx *ctx, wick_rocm_graph *g);
+
+/* ---- GPU timestamps -----------------------------------------------------
+ * Counterpart of the reference's GpuTimer (MTLCounterSampleBuffer timestamps,
+ * wick/src/model/metal_lfm2.rs:3367-4116): events recorded on the context's stream. */
+int wick_rocm_event_create(wick_rocm_ctx *ctx, wick_rocm_event **out);
+int wick_rocm_event_record(wick_rocm_ctx *ctx, wick_rocm_event *e);
+int wick_rocm_event_elapsed_ms(wick_rocm_ctx *ctx, wick_rocm_event *start, wick_rocm_event *stop, float *ms); /* waits for stop */
+int wick_rocm_event_destroy(wick_rocm_ctx *ctx, wick_rocm_event *e);
+
+/* Library version string, e.g. "wick-rocm 0.1 (gfx950)". */
+const char *wick_rocm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WICK_ROCM_H */

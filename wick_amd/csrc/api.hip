@@ -1,0 +1,469 @@
+// C ABI of the gfx950 backend (see include/wick_rocm.h for the contract and the
+// reference interfaces each entry point stands in for).  Host code only: argument
+// validation, ownership, stream / graph / event plumbing, kernel routing.
+#include "../../include/wick_rocm.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+
+#include "wick_rocm_internal.h"
+
+using namespace wick_rocm;
+
+struct wick_rocm_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::mutex mu;  // serialises calls on this context, like the reference's infer_lock
+    std::string err;
+    std::string name;
+    int num_cus = 0;
+    size_t hbm_bytes = 0;
+    bool capturing = false;
+    // scratch for wick_rocm_matmul_f32 (quantized activations)
+    int8_t* scratch_q = nullptr;
+    float* scratch_s = nullptr;
+    size_t scratch_q_cap = 0;  // bytes
+    size_t scratch_s_cap = 0;  // floats
+};
+
+struct wick_rocm_weight {
+    void* d = nullptr;
+    size_t nbytes = 0;
+    int type = 0;
+    uint32_t m = 0, k = 0;
+};
+
+struct wick_rocm_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+struct wick_rocm_event {
+    hipEvent_t ev = nullptr;
+};
+
+namespace {
+
+int fail(wick_rocm_ctx* ctx, int code, const char* what) {
+    if (ctx) ctx->err = what;
+    return code;
+}
+
+int fail_hip(wick_rocm_ctx* ctx, hipError_t e, const char* where) {
+    if (ctx) {
+        ctx->err = std::string(where) + ": " + hipGetErrorString(e);
+    }
+    return WICK_ROCM_ERR_HIP;
+}
+
+#define WR_HIP(ctx, call)                                      \
+    do {                                                       \
+        hipError_t e_ = (call);                                \
+        if (e_ != hipSuccess) return fail_hip(ctx, e_, #call); \
+    } while (0)
+
+// Takes the context lock and makes its device current for the calling thread.
+struct Guard {
+    std::unique_lock<std::mutex> lk;
+    hipError_t status;
+    explicit Guard(wick_rocm_ctx* ctx) : lk(ctx->mu), status(hipSetDevice(ctx->device)) {}
+};
+
+#define WR_ENTER(ctx)                                                   \
+    if (!(ctx)) return WICK_ROCM_ERR_INVALID_ARG;                       \
+    Guard guard_(ctx);                                                  \
+    if (guard_.status != hipSuccess) return fail_hip(ctx, guard_.status, "hipSetDevice")
+
+int check_weight(wick_rocm_ctx* ctx, const wick_rocm_weight* w) {
+    if (!w || !w->d) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "null weight handle");
+    return WICK_ROCM_OK;
+}
+
+int ensure_scratch(wick_rocm_ctx* ctx, size_t q_bytes, size_t s_floats) {
+    if (q_bytes <= ctx->scratch_q_cap && s_floats <= ctx->scratch_s_cap) return WICK_ROCM_OK;
+    if (ctx->capturing)
+        return fail(ctx, WICK_ROCM_ERR_STATE, "activation scratch too small during graph capture; call wick_rocm_reserve_scratch first");
+    WR_HIP(ctx, hipStreamSynchronize(ctx->stream));  // earlier launches may still read the old scratch
+    if (q_bytes > ctx->scratch_q_cap) {
+        if (ctx->scratch_q) WR_HIP(ctx, hipFree(ctx->scratch_q));
+        ctx->scratch_q = nullptr, ctx->scratch_q_cap = 0;
+        WR_HIP(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->scratch_q), q_bytes));
+        ctx->scratch_q_cap = q_bytes;
+    }
+    if (s_floats > ctx->scratch_s_cap) {
+        if (ctx->scratch_s) WR_HIP(ctx, hipFree(ctx->scratch_s));
+        ctx->scratch_s = nullptr, ctx->scratch_s_cap = 0;
+        WR_HIP(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->scratch_s), s_floats * sizeof(float)));
+        ctx->scratch_s_cap = s_floats;
+    }
+    return WICK_ROCM_OK;
+}
+
+// Routing shared by wick_rocm_gemm_q8 and wick_rocm_matmul_f32 (lock already held).
+int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q, const float* d_s, uint32_t n,
+                float* d_y, uint32_t y_stride, int y_layout, int accumulate) {
+    if (!d_q || !d_s || !d_y) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "null device pointer");
+    if (n == 0) return WICK_ROCM_OK;
+    if (y_layout != WICK_ROCM_LAYOUT_TOKEN_MAJOR && y_layout != WICK_ROCM_LAYOUT_ROW_MAJOR)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "unknown output layout");
+    if (y_layout == WICK_ROCM_LAYOUT_TOKEN_MAJOR ? (y_stride < w->m && n > 1) : (y_stride < n))
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "y_stride smaller than the output extent");
+    const bool mfma_ok = (w->k % 256u == 0) && (reinterpret_cast<uintptr_t>(d_q) % 16u == 0) &&
+                         (reinterpret_cast<uintptr_t>(d_s) % 16u == 0);
+    hipError_t e;
+    if (n >= kGemmMinN && mfma_ok)
+        e = launch_gemm_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
+                             y_layout, accumulate, ctx->stream);
+    else
+        e = launch_gemv_tokens(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
+                               y_layout, accumulate, ctx->num_cus, ctx->stream);
+    if (e != hipSuccess) return fail_hip(ctx, e, "gemm launch");
+    return WICK_ROCM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* wick_rocm_version(void) { return "wick-rocm 0.1 (gfx950)"; }
+
+int wick_rocm_device_count(int* count) {
+    if (!count) return WICK_ROCM_ERR_INVALID_ARG;
+    int c = 0;
+    hipError_t e = hipGetDeviceCount(&c);
+    if (e != hipSuccess) {
+        *count = 0;
+        return e == hipErrorNoDevice ? WICK_ROCM_OK : WICK_ROCM_ERR_HIP;
+    }
+    *count = c;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_ctx_create(int device_id, wick_rocm_ctx** out) {
+    if (!out) return WICK_ROCM_ERR_INVALID_ARG;
+    *out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || device_id < 0 || device_id >= count) return WICK_ROCM_ERR_NO_DEVICE;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device_id) != hipSuccess) return WICK_ROCM_ERR_HIP;
+    // The kernels are built for gfx950 only; refuse anything else up front instead
+    // of failing at the first launch.
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) return WICK_ROCM_ERR_NO_DEVICE;
+    wick_rocm_ctx* ctx = new (std::nothrow) wick_rocm_ctx();
+    if (!ctx) return WICK_ROCM_ERR_HIP;
+    ctx->device = device_id;
+    ctx->name = std::string(prop.gcnArchName) + " " + prop.name;
+    ctx->num_cus = prop.multiProcessorCount;
+    ctx->hbm_bytes = prop.totalGlobalMem;
+    if (hipSetDevice(device_id) != hipSuccess || hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
+        delete ctx;
+        return WICK_ROCM_ERR_HIP;
+    }
+    *out = ctx;
+    return WICK_ROCM_OK;
+}
+
+void wick_rocm_ctx_destroy(wick_rocm_ctx* ctx) {
+    if (!ctx) return;
+    {
+        Guard g(ctx);
+        if (ctx->stream) {
+            (void)hipStreamSynchronize(ctx->stream);
+            (void)hipStreamDestroy(ctx->stream);
+        }
+        if (ctx->scratch_q) (void)hipFree(ctx->scratch_q);
+        if (ctx->scratch_s) (void)hipFree(ctx->scratch_s);
+    }
+    delete ctx;
+}
+
+int wick_rocm_last_error(wick_rocm_ctx* ctx, char* buf, size_t buf_len) {
+    if (!ctx || !buf || buf_len == 0) return WICK_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    std::snprintf(buf, buf_len, "%s", ctx->err.c_str());
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_device_info(wick_rocm_ctx* ctx, char* name_buf, size_t name_len, int* compute_units, size_t* hbm_bytes) {
+    if (!ctx) return WICK_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    if (name_buf && name_len) std::snprintf(name_buf, name_len, "%s", ctx->name.c_str());
+    if (compute_units) *compute_units = ctx->num_cus;
+    if (hbm_bytes) *hbm_bytes = ctx->hbm_bytes;
+    return WICK_ROCM_OK;
+}
+
+void* wick_rocm_ctx_stream(wick_rocm_ctx* ctx) { return ctx ? static_cast<void*>(ctx->stream) : nullptr; }
+
+int wick_rocm_buffer_alloc(wick_rocm_ctx* ctx, size_t nbytes, void** d_ptr) {
+    WR_ENTER(ctx);
+    if (!d_ptr || nbytes == 0) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "buffer_alloc: null out pointer or zero size");
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "buffer_alloc during graph capture");
+    *d_ptr = nullptr;
+    WR_HIP(ctx, hipMalloc(d_ptr, nbytes));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_buffer_free(wick_rocm_ctx* ctx, void* d_ptr) {
+    WR_ENTER(ctx);
+    if (!d_ptr) return WICK_ROCM_OK;
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "buffer_free during graph capture");
+    WR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    WR_HIP(ctx, hipFree(d_ptr));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_upload(wick_rocm_ctx* ctx, void* d_dst, const void* src, size_t nbytes) {
+    WR_ENTER(ctx);
+    if (nbytes == 0) return WICK_ROCM_OK;
+    if (!d_dst || !src) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "upload: null pointer");
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "upload during graph capture");
+    WR_HIP(ctx, hipMemcpyAsync(d_dst, src, nbytes, hipMemcpyHostToDevice, ctx->stream));
+    WR_HIP(ctx, hipStreamSynchronize(ctx->stream));  // the host buffer may be reused on return
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_download(wick_rocm_ctx* ctx, void* dst, const void* d_src, size_t nbytes) {
+    WR_ENTER(ctx);
+    if (nbytes == 0) return WICK_ROCM_OK;
+    if (!dst || !d_src) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "download: null pointer");
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "download during graph capture");
+    WR_HIP(ctx, hipMemcpyAsync(dst, d_src, nbytes, hipMemcpyDeviceToHost, ctx->stream));
+    WR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_sync(wick_rocm_ctx* ctx) {
+    WR_ENTER(ctx);
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "sync during graph capture");
+    WR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_weight_upload(wick_rocm_ctx* ctx, const void* host_blocks, size_t nbytes, int ggml_type, uint32_t m,
+                            uint32_t k, wick_rocm_weight** out) {
+    WR_ENTER(ctx);
+    if (!out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "weight_upload: null out pointer");
+    *out = nullptr;
+    if (!host_blocks) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "weight_upload: null host pointer");
+    const int bb = block_bytes(ggml_type);
+    if (bb == 0) return fail(ctx, WICK_ROCM_ERR_UNSUPPORTED_DTYPE, "weight_upload: only Q4_0 (2) and Q8_0 (8) are supported");
+    if (m == 0 || k == 0 || k % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "weight_upload: m, k must be > 0 and k % 32 == 0");
+    if (nbytes != (size_t)m * (k / 32u) * (size_t)bb)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "weight_upload: nbytes != m * (k/32) * block_bytes");
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "weight_upload during graph capture");
+    wick_rocm_weight* w = new (std::nothrow) wick_rocm_weight();
+    if (!w) return fail(ctx, WICK_ROCM_ERR_HIP, "out of host memory");
+    hipError_t e = hipMalloc(&w->d, nbytes);
+    if (e == hipSuccess) e = hipMemcpyAsync(w->d, host_blocks, nbytes, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        if (w->d) (void)hipFree(w->d);
+        delete w;
+        return fail_hip(ctx, e, "weight_upload");
+    }
+    w->nbytes = nbytes, w->type = ggml_type, w->m = m, w->k = k;
+    *out = w;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_weight_free(wick_rocm_ctx* ctx, wick_rocm_weight* w) {
+    WR_ENTER(ctx);
+    if (!w) return WICK_ROCM_OK;
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "weight_free during graph capture");
+    WR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (w->d) WR_HIP(ctx, hipFree(w->d));
+    delete w;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_weight_info(const wick_rocm_weight* w, int* ggml_type, uint32_t* m, uint32_t* k, size_t* nbytes) {
+    if (!w) return WICK_ROCM_ERR_INVALID_ARG;
+    if (ggml_type) *ggml_type = w->type;
+    if (m) *m = w->m;
+    if (k) *k = w->k;
+    if (nbytes) *nbytes = w->nbytes;
+    return WICK_ROCM_OK;
+}
+
+const void* wick_rocm_weight_device_ptr(const wick_rocm_weight* w) { return w ? w->d : nullptr; }
+
+int wick_rocm_quantize_q8_0(wick_rocm_ctx* ctx, const float* d_x, uint32_t n, uint32_t k, uint32_t x_stride,
+                            int8_t* d_quants, float* d_scales) {
+    WR_ENTER(ctx);
+    if (n == 0) return WICK_ROCM_OK;
+    if (!d_x || !d_quants || !d_scales) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "quantize_q8_0: null device pointer");
+    if (k == 0 || k % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "quantize_q8_0: k % 32 != 0");
+    if (x_stride < k && n > 1) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "quantize_q8_0: x_stride < k");
+    if (reinterpret_cast<uintptr_t>(d_x) % 4u || reinterpret_cast<uintptr_t>(d_quants) % 4u ||
+        reinterpret_cast<uintptr_t>(d_scales) % 4u)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "quantize_q8_0: pointers must be 4-byte aligned");
+    hipError_t e = launch_quantize_q8_0(d_x, n, k, x_stride, d_quants, d_scales, ctx->stream);
+    if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_gemv_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count,
+                            const int8_t* d_quants, const float* d_scales, int accumulate) {
+    WR_ENTER(ctx);
+    if (!ws || !d_ys || !d_quants || !d_scales) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv: null pointer");
+    if (count == 0 || count > (uint32_t)kMaxGemvBatch)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv_q8_multi: count must be 1..4");
+    GemvBatch b{};
+    uint32_t rows = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        if (int rc = check_weight(ctx, ws[i])) return rc;
+        if (!d_ys[i]) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv: null output pointer");
+        if (ws[i]->k != ws[0]->k || ws[i]->type != ws[0]->type)
+            return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "gemv_q8_multi: weights must share k and dtype");
+        if ((uint64_t)rows + ws[i]->m > 0xffffffffull) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "gemv_q8_multi: too many rows");
+        rows += ws[i]->m;
+        b.w[i] = static_cast<const uint8_t*>(ws[i]->d);
+        b.y[i] = d_ys[i];
+        b.row_end[i] = rows;
+    }
+    b.count = count;
+    hipError_t e = launch_gemv(ws[0]->type, b, ws[0]->k, d_quants, d_scales, accumulate, ctx->num_cus, ctx->stream);
+    if (e != hipSuccess) return fail_hip(ctx, e, "gemv launch");
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_gemv_q8(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_quants, const float* d_scales,
+                      float* d_y, int accumulate) {
+    const wick_rocm_weight* ws[1] = {w};
+    float* ys[1] = {d_y};
+    return wick_rocm_gemv_q8_multi(ctx, ws, ys, 1, d_quants, d_scales, accumulate);
+}
+
+int wick_rocm_gemm_q8(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_quants, const float* d_scales,
+                      uint32_t n, float* d_y, uint32_t y_stride, int y_layout, int accumulate) {
+    WR_ENTER(ctx);
+    if (int rc = check_weight(ctx, w)) return rc;
+    return gemm_locked(ctx, w, d_quants, d_scales, n, d_y, y_stride, y_layout, accumulate);
+}
+
+int wick_rocm_reserve_scratch(wick_rocm_ctx* ctx, uint32_t max_n, uint32_t max_k) {
+    WR_ENTER(ctx);
+    if (max_k % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "reserve_scratch: max_k % 32 != 0");
+    return ensure_scratch(ctx, (size_t)max_n * max_k, (size_t)max_n * (max_k / 32u));
+}
+
+int wick_rocm_matmul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const float* d_x, size_t x_off_bytes, uint32_t n,
+                         uint32_t x_stride, float* d_y, size_t y_off_bytes, uint32_t y_stride, int accumulate) {
+    WR_ENTER(ctx);
+    if (int rc = check_weight(ctx, w)) return rc;
+    if (!d_x || !d_y) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "matmul_f32: null device pointer");
+    if (n == 0) return WICK_ROCM_OK;
+    if (x_off_bytes % 4u || y_off_bytes % 4u) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "matmul_f32: offsets must be multiples of 4");
+    if (n > 1 && (x_stride < w->k || y_stride < w->m))
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "matmul_f32: stride smaller than the vector length");
+    const float* x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes);
+    float* y = reinterpret_cast<float*>(reinterpret_cast<char*>(d_y) + y_off_bytes);
+    if (int rc = ensure_scratch(ctx, (size_t)n * w->k, (size_t)n * (w->k / 32u))) return rc;
+    hipError_t e = launch_quantize_q8_0(x, n, w->k, x_stride, ctx->scratch_q, ctx->scratch_s, ctx->stream);
+    if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
+    return gemm_locked(ctx, w, ctx->scratch_q, ctx->scratch_s, n, y, n == 1 ? w->m : y_stride,
+                       WICK_ROCM_LAYOUT_TOKEN_MAJOR, accumulate);
+}
+
+int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_quants, uint32_t n,
+                             int32_t* d_out) {
+    WR_ENTER(ctx);
+    if (int rc = check_weight(ctx, w)) return rc;
+    if (!d_quants || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "block_dots: null device pointer");
+    if (n == 0) return WICK_ROCM_OK;
+    const bool mfma = n >= kGemmMinN && (w->k % 256u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
+    hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->stream)
+                        : launch_block_dots_dot4(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->stream);
+    if (e != hipSuccess) return fail_hip(ctx, e, "block_dots launch");
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_graph_begin(wick_rocm_ctx* ctx) {
+    WR_ENTER(ctx);
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "graph_begin: capture already in progress");
+    WR_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_graph_end(wick_rocm_ctx* ctx, wick_rocm_graph** out) {
+    WR_ENTER(ctx);
+    if (!out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "graph_end: null out pointer");
+    *out = nullptr;
+    if (!ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "graph_end: no capture in progress");
+    ctx->capturing = false;
+    wick_rocm_graph* g = new (std::nothrow) wick_rocm_graph();
+    if (!g) return fail(ctx, WICK_ROCM_ERR_HIP, "out of host memory");
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
+    if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        delete g;
+        return fail_hip(ctx, e, "graph_end");
+    }
+    *out = g;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_graph_launch(wick_rocm_ctx* ctx, wick_rocm_graph* g) {
+    WR_ENTER(ctx);
+    if (!g || !g->exec) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "graph_launch: null graph");
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "graph_launch during capture");
+    WR_HIP(ctx, hipGraphLaunch(g->exec, ctx->stream));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_graph_destroy(wick_rocm_ctx* ctx, wick_rocm_graph* g) {
+    WR_ENTER(ctx);
+    if (!g) return WICK_ROCM_OK;
+    WR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_event_create(wick_rocm_ctx* ctx, wick_rocm_event** out) {
+    WR_ENTER(ctx);
+    if (!out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "event_create: null out pointer");
+    wick_rocm_event* e = new (std::nothrow) wick_rocm_event();
+    if (!e) return fail(ctx, WICK_ROCM_ERR_HIP, "out of host memory");
+    hipError_t he = hipEventCreate(&e->ev);
+    if (he != hipSuccess) {
+        delete e;
+        return fail_hip(ctx, he, "hipEventCreate");
+    }
+    *out = e;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_event_record(wick_rocm_ctx* ctx, wick_rocm_event* e) {
+    WR_ENTER(ctx);
+    if (!e) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "event_record: null event");
+    WR_HIP(ctx, hipEventRecord(e->ev, ctx->stream));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_event_elapsed_ms(wick_rocm_ctx* ctx, wick_rocm_event* start, wick_rocm_event* stop, float* ms) {
+    WR_ENTER(ctx);
+    if (!start || !stop || !ms) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "event_elapsed_ms: null argument");
+    WR_HIP(ctx, hipEventSynchronize(stop->ev));
+    WR_HIP(ctx, hipEventElapsedTime(ms, start->ev, stop->ev));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_event_destroy(wick_rocm_ctx* ctx, wick_rocm_event* e) {
+    WR_ENTER(ctx);
+    if (!e) return WICK_ROCM_OK;
+    (void)hipEventDestroy(e->ev);
+    delete e;
+    return WICK_ROCM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,331 @@
+// Batched prefill GEMM: raw GGUF Q4_0 / Q8_0 weight blocks x Q8_0-quantized
+// activations -> f32, on the gfx950 int8 matrix cores.
+//
+// Arithmetic: gemm_q4_0_q8_0_neon / gemm_q8_0_q8_0_neon
+// (wick/src/backend/simd.rs:696-925, 937-1019):
+//   C[i,j] = sum_b f32(isum_{i,j,b}) * (f32(f16 d_w[i,b]) * xs[j,b]),  isum exact i32
+// with one scale pair per 32-element block, so i32 accumulation cannot run across
+// blocks: every v_mfma_i32_32x32x32_i8 covers exactly one block (K = 32) and its
+// 32x32 i32 result is scaled into f32 accumulators on the vector ALU.
+//
+// Workgroup = 256 threads = 4 waves, tile = 128 weight rows x 128 tokens, each
+// wave owns 64 x 64 (2 x 2 MFMA tiles).  One stage = 8 blocks (256 elements of K):
+//   * weights: each thread reads two 36/68-byte block pairs with dword-aligned
+//     wide loads (a row contributes 144/272 contiguous bytes per stage), unpacks
+//     nibbles to int8 and writes 16-byte operand rows to LDS;
+//   * activations: 16-byte chunks copied global -> LDS; scales alongside.
+// Global loads of stage s+1 are in flight (held in registers) while stage s is
+// computed from LDS.
+//
+// LDS operand layout: [block][khalf][row][16 bytes] (planes ordered the other
+// way round for weights; see Smem).  An MFMA lane supplies 16
+// consecutive K-bytes of one operand row, lanes 0-31 the first half of the block
+// and lanes 32-63 the second, so 32 consecutive lanes read 512 consecutive bytes:
+// conflict-free without padding.  For Q4_0 the low nibbles of a block ARE its
+// first 16 elements and the high nibbles its last 16 (wick/src/quant.rs:82-88),
+// so the two halves fall out of one and / shift each.
+//
+// Roles: tokens are the MFMA "A" (M) operand, weight rows the "B" (N) operand, so
+// in the 32x32 result a lane holds ONE weight row (n = lane % 32) and 16 tokens
+// (m = 8*(r/4) + 4*(lane/32) + r%4).  Its weight scale is one register per block;
+// the 16 token scales are LDS broadcast reads.
+//
+// Scaling cost is what bounds this kernel (vector ALU, not the matrix core), so it
+// is cut to two FMAs per result:
+//   * Q4_0 nibbles are stored as 16*(nibble-8) (the nibble moved to the top of the
+//     byte, sign bit flipped: two ALU ops per four weights, no per-byte subtract);
+//     the 1/16 is folded into the weight scale.
+//   * The MFMA accumulates onto C = 0x4B400000 in every lane, i.e. the bit pattern
+//     of 12582912.0f = 1.5 * 2^23.  Integer-adding v (|v| < 2^22) to that pattern
+//     gives exactly the f32 12582912 + v, so the i32 -> f32 conversion is free.
+//   * t = fma(D_as_f32, dw, -12582912*dw) = round(v * dw) exactly (single rounding;
+//     12582912*dw is exact because dw has an 11-bit significand);
+//     acc = fma(t, dx, acc).
+#include "wick_rocm_device.h"
+#include "wick_rocm_internal.h"
+
+namespace wick_rocm {
+
+namespace {
+
+constexpr int BM = 128;       // weight rows per workgroup
+constexpr int BN = 128;       // tokens per workgroup
+constexpr int KB = 8;         // blocks per stage
+constexpr int THREADS = 256;  // 4 waves: 2 (rows) x 2 (tokens)
+constexpr uint32_t kBiasBits = 0x4B400000u;  // 12582912.0f
+constexpr float kBias = 12582912.0f;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+struct GemmArgs {
+    const uint8_t* w;
+    const int8_t* xq;
+    const float* xs;
+    float* y;
+    int32_t* dots;  // parity hook output (DUMP only)
+    uint32_t m, n, k;
+    uint32_t y_stride;
+    uint32_t row_tiles, tok_tiles;
+    int y_row_major;
+    int accumulate;
+};
+
+// Row counts are padded (one 16-byte operand row per plane, four floats per scale
+// row) so that the stage WRITES, where neighbouring lanes hit different planes of
+// the same row, spread over the LDS banks; reads walk consecutive rows of one
+// plane and do not care.
+struct Smem {
+    uint4 wt[2][KB][BM + 1];  // [khalf][block][row]: int8 operand rows, 16 bytes each
+    uint4 xt[KB][2][BN + 1];  // [block][khalf][token]
+    float dw[KB][BM + 4];   // weight scale (x 1/16 for Q4_0)
+    float ndw[KB][BM + 4];  // -12582912 * dw
+    float dx[KB][BN + 4];   // activation scale
+};
+
+// 16*(nibble-8) for the four low / four high nibbles of each byte of q.
+__device__ __forceinline__ uint32_t q4_lo_x16(uint32_t q) { return ((q << 4) & 0xf0f0f0f0u) ^ 0x80808080u; }
+__device__ __forceinline__ uint32_t q4_hi_x16(uint32_t q) { return (q & 0xf0f0f0f0u) ^ 0x80808080u; }
+
+template <int TYPE>
+struct StageRegs {
+    uint32_t w[2][PairTraits<TYPE>::DWORDS];
+    uint4 x[8];
+    float4 dx;
+};
+
+template <int TYPE>
+__device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uint32_t tok0, uint32_t kb0,
+                                           StageRegs<TYPE>& r) {
+    using PT = PairTraits<TYPE>;
+    const uint32_t t = threadIdx.x;
+    const uint32_t nb = a.k >> 5;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const uint32_t id = t + i * THREADS;  // 512 pairs: 128 rows x 4 pairs
+        const uint32_t row = min(row0 + (id >> 2), a.m - 1);
+        const uint32_t pr = id & 3u;
+        const uint8_t* p = a.w + ((size_t)row * nb + kb0 + 2 * pr) * (PT::BYTES / 2);
+        load_pair<PT::DWORDS>(p, r.w[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t id = t + i * THREADS;  // 2048 chunks: 128 tokens x 16 chunks of 16 B
+        const uint32_t tok = min(tok0 + (id >> 4), a.n - 1);
+        const uint32_t c = id & 15u;
+        r.x[i] = *reinterpret_cast<const uint4*>(a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + c * 16);
+    }
+    if (a.xs) {  // null only for the parity hook, which never scales
+        const uint32_t tok = min(tok0 + (t >> 1), a.n - 1);
+        r.dx = *reinterpret_cast<const float4*>(a.xs + (size_t)tok * nb + kb0 + (t & 1u) * 4);
+    } else {
+        r.dx = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+
+template <int TYPE>
+__device__ __forceinline__ void store_stage(Smem& s, const StageRegs<TYPE>& r) {
+    using PT = PairTraits<TYPE>;
+    const uint32_t t = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const uint32_t id = t + i * THREADS;
+        const uint32_t row = id >> 2;
+        const uint32_t pr = id & 3u;
+        uint32_t d0, d1, q0[PT::NQ], q1[PT::NQ];
+        split_pair<TYPE>(r.w[i], d0, d1, q0, q1);
+        const float scale = (TYPE == 2) ? 0.0625f : 1.0f;
+        const float dw0 = f16_bits_to_f32(d0) * scale, dw1 = f16_bits_to_f32(d1) * scale;
+        s.dw[2 * pr][row] = dw0;
+        s.dw[2 * pr + 1][row] = dw1;
+        s.ndw[2 * pr][row] = -kBias * dw0;
+        s.ndw[2 * pr + 1][row] = -kBias * dw1;
+        if constexpr (TYPE == 2) {
+            s.wt[0][2 * pr][row] = make_uint4(q4_lo_x16(q0[0]), q4_lo_x16(q0[1]), q4_lo_x16(q0[2]), q4_lo_x16(q0[3]));
+            s.wt[1][2 * pr][row] = make_uint4(q4_hi_x16(q0[0]), q4_hi_x16(q0[1]), q4_hi_x16(q0[2]), q4_hi_x16(q0[3]));
+            s.wt[0][2 * pr + 1][row] = make_uint4(q4_lo_x16(q1[0]), q4_lo_x16(q1[1]), q4_lo_x16(q1[2]), q4_lo_x16(q1[3]));
+            s.wt[1][2 * pr + 1][row] = make_uint4(q4_hi_x16(q1[0]), q4_hi_x16(q1[1]), q4_hi_x16(q1[2]), q4_hi_x16(q1[3]));
+        } else {
+            s.wt[0][2 * pr][row] = make_uint4(q0[0], q0[1], q0[2], q0[3]);
+            s.wt[1][2 * pr][row] = make_uint4(q0[4], q0[5], q0[6], q0[7]);
+            s.wt[0][2 * pr + 1][row] = make_uint4(q1[0], q1[1], q1[2], q1[3]);
+            s.wt[1][2 * pr + 1][row] = make_uint4(q1[4], q1[5], q1[6], q1[7]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t id = t + i * THREADS;
+        const uint32_t tok = id >> 4;
+        const uint32_t c = id & 15u;
+        s.xt[c >> 1][c & 1u][tok] = r.x[i];
+    }
+    {
+        const uint32_t tok = t >> 1;
+        const uint32_t b4 = (t & 1u) * 4;
+        s.dx[b4 + 0][tok] = r.dx.x;
+        s.dx[b4 + 1][tok] = r.dx.y;
+        s.dx[b4 + 2][tok] = r.dx.z;
+        s.dx[b4 + 3][tok] = r.dx.w;
+    }
+}
+
+// Workgroup -> tile, XCD-aware: hardware hands consecutive workgroup ids to the 8
+// XCDs round-robin, so ids with equal (id % 8) share an L2.  Each XCD gets a
+// contiguous run of tiles; within a run the token tile varies fastest, so the
+// workgroups resident on one XCD share weight-row panels in that L2.
+__device__ __forceinline__ uint32_t tile_of_block(uint32_t bid, uint32_t tiles) {
+    const uint32_t per_xcd = (tiles + 7u) / 8u;
+    return (bid & 7u) * per_xcd + (bid >> 3);
+}
+
+template <int TYPE, bool DUMP>
+__global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
+    __shared__ Smem s;
+    const uint32_t tiles = a.row_tiles * a.tok_tiles;
+    const uint32_t tile = tile_of_block(blockIdx.x, tiles);
+    if (tile >= tiles) return;  // whole workgroup leaves together
+    const uint32_t row0 = (tile / a.tok_tiles) * BM;
+    const uint32_t tok0 = (tile % a.tok_tiles) * BN;
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t l32 = lane & 31u;
+    const uint32_t g = lane >> 5;            // which 16-byte half of the block this lane feeds
+    const uint32_t wrow0 = (wave >> 1) * 64;  // wave's rows within the tile
+    const uint32_t wtok0 = (wave & 1u) * 64;
+    const uint32_t nb = a.k >> 5;
+    const uint32_t stages = nb / KB;
+
+    float acc[2][2][16];
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+        for (int rt = 0; rt < 2; rt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[tt][rt][r] = 0.0f;
+
+    v16i cbias;
+#pragma unroll
+    for (int r = 0; r < 16; r++) cbias[r] = (int)kBiasBits;
+
+    StageRegs<TYPE> regs;
+    load_stage<TYPE>(a, row0, tok0, 0, regs);
+    store_stage<TYPE>(s, regs);
+    __syncthreads();
+
+    for (uint32_t st = 0; st < stages; st++) {
+        if (st + 1 < stages) load_stage<TYPE>(a, row0, tok0, (st + 1) * KB, regs);
+
+#pragma unroll 2
+        for (int b = 0; b < KB; b++) {
+            v4i av[2], bv[2];
+            float dwv[2], ndwv[2];
+            float4 dxv[2][4];
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+                const uint4 t4 = s.xt[b][g][wtok0 + tt * 32 + l32];
+                av[tt] = v4i{(int)t4.x, (int)t4.y, (int)t4.z, (int)t4.w};
+#pragma unroll
+                for (int gq = 0; gq < 4; gq++)
+                    dxv[tt][gq] = *reinterpret_cast<const float4*>(&s.dx[b][wtok0 + tt * 32 + 8 * gq + 4 * g]);
+            }
+#pragma unroll
+            for (int rt = 0; rt < 2; rt++) {
+                const uint4 t4 = s.wt[g][b][wrow0 + rt * 32 + l32];
+                bv[rt] = v4i{(int)t4.x, (int)t4.y, (int)t4.z, (int)t4.w};
+                dwv[rt] = s.dw[b][wrow0 + rt * 32 + l32];
+                ndwv[rt] = s.ndw[b][wrow0 + rt * 32 + l32];
+            }
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[tt], bv[rt], cbias, 0, 0, 0);
+                    if constexpr (DUMP) {
+                        const uint32_t row = row0 + wrow0 + rt * 32 + l32;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const uint32_t tok = tok0 + wtok0 + tt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+                            if (row < a.m && tok < a.n) {
+                                int v = d[r] - (int)kBiasBits;
+                                if (TYPE == 2) v >>= 4;  // weights were stored x16; exact
+                                a.dots[((size_t)tok * a.m + row) * nb + st * KB + b] = v;
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const float df = __int_as_float(d[r]);
+                            const float t = __builtin_fmaf(df, dwv[rt], ndwv[rt]);
+                            const float dxs = (r & 3) == 0   ? dxv[tt][r >> 2].x
+                                              : (r & 3) == 1 ? dxv[tt][r >> 2].y
+                                              : (r & 3) == 2 ? dxv[tt][r >> 2].z
+                                                             : dxv[tt][r >> 2].w;
+                            acc[tt][rt][r] = __builtin_fmaf(t, dxs, acc[tt][rt][r]);
+                        }
+                    }
+                }
+            }
+        }
+
+        __syncthreads();
+        if (st + 1 < stages) store_stage<TYPE>(s, regs);
+        __syncthreads();
+    }
+
+    if constexpr (!DUMP) {
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int rt = 0; rt < 2; rt++) {
+                const uint32_t row = row0 + wrow0 + rt * 32 + l32;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const uint32_t tok = tok0 + wtok0 + tt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+                    if (row < a.m && tok < a.n) {
+                        float* dst = a.y_row_major ? a.y + (size_t)row * a.y_stride + tok : a.y + (size_t)tok * a.y_stride + row;
+                        *dst = a.accumulate ? *dst + acc[tt][rt][r] : acc[tt][rt][r];
+                    }
+                }
+            }
+    }
+}
+
+template <bool DUMP>
+hipError_t launch(int type, GemmArgs& a, hipStream_t stream) {
+    if (a.m == 0 || a.n == 0) return hipSuccess;
+    a.row_tiles = (a.m + BM - 1) / BM;
+    a.tok_tiles = (a.n + BN - 1) / BN;
+    const uint32_t tiles = a.row_tiles * a.tok_tiles;
+    const uint32_t blocks = ((tiles + 7u) / 8u) * 8u;  // every XCD gets the same number of slots
+    if (type == kTypeQ4_0)
+        gemm_mfma_kernel<2, DUMP><<<blocks, THREADS, 0, stream>>>(a);
+    else
+        gemm_mfma_kernel<8, DUMP><<<blocks, THREADS, 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
+                            const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
+                            int accumulate, hipStream_t stream) {
+    GemmArgs a{};
+    a.w = d_w, a.xq = d_q, a.xs = d_scales, a.y = d_y, a.dots = nullptr;
+    a.m = m, a.n = n, a.k = k, a.y_stride = y_stride;
+    a.y_row_major = (y_layout == 1);
+    a.accumulate = accumulate;
+    return launch<false>(type, a, stream);
+}
+
+// Parity hook through the matrix-core path: the same loads, unpack, LDS layout and
+// MFMA as the GEMM, writing the raw i32 block dots instead of scaling them.
+hipError_t launch_block_dots_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,
+                                  int32_t* d_out, hipStream_t stream) {
+    GemmArgs a{};
+    a.w = d_w, a.xq = d_q, a.xs = nullptr, a.y = nullptr, a.dots = d_out;
+    a.m = m, a.n = n, a.k = k, a.y_stride = 0;
+    return launch<true>(type, a, stream);
+}
+
+}  // namespace wick_rocm

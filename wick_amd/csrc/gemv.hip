@@ -1,0 +1,290 @@
+// Decode GEMV (and small-n multi-token GEMV) over raw GGUF Q4_0 / Q8_0 blocks
+// against Q8_0-quantized activations, for gfx950.
+//
+// Arithmetic: gemv_q4_0_q8_0_neon / gemv_q8_0_q8_0_neon
+// (wick/src/backend/simd.rs:328-415, 440-524):
+//   y[i] = sum_b f32(isum_{i,b}) * (f32(f16 d_w[i,b]) * xs[b]),  isum exact i32.
+// The f32 summation order differs from NEON's (tree over lanes instead of
+// even/odd block accumulators); the contract is rel-L2 <= 1e-5, not bit equality.
+//
+// Shape of the kernel (HBM-bandwidth-bound, no matrix cores):
+//   * The weight matrix is a flat stream of 36-byte (Q4_0) / 68-byte (Q8_0)
+//     block PAIRS; a row of k elements is k/64 consecutive pairs and rows follow
+//     each other without padding, so 64 consecutive lanes read 64 consecutive
+//     pairs = one contiguous 2304 / 4352 byte span with dword-aligned wide loads.
+//   * A row is owned by LPR lanes (power of two, <= 64); a lane always meets the
+//     same pair index of every row it visits, so its slice of the activation
+//     vector (64 int8 + 2 scales per pair) lives in REGISTERS for the whole
+//     kernel.  Nothing is staged through LDS.
+//   * Nibbles are unpacked with and/shift and dotted with v_dot4_i32_i8; the
+//     "-8" of Q4_0 is folded into one subtraction of 8*sum(x) per block.
+//   * U rows are in flight per lane before any is consumed, and every wave is
+//     its own workgroup so small matrices still spread over all 256 CUs.
+//   * Rows are reduced across their LPR lanes with lane swaps.
+#include "wick_rocm_device.h"
+#include "wick_rocm_internal.h"
+
+namespace wick_rocm {
+
+namespace {
+
+struct GemvArgs {
+    GemvBatch batch;
+    const int8_t* xq;   // [n][k]
+    const float* xs;    // [n][k/32]
+    uint32_t k;
+    uint32_t n;         // tokens (1 for decode)
+    uint32_t y_stride;  // token-major: >= rows of that weight; row-major: >= n
+    uint32_t rows_per_wave;
+    int y_row_major;
+    int accumulate;
+};
+
+template <int TYPE, int NT>
+struct ActRegs {
+    uint32_t q[NT][2][8];  // two blocks of 32 int8
+    float s[NT][2];
+    int sum[NT][2];  // sum of the block's quants (used by Q4_0 only)
+};
+
+template <int TYPE, int LPR, int NCHUNK, int U, int NT>
+__global__ __launch_bounds__(64) void gemv_pairs_kernel(GemvArgs a) {
+    using PT = PairTraits<TYPE>;
+    constexpr int RPW = 64 / LPR;  // rows per wave pass
+    const uint32_t lane = threadIdx.x;
+    const uint32_t sub = lane % LPR;
+    const uint32_t rsel = lane / LPR;
+    const uint32_t ppr = a.k >> 6;  // pairs per row
+    const uint32_t nb = a.k >> 5;
+    const uint32_t total_rows = a.batch.row_end[a.batch.count - 1];
+    const uint32_t tok0 = blockIdx.y * NT;
+
+    // This lane's slice of the activations, kept in registers.
+    ActRegs<TYPE, NT> act[NCHUNK];
+    bool pvalid[NCHUNK];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; c++) {
+        const uint32_t p = c * LPR + sub;
+        pvalid[c] = p < ppr;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const bool ok = pvalid[c] && (tok0 + t < a.n);
+            const uint32_t tok = ok ? tok0 + t : 0;
+            const uint32_t pp = ok ? p : 0;
+            const uint4* src = reinterpret_cast<const uint4*>(a.xq + (size_t)tok * a.k + (size_t)pp * 64);
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                uint4 lo = src[2 * h], hi = src[2 * h + 1];
+                if (!ok) lo = hi = make_uint4(0, 0, 0, 0);
+                act[c].q[t][h][0] = lo.x, act[c].q[t][h][1] = lo.y, act[c].q[t][h][2] = lo.z, act[c].q[t][h][3] = lo.w;
+                act[c].q[t][h][4] = hi.x, act[c].q[t][h][5] = hi.y, act[c].q[t][h][6] = hi.z, act[c].q[t][h][7] = hi.w;
+                act[c].sum[t][h] = (TYPE == 2) ? block_xsum(act[c].q[t][h]) : 0;
+                const float sc = a.xs[(size_t)tok * nb + 2 * pp + h];
+                act[c].s[t][h] = ok ? sc : 0.0f;
+            }
+        }
+    }
+
+    const uint32_t wave_row0 = blockIdx.x * a.rows_per_wave;
+    const uint32_t wave_row1 = min(wave_row0 + a.rows_per_wave, total_rows);
+
+    for (uint32_t base = wave_row0; base < wave_row1; base += RPW * U) {
+        uint32_t w[U][NCHUNK][PT::DWORDS];
+        bool rvalid[U];
+        uint32_t lrow[U];
+        float* yp[U];
+        // Issue every load of this pass first.
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t r = base + u * RPW + rsel;
+            rvalid[u] = r < wave_row1;
+            const uint8_t* wp = a.batch.w[0];
+            yp[u] = a.batch.y[0];
+            uint32_t start = 0;
+#pragma unroll
+            for (int i = 1; i < kMaxGemvBatch; i++) {
+                if (i < (int)a.batch.count && r >= a.batch.row_end[i - 1]) {
+                    wp = a.batch.w[i];
+                    yp[u] = a.batch.y[i];
+                    start = a.batch.row_end[i - 1];
+                }
+            }
+            lrow[u] = r - start;
+            const uint8_t* rowp = wp + (size_t)lrow[u] * ppr * PT::BYTES;
+#pragma unroll
+            for (int c = 0; c < NCHUNK; c++) {
+                if (rvalid[u] && pvalid[c]) {
+                    load_pair<PT::DWORDS>(rowp + (size_t)(c * LPR + sub) * PT::BYTES, w[u][c]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < PT::DWORDS; i++) w[u][c][i] = 0;
+                }
+            }
+        }
+        // Consume.
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) acc[t] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < NCHUNK; c++) {
+                uint32_t d0, d1, q0[PT::NQ], q1[PT::NQ];
+                split_pair<TYPE>(w[u][c], d0, d1, q0, q1);
+                const float dw0 = f16_bits_to_f32(d0), dw1 = f16_bits_to_f32(d1);
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const int i0 = block_dot<TYPE>(q0, act[c].q[t][0], act[c].sum[t][0]);
+                    const int i1 = block_dot<TYPE>(q1, act[c].q[t][1], act[c].sum[t][1]);
+                    acc[t] += (float)i0 * (dw0 * act[c].s[t][0]);
+                    acc[t] += (float)i1 * (dw1 * act[c].s[t][1]);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const float tot = group_sum<LPR>(acc[t]);
+                if (sub == 0 && rvalid[u] && tok0 + t < a.n) {
+                    float* dst = a.y_row_major ? yp[u] + (size_t)lrow[u] * a.y_stride + (tok0 + t)
+                                               : yp[u] + (size_t)(tok0 + t) * a.y_stride + lrow[u];
+                    *dst = a.accumulate ? *dst + tot : tot;
+                }
+            }
+        }
+    }
+}
+
+// Any k % 32 == 0, any byte alignment: one wave per row, lanes stride over single
+// blocks, two-byte loads.  Correctness path for shapes the pair kernel does not
+// take (odd block count per row, k > 8192); not tuned.
+template <int TYPE, int NT>
+__global__ __launch_bounds__(64) void gemv_generic_kernel(GemvArgs a) {
+    constexpr int BB = (TYPE == 2) ? kQ4BlockBytes : kQ8BlockBytes;
+    constexpr int NQ = PairTraits<TYPE>::NQ;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t nb = a.k >> 5;
+    const uint32_t total_rows = a.batch.row_end[a.batch.count - 1];
+    const uint32_t tok0 = blockIdx.y * NT;
+    const uint32_t row0 = blockIdx.x * a.rows_per_wave;
+    const uint32_t row1 = min(row0 + a.rows_per_wave, total_rows);
+    for (uint32_t r = row0; r < row1; r++) {
+        const uint8_t* wp = a.batch.w[0];
+        float* yp = a.batch.y[0];
+        uint32_t start = 0;
+        for (uint32_t i = 1; i < a.batch.count; i++) {
+            if (r >= a.batch.row_end[i - 1]) {
+                wp = a.batch.w[i];
+                yp = a.batch.y[i];
+                start = a.batch.row_end[i - 1];
+            }
+        }
+        const uint32_t lrow = r - start;
+        const uint8_t* rowp = wp + (size_t)lrow * nb * BB;
+        float acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; t++) acc[t] = 0.0f;
+        for (uint32_t b = lane; b < nb; b += 64) {
+            const uint16_t* hp = reinterpret_cast<const uint16_t*>(rowp + (size_t)b * BB);
+            const float dw = f16_bits_to_f32(hp[0]);
+            uint32_t q[NQ];
+#pragma unroll
+            for (int j = 0; j < NQ; j++) q[j] = (uint32_t)hp[1 + 2 * j] | ((uint32_t)hp[2 + 2 * j] << 16);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                if (tok0 + t < a.n) {
+                    const uint32_t* xp = reinterpret_cast<const uint32_t*>(a.xq + (size_t)(tok0 + t) * a.k + (size_t)b * 32);
+                    uint32_t x[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) x[j] = xp[j];
+                    const int isum = block_dot<TYPE>(q, x, (TYPE == 2) ? block_xsum(x) : 0);
+                    acc[t] += (float)isum * (dw * a.xs[(size_t)(tok0 + t) * nb + b]);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const float tot = group_sum<64>(acc[t]);
+            if (lane == 0 && tok0 + t < a.n) {
+                float* dst = a.y_row_major ? yp + (size_t)lrow * a.y_stride + (tok0 + t)
+                                           : yp + (size_t)(tok0 + t) * a.y_stride + lrow;
+                *dst = a.accumulate ? *dst + tot : tot;
+            }
+        }
+    }
+}
+
+template <int TYPE, int LPR, int NCHUNK, int NT>
+hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, hipStream_t stream) {
+    // Rows in flight per lane: bounded by registers (a Q8_0 pair is 17 dwords).
+    constexpr int U = (TYPE == 2) ? (NCHUNK == 1 ? (NT == 1 ? 4 : 2) : (NT == 1 ? 2 : 1)) : (NCHUNK == 1 && NT == 1 ? 2 : 1);
+    constexpr uint32_t pass_rows = (64 / LPR) * U;
+    // Enough single-wave workgroups to give every CU ~16 waves, and every wave at
+    // least one full pass.
+    const uint32_t max_waves = (uint32_t)num_cus * 16u;
+    uint32_t passes = (total_rows + pass_rows - 1) / pass_rows;
+    uint32_t passes_per_wave = (passes + max_waves - 1) / max_waves;
+    if (passes_per_wave == 0) passes_per_wave = 1;
+    a.rows_per_wave = passes_per_wave * pass_rows;
+    const uint32_t waves = (total_rows + a.rows_per_wave - 1) / a.rows_per_wave;
+    dim3 grid(waves, (a.n + NT - 1) / NT);
+    gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT><<<grid, 64, 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+template <int TYPE, int NT>
+hipError_t dispatch(GemvArgs& a, int num_cus, hipStream_t stream) {
+    const uint32_t total_rows = a.batch.row_end[a.batch.count - 1];
+    if (total_rows == 0 || a.n == 0) return hipSuccess;
+    const uint32_t nb = a.k >> 5;
+    const uint32_t ppr = nb >> 1;
+    bool aligned = (nb % 2u) == 0 && (reinterpret_cast<uintptr_t>(a.xq) % 16u) == 0;
+    for (uint32_t i = 0; i < a.batch.count; i++) aligned = aligned && (reinterpret_cast<uintptr_t>(a.batch.w[i]) % 4u) == 0;
+    if (aligned && ppr <= 128) {
+        if (ppr <= 4) return launch_pairs<TYPE, 4, 1, NT>(a, total_rows, num_cus, stream);
+        if (ppr <= 8) return launch_pairs<TYPE, 8, 1, NT>(a, total_rows, num_cus, stream);
+        if (ppr <= 16) return launch_pairs<TYPE, 16, 1, NT>(a, total_rows, num_cus, stream);
+        if (ppr <= 32) return launch_pairs<TYPE, 32, 1, NT>(a, total_rows, num_cus, stream);
+        if (ppr <= 64) return launch_pairs<TYPE, 64, 1, NT>(a, total_rows, num_cus, stream);
+        return launch_pairs<TYPE, 64, 2, NT>(a, total_rows, num_cus, stream);
+    }
+    a.rows_per_wave = 1;
+    dim3 grid(total_rows, (a.n + NT - 1) / NT);
+    gemv_generic_kernel<TYPE, NT><<<grid, 64, 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_gemv(int type, const GemvBatch& batch, uint32_t k, const int8_t* d_q, const float* d_scales,
+                       int accumulate, int num_cus, hipStream_t stream) {
+    GemvArgs a{};
+    a.batch = batch;
+    a.xq = d_q;
+    a.xs = d_scales;
+    a.k = k;
+    a.n = 1;
+    a.y_stride = 0;
+    a.y_row_major = 0;
+    a.accumulate = accumulate;
+    return type == kTypeQ4_0 ? dispatch<2, 1>(a, num_cus, stream) : dispatch<8, 1>(a, num_cus, stream);
+}
+
+hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
+                              const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
+                              int accumulate, int num_cus, hipStream_t stream) {
+    GemvArgs a{};
+    a.batch.w[0] = d_w;
+    a.batch.y[0] = d_y;
+    a.batch.row_end[0] = m;
+    a.batch.count = 1;
+    a.xq = d_q;
+    a.xs = d_scales;
+    a.k = k;
+    a.n = n;
+    a.y_stride = y_stride;
+    a.y_row_major = (y_layout == 1);
+    a.accumulate = accumulate;
+    if (n == 1) return type == kTypeQ4_0 ? dispatch<2, 1>(a, num_cus, stream) : dispatch<8, 1>(a, num_cus, stream);
+    return type == kTypeQ4_0 ? dispatch<2, 4>(a, num_cus, stream) : dispatch<8, 4>(a, num_cus, stream);
+}
+
+}  // namespace wick_rocm

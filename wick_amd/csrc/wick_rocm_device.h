@@ -1,0 +1,130 @@
+// Device-side helpers shared by the GEMV, GEMM and parity-hook kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace wick_rocm {
+
+// f16 bit pattern -> f32 (v_cvt_f32_f16; exact, subnormals kept).
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits) {
+    uint16_t b = (uint16_t)bits;
+    _Float16 h;
+    __builtin_memcpy(&h, &b, 2);
+    return (float)h;
+}
+
+// 4- and 16-byte vectors that only promise 4-byte alignment, so the compiler may
+// still issue one wide global load for them.
+struct __attribute__((packed, aligned(4))) u32x4_a4 {
+    uint32_t v[4];
+};
+struct __attribute__((packed, aligned(4))) u32x2_a4 {
+    uint32_t v[2];
+};
+
+// A "pair" is two consecutive weight blocks of one row: 36 B (Q4_0) or 68 B
+// (Q8_0).  Rows hold an even number of blocks on the fast paths, so every pair
+// starts 4-byte aligned and is read as whole dwords:
+//   dword 0            = [ d0 (f16) | first two quant bytes of block 0 ]
+//   dwords 1 .. NQ-1   = block 0 quants, shifted by two bytes
+//   dword NQ           = [ last two quant bytes of block 0 | d1 (f16) ]
+//   dwords NQ+1 .. 2NQ = block 1 quants, dword aligned
+// NQ = quant dwords per block: 4 (Q4_0: 16 nibble bytes) or 8 (Q8_0: 32 int8).
+template <int TYPE>
+struct PairTraits;
+template <>
+struct PairTraits<2> {
+    static constexpr int NQ = 4;
+    static constexpr int DWORDS = 9;
+    static constexpr int BYTES = 36;
+};
+template <>
+struct PairTraits<8> {
+    static constexpr int NQ = 8;
+    static constexpr int DWORDS = 17;
+    static constexpr int BYTES = 68;
+};
+
+template <int DWORDS>
+__device__ __forceinline__ void load_pair(const uint8_t* __restrict__ p, uint32_t (&w)[DWORDS]) {
+    static_assert(DWORDS % 4 == 1, "pair = 4*j + 1 dwords");
+#pragma unroll
+    for (int i = 0; i < DWORDS / 4; i++) {
+        u32x4_a4 t = *reinterpret_cast<const u32x4_a4*>(p + 16 * i);
+        w[4 * i + 0] = t.v[0];
+        w[4 * i + 1] = t.v[1];
+        w[4 * i + 2] = t.v[2];
+        w[4 * i + 3] = t.v[3];
+    }
+    w[DWORDS - 1] = *reinterpret_cast<const uint32_t*>(p + 4 * (DWORDS - 1));
+}
+
+// Splits a pair into the two f16 scale bit patterns and the two blocks' quant
+// dwords (block 0 needs a two-byte funnel shift, v_alignbyte_b32).
+template <int TYPE>
+__device__ __forceinline__ void split_pair(const uint32_t (&w)[PairTraits<TYPE>::DWORDS], uint32_t& d0, uint32_t& d1,
+                                           uint32_t (&q0)[PairTraits<TYPE>::NQ], uint32_t (&q1)[PairTraits<TYPE>::NQ]) {
+    constexpr int NQ = PairTraits<TYPE>::NQ;
+    d0 = w[0] & 0xffffu;
+    d1 = w[NQ] >> 16;
+#pragma unroll
+    for (int j = 0; j < NQ; j++) {
+        q0[j] = __builtin_amdgcn_alignbyte(w[j + 1], w[j], 2);
+        q1[j] = w[NQ + 1 + j];
+    }
+}
+
+// Exact i32 dot of one weight block with one Q8_0 activation block (8 dwords of
+// int8: x[0..3] = elements 0..15, x[4..7] = elements 16..31).
+//
+// Q4_0 (wick/src/quant.rs:82-88): byte i of qs holds element i in its low nibble
+// and element i+16 in its high nibble, value = nibble - 8.  The unsigned nibbles
+// are dotted as they are and 8 * sum(x) is subtracted once; `xsum` is that
+// block's sum of activation quants.
+__device__ __forceinline__ int block_dot_q4_0(const uint32_t (&q)[4], const uint32_t (&x)[8], int xsum) {
+    int s = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint32_t lo = q[j] & 0x0f0f0f0fu;
+        uint32_t hi = (q[j] >> 4) & 0x0f0f0f0fu;
+        s = __builtin_amdgcn_sdot4((int)lo, (int)x[j], s, false);
+        s = __builtin_amdgcn_sdot4((int)hi, (int)x[4 + j], s, false);
+    }
+    return s - 8 * xsum;
+}
+
+__device__ __forceinline__ int block_dot_q8_0(const uint32_t (&q)[8], const uint32_t (&x)[8]) {
+    int s = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) s = __builtin_amdgcn_sdot4((int)q[j], (int)x[j], s, false);
+    return s;
+}
+
+__device__ __forceinline__ int block_xsum(const uint32_t (&x)[8]) {
+    int s = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) s = __builtin_amdgcn_sdot4(0x01010101, (int)x[j], s, false);
+    return s;
+}
+
+template <int TYPE>
+__device__ __forceinline__ int block_dot(const uint32_t (&q)[PairTraits<TYPE>::NQ], const uint32_t (&x)[8], int xsum) {
+    if constexpr (TYPE == 2) {
+        return block_dot_q4_0(q, x, xsum);
+    } else {
+        (void)xsum;
+        return block_dot_q8_0(q, x);
+    }
+}
+
+// Sum over groups of WIDTH consecutive lanes (WIDTH a power of two <= 64); every
+// lane of a group ends with the group's total.
+template <int WIDTH>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int off = WIDTH / 2; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+}  // namespace wick_rocm
