@@ -176,6 +176,16 @@ int wick_rocm_event_record(wick_rocm_ctx *ctx, wick_rocm_event *e);
 int wick_rocm_event_elapsed_ms(wick_rocm_ctx *ctx, wick_rocm_event *start, wick_rocm_event *stop, float *ms); /* waits for stop */
 int wick_rocm_event_destroy(wick_rocm_ctx *ctx, wick_rocm_event *e);
 
+/* Per-dispatch kernel timestamps, the counterpart of WICK_PROFILE=gpu
+ * (per-dispatch counter samples, wick/src/model/metal_lfm2.rs:3367-4116).  Between
+ * begin and end every kernel the hot-path calls launch carries its own start/stop
+ * timestamps; end waits for the stream and returns, per kernel family
+ * (0 = quantizer, 1 = GEMV, 2 = GEMM, 3 = other), the summed execution time in ms
+ * and the number of launches.  Arrays hold n_families (<= 4) entries.  Not usable
+ * during graph capture. */
+int wick_rocm_kernel_timing_begin(wick_rocm_ctx *ctx);
+int wick_rocm_kernel_timing_end(wick_rocm_ctx *ctx, double *total_ms, uint64_t *launches, int n_families);
+
 /* Library version string, e.g. "wick-rocm 0.1 (gfx950)". */
 const char *wick_rocm_version(void);
 

@@ -1,0 +1,135 @@
+"""Batched prefill GEMM on the GPU against the oracle, both output layouts, both
+kernel paths (multi-token GEMV below GEMM_MIN_N or when k % 256 != 0; int8 MFMA
+otherwise).  Block dots BIT-EXACT, f32 within rel-L2 1e-5 / max-abs 1e-4 x RMS."""
+import numpy as np
+import pytest
+
+import wick_amd as W
+from conftest import assert_f32_parity, rel_l2
+from gpu_util import Problem, fetch_gemm
+from test_oracle_matmul import ref_inputs, ref_weights
+
+pytestmark = pytest.mark.gpu
+
+# (m, n, k)
+SHAPES = [
+    (8, 1, 64), (8, 5, 64), (8, 7, 64), (8, 8, 64), (8, 11, 64), (8, 16, 64),  # the reference's own test shapes
+    (4, 1, 32), (64, 4, 32), (64, 20, 96), (33, 3, 2080),                        # generic path
+    (64, 2, 256), (100, 15, 512),                                                # multi-token GEMV
+    (128, 16, 256), (128, 128, 256), (1, 16, 256), (130, 129, 512), (200, 50, 512), (256, 300, 1024),
+    (512, 100, 2048), (1000, 257, 4608), (300, 64, 6912),                        # MFMA, ragged tiles
+]
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_gemm_parity(ctx, oracle, dtype, m, n, k):
+    with Problem(ctx, oracle, dtype, m, k, n, seed=m + 5 * n + 11 * k + dtype) as p:
+        ref = oracle.gemm_q8(dtype, p.wb, p.s, p.q, m, n, k)
+        for layout, stride in ((W.LAYOUT_ROW_MAJOR, n), (W.LAYOUT_TOKEN_MAJOR, m), (W.LAYOUT_ROW_MAJOR, n + 3), (W.LAYOUT_TOKEN_MAJOR, m + 5)):
+            rows = m if layout == W.LAYOUT_ROW_MAJOR else n
+            d_y = p.to_device(np.full(rows * stride, -7.0, np.float32))
+            ctx.gemm_preq(p.w, p.d_s, p.d_q, n, d_y, y_stride=stride, layout=layout)
+            assert_f32_parity(fetch_gemm(d_y, m, n, stride, layout), ref, f"gemm {dtype} {m}x{n}x{k} layout {layout}")
+            # padding between rows is left untouched
+            full = d_y.download(np.float32, rows * stride).reshape(rows, stride)
+            used = n if layout == W.LAYOUT_ROW_MAJOR else m
+            assert np.all(full[:, used:] == -7.0)
+        d_d = p.alloc(n * m * (k // 32) * 4)
+        ctx.block_dots_i32(p.w, p.d_q, n, d_d)
+        dots = d_d.download(np.int32, n * m * (k // 32)).reshape(n, m, k // 32)
+        assert np.array_equal(dots, oracle.block_dots_i32(dtype, p.wb, p.q, m, n, k))
+
+
+@pytest.mark.parametrize("dtype,n", [(W.Q4_0, 7), (W.Q8_0, 5), (W.Q4_0, 8), (W.Q4_0, 11), (W.Q4_0, 16)])
+def test_reference_gemm_vs_gemv_inputs(ctx, oracle, dtype, n):
+    """The reference's GEMM == sequential GEMV tests (simd.rs:1440-1623) on their own
+    weights/inputs: GPU GEMM column j vs GPU GEMV of column j within the reference's 1e-4."""
+    m, k = 8, 64
+    wb = oracle.build_matrix(dtype, ref_weights(m, k), m, k)
+    s, q = oracle.quantize_q8_0_batch(ref_inputs(n, k), n, k)
+    w = ctx.upload_weight(wb, dtype, m, k)
+    d_q, d_s = ctx.to_device(q), ctx.to_device(s)
+    d_c, d_y = ctx.alloc(m * n * 4), ctx.alloc(m * 4)
+    ctx.gemm_preq(w, d_s, d_q, n, d_c, layout=W.LAYOUT_ROW_MAJOR)
+    c = d_c.download(np.float32, m * n).reshape(m, n)
+    assert_f32_parity(c, oracle.gemm_q8(dtype, wb, s, q, m, n, k), "reference inputs")
+    for j in range(n):
+        ctx.gemv_with_preq(w, d_s.ptr + j * (k // 32) * 4, d_q.ptr + j * k, d_y)
+        assert np.abs(c[:, j] - d_y.download(np.float32, m)).max() < 1e-4
+    w.free()
+    for b in (d_q, d_s, d_c, d_y):
+        b.free()
+
+
+def test_q8_0_closed_form(ctx, oracle):
+    """test_q8_0_gemm_standalone (wick/tests/bench_perf.rs:852-971): m=64, k=32, n=4,
+    scale 1/(row+1), quants -16..15, x == 1, x_stride = k, y_stride = m, through the
+    f32 call-site entry point."""
+    m, k, n = 64, 32, 4
+    rows = []
+    for r in range(m):
+        h = int(np.float16(1.0 / (r + 1.0)).view(np.uint16))
+        rows.append(np.concatenate([np.array([h & 0xFF, h >> 8], np.uint8), (np.arange(32) - 16).astype(np.int8).view(np.uint8)]))
+    w = ctx.upload_weight(np.concatenate(rows), W.Q8_0, m, k)
+    d_x = ctx.to_device(np.ones(n * k, np.float32))
+    d_y = ctx.alloc(m * n * 4)
+    ctx.encode_gemm(w, d_x, 0, d_y, 0, n, k, m)
+    y = d_y.download(np.float32, m * n).reshape(n, m)
+    expect = np.array([-16.0 * float(np.float16(1.0 / (r + 1.0))) for r in range(m)]) * 127.0 * float(np.float16(1.0 / 127.0))
+    for col in range(n):
+        assert np.abs(y[col] - (-16.0 / (np.arange(m) + 1.0))).max() < 1.0  # the reference's bound
+        assert np.allclose(y[col], expect, rtol=1e-6)
+    w.free(), d_x.free(), d_y.free()
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+@pytest.mark.parametrize("n", [3, 40])
+def test_accumulate(ctx, oracle, dtype, n):
+    m, k = 256, 512
+    with Problem(ctx, oracle, dtype, m, k, n, seed=8) as p:
+        y0 = oracle.fill_normal(4, 1.0, n * m)
+        d_y = p.to_device(y0)
+        ctx.gemm_preq(p.w, p.d_s, p.d_q, n, d_y, layout=W.LAYOUT_TOKEN_MAJOR, accumulate=True)
+        ref = y0.reshape(n, m).T.astype(np.float64) + oracle.gemm_q8(dtype, p.wb, p.s, p.q, m, n, k, f64=True)
+        assert_f32_parity(fetch_gemm(d_y, m, n, m, W.LAYOUT_TOKEN_MAJOR), ref, "gemm accumulate")
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+def test_full_size_prefill_shape(ctx, oracle, dtype):
+    """m=6912, n=2002, k=2048 (the LFM2-1.2B ffn_up prefill shape).  The oracle checks a
+    band of rows across ALL tokens plus scattered rows; size-independent properties cover
+    the rest: column j of the GEMM equals the GEMV of column j, and both layouts agree."""
+    m, n, k = 6912, 2002, 2048
+    with Problem(ctx, oracle, dtype, m, k, n, seed=2026) as p:
+        d_y = p.alloc(m * n * 4)
+        ctx.gemm_preq(p.w, p.d_s, p.d_q, n, d_y, layout=W.LAYOUT_TOKEN_MAJOR)
+        y = fetch_gemm(d_y, m, n, m, W.LAYOUT_TOKEN_MAJOR)
+        assert np.isfinite(y).all()
+        bb = 18 if dtype == W.Q4_0 else 34
+        rows = np.concatenate([np.arange(0, 40), np.arange(6890, 6912), np.arange(100, 6800, 397)])
+        sub = np.concatenate([p.wb.reshape(m, -1)[r] for r in rows])
+        assert sub.size == len(rows) * (k // 32) * bb
+        assert_f32_parity(y[rows], oracle.gemm_q8(dtype, sub, p.s, p.q, len(rows), n, k), "C3 row band")
+        d_v = p.alloc(m * 4)
+        for j in (0, 1, 127, 128, 1000, 1983, 1984, 2001):
+            ctx.gemv_with_preq(p.w, p.d_s.ptr + j * (k // 32) * 4, p.d_q.ptr + j * k, d_v)
+            assert rel_l2(y[:, j], d_v.download(np.float32, m)) < 1e-6
+        ctx.gemm_preq(p.w, p.d_s, p.d_q, n, d_y, layout=W.LAYOUT_ROW_MAJOR)
+        y2 = fetch_gemm(d_y, m, n, n, W.LAYOUT_ROW_MAJOR)
+        assert np.array_equal(y, y2)
+
+
+def test_argument_errors(ctx, oracle):
+    with Problem(ctx, oracle, W.Q4_0, 64, 256, 20) as p:
+        d_y = p.alloc(64 * 20 * 4)
+        with pytest.raises(W.RocmError) as e:
+            ctx.gemm_preq(p.w, p.d_s, p.d_q, 20, d_y, y_stride=10, layout=W.LAYOUT_ROW_MAJOR)
+        assert e.value.status == -1
+        with pytest.raises(W.RocmError) as e:
+            ctx.gemm_preq(p.w, p.d_s, p.d_q, 20, d_y, y_stride=63, layout=W.LAYOUT_TOKEN_MAJOR)
+        assert e.value.status == -1
+        with pytest.raises(W.RocmError) as e:
+            ctx.gemm_preq(p.w, p.d_s, p.d_q, 20, d_y, y_stride=64, layout=5)
+        assert e.value.status == -1
+        ctx.gemm_preq(p.w, p.d_s, p.d_q, 0, d_y, y_stride=64, layout=W.LAYOUT_TOKEN_MAJOR)  # n = 0: no-op

@@ -29,6 +29,8 @@ struct wick_rocm_ctx {
     float* scratch_s = nullptr;
     size_t scratch_q_cap = 0;  // bytes
     size_t scratch_s_cap = 0;  // floats
+    KernelTimer timer;
+    Launch launch() { return Launch{stream, &timer}; }
 };
 
 struct wick_rocm_weight {
@@ -118,10 +120,10 @@ int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q
     hipError_t e;
     if (n >= kGemmMinN && mfma_ok)
         e = launch_gemm_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
-                             y_layout, accumulate, ctx->stream);
+                             y_layout, accumulate, ctx->launch());
     else
         e = launch_gemv_tokens(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
-                               y_layout, accumulate, ctx->num_cus, ctx->stream);
+                               y_layout, accumulate, ctx->num_cus, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "gemm launch");
     return WICK_ROCM_OK;
 }
@@ -178,6 +180,11 @@ void wick_rocm_ctx_destroy(wick_rocm_ctx* ctx) {
         }
         if (ctx->scratch_q) (void)hipFree(ctx->scratch_q);
         if (ctx->scratch_s) (void)hipFree(ctx->scratch_s);
+        for (auto* v : {&ctx->timer.recs, &ctx->timer.spares})
+            for (KernelTimer::Rec& r : *v) {
+                (void)hipEventDestroy(r.start);
+                (void)hipEventDestroy(r.stop);
+            }
     }
     delete ctx;
 }
@@ -303,7 +310,7 @@ int wick_rocm_quantize_q8_0(wick_rocm_ctx* ctx, const float* d_x, uint32_t n, ui
     if (reinterpret_cast<uintptr_t>(d_x) % 4u || reinterpret_cast<uintptr_t>(d_quants) % 4u ||
         reinterpret_cast<uintptr_t>(d_scales) % 4u)
         return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "quantize_q8_0: pointers must be 4-byte aligned");
-    hipError_t e = launch_quantize_q8_0(d_x, n, k, x_stride, d_quants, d_scales, ctx->stream);
+    hipError_t e = launch_quantize_q8_0(d_x, n, k, x_stride, d_quants, d_scales, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
     return WICK_ROCM_OK;
 }
@@ -328,7 +335,7 @@ int wick_rocm_gemv_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* w
         b.row_end[i] = rows;
     }
     b.count = count;
-    hipError_t e = launch_gemv(ws[0]->type, b, ws[0]->k, d_quants, d_scales, accumulate, ctx->num_cus, ctx->stream);
+    hipError_t e = launch_gemv(ws[0]->type, b, ws[0]->k, d_quants, d_scales, accumulate, ctx->num_cus, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "gemv launch");
     return WICK_ROCM_OK;
 }
@@ -365,7 +372,7 @@ int wick_rocm_matmul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const fl
     const float* x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes);
     float* y = reinterpret_cast<float*>(reinterpret_cast<char*>(d_y) + y_off_bytes);
     if (int rc = ensure_scratch(ctx, (size_t)n * w->k, (size_t)n * (w->k / 32u))) return rc;
-    hipError_t e = launch_quantize_q8_0(x, n, w->k, x_stride, ctx->scratch_q, ctx->scratch_s, ctx->stream);
+    hipError_t e = launch_quantize_q8_0(x, n, w->k, x_stride, ctx->scratch_q, ctx->scratch_s, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
     return gemm_locked(ctx, w, ctx->scratch_q, ctx->scratch_s, n, y, n == 1 ? w->m : y_stride,
                        WICK_ROCM_LAYOUT_TOKEN_MAJOR, accumulate);
@@ -378,8 +385,8 @@ int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, cons
     if (!d_quants || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "block_dots: null device pointer");
     if (n == 0) return WICK_ROCM_OK;
     const bool mfma = n >= kGemmMinN && (w->k % 256u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
-    hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->stream)
-                        : launch_block_dots_dot4(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->stream);
+    hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch())
+                        : launch_block_dots_dot4(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "block_dots launch");
     return WICK_ROCM_OK;
 }
@@ -387,6 +394,7 @@ int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, cons
 int wick_rocm_graph_begin(wick_rocm_ctx* ctx) {
     WR_ENTER(ctx);
     if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "graph_begin: capture already in progress");
+    if (ctx->timer.enabled) return fail(ctx, WICK_ROCM_ERR_STATE, "graph_begin: kernel timing is on");
     WR_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     ctx->capturing = true;
     return WICK_ROCM_OK;
@@ -455,6 +463,38 @@ int wick_rocm_event_elapsed_ms(wick_rocm_ctx* ctx, wick_rocm_event* start, wick_
     if (!start || !stop || !ms) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "event_elapsed_ms: null argument");
     WR_HIP(ctx, hipEventSynchronize(stop->ev));
     WR_HIP(ctx, hipEventElapsedTime(ms, start->ev, stop->ev));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_kernel_timing_begin(wick_rocm_ctx* ctx) {
+    WR_ENTER(ctx);
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "kernel_timing_begin during graph capture");
+    if (ctx->timer.enabled) return fail(ctx, WICK_ROCM_ERR_STATE, "kernel timing already on");
+    ctx->timer.enabled = true;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_kernel_timing_end(wick_rocm_ctx* ctx, double* total_ms, uint64_t* launches, int n_families) {
+    WR_ENTER(ctx);
+    if (!ctx->timer.enabled) return fail(ctx, WICK_ROCM_ERR_STATE, "kernel timing is not on");
+    ctx->timer.enabled = false;
+    for (int f = 0; f < n_families; f++) {
+        if (total_ms) total_ms[f] = 0.0;
+        if (launches) launches[f] = 0;
+    }
+    hipError_t first = hipStreamSynchronize(ctx->stream);
+    for (KernelTimer::Rec& r : ctx->timer.recs) {
+        float ms = 0.f;
+        hipError_t e = hipEventElapsedTime(&ms, r.start, r.stop);
+        if (e != hipSuccess && first == hipSuccess) first = e;
+        if (e == hipSuccess && r.family < n_families) {
+            if (total_ms) total_ms[r.family] += (double)ms;
+            if (launches) launches[r.family] += 1;
+        }
+        ctx->timer.spares.push_back(r);
+    }
+    ctx->timer.recs.clear();
+    if (first != hipSuccess) return fail_hip(ctx, first, "kernel_timing_end");
     return WICK_ROCM_OK;
 }
 

@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void block_dots_generic_kernel(const uint8_t* 
 }  // namespace
 
 hipError_t launch_block_dots_dot4(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,
-                                  int32_t* d_out, hipStream_t stream) {
+                                  int32_t* d_out, const Launch& L) {
     const uint32_t nb = k >> 5;
     if ((uint64_t)m * n * nb == 0) return hipSuccess;
     const bool pairs = (nb % 2u == 0) && (reinterpret_cast<uintptr_t>(d_w) % 4u == 0);
@@ -68,14 +68,14 @@ hipError_t launch_block_dots_dot4(int type, const uint8_t* d_w, uint32_t m, uint
     const uint32_t blocks = (uint32_t)((total + 255) / 256);
     if (pairs) {
         if (type == kTypeQ4_0)
-            block_dots_pairs_kernel<2><<<blocks, 256, 0, stream>>>(d_w, d_q, m, n, k, d_out);
+            return launch_kernel(L, kFamOther, block_dots_pairs_kernel<2>, dim3(blocks), dim3(256), d_w, d_q, m, n, k, d_out);
         else
-            block_dots_pairs_kernel<8><<<blocks, 256, 0, stream>>>(d_w, d_q, m, n, k, d_out);
+            return launch_kernel(L, kFamOther, block_dots_pairs_kernel<8>, dim3(blocks), dim3(256), d_w, d_q, m, n, k, d_out);
     } else {
         if (type == kTypeQ4_0)
-            block_dots_generic_kernel<2><<<blocks, 256, 0, stream>>>(d_w, d_q, m, n, k, d_out);
+            return launch_kernel(L, kFamOther, block_dots_generic_kernel<2>, dim3(blocks), dim3(256), d_w, d_q, m, n, k, d_out);
         else
-            block_dots_generic_kernel<8><<<blocks, 256, 0, stream>>>(d_w, d_q, m, n, k, d_out);
+            return launch_kernel(L, kFamOther, block_dots_generic_kernel<8>, dim3(blocks), dim3(256), d_w, d_q, m, n, k, d_out);
     }
     return hipGetLastError();
 }

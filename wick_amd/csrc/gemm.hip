@@ -292,16 +292,16 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
 }
 
 template <bool DUMP>
-hipError_t launch(int type, GemmArgs& a, hipStream_t stream) {
+hipError_t launch(int type, GemmArgs& a, const Launch& L) {
     if (a.m == 0 || a.n == 0) return hipSuccess;
     a.row_tiles = (a.m + BM - 1) / BM;
     a.tok_tiles = (a.n + BN - 1) / BN;
     const uint32_t tiles = a.row_tiles * a.tok_tiles;
     const uint32_t blocks = ((tiles + 7u) / 8u) * 8u;  // every XCD gets the same number of slots
     if (type == kTypeQ4_0)
-        gemm_mfma_kernel<2, DUMP><<<blocks, THREADS, 0, stream>>>(a);
+        return launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
     else
-        gemm_mfma_kernel<8, DUMP><<<blocks, THREADS, 0, stream>>>(a);
+        return launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
     return hipGetLastError();
 }
 
@@ -309,23 +309,23 @@ hipError_t launch(int type, GemmArgs& a, hipStream_t stream) {
 
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                             const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
-                            int accumulate, hipStream_t stream) {
+                            int accumulate, const Launch& L) {
     GemmArgs a{};
     a.w = d_w, a.xq = d_q, a.xs = d_scales, a.y = d_y, a.dots = nullptr;
     a.m = m, a.n = n, a.k = k, a.y_stride = y_stride;
     a.y_row_major = (y_layout == 1);
     a.accumulate = accumulate;
-    return launch<false>(type, a, stream);
+    return launch<false>(type, a, L);
 }
 
 // Parity hook through the matrix-core path: the same loads, unpack, LDS layout and
 // MFMA as the GEMM, writing the raw i32 block dots instead of scaling them.
 hipError_t launch_block_dots_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,
-                                  int32_t* d_out, hipStream_t stream) {
+                                  int32_t* d_out, const Launch& L) {
     GemmArgs a{};
     a.w = d_w, a.xq = d_q, a.xs = nullptr, a.y = nullptr, a.dots = d_out;
     a.m = m, a.n = n, a.k = k, a.y_stride = 0;
-    return launch<true>(type, a, stream);
+    return launch<true>(type, a, L);
 }
 
 }  // namespace wick_rocm

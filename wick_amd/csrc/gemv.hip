@@ -213,7 +213,7 @@ __global__ __launch_bounds__(64) void gemv_generic_kernel(GemvArgs a) {
 }
 
 template <int TYPE, int LPR, int NCHUNK, int NT>
-hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, hipStream_t stream) {
+hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
     // Rows in flight per lane: bounded by registers (a Q8_0 pair is 17 dwords).
     constexpr int U = (TYPE == 2) ? (NCHUNK == 1 ? (NT == 1 ? 4 : 2) : (NT == 1 ? 2 : 1)) : (NCHUNK == 1 && NT == 1 ? 2 : 1);
     constexpr uint32_t pass_rows = (64 / LPR) * U;
@@ -226,12 +226,12 @@ hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, hipStream
     a.rows_per_wave = passes_per_wave * pass_rows;
     const uint32_t waves = (total_rows + a.rows_per_wave - 1) / a.rows_per_wave;
     dim3 grid(waves, (a.n + NT - 1) / NT);
-    gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT><<<grid, 64, 0, stream>>>(a);
+    return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT>, dim3(grid), dim3(64), a);
     return hipGetLastError();
 }
 
 template <int TYPE, int NT>
-hipError_t dispatch(GemvArgs& a, int num_cus, hipStream_t stream) {
+hipError_t dispatch(GemvArgs& a, int num_cus, const Launch& L) {
     const uint32_t total_rows = a.batch.row_end[a.batch.count - 1];
     if (total_rows == 0 || a.n == 0) return hipSuccess;
     const uint32_t nb = a.k >> 5;
@@ -239,23 +239,23 @@ hipError_t dispatch(GemvArgs& a, int num_cus, hipStream_t stream) {
     bool aligned = (nb % 2u) == 0 && (reinterpret_cast<uintptr_t>(a.xq) % 16u) == 0;
     for (uint32_t i = 0; i < a.batch.count; i++) aligned = aligned && (reinterpret_cast<uintptr_t>(a.batch.w[i]) % 4u) == 0;
     if (aligned && ppr <= 128) {
-        if (ppr <= 4) return launch_pairs<TYPE, 4, 1, NT>(a, total_rows, num_cus, stream);
-        if (ppr <= 8) return launch_pairs<TYPE, 8, 1, NT>(a, total_rows, num_cus, stream);
-        if (ppr <= 16) return launch_pairs<TYPE, 16, 1, NT>(a, total_rows, num_cus, stream);
-        if (ppr <= 32) return launch_pairs<TYPE, 32, 1, NT>(a, total_rows, num_cus, stream);
-        if (ppr <= 64) return launch_pairs<TYPE, 64, 1, NT>(a, total_rows, num_cus, stream);
-        return launch_pairs<TYPE, 64, 2, NT>(a, total_rows, num_cus, stream);
+        if (ppr <= 4) return launch_pairs<TYPE, 4, 1, NT>(a, total_rows, num_cus, L);
+        if (ppr <= 8) return launch_pairs<TYPE, 8, 1, NT>(a, total_rows, num_cus, L);
+        if (ppr <= 16) return launch_pairs<TYPE, 16, 1, NT>(a, total_rows, num_cus, L);
+        if (ppr <= 32) return launch_pairs<TYPE, 32, 1, NT>(a, total_rows, num_cus, L);
+        if (ppr <= 64) return launch_pairs<TYPE, 64, 1, NT>(a, total_rows, num_cus, L);
+        return launch_pairs<TYPE, 64, 2, NT>(a, total_rows, num_cus, L);
     }
     a.rows_per_wave = 1;
     dim3 grid(total_rows, (a.n + NT - 1) / NT);
-    gemv_generic_kernel<TYPE, NT><<<grid, 64, 0, stream>>>(a);
+    return launch_kernel(L, kFamGemv, gemv_generic_kernel<TYPE, NT>, dim3(grid), dim3(64), a);
     return hipGetLastError();
 }
 
 }  // namespace
 
 hipError_t launch_gemv(int type, const GemvBatch& batch, uint32_t k, const int8_t* d_q, const float* d_scales,
-                       int accumulate, int num_cus, hipStream_t stream) {
+                       int accumulate, int num_cus, const Launch& L) {
     GemvArgs a{};
     a.batch = batch;
     a.xq = d_q;
@@ -265,12 +265,12 @@ hipError_t launch_gemv(int type, const GemvBatch& batch, uint32_t k, const int8_
     a.y_stride = 0;
     a.y_row_major = 0;
     a.accumulate = accumulate;
-    return type == kTypeQ4_0 ? dispatch<2, 1>(a, num_cus, stream) : dispatch<8, 1>(a, num_cus, stream);
+    return type == kTypeQ4_0 ? dispatch<2, 1>(a, num_cus, L) : dispatch<8, 1>(a, num_cus, L);
 }
 
 hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                               const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
-                              int accumulate, int num_cus, hipStream_t stream) {
+                              int accumulate, int num_cus, const Launch& L) {
     GemvArgs a{};
     a.batch.w[0] = d_w;
     a.batch.y[0] = d_y;
@@ -283,8 +283,8 @@ hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t
     a.y_stride = y_stride;
     a.y_row_major = (y_layout == 1);
     a.accumulate = accumulate;
-    if (n == 1) return type == kTypeQ4_0 ? dispatch<2, 1>(a, num_cus, stream) : dispatch<8, 1>(a, num_cus, stream);
-    return type == kTypeQ4_0 ? dispatch<2, 4>(a, num_cus, stream) : dispatch<8, 4>(a, num_cus, stream);
+    if (n == 1) return type == kTypeQ4_0 ? dispatch<2, 1>(a, num_cus, L) : dispatch<8, 1>(a, num_cus, L);
+    return type == kTypeQ4_0 ? dispatch<2, 4>(a, num_cus, L) : dispatch<8, 4>(a, num_cus, L);
 }
 
 }  // namespace wick_rocm

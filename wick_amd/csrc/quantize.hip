@@ -61,15 +61,15 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* __restr
 }  // namespace
 
 hipError_t launch_quantize_q8_0(const float* d_x, uint32_t n, uint32_t k, uint32_t x_stride, int8_t* d_q,
-                                float* d_scales, hipStream_t stream) {
+                                float* d_scales, const Launch& L) {
     const uint64_t total = (uint64_t)n * (k >> 2);
     if (total == 0) return hipSuccess;
     const uint32_t blocks = (uint32_t)((total + 255) / 256);
     const bool vec4 = ((reinterpret_cast<uintptr_t>(d_x) & 15u) == 0) && (x_stride % 4u == 0);
     if (vec4)
-        quantize_q8_0_kernel<true><<<blocks, 256, 0, stream>>>(d_x, n, k, x_stride, d_q, d_scales);
+        return launch_kernel(L, kFamQuantize, quantize_q8_0_kernel<true>, dim3(blocks), dim3(256), d_x, n, k, x_stride, d_q, d_scales);
     else
-        quantize_q8_0_kernel<false><<<blocks, 256, 0, stream>>>(d_x, n, k, x_stride, d_q, d_scales);
+        return launch_kernel(L, kFamQuantize, quantize_q8_0_kernel<false>, dim3(blocks), dim3(256), d_x, n, k, x_stride, d_q, d_scales);
     return hipGetLastError();
 }
 

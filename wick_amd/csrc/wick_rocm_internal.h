@@ -2,8 +2,11 @@
 // layer.  Not installed; the public surface is include/wick_rocm.h.
 #pragma once
 
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <vector>
 
 namespace wick_rocm {
 
@@ -24,32 +27,77 @@ struct GemvBatch {
     uint32_t count;
 };
 
-// Launchers.  All only enqueue on `stream`; callers have validated shapes.
+// Per-dispatch GPU timestamps (the counterpart of the reference's GpuTimer,
+// wick/src/model/metal_lfm2.rs:3367-4116).  While enabled, every kernel is
+// launched with a start/stop event pair bound to its own dispatch packet
+// (hipExtLaunchKernelGGL), so the elapsed time is the kernel's execution time
+// alone, the same quantity a kernel trace reports.
+enum KernelFamily { kFamQuantize = 0, kFamGemv = 1, kFamGemm = 2, kFamOther = 3, kNumFamilies = 4 };
+
+struct KernelTimer {
+    struct Rec {
+        hipEvent_t start, stop;
+        int family;
+    };
+    bool enabled = false;
+    std::vector<Rec> recs;    // launches since timing began
+    std::vector<Rec> spares;  // event pairs kept for reuse
+};
+
+struct Launch {
+    hipStream_t stream;
+    KernelTimer* timer;  // may be null
+};
+
+template <typename... KArgs, typename... Args>
+inline hipError_t launch_kernel(const Launch& L, int family, void (*kernel)(KArgs...), dim3 grid, dim3 block,
+                                Args... args) {
+    if (L.timer && L.timer->enabled) {
+        KernelTimer::Rec r{};
+        if (!L.timer->spares.empty()) {
+            r = L.timer->spares.back();
+            L.timer->spares.pop_back();
+        } else {
+            hipError_t e = hipEventCreate(&r.start);
+            if (e != hipSuccess) return e;
+            e = hipEventCreate(&r.stop);
+            if (e != hipSuccess) return e;
+        }
+        r.family = family;
+        hipExtLaunchKernelGGL(kernel, grid, block, 0, L.stream, r.start, r.stop, 0, args...);
+        L.timer->recs.push_back(r);
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, 0, L.stream, args...);
+    }
+    return hipGetLastError();
+}
+
+// Launchers.  All only enqueue on L.stream; callers have validated shapes.
 // They return hipGetLastError() after the launch.
 
 hipError_t launch_quantize_q8_0(const float* d_x, uint32_t n, uint32_t k, uint32_t x_stride, int8_t* d_q,
-                                float* d_scales, hipStream_t stream);
+                                float* d_scales, const Launch& L);
 
 // Decode GEMV, one token.  k % 32 == 0.
 hipError_t launch_gemv(int type, const GemvBatch& batch, uint32_t k, const int8_t* d_q, const float* d_scales,
-                       int accumulate, int num_cus, hipStream_t stream);
+                       int accumulate, int num_cus, const Launch& L);
 
 // Small-n GEMM done as a multi-token GEMV (weights streamed once per 1..kGemvTokens tokens).
 hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                               const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
-                              int accumulate, int num_cus, hipStream_t stream);
+                              int accumulate, int num_cus, const Launch& L);
 
 // int8-MFMA GEMM.  Requires k % 256 == 0.
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                             const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
-                            int accumulate, hipStream_t stream);
+                            int accumulate, const Launch& L);
 
 // Per-block i32 dots, out[(j*m + i)*nb + b], through the same unpack + v_dot4 code
 // as the GEMV, or through the GEMM's loads / LDS layout / MFMA (k % 256 == 0).
 hipError_t launch_block_dots_dot4(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,
-                                  int32_t* d_out, hipStream_t stream);
+                                  int32_t* d_out, const Launch& L);
 hipError_t launch_block_dots_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,
-                                  int32_t* d_out, hipStream_t stream);
+                                  int32_t* d_out, const Launch& L);
 
 // n at and above which gemm_q8 uses the MFMA kernel (when k % 256 == 0).
 constexpr uint32_t kGemmMinN = 16;  // cf. GEMM_MIN_N, wick/src/model/metal_lfm2.rs:18-21

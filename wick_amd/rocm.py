@@ -89,6 +89,8 @@ _SIGNATURES = {
     "wick_rocm_event_record": (C.c_int, [_P, _P]),
     "wick_rocm_event_elapsed_ms": (C.c_int, [_P, _P, _P, C.POINTER(C.c_float)]),
     "wick_rocm_event_destroy": (C.c_int, [_P, _P]),
+    "wick_rocm_kernel_timing_begin": (C.c_int, [_P]),
+    "wick_rocm_kernel_timing_end": (C.c_int, [_P, C.POINTER(C.c_double), C.POINTER(C.c_uint64), C.c_int]),
 }
 
 
@@ -285,6 +287,18 @@ class RocmContext:
         ms = C.c_float(0)
         self._check(self._lib.wick_rocm_event_elapsed_ms(self._h, start, stop, C.byref(ms)))
         return ms.value
+
+    FAMILIES = ("quantize", "gemv", "gemm", "other")
+
+    def kernel_timing_begin(self) -> None:
+        self._check(self._lib.wick_rocm_kernel_timing_begin(self._h))
+
+    def kernel_timing_end(self) -> dict:
+        """{family: (total_ms, launches)} of the kernels launched since kernel_timing_begin."""
+        ms = (C.c_double * 4)()
+        cnt = (C.c_uint64 * 4)()
+        self._check(self._lib.wick_rocm_kernel_timing_end(self._h, ms, cnt, 4))
+        return {f: (ms[i], int(cnt[i])) for i, f in enumerate(self.FAMILIES)}
 
     def event_destroy(self, e: int) -> None:
         self._check(self._lib.wick_rocm_event_destroy(self._h, e))
