@@ -3,10 +3,10 @@
 
 A "step" is one pass of the decode hot path over the LFM2-350M-shaped weight set
 (hidden 1024, 10 short-conv + 6 attention layers, FFN 4608, tied LM head
-65536 x 1024) at n = 1: 65 Q8_0 activation quantizations and 65 GEMV launches
+65536 x 1024) at n = 1: 65 Q8_0 activation quantizations fused into 65 GEMV launches
 covering 93 weight matrices ({Q,K,V} and {gate,up} share one quantized activation
-and one launch, like the reference's call sites), submitted as ONE HIP graph per
-token.  Two distinct device copies of the weight set are alternated so every step
+and one launch, like the reference's call sites; the quantization runs inside the
+GEMV kernel), submitted as ONE HIP graph per token.  Two distinct device copies of the weight set are alternated so every step
 streams its weights from HBM, not from the 256 MB Infinity Cache.
 
 Prints one JSON line: `value` = algorithmic GEMV bytes per step / step time, plus
@@ -93,13 +93,15 @@ class DecodeStep:
         self.d_q = ctx.alloc(IS)
         self.d_s = ctx.alloc(IS // 32 * 4)
 
-    def enqueue(self):
+    def enqueue(self, fused=True):
+        """fused: one launch per call site, the Q8_0 quantization of the activation is done
+        inside the GEMV kernel.  Otherwise quantize and GEMV are separate launches."""
         ctx = self.ctx
         for ws, ys, k in self.sites:
-            ctx.quantize_q8_0(self.d_x[k], 1, k, k, self.d_q, self.d_s)
-            if len(ws) == 1:
-                ctx.gemv_with_preq(ws[0], self.d_s, self.d_q, ys[0])
+            if fused:
+                ctx.encode_gemv_fused(ws, self.d_x[k], 0, ys)
             else:
+                ctx.quantize_q8_0(self.d_x[k], 1, k, k, self.d_q, self.d_s)
                 ctx.gemv_with_preq_multi(ws, self.d_s, self.d_q, ys)
 
 
@@ -149,9 +151,16 @@ def bench_decode(ctx, W, O, dtype, steps, warmup, host_weights):
         "gemv_kernel_ms_per_step": kt["gemv"][0] / steps,
         "gemv_kernel_GBps": gbytes / (kt["gemv"][0] / steps) / 1e6,
         "gemv_kernel_avg_us": kt["gemv"][0] / kt["gemv"][1] * 1e3,
-        "quantize_kernel_ms_per_step": kt["quantize"][0] / steps,
-        "quantize_kernel_avg_us": kt["quantize"][0] / kt["quantize"][1] * 1e3,
     }
+    # the same step with the quantizer as its own launch (two launches per call site)
+    graphs2 = []
+    for c in copies:
+        ctx.graph_begin()
+        c.enqueue(fused=False)
+        graphs2.append(ctx.graph_end())
+    res["ms_per_step_unfused_quantizer"] = time_graphs(ctx, graphs2, steps, warmup)
+    for g in graphs2:
+        ctx.graph_destroy(g)
     for g in graphs:
         ctx.graph_destroy(g)
     for c in copies:
@@ -288,10 +297,10 @@ def main():
         "dtype": "i8",
         "data": "synthetic",
         "config": {
-            "workload": "LFM2-350M-shaped decode-step weight set, Q4_0 weights x Q8_0 activations, n=1: 93 GEMVs in 65 launches "
-                        "+ 65 activation quantizations per step, one HIP graph per step, two weight copies alternated (HBM-cold)",
+            "workload": "LFM2-350M-shaped decode-step weight set, Q4_0 weights x Q8_0 activations, n=1: 93 GEMVs in 65 launches, "
+                        "each quantizing its f32 activation in-kernel; one HIP graph per step, two weight copies alternated (HBM-cold)",
             "device": ctx.device_name,
-            "value_definition": "algorithmic GEMV bytes per step (weights + Q8_0 activations + f32 outputs) / step time, quantizer launches included in the time",
+            "value_definition": "algorithmic GEMV bytes per step (weights + Q8_0 activations + f32 outputs) / step time, activation quantization included in the time",
         },
         "roofline": {
             "bound": "hbm",

@@ -148,6 +148,16 @@ int wick_rocm_gemm_q8(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_
  * Offsets are in bytes like the reference's. */
 int wick_rocm_matmul_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const float *d_x, size_t x_off_bytes, uint32_t n,
                          uint32_t x_stride, float *d_y, size_t y_off_bytes, uint32_t y_stride, int accumulate);
+/* encode_gemv_qkv / encode_gemv_gate_up (wick/src/model/metal_lfm2.rs:1043-1119):
+ * up to four weights sharing k and dtype against ONE f32 activation vector read at
+ * d_x + x_off_bytes, y_i (+)= W_i x, in a single launch.  The Q8_0 quantization of x
+ * happens inside the GEMV kernel (bit-identical to wick_rocm_quantize_q8_0); shapes
+ * the fused kernel does not take (odd block count per row, k > 8192, x not 16-byte
+ * aligned) quantize into context scratch first.  wick_rocm_matmul_f32 with n = 1
+ * takes the same route. */
+int wick_rocm_gemv_f32_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *ws, float *const *d_ys, uint32_t count,
+                             const float *d_x, size_t x_off_bytes, int accumulate);
+
 /* Pre-sizes the scratch used by wick_rocm_matmul_f32 for up to max_n columns of
  * up to max_k elements (call before capturing a graph). */
 int wick_rocm_reserve_scratch(wick_rocm_ctx *ctx, uint32_t max_n, uint32_t max_k);

@@ -92,3 +92,52 @@ def test_graph_replay_matches_eager(ctx, oracle):
         w.free()
     for b in (d_x, d_q, d_s, d_g, d_u, d_o):
         b.free()
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+@pytest.mark.parametrize("ms,k", [((1024, 512, 512), 1024), ((4608, 4608), 1024), ((1024,), 4608), ((2048,), 6912), ((300,), 2048),
+                                  ((7, 5), 96), ((16,), 16384), ((9,), 64)])
+def test_fused_quantize_gemv_is_bit_identical_to_two_steps(ctx, oracle, dtype, ms, k):
+    """encode_gemv_qkv / encode_gemv_gate_up shape: f32 activation in, the Q8_0
+    quantization done inside the GEMV kernel.  The result must be BIT-identical to
+    quantize_q8_0 followed by gemv_with_preq (same quants, same arithmetic), for the
+    shapes the fused kernel takes and for the ones that fall back."""
+    x = oracle.fill_normal(k + len(ms), 1.0, k + 8)
+    d_x = ctx.to_device(x)
+    wbs = [oracle.synth_weight(dtype, m, k, seed=200 + i) for i, m in enumerate(ms)]
+    ws = [ctx.upload_weight(wb, dtype, m, k) for wb, m in zip(wbs, ms)]
+    ys = [ctx.alloc(m * 4) for m in ms]
+    ys2 = [ctx.alloc(m * 4) for m in ms]
+    for off in (0, 8 * 4, 4):  # 16-byte aligned twice, then a 4-byte-aligned source (fallback)
+        ctx.encode_gemv_fused(ws, d_x, off, ys)
+        d_q, d_s = ctx.alloc(k), ctx.alloc(k // 32 * 4)
+        ctx.quantize_q8_0(d_x.ptr + off, 1, k, k, d_q, d_s)
+        ctx.gemv_with_preq_multi(ws, d_s, d_q, ys2)
+        s, q = oracle.quantize_q8_0(x[off // 4:off // 4 + k])
+        for wb, m, y, y2 in zip(wbs, ms, ys, ys2):
+            got = y.download(np.float32, m)
+            assert np.array_equal(got.view(np.uint32), y2.download(np.float32, m).view(np.uint32))
+            assert_f32_parity(got, oracle.gemv_q8(dtype, wb, s, q, m, k), f"fused m={m} k={k} off={off}")
+        d_q.free(), d_s.free()
+    for w in ws:
+        w.free()
+    for b in [d_x] + ys + ys2:
+        b.free()
+
+
+def test_fused_gemv_edge_activations(ctx, oracle):
+    """All-zero blocks, one huge element, tiny values: the in-kernel quantizer follows
+    the same edge rules as the stand-alone one."""
+    m, k = 64, 256
+    x = oracle.fill_normal(3, 1.0, k)
+    x[0:32] = 0.0
+    x[40] = 1e4
+    x[64:96] *= 1e-20
+    x[100] = -0.0
+    wb = oracle.synth_weight(W.Q4_0, m, k, seed=6)
+    w = ctx.upload_weight(wb, W.Q4_0, m, k)
+    d_x, d_y = ctx.to_device(x), ctx.alloc(m * 4)
+    ctx.encode_gemv(w, d_x, 0, d_y, 0)
+    s, q = oracle.quantize_q8_0(x)
+    assert_f32_parity(d_y.download(np.float32, m), oracle.gemv_q8(W.Q4_0, wb, s, q, m, k), "fused edge")
+    w.free(), d_x.free(), d_y.free()

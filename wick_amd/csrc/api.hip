@@ -115,7 +115,7 @@ int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q
         return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "unknown output layout");
     if (y_layout == WICK_ROCM_LAYOUT_TOKEN_MAJOR ? (y_stride < w->m && n > 1) : (y_stride < n))
         return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "y_stride smaller than the output extent");
-    const bool mfma_ok = (w->k % 256u == 0) && (reinterpret_cast<uintptr_t>(d_q) % 16u == 0) &&
+    const bool mfma_ok = (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_q) % 16u == 0) &&
                          (reinterpret_cast<uintptr_t>(d_s) % 16u == 0);
     hipError_t e;
     if (n >= kGemmMinN && mfma_ok)
@@ -315,29 +315,66 @@ int wick_rocm_quantize_q8_0(wick_rocm_ctx* ctx, const float* d_x, uint32_t n, ui
     return WICK_ROCM_OK;
 }
 
-int wick_rocm_gemv_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count,
-                            const int8_t* d_quants, const float* d_scales, int accumulate) {
-    WR_ENTER(ctx);
-    if (!ws || !d_ys || !d_quants || !d_scales) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv: null pointer");
-    if (count == 0 || count > (uint32_t)kMaxGemvBatch)
-        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv_q8_multi: count must be 1..4");
-    GemvBatch b{};
+namespace {
+
+// Validates a group of weights sharing one activation and fills the launch batch.
+int make_batch(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count, GemvBatch& b) {
+    if (!ws || !d_ys) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv: null pointer");
+    if (count == 0 || count > (uint32_t)kMaxGemvBatch) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv multi: count must be 1..4");
     uint32_t rows = 0;
     for (uint32_t i = 0; i < count; i++) {
         if (int rc = check_weight(ctx, ws[i])) return rc;
         if (!d_ys[i]) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv: null output pointer");
         if (ws[i]->k != ws[0]->k || ws[i]->type != ws[0]->type)
-            return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "gemv_q8_multi: weights must share k and dtype");
-        if ((uint64_t)rows + ws[i]->m > 0xffffffffull) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "gemv_q8_multi: too many rows");
+            return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "gemv multi: weights must share k and dtype");
+        if ((uint64_t)rows + ws[i]->m > 0xffffffffull) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "gemv multi: too many rows");
         rows += ws[i]->m;
         b.w[i] = static_cast<const uint8_t*>(ws[i]->d);
         b.y[i] = d_ys[i];
         b.row_end[i] = rows;
     }
     b.count = count;
+    return WICK_ROCM_OK;
+}
+
+// f32 activations -> y for a group of weights (lock held): fused quantize+GEMV when
+// the pair kernel takes the shape, otherwise quantize into scratch, then GEMV.
+int gemv_f32_locked(wick_rocm_ctx* ctx, const GemvBatch& b, int type, uint32_t k, const float* x, int accumulate) {
+    if (pairs_kernel_applies(b, k) && reinterpret_cast<uintptr_t>(x) % 16u == 0) {
+        hipError_t e = launch_gemv_f32(type, b, k, x, accumulate, ctx->num_cus, ctx->launch());
+        if (e != hipSuccess) return fail_hip(ctx, e, "fused gemv launch");
+        return WICK_ROCM_OK;
+    }
+    if (int rc = ensure_scratch(ctx, k, k / 32u)) return rc;
+    hipError_t e = launch_quantize_q8_0(x, 1, k, k, ctx->scratch_q, ctx->scratch_s, ctx->launch());
+    if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
+    e = launch_gemv(type, b, k, ctx->scratch_q, ctx->scratch_s, accumulate, ctx->num_cus, ctx->launch());
+    if (e != hipSuccess) return fail_hip(ctx, e, "gemv launch");
+    return WICK_ROCM_OK;
+}
+
+}  // namespace
+
+int wick_rocm_gemv_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count,
+                            const int8_t* d_quants, const float* d_scales, int accumulate) {
+    WR_ENTER(ctx);
+    if (!d_quants || !d_scales) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv: null pointer");
+    GemvBatch b{};
+    if (int rc = make_batch(ctx, ws, d_ys, count, b)) return rc;
     hipError_t e = launch_gemv(ws[0]->type, b, ws[0]->k, d_quants, d_scales, accumulate, ctx->num_cus, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "gemv launch");
     return WICK_ROCM_OK;
+}
+
+int wick_rocm_gemv_f32_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count,
+                             const float* d_x, size_t x_off_bytes, int accumulate) {
+    WR_ENTER(ctx);
+    if (!d_x) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv_f32_multi: null activation pointer");
+    if (x_off_bytes % 4u) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv_f32_multi: offset must be a multiple of 4");
+    GemvBatch b{};
+    if (int rc = make_batch(ctx, ws, d_ys, count, b)) return rc;
+    const float* x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes);
+    return gemv_f32_locked(ctx, b, ws[0]->type, ws[0]->k, x, accumulate);
 }
 
 int wick_rocm_gemv_q8(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_quants, const float* d_scales,
@@ -371,6 +408,11 @@ int wick_rocm_matmul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const fl
         return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "matmul_f32: stride smaller than the vector length");
     const float* x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes);
     float* y = reinterpret_cast<float*>(reinterpret_cast<char*>(d_y) + y_off_bytes);
+    if (n == 1) {
+        GemvBatch b{};
+        b.w[0] = static_cast<const uint8_t*>(w->d), b.y[0] = y, b.row_end[0] = w->m, b.count = 1;
+        return gemv_f32_locked(ctx, b, w->type, w->k, x, accumulate);
+    }
     if (int rc = ensure_scratch(ctx, (size_t)n * w->k, (size_t)n * (w->k / 32u))) return rc;
     hipError_t e = launch_quantize_q8_0(x, n, w->k, x_stride, ctx->scratch_q, ctx->scratch_s, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
@@ -384,7 +426,7 @@ int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, cons
     if (int rc = check_weight(ctx, w)) return rc;
     if (!d_quants || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "block_dots: null device pointer");
     if (n == 0) return WICK_ROCM_OK;
-    const bool mfma = n >= kGemmMinN && (w->k % 256u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
+    const bool mfma = n >= kGemmMinN && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
     hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch())
                         : launch_block_dots_dot4(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "block_dots launch");

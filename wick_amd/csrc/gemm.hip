@@ -9,29 +9,31 @@
 // 32x32 i32 result is scaled into f32 accumulators on the vector ALU.
 //
 // Workgroup = 256 threads = 4 waves, tile = 128 weight rows x 128 tokens, each
-// wave owns 64 x 64 (2 x 2 MFMA tiles).  One stage = 8 blocks (256 elements of K):
-//   * weights: each thread reads two 36/68-byte block pairs with dword-aligned
-//     wide loads (a row contributes 144/272 contiguous bytes per stage), unpacks
-//     nibbles to int8 and writes 16-byte operand rows to LDS;
+// wave owns 64 x 64 (2 x 2 MFMA tiles).  One stage = 4 blocks (128 elements of K):
+//   * weights: each thread reads one 36/68-byte block pair with dword-aligned wide
+//     loads, unpacks nibbles to int8 and writes 16-byte operand rows to LDS;
 //   * activations: 16-byte chunks copied global -> LDS; scales alongside.
-// Global loads of stage s+1 are in flight (held in registers) while stage s is
-// computed from LDS.
+// LDS holds two stages.  The global loads of stage s+1 are issued before stage s is
+// computed and written to the other LDS buffer after it, so there is one barrier
+// per stage and the load latency hides behind the stage's ALU work.
 //
-// LDS operand layout: [block][khalf][row][16 bytes] (planes ordered the other
-// way round for weights; see Smem).  An MFMA lane supplies 16
+// LDS operand layout: [block][khalf][row][16 bytes].  An MFMA lane supplies 16
 // consecutive K-bytes of one operand row, lanes 0-31 the first half of the block
 // and lanes 32-63 the second, so 32 consecutive lanes read 512 consecutive bytes:
-// conflict-free without padding.  For Q4_0 the low nibbles of a block ARE its
-// first 16 elements and the high nibbles its last 16 (wick/src/quant.rs:82-88),
-// so the two halves fall out of one and / shift each.
+// conflict-free.  For Q4_0 the low nibbles of a block ARE its first 16 elements and
+// the high nibbles its last 16 (wick/src/quant.rs:82-88), so the two halves fall
+// out of one and / shift each.  (The K order inside an MFMA is irrelevant as long
+// as both operands use the same one.)
 //
 // Roles: tokens are the MFMA "A" (M) operand, weight rows the "B" (N) operand, so
 // in the 32x32 result a lane holds ONE weight row (n = lane % 32) and 16 tokens
 // (m = 8*(r/4) + 4*(lane/32) + r%4).  Its weight scale is one register per block;
-// the 16 token scales are LDS broadcast reads.
+// the 16 token scales are kept as f16 in LDS, stored in the order a lane consumes
+// them (32 contiguous bytes per lane half, tile and block) and fed to the FMA as
+// f16 operands (v_fma_mix_f32), which is exact because they ARE f16 values.
 //
-// Scaling cost is what bounds this kernel (vector ALU, not the matrix core), so it
-// is cut to two FMAs per result:
+// Scaling is what bounds this kernel (vector ALU, not the matrix core), so it is
+// cut to two FMAs per result:
 //   * Q4_0 nibbles are stored as 16*(nibble-8) (the nibble moved to the top of the
 //     byte, sign bit flipped: two ALU ops per four weights, no per-byte subtract);
 //     the 1/16 is folded into the weight scale.
@@ -50,13 +52,14 @@ namespace {
 
 constexpr int BM = 128;       // weight rows per workgroup
 constexpr int BN = 128;       // tokens per workgroup
-constexpr int KB = 8;         // blocks per stage
+constexpr int KB = 4;         // blocks per stage
 constexpr int THREADS = 256;  // 4 waves: 2 (rows) x 2 (tokens)
 constexpr uint32_t kBiasBits = 0x4B400000u;  // 12582912.0f
 constexpr float kBias = 12582912.0f;
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 
 struct GemmArgs {
     const uint8_t* w;
@@ -71,16 +74,19 @@ struct GemmArgs {
     int accumulate;
 };
 
-// Row counts are padded (one 16-byte operand row per plane, four floats per scale
-// row) so that the stage WRITES, where neighbouring lanes hit different planes of
-// the same row, spread over the LDS banks; reads walk consecutive rows of one
-// plane and do not care.
+// One stage of operands.  Row counts are padded (one 16-byte operand row per
+// plane, two float2 per scale row) so that the stage WRITES, where neighbouring
+// lanes hit different planes of the same row, spread over the LDS banks; reads
+// walk consecutive rows of one plane.
+struct Stage {
+    uint4 wt[2][KB][BM + 2];    // [khalf][block][row]  int8 weights (Q4_0: x16)
+    uint4 xt[KB][2][BN + 1];    // [block][khalf][token] int8 activations
+    float2 dws[KB][BM + 2];     // {dw, -12582912*dw} per block and row (dw x 1/16 for Q4_0)
+    h8 dxh[KB][BN / 32][2][2];  // [block][token tile][lane half][2 x 8 halves]: token scales in lane order
+};
+
 struct Smem {
-    uint4 wt[2][KB][BM + 1];  // [khalf][block][row]: int8 operand rows, 16 bytes each
-    uint4 xt[KB][2][BN + 1];  // [block][khalf][token]
-    float dw[KB][BM + 4];   // weight scale (x 1/16 for Q4_0)
-    float ndw[KB][BM + 4];  // -12582912 * dw
-    float dx[KB][BN + 4];   // activation scale
+    Stage st[2];
 };
 
 // 16*(nibble-8) for the four low / four high nibbles of each byte of q.
@@ -89,83 +95,80 @@ __device__ __forceinline__ uint32_t q4_hi_x16(uint32_t q) { return (q & 0xf0f0f0
 
 template <int TYPE>
 struct StageRegs {
-    uint32_t w[2][PairTraits<TYPE>::DWORDS];
-    uint4 x[8];
+    uint32_t w[PairTraits<TYPE>::DWORDS];
+    uint4 x[4];
     float4 dx;
 };
 
+// Thread -> work of one stage:
+//   weights      256 pairs   = 128 rows x 2 pairs             : row = t >> 1, pair = t & 1
+//   activations  1024 chunks = 128 tokens x 8 chunks of 16 B  : id = t + 256 i, token = id >> 3, chunk = id & 7
+//   token scales 128 tokens x 4 blocks (one float4)           : threads 0..127, token = t
 template <int TYPE>
 __device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uint32_t tok0, uint32_t kb0,
                                            StageRegs<TYPE>& r) {
     using PT = PairTraits<TYPE>;
     const uint32_t t = threadIdx.x;
     const uint32_t nb = a.k >> 5;
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const uint32_t id = t + i * THREADS;  // 512 pairs: 128 rows x 4 pairs
-        const uint32_t row = min(row0 + (id >> 2), a.m - 1);
-        const uint32_t pr = id & 3u;
-        const uint8_t* p = a.w + ((size_t)row * nb + kb0 + 2 * pr) * (PT::BYTES / 2);
-        load_pair<PT::DWORDS>(p, r.w[i]);
+    {
+        const uint32_t row = min(row0 + (t >> 1), a.m - 1);
+        const uint8_t* p = a.w + ((size_t)row * nb + kb0 + 2 * (t & 1u)) * (PT::BYTES / 2);
+        load_pair<PT::DWORDS>(p, r.w);
     }
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const uint32_t id = t + i * THREADS;  // 2048 chunks: 128 tokens x 16 chunks of 16 B
-        const uint32_t tok = min(tok0 + (id >> 4), a.n - 1);
-        const uint32_t c = id & 15u;
-        r.x[i] = *reinterpret_cast<const uint4*>(a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + c * 16);
+    for (int i = 0; i < 4; i++) {
+        const uint32_t id = t + i * THREADS;
+        const uint32_t tok = min(tok0 + (id >> 3), a.n - 1);
+        r.x[i] = *reinterpret_cast<const uint4*>(a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + (id & 7u) * 16);
     }
-    if (a.xs) {  // null only for the parity hook, which never scales
-        const uint32_t tok = min(tok0 + (t >> 1), a.n - 1);
-        r.dx = *reinterpret_cast<const float4*>(a.xs + (size_t)tok * nb + kb0 + (t & 1u) * 4);
+    if (t < BN && a.xs) {  // xs is null only for the parity hook, which never scales
+        const uint32_t tok = min(tok0 + t, a.n - 1);
+        r.dx = *reinterpret_cast<const float4*>(a.xs + (size_t)tok * nb + kb0);
     } else {
         r.dx = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 }
 
 template <int TYPE>
-__device__ __forceinline__ void store_stage(Smem& s, const StageRegs<TYPE>& r) {
+__device__ __forceinline__ void store_stage(Stage& s, const StageRegs<TYPE>& r) {
     using PT = PairTraits<TYPE>;
     const uint32_t t = threadIdx.x;
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const uint32_t id = t + i * THREADS;
-        const uint32_t row = id >> 2;
-        const uint32_t pr = id & 3u;
+    {
+        const uint32_t row = t >> 1;
+        const uint32_t b0 = 2 * (t & 1u);
         uint32_t d0, d1, q0[PT::NQ], q1[PT::NQ];
-        split_pair<TYPE>(r.w[i], d0, d1, q0, q1);
+        split_pair<TYPE>(r.w, d0, d1, q0, q1);
         const float scale = (TYPE == 2) ? 0.0625f : 1.0f;
         const float dw0 = f16_bits_to_f32(d0) * scale, dw1 = f16_bits_to_f32(d1) * scale;
-        s.dw[2 * pr][row] = dw0;
-        s.dw[2 * pr + 1][row] = dw1;
-        s.ndw[2 * pr][row] = -kBias * dw0;
-        s.ndw[2 * pr + 1][row] = -kBias * dw1;
+        s.dws[b0][row] = make_float2(dw0, -kBias * dw0);
+        s.dws[b0 + 1][row] = make_float2(dw1, -kBias * dw1);
         if constexpr (TYPE == 2) {
-            s.wt[0][2 * pr][row] = make_uint4(q4_lo_x16(q0[0]), q4_lo_x16(q0[1]), q4_lo_x16(q0[2]), q4_lo_x16(q0[3]));
-            s.wt[1][2 * pr][row] = make_uint4(q4_hi_x16(q0[0]), q4_hi_x16(q0[1]), q4_hi_x16(q0[2]), q4_hi_x16(q0[3]));
-            s.wt[0][2 * pr + 1][row] = make_uint4(q4_lo_x16(q1[0]), q4_lo_x16(q1[1]), q4_lo_x16(q1[2]), q4_lo_x16(q1[3]));
-            s.wt[1][2 * pr + 1][row] = make_uint4(q4_hi_x16(q1[0]), q4_hi_x16(q1[1]), q4_hi_x16(q1[2]), q4_hi_x16(q1[3]));
+            s.wt[0][b0][row] = make_uint4(q4_lo_x16(q0[0]), q4_lo_x16(q0[1]), q4_lo_x16(q0[2]), q4_lo_x16(q0[3]));
+            s.wt[1][b0][row] = make_uint4(q4_hi_x16(q0[0]), q4_hi_x16(q0[1]), q4_hi_x16(q0[2]), q4_hi_x16(q0[3]));
+            s.wt[0][b0 + 1][row] = make_uint4(q4_lo_x16(q1[0]), q4_lo_x16(q1[1]), q4_lo_x16(q1[2]), q4_lo_x16(q1[3]));
+            s.wt[1][b0 + 1][row] = make_uint4(q4_hi_x16(q1[0]), q4_hi_x16(q1[1]), q4_hi_x16(q1[2]), q4_hi_x16(q1[3]));
         } else {
-            s.wt[0][2 * pr][row] = make_uint4(q0[0], q0[1], q0[2], q0[3]);
-            s.wt[1][2 * pr][row] = make_uint4(q0[4], q0[5], q0[6], q0[7]);
-            s.wt[0][2 * pr + 1][row] = make_uint4(q1[0], q1[1], q1[2], q1[3]);
-            s.wt[1][2 * pr + 1][row] = make_uint4(q1[4], q1[5], q1[6], q1[7]);
+            s.wt[0][b0][row] = make_uint4(q0[0], q0[1], q0[2], q0[3]);
+            s.wt[1][b0][row] = make_uint4(q0[4], q0[5], q0[6], q0[7]);
+            s.wt[0][b0 + 1][row] = make_uint4(q1[0], q1[1], q1[2], q1[3]);
+            s.wt[1][b0 + 1][row] = make_uint4(q1[4], q1[5], q1[6], q1[7]);
         }
     }
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < 4; i++) {
         const uint32_t id = t + i * THREADS;
-        const uint32_t tok = id >> 4;
-        const uint32_t c = id & 15u;
-        s.xt[c >> 1][c & 1u][tok] = r.x[i];
+        const uint32_t c = id & 7u;
+        s.xt[c >> 1][c & 1u][id >> 3] = r.x[i];
     }
-    {
-        const uint32_t tok = t >> 1;
-        const uint32_t b4 = (t & 1u) * 4;
-        s.dx[b4 + 0][tok] = r.dx.x;
-        s.dx[b4 + 1][tok] = r.dx.y;
-        s.dx[b4 + 2][tok] = r.dx.z;
-        s.dx[b4 + 3][tok] = r.dx.w;
+    if (t < BN) {
+        // token t of the tile sits at MFMA row t % 32 = 8*gq + 4*g + e -> lane half g, slot 4*gq + e
+        const uint32_t tile = t >> 5, g = (t >> 2) & 1u, slot = ((t >> 3) & 3u) * 4 + (t & 3u);
+        _Float16* base = reinterpret_cast<_Float16*>(&s.dxh[0][tile][g][0]) + slot;
+        constexpr int kBlockStride = sizeof(s.dxh[0]) / sizeof(_Float16);
+        base[0 * kBlockStride] = (_Float16)r.dx.x;  // exact: the scales are f16 values
+        base[1 * kBlockStride] = (_Float16)r.dx.y;
+        base[2 * kBlockStride] = (_Float16)r.dx.z;
+        base[3 * kBlockStride] = (_Float16)r.dx.w;
     }
 }
 
@@ -180,7 +183,7 @@ __device__ __forceinline__ uint32_t tile_of_block(uint32_t bid, uint32_t tiles) 
 
 template <int TYPE, bool DUMP>
 __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
-    __shared__ Smem s;
+    __shared__ Smem sm;
     const uint32_t tiles = a.row_tiles * a.tok_tiles;
     const uint32_t tile = tile_of_block(blockIdx.x, tiles);
     if (tile >= tiles) return;  // whole workgroup leaves together
@@ -190,7 +193,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t l32 = lane & 31u;
-    const uint32_t g = lane >> 5;            // which 16-byte half of the block this lane feeds
+    const uint32_t g = lane >> 5;             // which 16-byte half of the block this lane feeds
     const uint32_t wrow0 = (wave >> 1) * 64;  // wave's rows within the tile
     const uint32_t wtok0 = (wave & 1u) * 64;
     const uint32_t nb = a.k >> 5;
@@ -210,31 +213,35 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
 
     StageRegs<TYPE> regs;
     load_stage<TYPE>(a, row0, tok0, 0, regs);
-    store_stage<TYPE>(s, regs);
+    store_stage<TYPE>(sm.st[0], regs);
     __syncthreads();
 
     for (uint32_t st = 0; st < stages; st++) {
+        const Stage& s = sm.st[st & 1u];
         if (st + 1 < stages) load_stage<TYPE>(a, row0, tok0, (st + 1) * KB, regs);
 
-#pragma unroll 2
+        // 16 MFMA tiles per stage.  Within a wave each MFMA is followed by its 32 FMAs;
+        // the matrix core of a SIMD is kept busy by the other resident wave(s), whose FMA
+        // phases fall into this wave's MFMA latency and vice versa.  The block loop is kept
+        // rolled on purpose: unrolled, the compiler issues all 16 MFMAs of the stage up
+        // front and spills their results.
+#pragma unroll 1
         for (int b = 0; b < KB; b++) {
             v4i av[2], bv[2];
-            float dwv[2], ndwv[2];
-            float4 dxv[2][4];
+            float2 dw[2];
+            h8 dx[2][2];
 #pragma unroll
             for (int tt = 0; tt < 2; tt++) {
                 const uint4 t4 = s.xt[b][g][wtok0 + tt * 32 + l32];
                 av[tt] = v4i{(int)t4.x, (int)t4.y, (int)t4.z, (int)t4.w};
-#pragma unroll
-                for (int gq = 0; gq < 4; gq++)
-                    dxv[tt][gq] = *reinterpret_cast<const float4*>(&s.dx[b][wtok0 + tt * 32 + 8 * gq + 4 * g]);
+                dx[tt][0] = s.dxh[b][(wtok0 >> 5) + tt][g][0];
+                dx[tt][1] = s.dxh[b][(wtok0 >> 5) + tt][g][1];
             }
 #pragma unroll
             for (int rt = 0; rt < 2; rt++) {
                 const uint4 t4 = s.wt[g][b][wrow0 + rt * 32 + l32];
                 bv[rt] = v4i{(int)t4.x, (int)t4.y, (int)t4.z, (int)t4.w};
-                dwv[rt] = s.dw[b][wrow0 + rt * 32 + l32];
-                ndwv[rt] = s.ndw[b][wrow0 + rt * 32 + l32];
+                dw[rt] = s.dws[b][wrow0 + rt * 32 + l32];
             }
 #pragma unroll
             for (int tt = 0; tt < 2; tt++) {
@@ -255,21 +262,17 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
                     } else {
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
-                            const float df = __int_as_float(d[r]);
-                            const float t = __builtin_fmaf(df, dwv[rt], ndwv[rt]);
-                            const float dxs = (r & 3) == 0   ? dxv[tt][r >> 2].x
-                                              : (r & 3) == 1 ? dxv[tt][r >> 2].y
-                                              : (r & 3) == 2 ? dxv[tt][r >> 2].z
-                                                             : dxv[tt][r >> 2].w;
-                            acc[tt][rt][r] = __builtin_fmaf(t, dxs, acc[tt][rt][r]);
+                            const float t = __builtin_fmaf(__int_as_float(d[r]), dw[rt].x, dw[rt].y);
+                            acc[tt][rt][r] = __builtin_fmaf(t, (float)dx[tt][r >> 3][r & 7], acc[tt][rt][r]);
                         }
                     }
                 }
             }
         }
 
-        __syncthreads();
-        if (st + 1 < stages) store_stage<TYPE>(s, regs);
+        // The other buffer was last read in stage st-1; every wave has passed the barrier
+        // that ended that stage, so it is free to be refilled now.
+        if (st + 1 < stages) store_stage<TYPE>(sm.st[(st + 1) & 1u], regs);
         __syncthreads();
     }
 
@@ -300,9 +303,7 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L) {
     const uint32_t blocks = ((tiles + 7u) / 8u) * 8u;  // every XCD gets the same number of slots
     if (type == kTypeQ4_0)
         return launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
-    else
-        return launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
-    return hipGetLastError();
+    return launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
 }
 
 }  // namespace

@@ -30,12 +30,15 @@ namespace {
 
 struct GemvArgs {
     GemvBatch batch;
-    const int8_t* xq;   // [n][k]
+    const int8_t* xq;   // [n][k]      (pre-quantized activations)
     const float* xs;    // [n][k/32]
+    const float* xf;    // [n][x_stride] f32 activations, quantized in-kernel (FUSEQ variants)
+    uint32_t x_stride;
     uint32_t k;
     uint32_t n;         // tokens (1 for decode)
     uint32_t y_stride;  // token-major: >= rows of that weight; row-major: >= n
     uint32_t rows_per_wave;
+    uint32_t wave_end[kMaxGemvBatch];  // running total of waves (workgroups) per weight: a wave never straddles weights
     int y_row_major;
     int accumulate;
 };
@@ -47,80 +50,156 @@ struct ActRegs {
     int sum[NT][2];  // sum of the block's quants (used by Q4_0 only)
 };
 
-template <int TYPE, int LPR, int NCHUNK, int U, int NT>
-__global__ __launch_bounds__(64) void gemv_pairs_kernel(GemvArgs a) {
+// FUSEQ workgroups have four waves that quantize the activation vector together.
+constexpr int kFusedWaves = 4;
+constexpr int kFusedMaxK = 8192;
+
+template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ>
+__global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kernel(GemvArgs a) {
     using PT = PairTraits<TYPE>;
     constexpr int RPW = 64 / LPR;  // rows per wave pass
-    const uint32_t lane = threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u;
     const uint32_t sub = lane % LPR;
     const uint32_t rsel = lane / LPR;
     const uint32_t ppr = a.k >> 6;  // pairs per row
     const uint32_t nb = a.k >> 5;
-    const uint32_t total_rows = a.batch.row_end[a.batch.count - 1];
     const uint32_t tok0 = blockIdx.y * NT;
+
+    // Which weight of the batch this wave works on: scalar, once per wave, and
+    // branch-free so that all kernel arguments arrive in one scalar-load round trip.
+    const uint32_t gwave =
+        FUSEQ ? blockIdx.x * kFusedWaves + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) : blockIdx.x;
+    const uint32_t cnt = a.batch.count;
+    const uint32_t widx = (uint32_t)(cnt > 1 && gwave >= a.wave_end[0]) + (uint32_t)(cnt > 2 && gwave >= a.wave_end[1]) +
+                          (uint32_t)(cnt > 3 && gwave >= a.wave_end[2]);
+    // widx is wave-uniform: these are scalar loads from the argument block at a computed offset.
+    const uint8_t* wbase = a.batch.w[widx];
+    float* ybase = a.batch.y[widx];
+    const uint32_t rows = a.batch.row_end[widx] - (widx ? a.batch.row_end[widx - 1] : 0u);
+    const uint32_t wave = gwave - (widx ? a.wave_end[widx - 1] : 0u);
+    // Waves past the end of the batch (last workgroup of a fused launch) get an empty row
+    // range but still take part in the cooperative quantization and its barrier.
+    const bool live_wave = gwave < a.wave_end[cnt - 1];
+    const uint32_t wave_row0 = live_wave ? wave * a.rows_per_wave : 0;
+    const uint32_t wave_row1 = live_wave ? min(wave_row0 + a.rows_per_wave, rows) : 0;
+
+    bool pvalid[NCHUNK];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; c++) pvalid[c] = c * LPR + sub < ppr;
+
+    // Weight registers of one pass (U rows per lane) and where each row's result goes.
+    uint32_t w[U][NCHUNK][PT::DWORDS];
+    bool rvalid[U];
+    uint32_t lrow[U];
+    // Loads are unconditional (row and pair indices clamped into range) so that the number
+    // of outstanding loads is known at every wait; a clamped load's data is neutralised by
+    // zero activation scales (pair out of range) or simply not stored (row out of range).
+    auto issue_pass = [&](uint32_t base) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            lrow[u] = base + u * RPW + rsel;
+            rvalid[u] = lrow[u] < wave_row1;
+            const uint8_t* rowp = wbase + (size_t)min(lrow[u], rows - 1) * ppr * PT::BYTES;
+#pragma unroll
+            for (int c = 0; c < NCHUNK; c++) {
+                const uint32_t p = pvalid[c] ? c * LPR + sub : 0;
+                load_pair<PT::DWORDS>(rowp + (size_t)p * PT::BYTES, w[u][c]);
+            }
+        }
+    };
+
+    // Order of the memory operations matters because the load counter retires in order:
+    //   1. (fused) this thread's share of the f32 activation vector,
+    //   2. the weight loads of the first pass (the long pole, HBM),
+    //   3. wait for (1) only, quantize into LDS, barrier -- all under the latency of (2).
+    __shared__ __align__(16) uint32_t fq[FUSEQ ? kFusedMaxK / 4 : 4];
+    __shared__ float fs[FUSEQ ? kFusedMaxK / 32 : 1];
+    constexpr int kQuadRounds = kFusedMaxK / 4 / (64 * kFusedWaves);  // 8
+    float4 xv[FUSEQ ? kQuadRounds : 1];
+    if constexpr (FUSEQ) {
+        const uint32_t quads = a.k >> 2;
+#pragma unroll
+        for (int i = 0; i < kQuadRounds; i++) {
+            const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
+            xv[i] = reinterpret_cast<const float4*>(a.xf)[min(quad, quads - 1)];  // clamped, unconditional
+        }
+        // keep the compiler from moving the weight loads in front of these
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    issue_pass(wave_row0);
+    if constexpr (FUSEQ) {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // Fused variant: the workgroup quantizes the f32 activation vector ONCE, together,
+    // into LDS (eight lanes per 32-element block, exactly like the stand-alone quantizer
+    // kernel), instead of every wave redoing it.  Only n = 1 uses this variant.
+    if constexpr (FUSEQ) {
+        const uint32_t quads = a.k >> 2;
+#pragma unroll
+        for (int i = 0; i < kQuadRounds; i++) {
+            const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
+            if (i * 64 * kFusedWaves < quads) {  // uniform: whole rounds only differ in their tail
+                const float4 v = xv[i];
+                float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+                amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+                float id;
+                const float scale = q8_scale_and_inverse(amax, id);
+                if (quad < quads) {
+                    fq[quad] = q8_pack4(v.x, v.y, v.z, v.w, id);
+                    if ((quad & 7u) == 0) fs[quad >> 3] = scale;
+                }
+            }
+        }
+        __syncthreads();
+    }
 
     // This lane's slice of the activations, kept in registers.
     ActRegs<TYPE, NT> act[NCHUNK];
-    bool pvalid[NCHUNK];
 #pragma unroll
     for (int c = 0; c < NCHUNK; c++) {
         const uint32_t p = c * LPR + sub;
-        pvalid[c] = p < ppr;
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             const bool ok = pvalid[c] && (tok0 + t < a.n);
             const uint32_t tok = ok ? tok0 + t : 0;
             const uint32_t pp = ok ? p : 0;
-            const uint4* src = reinterpret_cast<const uint4*>(a.xq + (size_t)tok * a.k + (size_t)pp * 64);
+            if constexpr (FUSEQ) {
+                // This lane's two blocks, from the copy the workgroup quantized into LDS.
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                uint4 lo = src[2 * h], hi = src[2 * h + 1];
-                if (!ok) lo = hi = make_uint4(0, 0, 0, 0);
-                act[c].q[t][h][0] = lo.x, act[c].q[t][h][1] = lo.y, act[c].q[t][h][2] = lo.z, act[c].q[t][h][3] = lo.w;
-                act[c].q[t][h][4] = hi.x, act[c].q[t][h][5] = hi.y, act[c].q[t][h][6] = hi.z, act[c].q[t][h][7] = hi.w;
-                act[c].sum[t][h] = (TYPE == 2) ? block_xsum(act[c].q[t][h]) : 0;
-                const float sc = a.xs[(size_t)tok * nb + 2 * pp + h];
-                act[c].s[t][h] = ok ? sc : 0.0f;
+                for (int h = 0; h < 2; h++) {
+                    const uint4 lo = *reinterpret_cast<const uint4*>(&fq[pp * 16 + h * 8]);
+                    const uint4 hi = *reinterpret_cast<const uint4*>(&fq[pp * 16 + h * 8 + 4]);
+                    act[c].q[t][h][0] = ok ? lo.x : 0, act[c].q[t][h][1] = ok ? lo.y : 0;
+                    act[c].q[t][h][2] = ok ? lo.z : 0, act[c].q[t][h][3] = ok ? lo.w : 0;
+                    act[c].q[t][h][4] = ok ? hi.x : 0, act[c].q[t][h][5] = ok ? hi.y : 0;
+                    act[c].q[t][h][6] = ok ? hi.z : 0, act[c].q[t][h][7] = ok ? hi.w : 0;
+                    act[c].sum[t][h] = (TYPE == 2) ? block_xsum(act[c].q[t][h]) : 0;
+                    act[c].s[t][h] = ok ? fs[2 * pp + h] : 0.0f;
+                }
+            } else {
+                const uint4* src = reinterpret_cast<const uint4*>(a.xq + (size_t)tok * a.k + (size_t)pp * 64);
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    uint4 lo = src[2 * h], hi = src[2 * h + 1];
+                    if (!ok) lo = hi = make_uint4(0, 0, 0, 0);
+                    act[c].q[t][h][0] = lo.x, act[c].q[t][h][1] = lo.y, act[c].q[t][h][2] = lo.z, act[c].q[t][h][3] = lo.w;
+                    act[c].q[t][h][4] = hi.x, act[c].q[t][h][5] = hi.y, act[c].q[t][h][6] = hi.z, act[c].q[t][h][7] = hi.w;
+                    act[c].sum[t][h] = (TYPE == 2) ? block_xsum(act[c].q[t][h]) : 0;
+                    const float sc = a.xs[(size_t)tok * nb + 2 * pp + h];
+                    act[c].s[t][h] = ok ? sc : 0.0f;
+                }
             }
         }
     }
 
-    const uint32_t wave_row0 = blockIdx.x * a.rows_per_wave;
-    const uint32_t wave_row1 = min(wave_row0 + a.rows_per_wave, total_rows);
-
     for (uint32_t base = wave_row0; base < wave_row1; base += RPW * U) {
-        uint32_t w[U][NCHUNK][PT::DWORDS];
-        bool rvalid[U];
-        uint32_t lrow[U];
-        float* yp[U];
-        // Issue every load of this pass first.
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const uint32_t r = base + u * RPW + rsel;
-            rvalid[u] = r < wave_row1;
-            const uint8_t* wp = a.batch.w[0];
-            yp[u] = a.batch.y[0];
-            uint32_t start = 0;
-#pragma unroll
-            for (int i = 1; i < kMaxGemvBatch; i++) {
-                if (i < (int)a.batch.count && r >= a.batch.row_end[i - 1]) {
-                    wp = a.batch.w[i];
-                    yp[u] = a.batch.y[i];
-                    start = a.batch.row_end[i - 1];
-                }
-            }
-            lrow[u] = r - start;
-            const uint8_t* rowp = wp + (size_t)lrow[u] * ppr * PT::BYTES;
-#pragma unroll
-            for (int c = 0; c < NCHUNK; c++) {
-                if (rvalid[u] && pvalid[c]) {
-                    load_pair<PT::DWORDS>(rowp + (size_t)(c * LPR + sub) * PT::BYTES, w[u][c]);
-                } else {
-#pragma unroll
-                    for (int i = 0; i < PT::DWORDS; i++) w[u][c][i] = 0;
-                }
-            }
-        }
+        if (base != wave_row0) issue_pass(base);
         // Consume.
 #pragma unroll
         for (int u = 0; u < U; u++) {
@@ -131,7 +210,7 @@ __global__ __launch_bounds__(64) void gemv_pairs_kernel(GemvArgs a) {
             for (int c = 0; c < NCHUNK; c++) {
                 uint32_t d0, d1, q0[PT::NQ], q1[PT::NQ];
                 split_pair<TYPE>(w[u][c], d0, d1, q0, q1);
-                const float dw0 = f16_bits_to_f32(d0), dw1 = f16_bits_to_f32(d1);
+                const float dw0 = pvalid[c] ? f16_bits_to_f32(d0) : 0.0f, dw1 = pvalid[c] ? f16_bits_to_f32(d1) : 0.0f;
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
                     const int i0 = block_dot<TYPE>(q0, act[c].q[t][0], act[c].sum[t][0]);
@@ -144,8 +223,8 @@ __global__ __launch_bounds__(64) void gemv_pairs_kernel(GemvArgs a) {
             for (int t = 0; t < NT; t++) {
                 const float tot = group_sum<LPR>(acc[t]);
                 if (sub == 0 && rvalid[u] && tok0 + t < a.n) {
-                    float* dst = a.y_row_major ? yp[u] + (size_t)lrow[u] * a.y_stride + (tok0 + t)
-                                               : yp[u] + (size_t)(tok0 + t) * a.y_stride + lrow[u];
+                    float* dst = a.y_row_major ? ybase + (size_t)lrow[u] * a.y_stride + (tok0 + t)
+                                               : ybase + (size_t)(tok0 + t) * a.y_stride + lrow[u];
                     *dst = a.accumulate ? *dst + tot : tot;
                 }
             }
@@ -162,22 +241,22 @@ __global__ __launch_bounds__(64) void gemv_generic_kernel(GemvArgs a) {
     constexpr int NQ = PairTraits<TYPE>::NQ;
     const uint32_t lane = threadIdx.x;
     const uint32_t nb = a.k >> 5;
-    const uint32_t total_rows = a.batch.row_end[a.batch.count - 1];
     const uint32_t tok0 = blockIdx.y * NT;
-    const uint32_t row0 = blockIdx.x * a.rows_per_wave;
-    const uint32_t row1 = min(row0 + a.rows_per_wave, total_rows);
-    for (uint32_t r = row0; r < row1; r++) {
-        const uint8_t* wp = a.batch.w[0];
-        float* yp = a.batch.y[0];
-        uint32_t start = 0;
-        for (uint32_t i = 1; i < a.batch.count; i++) {
-            if (r >= a.batch.row_end[i - 1]) {
-                wp = a.batch.w[i];
-                yp = a.batch.y[i];
-                start = a.batch.row_end[i - 1];
-            }
+    const uint8_t* wp = a.batch.w[0];
+    float* yp = a.batch.y[0];
+    uint32_t rows = a.batch.row_end[0];
+    uint32_t wave = blockIdx.x;
+    for (uint32_t i = 1; i < a.batch.count; i++) {
+        if (blockIdx.x >= a.wave_end[i - 1]) {
+            wp = a.batch.w[i];
+            yp = a.batch.y[i];
+            rows = a.batch.row_end[i] - a.batch.row_end[i - 1];
+            wave = blockIdx.x - a.wave_end[i - 1];
         }
-        const uint32_t lrow = r - start;
+    }
+    const uint32_t row0 = wave * a.rows_per_wave;
+    const uint32_t row1 = min(row0 + a.rows_per_wave, rows);
+    for (uint32_t lrow = row0; lrow < row1; lrow++) {
         const uint8_t* rowp = wp + (size_t)lrow * nb * BB;
         float acc[NT];
 #pragma unroll
@@ -212,7 +291,19 @@ __global__ __launch_bounds__(64) void gemv_generic_kernel(GemvArgs a) {
     }
 }
 
-template <int TYPE, int LPR, int NCHUNK, int NT>
+// Every weight of the batch gets its own whole number of waves.
+inline uint32_t set_wave_ends(GemvArgs& a) {
+    uint32_t waves = 0, prev = 0;
+    for (uint32_t i = 0; i < a.batch.count; i++) {
+        const uint32_t rows = a.batch.row_end[i] - prev;
+        prev = a.batch.row_end[i];
+        waves += (rows + a.rows_per_wave - 1) / a.rows_per_wave;
+        a.wave_end[i] = waves;
+    }
+    return waves;
+}
+
+template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ>
 hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
     // Rows in flight per lane: bounded by registers (a Q8_0 pair is 17 dwords).
     constexpr int U = (TYPE == 2) ? (NCHUNK == 1 ? (NT == 1 ? 4 : 2) : (NT == 1 ? 2 : 1)) : (NCHUNK == 1 && NT == 1 ? 2 : 1);
@@ -224,35 +315,62 @@ hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, const Lau
     uint32_t passes_per_wave = (passes + max_waves - 1) / max_waves;
     if (passes_per_wave == 0) passes_per_wave = 1;
     a.rows_per_wave = passes_per_wave * pass_rows;
-    const uint32_t waves = (total_rows + a.rows_per_wave - 1) / a.rows_per_wave;
+    const uint32_t waves = set_wave_ends(a);
+    if (FUSEQ) {
+        dim3 grid((waves + kFusedWaves - 1) / kFusedWaves, 1);
+        return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ>, grid, dim3(64 * kFusedWaves), a);
+    }
     dim3 grid(waves, (a.n + NT - 1) / NT);
-    return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT>, dim3(grid), dim3(64), a);
+    return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ>, dim3(grid), dim3(64), a);
     return hipGetLastError();
 }
 
-template <int TYPE, int NT>
+// FUSEQ callers have checked that the pair kernel applies (pairs_kernel_applies).
+template <int TYPE, int NT, bool FUSEQ = false>
 hipError_t dispatch(GemvArgs& a, int num_cus, const Launch& L) {
     const uint32_t total_rows = a.batch.row_end[a.batch.count - 1];
     if (total_rows == 0 || a.n == 0) return hipSuccess;
     const uint32_t nb = a.k >> 5;
     const uint32_t ppr = nb >> 1;
-    bool aligned = (nb % 2u) == 0 && (reinterpret_cast<uintptr_t>(a.xq) % 16u) == 0;
+    bool aligned = (nb % 2u) == 0 && (FUSEQ || (reinterpret_cast<uintptr_t>(a.xq) % 16u) == 0);
     for (uint32_t i = 0; i < a.batch.count; i++) aligned = aligned && (reinterpret_cast<uintptr_t>(a.batch.w[i]) % 4u) == 0;
     if (aligned && ppr <= 128) {
-        if (ppr <= 4) return launch_pairs<TYPE, 4, 1, NT>(a, total_rows, num_cus, L);
-        if (ppr <= 8) return launch_pairs<TYPE, 8, 1, NT>(a, total_rows, num_cus, L);
-        if (ppr <= 16) return launch_pairs<TYPE, 16, 1, NT>(a, total_rows, num_cus, L);
-        if (ppr <= 32) return launch_pairs<TYPE, 32, 1, NT>(a, total_rows, num_cus, L);
-        if (ppr <= 64) return launch_pairs<TYPE, 64, 1, NT>(a, total_rows, num_cus, L);
-        return launch_pairs<TYPE, 64, 2, NT>(a, total_rows, num_cus, L);
+        if (ppr <= 4) return launch_pairs<TYPE, 4, 1, NT, FUSEQ>(a, total_rows, num_cus, L);
+        if (ppr <= 8) return launch_pairs<TYPE, 8, 1, NT, FUSEQ>(a, total_rows, num_cus, L);
+        if (ppr <= 16) return launch_pairs<TYPE, 16, 1, NT, FUSEQ>(a, total_rows, num_cus, L);
+        if (ppr <= 32) return launch_pairs<TYPE, 32, 1, NT, FUSEQ>(a, total_rows, num_cus, L);
+        if (ppr <= 64) return launch_pairs<TYPE, 64, 1, NT, FUSEQ>(a, total_rows, num_cus, L);
+        return launch_pairs<TYPE, 64, 2, NT, FUSEQ>(a, total_rows, num_cus, L);
     }
+    if (FUSEQ) return hipErrorInvalidValue;  // unreachable: see pairs_kernel_applies
     a.rows_per_wave = 1;
-    dim3 grid(total_rows, (a.n + NT - 1) / NT);
+    dim3 grid(set_wave_ends(a), (a.n + NT - 1) / NT);
     return launch_kernel(L, kFamGemv, gemv_generic_kernel<TYPE, NT>, dim3(grid), dim3(64), a);
     return hipGetLastError();
 }
 
 }  // namespace
+
+bool pairs_kernel_applies(const GemvBatch& batch, uint32_t k) {
+    const uint32_t nb = k >> 5;
+    if (nb % 2u != 0 || (nb >> 1) > 128) return false;
+    for (uint32_t i = 0; i < batch.count; i++)
+        if (reinterpret_cast<uintptr_t>(batch.w[i]) % 4u != 0) return false;
+    return true;
+}
+
+// f32 activations in, quantized inside the GEMV kernel: one launch instead of two.
+hipError_t launch_gemv_f32(int type, const GemvBatch& batch, uint32_t k, const float* d_x, int accumulate, int num_cus,
+                           const Launch& L) {
+    GemvArgs a{};
+    a.batch = batch;
+    a.xf = d_x;
+    a.x_stride = k;
+    a.k = k;
+    a.n = 1;
+    a.accumulate = accumulate;
+    return type == kTypeQ4_0 ? dispatch<2, 1, true>(a, num_cus, L) : dispatch<8, 1, true>(a, num_cus, L);
+}
 
 hipError_t launch_gemv(int type, const GemvBatch& batch, uint32_t k, const int8_t* d_q, const float* d_scales,
                        int accumulate, int num_cus, const Launch& L) {

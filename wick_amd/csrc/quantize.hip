@@ -9,6 +9,7 @@
 //
 // HBM-bound: reads 4*n*k bytes, writes n*k + 4*n*k/32.  Eight lanes own one
 // 32-element block (one float4 each); amax is reduced with three lane swaps.
+#include "wick_rocm_device.h"
 #include "wick_rocm_internal.h"
 
 namespace wick_rocm {
@@ -41,20 +42,12 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* __restr
     amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
     amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
 
-    const float d = __fdiv_rn(amax, 127.0f);                  // correctly rounded
-    const float id = (d != 0.0f) ? __fdiv_rn(1.0f, d) : 0.0f;  // from the UNROUNDED d
-    const _Float16 dh = (_Float16)d;                           // v_cvt_f16_f32, RNE, subnormals kept
-
-    // x * id, then round-to-nearest-even (v_rndne_f32), then the i32 -> i8 truncation.
-    const int q0 = (int)__builtin_rintf(__fmul_rn(v0, id));
-    const int q1 = (int)__builtin_rintf(__fmul_rn(v1, id));
-    const int q2 = (int)__builtin_rintf(__fmul_rn(v2, id));
-    const int q3 = (int)__builtin_rintf(__fmul_rn(v3, id));
-    const uint32_t packed = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) |
-                            ((uint32_t)(q3 & 0xff) << 24);
+    float id;
+    const float scale = q8_scale_and_inverse(amax, id);
+    const uint32_t packed = q8_pack4(v0, v1, v2, v3, id);
     if (live) {
         *reinterpret_cast<uint32_t*>(q + (size_t)col * k + 4u * quad) = packed;
-        if ((quad & 7u) == 0) scales[(size_t)col * (k >> 5) + (quad >> 3)] = (float)dh;
+        if ((quad & 7u) == 0) scales[(size_t)col * (k >> 5) + (quad >> 3)] = scale;
     }
 }
 

@@ -118,6 +118,25 @@ __device__ __forceinline__ int block_dot(const uint32_t (&q)[PairTraits<TYPE>::N
     }
 }
 
+// Q8_0 activation quantization arithmetic shared by the stand-alone quantizer and the
+// fused GEMV (quantize_f32_to_q8_0_neon, wick/src/backend/simd.rs:255-323): d = amax/127,
+// id = 1/d from the unrounded d, stored scale = f32(f16(d)),
+// q = (i8)(i32) round-ties-even(x * id).  Every step is one correctly rounded
+// binary32 operation.
+__device__ __forceinline__ float q8_scale_and_inverse(float amax, float& id) {
+    const float d = __fdiv_rn(amax, 127.0f);
+    id = (d != 0.0f) ? __fdiv_rn(1.0f, d) : 0.0f;
+    return (float)(_Float16)d;
+}
+
+__device__ __forceinline__ uint32_t q8_pack4(float v0, float v1, float v2, float v3, float id) {
+    const int q0 = (int)__builtin_rintf(__fmul_rn(v0, id));
+    const int q1 = (int)__builtin_rintf(__fmul_rn(v1, id));
+    const int q2 = (int)__builtin_rintf(__fmul_rn(v2, id));
+    const int q3 = (int)__builtin_rintf(__fmul_rn(v3, id));
+    return (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) | ((uint32_t)(q3 & 0xff) << 24);
+}
+
 // Sum over groups of WIDTH consecutive lanes (WIDTH a power of two <= 64); every
 // lane of a group ends with the group's total.
 template <int WIDTH>

@@ -18,8 +18,8 @@ constexpr int kMaxGemvBatch = 4;
 
 inline int block_bytes(int type) { return type == kTypeQ4_0 ? kQ4BlockBytes : (type == kTypeQ8_0 ? kQ8BlockBytes : 0); }
 
-// Up to kMaxGemvBatch weights that share one quantized activation.  Rows of all
-// weights form one concatenated row space [0, row_end[count-1]).
+// Up to kMaxGemvBatch weights that share one quantized activation.  row_end is the
+// running total of rows (row_end[i] - row_end[i-1] = rows of weight i).
 struct GemvBatch {
     const uint8_t* w[kMaxGemvBatch];
     float* y[kMaxGemvBatch];
@@ -81,6 +81,12 @@ hipError_t launch_quantize_q8_0(const float* d_x, uint32_t n, uint32_t k, uint32
 // Decode GEMV, one token.  k % 32 == 0.
 hipError_t launch_gemv(int type, const GemvBatch& batch, uint32_t k, const int8_t* d_q, const float* d_scales,
                        int accumulate, int num_cus, const Launch& L);
+
+// Decode GEMV straight from f32 activations (Q8_0 quantization fused into the
+// kernel).  Only when pairs_kernel_applies() and d_x is 16-byte aligned.
+bool pairs_kernel_applies(const GemvBatch& batch, uint32_t k);
+hipError_t launch_gemv_f32(int type, const GemvBatch& batch, uint32_t k, const float* d_x, int accumulate, int num_cus,
+                           const Launch& L);
 
 // Small-n GEMM done as a multi-token GEMV (weights streamed once per 1..kGemvTokens tokens).
 hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,

@@ -79,6 +79,7 @@ _SIGNATURES = {
     "wick_rocm_gemv_q8_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, _P, C.c_int]),
     "wick_rocm_gemm_q8": (C.c_int, [_P, _P, _P, _P, C.c_uint32, _P, C.c_uint32, C.c_int, C.c_int]),
     "wick_rocm_matmul_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_uint32, C.c_uint32, _P, C.c_size_t, C.c_uint32, C.c_int]),
+    "wick_rocm_gemv_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, C.c_size_t, C.c_int]),
     "wick_rocm_reserve_scratch": (C.c_int, [_P, C.c_uint32, C.c_uint32]),
     "wick_rocm_block_dots_i32": (C.c_int, [_P, _P, _P, C.c_uint32, _P]),
     "wick_rocm_graph_begin": (C.c_int, [_P]),
@@ -255,6 +256,13 @@ class RocmContext:
                     accumulate: bool = False) -> None:
         self._check(self._lib.wick_rocm_matmul_f32(self._h, w.handle, _ptr(x), x_off_bytes, n, x_stride, _ptr(y),
                                                    y_off_bytes, y_stride, int(accumulate)))
+
+    def encode_gemv_fused(self, ws: Sequence[RocmWeight], x, x_off_bytes: int, ys, accumulate: bool = False) -> None:
+        """encode_gemv_qkv / encode_gemv_gate_up: several weights, one f32 activation, one launch."""
+        n = len(ws)
+        wa = (_P * n)(*[w.handle for w in ws])
+        ya = (_P * n)(*[_ptr(y) for y in ys])
+        self._check(self._lib.wick_rocm_gemv_f32_multi(self._h, wa, ya, n, _ptr(x), x_off_bytes, int(accumulate)))
 
     def reserve_scratch(self, max_n: int, max_k: int) -> None:
         self._check(self._lib.wick_rocm_reserve_scratch(self._h, max_n, max_k))
