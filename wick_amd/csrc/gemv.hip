@@ -24,6 +24,8 @@
 #include "wick_rocm_device.h"
 #include "wick_rocm_internal.h"
 
+#include <cstdlib>
+
 namespace wick_rocm {
 
 namespace {
@@ -54,7 +56,7 @@ struct ActRegs {
 constexpr int kFusedWaves = 4;
 constexpr int kFusedMaxK = 8192;
 
-template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ>
+template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI>
 __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kernel(GemvArgs a) {
     using PT = PairTraits<TYPE>;
     constexpr int RPW = 64 / LPR;  // rows per wave pass
@@ -69,10 +71,13 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     // branch-free so that all kernel arguments arrive in one scalar-load round trip.
     const uint32_t gwave =
         FUSEQ ? blockIdx.x * kFusedWaves + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) : blockIdx.x;
-    const uint32_t cnt = a.batch.count;
-    const uint32_t widx = (uint32_t)(cnt > 1 && gwave >= a.wave_end[0]) + (uint32_t)(cnt > 2 && gwave >= a.wave_end[1]) +
-                          (uint32_t)(cnt > 3 && gwave >= a.wave_end[2]);
-    // widx is wave-uniform: these are scalar loads from the argument block at a computed offset.
+    const uint32_t cnt = MULTI ? a.batch.count : 1u;
+    uint32_t widx = 0;
+    if constexpr (MULTI)
+        widx = (uint32_t)(cnt > 1 && gwave >= a.wave_end[0]) + (uint32_t)(cnt > 2 && gwave >= a.wave_end[1]) +
+               (uint32_t)(cnt > 3 && gwave >= a.wave_end[2]);
+    // widx is wave-uniform: these are scalar loads from the argument block at a computed
+    // offset (a second round trip, which single-weight launches do not pay).
     const uint8_t* wbase = a.batch.w[widx];
     float* ybase = a.batch.y[widx];
     const uint32_t rows = a.batch.row_end[widx] - (widx ? a.batch.row_end[widx - 1] : 0u);
@@ -303,26 +308,48 @@ inline uint32_t set_wave_ends(GemvArgs& a) {
     return waves;
 }
 
-template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ>
-hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
-    // Rows in flight per lane: bounded by registers (a Q8_0 pair is 17 dwords).
-    constexpr int U = (TYPE == 2) ? (NCHUNK == 1 ? (NT == 1 ? 4 : 2) : (NT == 1 ? 2 : 1)) : (NCHUNK == 1 && NT == 1 ? 2 : 1);
+template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ, int U>
+hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
     constexpr uint32_t pass_rows = (64 / LPR) * U;
-    // Enough single-wave workgroups to give every CU ~16 waves, and every wave at
-    // least one full pass.
+    // Enough waves to give every CU ~16, and every wave at least one full pass.
     const uint32_t max_waves = (uint32_t)num_cus * 16u;
     uint32_t passes = (total_rows + pass_rows - 1) / pass_rows;
     uint32_t passes_per_wave = (passes + max_waves - 1) / max_waves;
     if (passes_per_wave == 0) passes_per_wave = 1;
     a.rows_per_wave = passes_per_wave * pass_rows;
     const uint32_t waves = set_wave_ends(a);
-    if (FUSEQ) {
-        dim3 grid((waves + kFusedWaves - 1) / kFusedWaves, 1);
-        return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ>, grid, dim3(64 * kFusedWaves), a);
-    }
-    dim3 grid(waves, (a.n + NT - 1) / NT);
-    return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ>, dim3(grid), dim3(64), a);
-    return hipGetLastError();
+    const dim3 grid = FUSEQ ? dim3((waves + kFusedWaves - 1) / kFusedWaves, 1) : dim3(waves, (a.n + NT - 1) / NT);
+    const dim3 block(FUSEQ ? 64 * kFusedWaves : 64);
+    if (a.batch.count > 1)
+        return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true>, grid, block, a);
+    return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false>, grid, block, a);
+}
+
+// Rows in flight per lane (U).  Small matrices are latency-bound: the finer the waves,
+// the sooner every byte is requested and the shorter each wave's unpack/dot tail, so U
+// drops until there are enough waves to cover the chip; big matrices stream with U = 4
+// (Q4_0) / 2 (Q8_0, whose pairs are 17 dwords).  WICK_ROCM_GEMV_U overrides (tuning knob,
+// like the reference's WICK_Q4_FAST / WICK_SPLITS environment switches).
+inline int gemv_u_override() {
+    static const int v = [] {
+        const char* e = getenv("WICK_ROCM_GEMV_U");
+        return e ? atoi(e) : 0;
+    }();
+    return v;
+}
+
+template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ>
+hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
+    constexpr int UMAX = (NT > 1 || NCHUNK > 1) ? (TYPE == 2 && NT == 1 ? 2 : 1) : (TYPE == 2 ? 4 : 2);
+    int u = UMAX;
+    const uint32_t want_waves = (uint32_t)num_cus * 8u;
+    while (u > 1 && total_rows / ((64 / LPR) * u) < want_waves) u >>= 1;
+    if (gemv_u_override() > 0) u = gemv_u_override() < UMAX ? gemv_u_override() : UMAX;
+    if constexpr (UMAX >= 4)
+        if (u >= 4) return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 4>(a, total_rows, num_cus, L);
+    if constexpr (UMAX >= 2)
+        if (u >= 2) return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 2>(a, total_rows, num_cus, L);
+    return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 1>(a, total_rows, num_cus, L);
 }
 
 // FUSEQ callers have checked that the pair kernel applies (pairs_kernel_applies).

@@ -138,11 +138,25 @@ __device__ __forceinline__ uint32_t q8_pack4(float v0, float v1, float v2, float
 }
 
 // Sum over groups of WIDTH consecutive lanes (WIDTH a power of two <= 64); every
-// lane of a group ends with the group's total.
+// lane of a group ends with the group's total.  Within a row of 16 lanes the four
+// butterfly steps are DPP operand modifiers on the add itself (no LDS crossbar, no
+// wait): xor 1 and xor 2 as quad permutes, then the two mirror patterns, which
+// complete the 8- and 16-lane sums because the smaller groups are already uniform.
+// Only the 32- and 64-lane steps go through ds_bpermute.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
+    return v + __builtin_bit_cast(float, moved);
+}
+
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-    for (int off = WIDTH / 2; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    if constexpr (WIDTH >= 2) v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    if constexpr (WIDTH >= 4) v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    if constexpr (WIDTH >= 8) v = dpp_add<0x141>(v);  // row_half_mirror
+    if constexpr (WIDTH >= 16) v = dpp_add<0x140>(v); // row_mirror
+    if constexpr (WIDTH >= 32) v += __shfl_xor(v, 16, 64);
+    if constexpr (WIDTH >= 64) v += __shfl_xor(v, 32, 64);
     return v;
 }
 
