@@ -141,3 +141,17 @@ def test_fused_gemv_edge_activations(ctx, oracle):
     s, q = oracle.quantize_q8_0(x)
     assert_f32_parity(d_y.download(np.float32, m), oracle.gemv_q8(W.Q4_0, wb, s, q, m, k), "fused edge")
     w.free(), d_x.free(), d_y.free()
+
+
+def test_cpp_host_mirror_selftest():
+    """The C++ host layer (wick_amd/host/rocm_backend.hpp) linked statically against
+    libwick_rocm.a: closed form, GEMM column == GEMV, fused == two-step, error statuses."""
+    import os
+    import subprocess
+
+    from conftest import ROOT
+
+    exe = os.path.join(ROOT, "wick_amd", "lib", "host_selftest")
+    assert os.path.exists(exe), "host_selftest has not been built (make -C wick_amd/csrc)"
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0 and "selftest OK" in out.stdout, out.stdout + out.stderr

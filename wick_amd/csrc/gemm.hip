@@ -172,23 +172,41 @@ __device__ __forceinline__ void store_stage(Stage& s, const StageRegs<TYPE>& r) 
     }
 }
 
-// Workgroup -> tile, XCD-aware: hardware hands consecutive workgroup ids to the 8
-// XCDs round-robin, so ids with equal (id % 8) share an L2.  Each XCD gets a
-// contiguous run of tiles; within a run the token tile varies fastest, so the
-// workgroups resident on one XCD share weight-row panels in that L2.
-__device__ __forceinline__ uint32_t tile_of_block(uint32_t bid, uint32_t tiles) {
+// Workgroup -> tile, XCD- and L2-aware.  Hardware hands consecutive workgroup ids to
+// the 8 XCDs round-robin, so ids with equal (id % 8) share an L2 (4 MB).  Each XCD
+// takes a contiguous run of a tile list that walks the output in 8 x 8 "supertiles"
+// (8 row tiles x 8 token tiles, row-major inside): the ~64 workgroups resident on an
+// XCD at one time then touch 8 weight panels + 8 activation panels (~3.3 MB at
+// k = 2048), which fit its L2, instead of a 4 x 16 strip whose activation panels
+// alone overflow it.
+__device__ __forceinline__ void tile_of_block(uint32_t bid, uint32_t row_tiles, uint32_t tok_tiles, uint32_t& row_tile,
+                                              uint32_t& tok_tile, bool& valid) {
+    constexpr uint32_t S = 8;
+    const uint32_t tiles = row_tiles * tok_tiles;
     const uint32_t per_xcd = (tiles + 7u) / 8u;
-    return (bid & 7u) * per_xcd + (bid >> 3);
+    const uint32_t t = (bid & 7u) * per_xcd + (bid >> 3);
+    valid = (bid >> 3) < per_xcd && t < tiles;
+    const uint32_t tt = valid ? t : 0;
+    const uint32_t sr_count = (row_tiles + S - 1) / S, sc_count = (tok_tiles + S - 1) / S;
+    const uint32_t sr = min(tt / (S * tok_tiles), sr_count - 1);  // supertile row (all but the last hold S*tok_tiles tiles)
+    const uint32_t t1 = tt - sr * S * tok_tiles;
+    const uint32_t h = min(S, row_tiles - sr * S);
+    const uint32_t sc = min(t1 / (h * S), sc_count - 1);
+    const uint32_t t2 = t1 - sc * h * S;
+    const uint32_t w = min(S, tok_tiles - sc * S);
+    row_tile = sr * S + t2 / w;
+    tok_tile = sc * S + t2 % w;
 }
 
 template <int TYPE, bool DUMP>
 __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
     __shared__ Smem sm;
-    const uint32_t tiles = a.row_tiles * a.tok_tiles;
-    const uint32_t tile = tile_of_block(blockIdx.x, tiles);
-    if (tile >= tiles) return;  // whole workgroup leaves together
-    const uint32_t row0 = (tile / a.tok_tiles) * BM;
-    const uint32_t tok0 = (tile % a.tok_tiles) * BN;
+    uint32_t row_tile, tok_tile;
+    bool valid_tile;
+    tile_of_block(blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
+    if (!valid_tile) return;  // whole workgroup leaves together
+    const uint32_t row0 = row_tile * BM;
+    const uint32_t tok0 = tok_tile * BN;
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;

@@ -1,0 +1,141 @@
+// Host-side C++ mirror of wick's GPU-backend matmul call sites over the C ABI in
+// include/wick_rocm.h.  This is the role `backend/rocm.rs` + `model/rocm_lfm2.rs`
+// play in the Rust tree (which cannot be compiled in this environment): same
+// method names, argument order and error behaviour as the reference's
+//   MetalWeight                       wick/src/model/metal_lfm2.rs:28-36
+//   encode_gemv_impl                  wick/src/model/metal_lfm2.rs:1231-1335
+//   encode_gemm                       wick/src/model/metal_lfm2.rs:881-992
+//   encode_gemv_qkv / _gate_up        wick/src/model/metal_lfm2.rs:1043-1119
+//   quantize_to_scratch / _columns    wick/src/model/lfm2.rs:571-612
+//   gemv_with_preq                    wick/src/backend/cpu.rs:334-354
+//   gemm_preq                         wick/src/model/lfm2.rs:539-565
+// Errors become exceptions here (anyhow::Result on the Rust side); contract
+// violations the reference asserts on (null buffers, bad strides) are reported the
+// same way instead of aborting.
+#pragma once
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/wick_rocm.h"
+
+namespace wick {
+
+enum class DType : int { Q4_0 = WICK_ROCM_TYPE_Q4_0, Q8_0 = WICK_ROCM_TYPE_Q8_0 };
+
+struct BackendError : std::runtime_error {
+    int status;
+    BackendError(int s, const std::string& m) : std::runtime_error("rocm backend: " + m + " (status " + std::to_string(s) + ")"), status(s) {}
+};
+
+class RocmContext;
+
+// Device-resident weight: GGUF block bytes verbatim.
+struct RocmWeight {
+    wick_rocm_weight* handle = nullptr;
+    DType dtype = DType::Q4_0;
+    uint32_t m = 0, k = 0;
+};
+
+// A caller-owned device buffer (a Metal `Buffer` in the reference).
+struct Buffer {
+    void* ptr = nullptr;
+    size_t nbytes = 0;
+};
+
+class RocmContext {
+public:
+    explicit RocmContext(int device = 0) {
+        int rc = wick_rocm_ctx_create(device, &ctx_);
+        if (rc != 0) throw BackendError(rc, rc == WICK_ROCM_ERR_NO_DEVICE ? "no gfx950 device" : "context creation failed");
+    }
+    ~RocmContext() { wick_rocm_ctx_destroy(ctx_); }
+    RocmContext(const RocmContext&) = delete;
+    RocmContext& operator=(const RocmContext&) = delete;
+
+    Buffer create_buffer(size_t nbytes) {
+        Buffer b;
+        b.nbytes = nbytes;
+        check(wick_rocm_buffer_alloc(ctx_, nbytes, &b.ptr));
+        return b;
+    }
+    void free_buffer(Buffer& b) {
+        check(wick_rocm_buffer_free(ctx_, b.ptr));
+        b.ptr = nullptr;
+    }
+    void write(const Buffer& b, const void* src, size_t nbytes, size_t off = 0) {
+        check(wick_rocm_upload(ctx_, static_cast<char*>(b.ptr) + off, src, nbytes));
+    }
+    void read(const Buffer& b, void* dst, size_t nbytes, size_t off = 0) {
+        check(wick_rocm_download(ctx_, dst, static_cast<const char*>(b.ptr) + off, nbytes));
+    }
+    std::vector<float> read_f32(const Buffer& b, size_t count, size_t off = 0) {
+        std::vector<float> v(count);
+        read(b, v.data(), count * sizeof(float), off);
+        return v;
+    }
+    void sync() { check(wick_rocm_sync(ctx_)); }
+
+    RocmWeight upload_weight(const void* blocks, size_t nbytes, DType dtype, uint32_t m, uint32_t k) {
+        RocmWeight w;
+        w.dtype = dtype, w.m = m, w.k = k;
+        check(wick_rocm_weight_upload(ctx_, blocks, nbytes, static_cast<int>(dtype), m, k, &w.handle));
+        return w;
+    }
+    void free_weight(RocmWeight& w) {
+        check(wick_rocm_weight_free(ctx_, w.handle));
+        w.handle = nullptr;
+    }
+
+    // ---- GPU call sites: f32 activations in, f32 out, byte offsets ------------------
+    void encode_gemv(const RocmWeight& w, const Buffer& input, uint64_t input_off_bytes, const Buffer& output,
+                     uint64_t output_off_bytes, bool accumulate = false) {
+        check(wick_rocm_matmul_f32(ctx_, w.handle, static_cast<const float*>(input.ptr), input_off_bytes, 1, w.k,
+                                   static_cast<float*>(output.ptr), output_off_bytes, w.m, accumulate));
+    }
+    void encode_gemm(const RocmWeight& w, const Buffer& x, uint64_t x_off_bytes, const Buffer& y, uint64_t y_off_bytes,
+                     uint32_t n, uint32_t x_stride, uint32_t y_stride, bool accumulate = false) {
+        check(wick_rocm_matmul_f32(ctx_, w.handle, static_cast<const float*>(x.ptr), x_off_bytes, n, x_stride,
+                                   static_cast<float*>(y.ptr), y_off_bytes, y_stride, accumulate));
+    }
+    // {Q,K,V} or {gate,up}: one activation, several weights, one launch.
+    void encode_gemv_fused(const std::vector<const RocmWeight*>& ws, const Buffer& x, uint64_t x_off_bytes,
+                           const std::vector<Buffer>& ys, bool accumulate = false) {
+        std::vector<const wick_rocm_weight*> hs;
+        std::vector<float*> ps;
+        for (auto* w : ws) hs.push_back(w->handle);
+        for (auto& y : ys) ps.push_back(static_cast<float*>(y.ptr));
+        check(wick_rocm_gemv_f32_multi(ctx_, hs.data(), ps.data(), static_cast<uint32_t>(hs.size()),
+                                       static_cast<const float*>(x.ptr), x_off_bytes, accumulate));
+    }
+
+    // ---- CPU call sites on pre-quantized activations ---------------------------------
+    void quantize_columns(const Buffer& x, uint32_t n, uint32_t k, uint32_t x_stride, const Buffer& quants, const Buffer& scales) {
+        check(wick_rocm_quantize_q8_0(ctx_, static_cast<const float*>(x.ptr), n, k, x_stride, static_cast<int8_t*>(quants.ptr),
+                                      static_cast<float*>(scales.ptr)));
+    }
+    void gemv_with_preq(const RocmWeight& w, const Buffer& scales, const Buffer& quants, const Buffer& y, bool accumulate = false) {
+        check(wick_rocm_gemv_q8(ctx_, w.handle, static_cast<const int8_t*>(quants.ptr), static_cast<const float*>(scales.ptr),
+                                static_cast<float*>(y.ptr), accumulate));
+    }
+    // out[i*n + j], like gemm_*_q8_0_neon
+    void gemm_preq(const RocmWeight& w, const Buffer& scales, const Buffer& quants, uint32_t n, const Buffer& out) {
+        check(wick_rocm_gemm_q8(ctx_, w.handle, static_cast<const int8_t*>(quants.ptr), static_cast<const float*>(scales.ptr), n,
+                                static_cast<float*>(out.ptr), n, WICK_ROCM_LAYOUT_ROW_MAJOR, 0));
+    }
+
+    wick_rocm_ctx* raw() { return ctx_; }
+
+private:
+    void check(int rc) {
+        if (rc == 0) return;
+        char buf[512] = {0};
+        wick_rocm_last_error(ctx_, buf, sizeof buf);
+        throw BackendError(rc, buf);
+    }
+    wick_rocm_ctx* ctx_ = nullptr;
+};
+
+}  // namespace wick
