@@ -3,19 +3,23 @@
 
 A "step" is one pass of the decode hot path over the LFM2-350M-shaped weight set
 (hidden 1024, 10 short-conv + 6 attention layers, FFN 4608, tied LM head
-65536 x 1024) at n = 1: 65 Q8_0 activation quantizations fused into 65 GEMV launches
-covering 93 weight matrices ({Q,K,V} and {gate,up} share one quantized activation
-and one launch, like the reference's call sites; the quantization runs inside the
-GEMV kernel), submitted as ONE HIP graph per token.  Two distinct device copies of the weight set are alternated so every step
-streams its weights from HBM, not from the 256 MB Infinity Cache.
+65536 x 1024) at n = 1: 93 weight matrices in 65 GEMV launches ({Q,K,V} and
+{gate,up} share one activation and one launch, like the reference's call sites; the
+Q8_0 quantization of the activation runs inside the GEMV kernel), submitted as ONE
+HIP graph per token.  Two distinct device copies of the weight set are alternated
+so every step streams its weights from HBM, not from the 256 MB Infinity Cache.
 
 Prints one JSON line: `value` = algorithmic GEMV bytes per step / step time, plus
-  roofline      the GEMV kernel: algorithmic bytes / summed kernel execution time
-                (per-dispatch timestamps taken live, same quantity as a kernel trace)
-  gemm          the prefill GEMM leg (Q4_0, m=6912, n=2002, k=2048) with its own roofline
+  roofline        the GEMV kernel over the timed steps: algorithmic bytes / summed kernel
+                  execution time (per-dispatch timestamps, the quantity a kernel trace reports)
+  gemm            prefill GEMM leg (Q4_0, m=6912, n=2002, k=2048) with its own roofline
   gemv_6912x2048  the single-GEMV shape the HBM target is quoted on, HBM-cold
-  cpu_baseline  the reference's x86 CPU path (f32 per-token GEMV, serial for Q4_0)
-                timed on this host on a bounded sample of the same step
+  decode_step_q8_0, prefill_sites, lm_head_sweep   the other configurations
+  cpu_baseline    the reference's x86 CPU path (f32 per-token GEMV, serial for Q4_0)
+                  timed on this host on a bounded sample of the same step
+
+`--leg NAME` runs one leg only (used for profiling): decode, decode_q8, gemv, gemm,
+prefill_sites, lm_head, copy, cpu.
 """
 from __future__ import annotations
 
@@ -65,16 +69,21 @@ def decode_call_sites():
     return sites
 
 
+def synth_many(O, jobs):
+    """jobs: [(dtype, m, k, seed)] -> block bytes, generated on a thread pool (N(0, 0.02^2))."""
+    with ThreadPoolExecutor(max_workers=min(16, os.cpu_count() or 4)) as pool:
+        return list(pool.map(lambda j: O.synth_weight(j[0], j[1], j[2], seed=j[3]), jobs))
+
+
 def synth_decode_weights(O, dtype: int):
-    """Host block bytes for every weight of the step: {site: [bytes per matrix]}.  N(0, 0.02^2)."""
-    jobs = []
+    """Host block bytes for every weight of the step: {site: [bytes per matrix]}."""
+    jobs, keys = [], []
     for si, (name, ms, k) in enumerate(decode_call_sites()):
         for wi, m in enumerate(ms):
-            jobs.append((name, wi, m, k, 1000 * dtype + 17 * si + wi))
-    with ThreadPoolExecutor(max_workers=min(16, os.cpu_count() or 4)) as pool:
-        blobs = list(pool.map(lambda j: O.synth_weight(dtype, j[2], j[3], seed=j[4]), jobs))
+            jobs.append((dtype, m, k, 1000 * dtype + 17 * si + wi))
+            keys.append(name)
     out = {}
-    for (name, wi, m, k, _), b in zip(jobs, blobs):
+    for name, b in zip(keys, synth_many(O, jobs)):
         out.setdefault(name, []).append(b)
     return out
 
@@ -82,8 +91,8 @@ def synth_decode_weights(O, dtype: int):
 class DecodeStep:
     """Device state of one copy of the weight set + the enqueue order of a step."""
 
-    def __init__(self, ctx, W, dtype, host_weights, d_x_hs, d_x_is):
-        self.ctx, self.W, self.dtype = ctx, W, dtype
+    def __init__(self, ctx, dtype, host_weights, d_x_hs, d_x_is):
+        self.ctx, self.dtype = ctx, dtype
         self.sites = []
         for name, ms, k in decode_call_sites():
             ws = [ctx.upload_weight(b, dtype, m, k) for b, m in zip(host_weights[name], ms)]
@@ -104,6 +113,14 @@ class DecodeStep:
                 ctx.quantize_q8_0(self.d_x[k], 1, k, k, self.d_q, self.d_s)
                 ctx.gemv_with_preq_multi(ws, self.d_s, self.d_q, ys)
 
+    def free(self):
+        for ws, ys, _ in self.sites:
+            for w in ws:
+                w.free()
+            for y in ys:
+                y.free()
+        self.d_q.free(), self.d_s.free()
+
 
 def time_graphs(ctx, graphs, steps, warmup):
     """Events around `steps` graph launches (round-robin over `graphs`); returns ms per step."""
@@ -121,10 +138,10 @@ def time_graphs(ctx, graphs, steps, warmup):
     return ms / steps
 
 
-def bench_decode(ctx, W, O, dtype, steps, warmup, host_weights):
+def bench_decode(ctx, W, O, dtype, steps, warmup, host_weights, with_unfused=True):
     x_hs = ctx.to_device(O.fill_normal(1, 1.0, HS))
     x_is = ctx.to_device(O.fill_normal(2, 1.0, IS))
-    copies = [DecodeStep(ctx, W, dtype, host_weights, x_hs, x_is) for _ in range(2)]
+    copies = [DecodeStep(ctx, dtype, host_weights, x_hs, x_is) for _ in range(2)]
     graphs = []
     for c in copies:
         ctx.graph_begin()
@@ -139,44 +156,40 @@ def bench_decode(ctx, W, O, dtype, steps, warmup, host_weights):
     sites = decode_call_sites()
     gbytes = sum(gemv_bytes(dtype, m, k) for _, ms, k in sites for m in ms)
     wbytes = sum(m * (k // 32) * BW[dtype] for _, ms, k in sites for m in ms)
-    qbytes = sum(quant_bytes(1, k) for _, _, k in sites)
     res = {
+        "dtype": dtype,
         "ms_per_step": ms_step,
         "gemv_bytes_per_step": gbytes,
         "weight_bytes_per_step": wbytes,
-        "quantize_bytes_per_step": qbytes,
+        "quantize_bytes_per_step": sum(quant_bytes(1, k) for _, _, k in sites),
         "gemv_launches_per_step": len(sites),
         "gemvs_per_step": sum(len(ms) for _, ms, _ in sites),
         "step_GBps": gbytes / ms_step / 1e6,
+        "us_per_launch_in_graph": ms_step * 1e3 / len(sites),
         "gemv_kernel_ms_per_step": kt["gemv"][0] / steps,
         "gemv_kernel_GBps": gbytes / (kt["gemv"][0] / steps) / 1e6,
         "gemv_kernel_avg_us": kt["gemv"][0] / kt["gemv"][1] * 1e3,
     }
-    # the same step with the quantizer as its own launch (two launches per call site)
-    graphs2 = []
-    for c in copies:
-        ctx.graph_begin()
-        c.enqueue(fused=False)
-        graphs2.append(ctx.graph_end())
-    res["ms_per_step_unfused_quantizer"] = time_graphs(ctx, graphs2, steps, warmup)
-    for g in graphs2:
-        ctx.graph_destroy(g)
+    if with_unfused:  # the same step with the quantizer as its own launch (two launches per call site)
+        graphs2 = []
+        for c in copies:
+            ctx.graph_begin()
+            c.enqueue(fused=False)
+            graphs2.append(ctx.graph_end())
+        res["ms_per_step_unfused_quantizer"] = time_graphs(ctx, graphs2, steps, warmup)
+        for g in graphs2:
+            ctx.graph_destroy(g)
     for g in graphs:
         ctx.graph_destroy(g)
     for c in copies:
-        for ws, ys, _ in c.sites:
-            for w in ws:
-                w.free()
-            for y in ys:
-                y.free()
-        c.d_q.free(), c.d_s.free()
+        c.free()
     x_hs.free(), x_is.free()
     return res
 
 
-def bench_single_gemv(ctx, W, O, dtype, m, k, launches=200):
+def bench_single_gemv(ctx, W, O, dtype, m, k, launches=200, wb=None):
     """One GEMV shape, HBM-cold: rotate over enough weight copies to exceed the Infinity Cache."""
-    wb = O.synth_weight(dtype, m, k, seed=4242)
+    wb = O.synth_weight(dtype, m, k, seed=4242) if wb is None else wb
     copies = max(3, int(300e6 // wb.nbytes) + 1)
     ws = [ctx.upload_weight(wb, dtype, m, k) for _ in range(copies)]
     s, q = O.quantize_q8_0(O.fill_normal(3, 1.0, k))
@@ -199,12 +212,12 @@ def bench_single_gemv(ctx, W, O, dtype, m, k, launches=200):
         w.free()
     d_q.free(), d_s.free(), d_y.free()
     return {"m": m, "k": k, "dtype": dtype, "bytes": b, "weight_copies": copies, "us_per_launch_in_graph": ms * 1e3,
-            "GBps_in_graph": b / ms / 1e6, "kernel_us": kus, "kernel_GBps": b / kus / 1e3,
-            "kernel_frac_of_hbm_peak": b / kus / 1e3 / HBM_PEAK_GBS}
+            "GBps_in_graph": b / ms / 1e6, "frac_of_hbm_peak_in_graph": b / ms / 1e6 / HBM_PEAK_GBS,
+            "kernel_us": kus, "kernel_GBps": b / kus / 1e3, "kernel_frac_of_hbm_peak": b / kus / 1e3 / HBM_PEAK_GBS}
 
 
-def bench_gemm(ctx, W, O, dtype, m, n, k, reps=20):
-    wb = O.synth_weight(dtype, m, k, seed=777)
+def bench_gemm(ctx, W, O, dtype, m, n, k, reps=20, wb=None, with_quantize=True):
+    wb = O.synth_weight(dtype, m, k, seed=777) if wb is None else wb
     w = ctx.upload_weight(wb, dtype, m, k)
     d_x = ctx.to_device(O.fill_normal(9, 1.0, n * k))
     d_q, d_s, d_y = ctx.alloc(n * k), ctx.alloc(n * (k // 32) * 4), ctx.alloc(m * n * 4)
@@ -227,14 +240,79 @@ def bench_gemm(ctx, W, O, dtype, m, n, k, reps=20):
         run()
     kt = ctx.kernel_timing_end()
     ops = 2.0 * m * n * k
-    gemm_ms = kt["gemm"][0] / kt["gemm"][1]
+    fam = "gemm" if kt["gemm"][1] else "gemv"  # small n is served by the multi-token GEMV
+    gemm_ms = kt[fam][0] / kt[fam][1]
     quant_ms = kt["quantize"][0] / kt["quantize"][1]
     w.free()
     for b in (d_x, d_q, d_s, d_y):
         b.free()
-    return {"m": m, "n": n, "k": k, "dtype": dtype, "ops": ops, "quantize_plus_gemm_ms": ms_both,
+    return {"m": m, "n": n, "k": k, "dtype": dtype, "ops": ops, "kernel_family": fam, "quantize_plus_gemm_ms": ms_both,
             "quantize_plus_gemm_TOPS": ops / ms_both / 1e9, "gemm_kernel_ms": gemm_ms, "gemm_kernel_TOPS": ops / gemm_ms / 1e9,
+            "frac_of_int8_peak": ops / gemm_ms / 1e9 / INT8_PEAK_TOPS,
             "quantize_kernel_ms": quant_ms, "quantize_kernel_GBps": quant_bytes(n, k) / quant_ms / 1e6}
+
+
+def bench_prefill_sites(ctx, W, O, n=4096, dtype=8):
+    """The nine per-layer prefill GEMMs of an LFM2-1.2B-shaped layer at n tokens (Q8_0)."""
+    hs, is_, kv = 2048, 6912, 512
+    sites = [("conv_in", 3 * hs, hs), ("conv_out", hs, hs), ("attn_q", hs, hs), ("attn_k", kv, hs), ("attn_v", kv, hs),
+             ("attn_o", hs, hs), ("ffn_gate", is_, hs), ("ffn_up", is_, hs), ("ffn_down", hs, is_)]
+    blobs = synth_many(O, [(dtype, m, k, 300 + i) for i, (_, m, k) in enumerate(sites)])
+    out, tot_ops, tot_ms = [], 0.0, 0.0
+    for (name, m, k), wb in zip(sites, blobs):
+        r = bench_gemm(ctx, W, O, dtype, m, n, k, reps=5, wb=wb)
+        out.append({"site": name, "m": m, "k": k, "gemm_kernel_ms": r["gemm_kernel_ms"], "TOPS": r["gemm_kernel_TOPS"],
+                    "frac_of_int8_peak": r["frac_of_int8_peak"]})
+        tot_ops += r["ops"]
+        tot_ms += r["gemm_kernel_ms"]
+    return {"n": n, "dtype": dtype, "sites": out, "total_ops": tot_ops, "total_gemm_ms": tot_ms, "TOPS": tot_ops / tot_ms / 1e9}
+
+
+def bench_lm_head_sweep(ctx, W, O, dtype=8, m=65536, k=2048, ns=(1, 4, 16, 64)):
+    """Tied LM head: where the bandwidth-bound multi-token GEMV hands off to the MFMA GEMM.
+    Each n is timed through both kernels (hand-off forced), HBM-cold over three weight copies."""
+    wb = O.synth_weight(dtype, m, k, seed=999)
+    ws = [ctx.upload_weight(wb, dtype, m, k) for _ in range(3)]
+    nmax = max(ns)
+    x = O.fill_normal(5, 1.0, nmax * k)
+    s, q = O.quantize_q8_0_batch(x, nmax, k)
+    d_q, d_s, d_y = ctx.to_device(q), ctx.to_device(s), ctx.alloc(m * nmax * 4)
+    rows = []
+    for n in ns:
+        row = {"n": n, "bytes": gemv_bytes(dtype, m, k, n), "ops": 2.0 * m * n * k}
+        for label, min_n in (("gemv", 1 << 30), ("mfma", 1)):
+            if label == "mfma" and n == 1:
+                continue
+            ctx.set_gemm_min_n(min_n)
+            ctx.graph_begin()
+            for w in ws:
+                ctx.gemm_preq(w, d_s, d_q, n, d_y, y_stride=m, layout=W.LAYOUT_TOKEN_MAJOR)
+            g = ctx.graph_end()
+            ms = time_graphs(ctx, [g], 4, 1) / len(ws)
+            ctx.graph_destroy(g)
+            row[label] = {"us": ms * 1e3, "GBps": row["bytes"] / ms / 1e6, "TOPS": row["ops"] / ms / 1e9}
+        ctx.set_gemm_min_n(0)
+        rows.append(row)
+    for w in ws:
+        w.free()
+    d_q.free(), d_s.free(), d_y.free()
+    crossover = next((r["n"] for r in rows if "mfma" in r and r["mfma"]["us"] < r["gemv"]["us"]), None)
+    return {"dtype": dtype, "m": m, "k": k, "rows": rows, "first_n_where_mfma_wins": crossover, "library_hand_off_n": W.GEMM_MIN_N}
+
+
+def bench_copy(ctx, nbytes=256 << 20, reps=10):
+    """Device-to-device copy of a known size: calibration of the FETCH_SIZE / WRITE_SIZE counters."""
+    a, b = ctx.alloc(nbytes), ctx.alloc(nbytes)
+    ctx.copy(b, a, nbytes)
+    ctx.sync()
+    e0, e1 = ctx.event(), ctx.event()
+    ctx.record(e0)
+    for _ in range(reps):
+        ctx.copy(b, a, nbytes)
+    ctx.record(e1)
+    ms = ctx.elapsed_ms(e0, e1) / reps
+    a.free(), b.free()
+    return {"bytes": nbytes, "ms": ms, "GBps_read_plus_write": 2 * nbytes / ms / 1e6}
 
 
 def cpu_baseline(O, dtype, host_weights, budget_s=12.0):
@@ -269,7 +347,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--skip-extra", action="store_true", help="only the headline decode step")
+    ap.add_argument("--skip-extra", action="store_true", help="only the headline decode step (+ CPU baseline)")
+    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | copy | cpu")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -278,7 +357,28 @@ def main():
     import wick_amd as W
     from oracle import oracle as O  # cpu_baseline leg + synthetic inputs only; never in the timed GPU path
 
+    leg = args.leg
+    if leg == "cpu":
+        print(json.dumps({"cpu_baseline": cpu_baseline(O, W.Q4_0, synth_decode_weights(O, W.Q4_0))}))
+        return
     ctx = W.RocmContext(0)
+    if leg != "all":
+        one = {
+            "decode": lambda: bench_decode(ctx, W, O, W.Q4_0, args.steps, args.warmup, synth_decode_weights(O, W.Q4_0), with_unfused=False),
+            "decode_q8": lambda: bench_decode(ctx, W, O, W.Q8_0, args.steps, args.warmup, synth_decode_weights(O, W.Q8_0), with_unfused=False),
+            "gemv": lambda: bench_single_gemv(ctx, W, O, W.Q4_0, 6912, 2048),
+            "gemm": lambda: bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048),
+            "prefill_sites": lambda: bench_prefill_sites(ctx, W, O),
+            "lm_head": lambda: bench_lm_head_sweep(ctx, W, O),
+            "copy": lambda: bench_copy(ctx),
+        }
+        if leg not in one:
+            print(f"bench.py: unknown leg {leg}", file=sys.stderr)
+            sys.exit(2)
+        print(json.dumps({leg: one[leg]()}))
+        ctx.close()
+        return
+
     dtype = W.Q4_0
     host_weights = synth_decode_weights(O, dtype)
     dec = bench_decode(ctx, W, O, dtype, args.steps, args.warmup, host_weights)
@@ -304,14 +404,19 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_pairs_kernel (all instantiations of the step)",
+            "kernel": "gemv_pairs_kernel (all instantiations of the step, fused quantizer)",
             "achieved": dec["gemv_kernel_GBps"],
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": dec["gemv_kernel_GBps"] / HBM_PEAK_GBS,
-            "traffic": None,
+            # HBM bytes per launch (average over the 65 launches of a step) from the calibrated FETCH_SIZE / WRITE_SIZE passes
+            # recorded in profiles/decode_step_lfm2_350m_q4_0.txt: (22*4.29 + 16*2.93 + 37.88 + 26*1.15 MB read + ~1.2 MB written) / 65
+            "traffic": 3.24e6,
+            "traffic_source": "profiles/decode_step_lfm2_350m_q4_0.txt (rocprofv3 --pmc FETCH_SIZE x2.0, WRITE_SIZE x1.0; copy-calibrated)",
             "bytes_per_launch_avg": dec["gemv_bytes_per_step"] / dec["gemv_launches_per_step"],
             "avg_launch_us": dec["gemv_kernel_avg_us"],
+            "note": "per-dispatch timestamps include ~4 us of fixed dispatch cost per launch; in the graph the same launches average "
+                    f"{dec['us_per_launch_in_graph']:.2f} us each",
         },
         "decode_step": dec,
     }
@@ -320,11 +425,19 @@ def main():
         out["gemv_6912x2048"] = bench_single_gemv(ctx, W, O, W.Q4_0, 6912, 2048)
         g = bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048)
         g["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma_kernel<Q4_0>", "achieved": g["gemm_kernel_TOPS"], "peak": INT8_PEAK_TOPS,
-                         "unit": "TOP/s", "frac": g["gemm_kernel_TOPS"] / INT8_PEAK_TOPS, "traffic": None}
+                         "unit": "TOP/s", "frac": g["gemm_kernel_TOPS"] / INT8_PEAK_TOPS,
+                         # 84.84 MB read + 60.04 MB written per launch (algorithmic 12.57 + 55.35 MB), profiles/gemm_q4_0_6912x2002x2048.txt
+                         "traffic": 144.9e6, "traffic_source": "profiles/gemm_q4_0_6912x2002x2048.txt"}
         out["gemm"] = g
-    if not args.skip_cpu:
-        out["cpu_baseline"] = cpu_baseline(O, dtype, host_weights)
+        del host_weights  # the CPU leg regenerates what it needs; keep host memory low
+        dq = bench_decode(ctx, W, O, W.Q8_0, max(10, args.steps // 2), args.warmup, synth_decode_weights(O, W.Q8_0), with_unfused=False)
+        out["decode_step_q8_0"] = dq
+        out["prefill_sites"] = bench_prefill_sites(ctx, W, O)
+        out["lm_head_sweep"] = bench_lm_head_sweep(ctx, W, O)
+        host_weights = None
     ctx.close()
+    if not args.skip_cpu:
+        out["cpu_baseline"] = cpu_baseline(O, dtype, host_weights or synth_decode_weights(O, dtype))
     print(json.dumps(out))
 
 

@@ -88,6 +88,9 @@ int wick_rocm_buffer_free(wick_rocm_ctx *ctx, void *d_ptr);
 int wick_rocm_upload(wick_rocm_ctx *ctx, void *d_dst, const void *src, size_t nbytes);   /* H2D, ordered on the stream */
 int wick_rocm_download(wick_rocm_ctx *ctx, void *dst, const void *d_src, size_t nbytes); /* D2H, waits for the stream */
 int wick_rocm_sync(wick_rocm_ctx *ctx);
+/* Device-to-device copy enqueued on the context's stream (the counterpart of a Metal
+ * blit between the reference's scratch buffers). */
+int wick_rocm_copy(wick_rocm_ctx *ctx, void *d_dst, const void *d_src, size_t nbytes);
 
 /* ---- weights ----------------------------------------------------------------
  * Stands in for MetalWeight {mmap_offset, dtype, m, k} (wick/src/model/metal_lfm2.rs:28-36,
@@ -138,6 +141,12 @@ int wick_rocm_gemv_q8_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *w
  * mirrors GEMM_MIN_N, wick/src/model/metal_lfm2.rs:18-21, 899-927). */
 int wick_rocm_gemm_q8(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_t *d_quants, const float *d_scales,
                       uint32_t n, float *d_y, uint32_t y_stride, int y_layout, int accumulate);
+
+/* The n at and above which wick_rocm_gemm_q8 / wick_rocm_matmul_f32 hand off from the
+ * multi-token GEMV to the MFMA GEMM (default 16, the reference's GEMM_MIN_N,
+ * wick/src/model/metal_lfm2.rs:18-21); 0 restores the default.  A tuning knob, like
+ * the reference's WICK_Q4_FAST / WICK_SPLITS switches (wick/src/backend/cpu.rs:23-27). */
+int wick_rocm_set_gemm_min_n(wick_rocm_ctx *ctx, uint32_t min_n);
 
 /* ---- the literal call-site shape ---------------------------------------
  * encode_gemm(w, x, x_off_bytes, y, y_off_bytes, n, x_stride, y_stride, accumulate)

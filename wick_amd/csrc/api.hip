@@ -29,6 +29,7 @@ struct wick_rocm_ctx {
     float* scratch_s = nullptr;
     size_t scratch_q_cap = 0;  // bytes
     size_t scratch_s_cap = 0;  // floats
+    uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
     KernelTimer timer;
     Launch launch() { return Launch{stream, &timer}; }
 };
@@ -118,7 +119,7 @@ int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q
     const bool mfma_ok = (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_q) % 16u == 0) &&
                          (reinterpret_cast<uintptr_t>(d_s) % 16u == 0);
     hipError_t e;
-    if (n >= kGemmMinN && mfma_ok)
+    if (n >= ctx->gemm_min_n && mfma_ok)
         e = launch_gemm_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
                              y_layout, accumulate, ctx->launch());
     else
@@ -242,6 +243,20 @@ int wick_rocm_download(wick_rocm_ctx* ctx, void* dst, const void* d_src, size_t 
     if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "download during graph capture");
     WR_HIP(ctx, hipMemcpyAsync(dst, d_src, nbytes, hipMemcpyDeviceToHost, ctx->stream));
     WR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_copy(wick_rocm_ctx* ctx, void* d_dst, const void* d_src, size_t nbytes) {
+    WR_ENTER(ctx);
+    if (nbytes == 0) return WICK_ROCM_OK;
+    if (!d_dst || !d_src) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "copy: null pointer");
+    WR_HIP(ctx, hipMemcpyAsync(d_dst, d_src, nbytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_set_gemm_min_n(wick_rocm_ctx* ctx, uint32_t min_n) {
+    WR_ENTER(ctx);
+    ctx->gemm_min_n = min_n == 0 ? kGemmMinN : min_n;
     return WICK_ROCM_OK;
 }
 
@@ -426,7 +441,7 @@ int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, cons
     if (int rc = check_weight(ctx, w)) return rc;
     if (!d_quants || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "block_dots: null device pointer");
     if (n == 0) return WICK_ROCM_OK;
-    const bool mfma = n >= kGemmMinN && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
+    const bool mfma = n >= ctx->gemm_min_n && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
     hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch())
                         : launch_block_dots_dot4(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "block_dots launch");

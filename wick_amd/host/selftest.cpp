@@ -1,5 +1,5 @@
 // Self-test of the C++ host mirror, linked STATICALLY against libwick_rocm.a the way a
-// Rust build.rs would link it.  Checks that need no oracle:
+// Rust build.rs would link it.  Self-contained checks (closed forms and invariants):
 //   * the Q8_0 closed form of the reference's test_q8_0_gemm_standalone
 //     (wick/tests/bench_perf.rs:852-971): m=64, k=32, n=4, scale 1/(row+1),
 //     quants -16..15, x == 1  ->  y[col*m + row] ~= -16/(row+1);

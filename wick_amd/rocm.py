@@ -70,6 +70,8 @@ _SIGNATURES = {
     "wick_rocm_upload": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_download": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_sync": (C.c_int, [_P]),
+    "wick_rocm_copy": (C.c_int, [_P, _P, _P, C.c_size_t]),
+    "wick_rocm_set_gemm_min_n": (C.c_int, [_P, C.c_uint32]),
     "wick_rocm_weight_upload": (C.c_int, [_P, _P, C.c_size_t, C.c_int, C.c_uint32, C.c_uint32, C.POINTER(_P)]),
     "wick_rocm_weight_free": (C.c_int, [_P, _P]),
     "wick_rocm_weight_info": (C.c_int, [_P, C.POINTER(C.c_int), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_size_t)]),
@@ -209,6 +211,12 @@ class RocmContext:
 
     def sync(self) -> None:
         self._check(self._lib.wick_rocm_sync(self._h))
+
+    def copy(self, dst, src, nbytes: int) -> None:
+        self._check(self._lib.wick_rocm_copy(self._h, _ptr(dst), _ptr(src), nbytes))
+
+    def set_gemm_min_n(self, min_n: int) -> None:
+        self._check(self._lib.wick_rocm_set_gemm_min_n(self._h, min_n))
 
     def alloc(self, nbytes: int) -> DeviceBuffer:
         return DeviceBuffer(self, nbytes)
