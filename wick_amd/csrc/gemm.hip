@@ -12,7 +12,8 @@
 // wave owns 64 x 64 (2 x 2 MFMA tiles).  One stage = 4 blocks (128 elements of K):
 //   * weights: each thread reads one 36/68-byte block pair with dword-aligned wide
 //     loads, unpacks nibbles to int8 and writes 16-byte operand rows to LDS;
-//   * activations: 16-byte chunks copied global -> LDS; scales alongside.
+//   * activations: copied global -> LDS directly (global_load_lds_dwordx4, asynchronous,
+//     no registers); token scales through registers (f32 -> f16, lane order).
 // LDS holds two stages.  The global loads of stage s+1 are issued before stage s is
 // computed and written to the other LDS buffer after it, so there is one barrier
 // per stage and the load latency hides behind the stage's ALU work.
@@ -96,13 +97,32 @@ __device__ __forceinline__ uint32_t q4_hi_x16(uint32_t q) { return (q & 0xf0f0f0
 template <int TYPE>
 struct StageRegs {
     uint32_t w[PairTraits<TYPE>::DWORDS];
-    uint4 x[4];
     float4 dx;
 };
 
+// Activation tiles go global -> LDS directly (global_load_lds_dwordx4): no staging
+// registers, no unpack, no ds_write, and the copy runs asynchronously under the stage's
+// ALU work.  One wave instruction fills 64 consecutive tokens of one [block][khalf]
+// plane (lane l -> token l, 16 bytes each, contiguous 1 KB in LDS); a stage has
+// 8 planes x 2 token halves = 16 such instructions, four per wave.
+__device__ __forceinline__ void dma_activations(const GemmArgs& a, Stage& s, uint32_t tok0, uint32_t kb0) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // = block of the stage
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        const uint32_t tok = min(tok0 + 64u * half + lane, a.n - 1);
+        const int8_t* src = a.xq + (size_t)tok * a.k + (size_t)(kb0 + wave) * 32;
+#pragma unroll
+        for (int kh = 0; kh < 2; kh++) {
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(src + 16 * kh),
+                                             (void __attribute__((address_space(3)))*)&s.xt[wave][kh][64 * half], 16, 0, 0);
+        }
+    }
+}
+
 // Thread -> work of one stage:
 //   weights      256 pairs   = 128 rows x 2 pairs             : row = t >> 1, pair = t & 1
-//   activations  1024 chunks = 128 tokens x 8 chunks of 16 B  : id = t + 256 i, token = id >> 3, chunk = id & 7
+//   activations  direct-to-LDS, see dma_activations
 //   token scales 128 tokens x 4 blocks (one float4)           : threads 0..127, token = t
 template <int TYPE>
 __device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uint32_t tok0, uint32_t kb0,
@@ -114,12 +134,6 @@ __device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uin
         const uint32_t row = min(row0 + (t >> 1), a.m - 1);
         const uint8_t* p = a.w + ((size_t)row * nb + kb0 + 2 * (t & 1u)) * (PT::BYTES / 2);
         load_pair<PT::DWORDS>(p, r.w);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t id = t + i * THREADS;
-        const uint32_t tok = min(tok0 + (id >> 3), a.n - 1);
-        r.x[i] = *reinterpret_cast<const uint4*>(a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + (id & 7u) * 16);
     }
     if (t < BN && a.xs) {  // xs is null only for the parity hook, which never scales
         const uint32_t tok = min(tok0 + t, a.n - 1);
@@ -153,12 +167,6 @@ __device__ __forceinline__ void store_stage(Stage& s, const StageRegs<TYPE>& r) 
             s.wt[0][b0 + 1][row] = make_uint4(q1[0], q1[1], q1[2], q1[3]);
             s.wt[1][b0 + 1][row] = make_uint4(q1[4], q1[5], q1[6], q1[7]);
         }
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t id = t + i * THREADS;
-        const uint32_t c = id & 7u;
-        s.xt[c >> 1][c & 1u][id >> 3] = r.x[i];
     }
     if (t < BN) {
         // token t of the tile sits at MFMA row t % 32 = 8*gq + 4*g + e -> lane half g, slot 4*gq + e
@@ -230,13 +238,20 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
     for (int r = 0; r < 16; r++) cbias[r] = (int)kBiasBits;
 
     StageRegs<TYPE> regs;
+    dma_activations(a, sm.st[0], tok0, 0);
     load_stage<TYPE>(a, row0, tok0, 0, regs);
     store_stage<TYPE>(sm.st[0], regs);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
     __syncthreads();
 
     for (uint32_t st = 0; st < stages; st++) {
         const Stage& s = sm.st[st & 1u];
-        if (st + 1 < stages) load_stage<TYPE>(a, row0, tok0, (st + 1) * KB, regs);
+        if (st + 1 < stages) {
+            // the other LDS stage was last read in stage st-1 and every wave has passed the
+            // barrier that ended it, so it can be refilled from here on
+            dma_activations(a, sm.st[(st + 1) & 1u], tok0, (st + 1) * KB);
+            load_stage<TYPE>(a, row0, tok0, (st + 1) * KB, regs);
+        }
 
         // 16 MFMA tiles per stage.  Within a wave each MFMA is followed by its 32 FMAs;
         // the matrix core of a SIMD is kept busy by the other resident wave(s), whose FMA
@@ -291,6 +306,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
         // The other buffer was last read in stage st-1; every wave has passed the barrier
         // that ended that stage, so it is free to be refilled now.
         if (st + 1 < stages) store_stage<TYPE>(sm.st[(st + 1) & 1u], regs);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS copies of the next stage have landed
         __syncthreads();
     }
 
