@@ -148,6 +148,13 @@ int wick_rocm_gemm_q8(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_
  * the reference's WICK_Q4_FAST / WICK_SPLITS switches (wick/src/backend/cpu.rs:23-27). */
 int wick_rocm_set_gemm_min_n(wick_rocm_ctx *ctx, uint32_t min_n);
 
+/* How the single-token GEMV fetches its weights, by bytes of weights in one launch: below
+ * direct_max_bytes every lane loads its own block pair; from there on a wave loads whole
+ * cache lines and redistributes them through LDS.  Negative = the built-in default (3 MiB
+ * for Q4_0, 512 KiB for Q8_0).  Results do not depend on it.  A tuning knob, like the
+ * reference's WICK_Q4_FAST / WICK_SPLITS switches (wick/src/backend/cpu.rs:23-27). */
+int wick_rocm_set_gemv_policy(wick_rocm_ctx *ctx, int64_t direct_max_bytes);
+
 /* ---- the literal call-site shape ---------------------------------------
  * encode_gemm(w, x, x_off_bytes, y, y_off_bytes, n, x_stride, y_stride, accumulate)
  * and, with n = 1, encode_gemv_impl(w, input, input_off, output, output_off, accumulate)

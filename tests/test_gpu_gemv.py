@@ -101,3 +101,50 @@ def test_argument_errors(ctx, oracle):
     with pytest.raises(W.RocmError) as e:
         ctx.upload_weight(blocks, W.Q4_0, 3, 64)  # byte count mismatch
     assert e.value.status == -3
+
+
+# Both ways of fetching the weights on: every lanes-per-row tier, k/64 not a power of two
+# (spans shorter than 64 pairs), two-chunk rows, m below one pass and not a multiple of the
+# rows per pass (the last span hangs over the matrix end), many passes per wave.
+STREAM_SHAPES = [(1, 64), (9, 128), (33, 192), (100, 256), (1, 512), (3, 512), (1000, 512), (2, 1024), (4, 1024), (37, 1024),
+                 (4099, 1024), (77, 1536), (1, 2048), (2, 2048), (515, 2048), (9001, 2048), (1, 4096), (7, 4096), (3001, 4096),
+                 (130, 4608), (1025, 4608), (65, 6912), (19, 8192), (70001, 1024)]
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+@pytest.mark.parametrize("m,k", STREAM_SHAPES)
+def test_gemv_streaming_variant(ctx, oracle, dtype, m, k):
+    """Both ways of fetching the weights (per-lane loads, whole-line span loads through LDS)
+    give the reference's result, pre-quantized and fused-quantizer entry points alike; the
+    fused and the pre-quantized launch of one policy agree bit for bit."""
+    with Problem(ctx, oracle, dtype, m, k, seed=5 * m + k + dtype) as p:
+        ref = oracle.gemv_q8(dtype, p.wb, p.s[0], p.q[0], m, k)
+        d_x = p.to_device(p.x)
+        d_y, d_yf = p.alloc(m * 4), p.alloc(m * 4)
+        try:
+            for direct_max in (1 << 62, 0):
+                ctx.set_gemv_policy(direct_max)
+                d_y.upload(np.full(m, np.nan, np.float32))
+                d_yf.upload(np.full(m, np.nan, np.float32))
+                ctx.gemv_with_preq(p.w, p.d_s, p.d_q, d_y)
+                ctx.encode_gemv_fused([p.w], d_x, 0, [d_yf])
+                y, yf = d_y.download(np.float32, m), d_yf.download(np.float32, m)
+                assert_f32_parity(y, ref, f"gemv direct_max={direct_max} {dtype} {m}x{k}")
+                assert np.array_equal(y, yf), "fused quantizer differs from pre-quantized launch"
+        finally:
+            ctx.set_gemv_policy(-1)
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+def test_gemv_streaming_accumulate(ctx, oracle, dtype):
+    m, k = 2051, 1024
+    with Problem(ctx, oracle, dtype, m, k, seed=31) as p:
+        y0 = oracle.fill_normal(78, 1.0, m)
+        d_y = p.to_device(y0)
+        try:
+            ctx.set_gemv_policy(0)
+            ctx.gemv_with_preq(p.w, p.d_s, p.d_q, d_y, accumulate=True)
+        finally:
+            ctx.set_gemv_policy(-1)
+        ref = y0 + oracle.gemv_q8(dtype, p.wb, p.s[0], p.q[0], m, k)
+        assert_f32_parity(d_y.download(np.float32, m), ref, "streaming gemv accumulate")

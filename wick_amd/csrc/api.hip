@@ -31,7 +31,8 @@ struct wick_rocm_ctx {
     size_t scratch_s_cap = 0;  // floats
     uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
     KernelTimer timer;
-    Launch launch() { return Launch{stream, &timer}; }
+    int64_t gemv_direct_max_bytes = -1;
+    Launch launch() { return Launch{stream, &timer, gemv_direct_max_bytes}; }
 };
 
 struct wick_rocm_weight {
@@ -251,6 +252,12 @@ int wick_rocm_copy(wick_rocm_ctx* ctx, void* d_dst, const void* d_src, size_t nb
     if (nbytes == 0) return WICK_ROCM_OK;
     if (!d_dst || !d_src) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "copy: null pointer");
     WR_HIP(ctx, hipMemcpyAsync(d_dst, d_src, nbytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_set_gemv_policy(wick_rocm_ctx* ctx, int64_t direct_max_bytes) {
+    WR_ENTER(ctx);
+    ctx->gemv_direct_max_bytes = direct_max_bytes < 0 ? -1 : direct_max_bytes;
     return WICK_ROCM_OK;
 }
 

@@ -56,7 +56,18 @@ struct ActRegs {
 constexpr int kFusedWaves = 4;
 constexpr int kFusedMaxK = 8192;
 
-template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI>
+// How a lane gets its pair (MODE):
+//   kDirect    each lane loads its own 36 / 68 bytes (two / four 16-byte loads + one dword);
+//   kDirectNT  the same, loads marked nontemporal;
+//   kSpan      the wave loads the contiguous span that holds its 64 pairs as whole consecutive
+//              16-byte pieces (lane l takes bytes 16 l .. 16 l + 15 of every KB: each load
+//              instruction covers whole cache lines once, nontemporal), parks the span in a
+//              wave-private LDS slot and every lane reads its pair back from there (lane
+//              stride 9 / 17 dwords: odd, conflict-free).  The same wave writes and reads the
+//              slot and LDS operations of a wave execute in order, so no barrier is involved.
+enum { kDirect = 0, kDirectNT = 1, kSpan = 2 };
+
+template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI, int MODE>
 __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kernel(GemvArgs a) {
     using PT = PairTraits<TYPE>;
     constexpr int RPW = 64 / LPR;  // rows per wave pass
@@ -93,9 +104,13 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     for (int c = 0; c < NCHUNK; c++) pvalid[c] = c * LPR + sub < ppr;
 
     // Weight registers of one pass (U rows per lane) and where each row's result goes.
-    uint32_t w[U][NCHUNK][PT::DWORDS];
+    constexpr int WREGS = PT::DWORDS;
+    constexpr int WIDE = PT::BYTES / 16;  // 16-byte pieces per lane and span (kSpan)
+    uint32_t w[U][NCHUNK][WREGS];
+    uint32_t span_tail[U][NCHUNK];  // kSpan: where the dword remainder of the span starts
     bool rvalid[U];
     uint32_t lrow[U];
+    __shared__ __align__(16) uint8_t span_lds[MODE == kSpan ? (FUSEQ ? kFusedWaves : 1) * 64 * PT::BYTES : 16];
     // Loads are unconditional (row and pair indices clamped into range) so that the number
     // of outstanding loads is known at every wait; a clamped load's data is neutralised by
     // zero activation scales (pair out of range) or simply not stored (row out of range).
@@ -104,12 +119,53 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
         for (int u = 0; u < U; u++) {
             lrow[u] = base + u * RPW + rsel;
             rvalid[u] = lrow[u] < wave_row1;
-            const uint8_t* rowp = wbase + (size_t)min(lrow[u], rows - 1) * ppr * PT::BYTES;
+            if constexpr (MODE == kSpan) {
+                // First row of this pass (wave-uniform) and the rows of it that exist.
+                const uint32_t row0 = base + u * RPW;
+                const uint32_t nrows = row0 < rows ? min((uint32_t)RPW, rows - row0) : 0u;
 #pragma unroll
-            for (int c = 0; c < NCHUNK; c++) {
-                const uint32_t p = pvalid[c] ? c * LPR + sub : 0;
-                load_pair<PT::DWORDS>(rowp + (size_t)p * PT::BYTES, w[u][c]);
+                for (int c = 0; c < NCHUNK; c++) {
+                    const uint32_t pairs = NCHUNK == 1 ? nrows * ppr : (nrows && ppr > 64u * c ? min(64u, ppr - 64u * c) : 0u);
+                    const uint32_t span = pairs * PT::BYTES;
+                    const uint8_t* sp = wbase + (span ? ((size_t)row0 * ppr + 64u * c) * PT::BYTES : 0);
+#pragma unroll
+                    for (int j = 0; j < WIDE; j++) {
+                        const uint32_t o = 1024u * j + 16u * lane;
+                        const u32x4_native_a4 t =
+                            __builtin_nontemporal_load(reinterpret_cast<const u32x4_native_a4*>(sp + (o + 16u <= span ? o : 0u)));
+                        w[u][c][4 * j + 0] = t.x, w[u][c][4 * j + 1] = t.y, w[u][c][4 * j + 2] = t.z, w[u][c][4 * j + 3] = t.w;
+                    }
+                    // What the 16-byte pieces leave over (256 bytes of a full span, the last
+                    // 4-12 bytes of a short one) goes as single dwords.
+                    const uint32_t o = (min(span, 1024u * WIDE) & ~15u) + 4u * lane;
+                    w[u][c][WREGS - 1] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(sp + (o + 4u <= span ? o : 0u)));
+                    span_tail[u][c] = min(span, 1024u * WIDE) & ~15u;
+                }
+            } else {
+                const uint8_t* rowp = wbase + (size_t)min(lrow[u], rows - 1) * ppr * PT::BYTES;
+#pragma unroll
+                for (int c = 0; c < NCHUNK; c++) {
+                    const uint32_t p = pvalid[c] ? c * LPR + sub : 0;
+                    load_pair<PT::DWORDS, MODE == kDirectNT>(rowp + (size_t)p * PT::BYTES, w[u][c]);
+                }
             }
+        }
+    };
+    // kSpan: the span pieces in w[u][c] go through this wave's LDS slot and come back as
+    // this lane's own pair (position rsel * ppr + sub of the span, or sub for a row chunk).
+    auto own_pair = [&](uint32_t (&piece)[WREGS], uint32_t tail) {
+        if constexpr (MODE == kSpan) {
+            uint8_t* slot = span_lds + (FUSEQ ? (threadIdx.x >> 6) * 64 * PT::BYTES : 0);
+#pragma unroll
+            for (int j = 0; j < WIDE; j++)
+                *reinterpret_cast<uint4*>(slot + 1024 * j + 16 * lane) =
+                    make_uint4(piece[4 * j], piece[4 * j + 1], piece[4 * j + 2], piece[4 * j + 3]);
+            // after the pieces: a piece that straddles the span's end holds filler
+            *reinterpret_cast<uint32_t*>(slot + tail + 4 * lane) = piece[WREGS - 1];
+            const uint32_t pos = NCHUNK == 1 ? rsel * ppr + sub : sub;
+            const uint32_t* mine = reinterpret_cast<const uint32_t*>(slot + (size_t)min(pos, 63u) * PT::BYTES);
+#pragma unroll
+            for (int i = 0; i < WREGS; i++) piece[i] = mine[i];
         }
     };
 
@@ -214,6 +270,7 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
 #pragma unroll
             for (int c = 0; c < NCHUNK; c++) {
                 uint32_t d0, d1, q0[PT::NQ], q1[PT::NQ];
+                own_pair(w[u][c], span_tail[u][c]);
                 split_pair<TYPE>(w[u][c], d0, d1, q0, q1);
                 const float dw0 = pvalid[c] ? f16_bits_to_f32(d0) : 0.0f, dw1 = pvalid[c] ? f16_bits_to_f32(d1) : 0.0f;
 #pragma unroll
@@ -308,6 +365,17 @@ inline uint32_t set_wave_ends(GemvArgs& a) {
     return waves;
 }
 
+// How the weights of a single-token launch are fetched, by bytes of weights in the launch
+// (measured on MI355X, HBM-cold, inside a graph):
+//   * small launches are latency-bound and per-lane loads save the LDS round trip.  For
+//     Q4_0 nontemporal per-lane loads are 0.3-0.4 us faster than ordinary ones; for Q8_0
+//     they are slower (a lane's 68 bytes take five load instructions that share cache
+//     lines, and without L1 retention every one of them goes to L2 again), so Q8_0 keeps
+//     ordinary loads and switches to span loads much earlier;
+//   * from the threshold on, whole-line span loads (kSpan): 10-25 % faster on 5-150 MB
+//     matrices, 6.4 TB/s kernel-time on a 142 MB Q8_0 matrix.
+constexpr uint64_t kDirectMaxBytesQ4 = 3ull << 20;
+constexpr uint64_t kDirectMaxBytesQ8 = 512ull << 10;
 template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ, int U>
 hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
     constexpr uint32_t pass_rows = (64 / LPR) * U;
@@ -320,9 +388,25 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
     const uint32_t waves = set_wave_ends(a);
     const dim3 grid = FUSEQ ? dim3((waves + kFusedWaves - 1) / kFusedWaves, 1) : dim3(waves, (a.n + NT - 1) / NT);
     const dim3 block(FUSEQ ? 64 * kFusedWaves : 64);
-    if (a.batch.count > 1)
-        return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true>, grid, block, a);
-    return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false>, grid, block, a);
+    // Several tokens re-read the weights: only single-token launches stream them.
+    const uint64_t bytes = (uint64_t)total_rows * (a.k >> 5) * (TYPE == 2 ? 18u : 34u);
+    constexpr int kSmall = TYPE == 2 ? kDirectNT : kDirect;
+    const uint64_t direct_max = L.gemv_direct_max_bytes >= 0 ? (uint64_t)L.gemv_direct_max_bytes : (TYPE == 2 ? kDirectMaxBytesQ4 : kDirectMaxBytesQ8);
+    const int mode = NT > 1 ? kDirect : (bytes < direct_max ? kSmall : kSpan);
+    const bool multi = a.batch.count > 1;
+    if constexpr (NT == 1) {
+        if (mode == kSpan && multi)
+            return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSpan>, grid, block, a);
+        if (mode == kSpan)
+            return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan>, grid, block, a);
+        if (multi)
+            return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSmall>, grid, block, a);
+        return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall>, grid, block, a);
+    } else {
+        if (multi)
+            return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kDirect>, grid, block, a);
+        return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kDirect>, grid, block, a);
+    }
 }
 
 // Rows in flight per lane (U).  Small matrices are latency-bound: the finer the waves,

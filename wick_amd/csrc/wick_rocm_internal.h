@@ -47,6 +47,7 @@ struct KernelTimer {
 struct Launch {
     hipStream_t stream;
     KernelTimer* timer;  // may be null
+    int64_t gemv_direct_max_bytes = -1;  // single-token GEMV: per-lane loads below, span loads from here on; < 0 = per-dtype default
 };
 
 template <typename... KArgs, typename... Args>

@@ -72,6 +72,7 @@ _SIGNATURES = {
     "wick_rocm_sync": (C.c_int, [_P]),
     "wick_rocm_copy": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_set_gemm_min_n": (C.c_int, [_P, C.c_uint32]),
+    "wick_rocm_set_gemv_policy": (C.c_int, [_P, C.c_int64]),
     "wick_rocm_weight_upload": (C.c_int, [_P, _P, C.c_size_t, C.c_int, C.c_uint32, C.c_uint32, C.POINTER(_P)]),
     "wick_rocm_weight_free": (C.c_int, [_P, _P]),
     "wick_rocm_weight_info": (C.c_int, [_P, C.POINTER(C.c_int), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_size_t)]),
@@ -214,6 +215,10 @@ class RocmContext:
 
     def copy(self, dst, src, nbytes: int) -> None:
         self._check(self._lib.wick_rocm_copy(self._h, _ptr(dst), _ptr(src), nbytes))
+
+    def set_gemv_policy(self, direct_max_bytes: int = -1) -> None:
+        """Weight-fetch threshold of the n = 1 GEMV (negative = default); results do not depend on it."""
+        self._check(self._lib.wick_rocm_set_gemv_policy(self._h, direct_max_bytes))
 
     def set_gemm_min_n(self, min_n: int) -> None:
         self._check(self._lib.wick_rocm_set_gemm_min_n(self._h, min_n))
