@@ -40,9 +40,10 @@ struct GemvArgs {
     uint32_t n;         // tokens (1 for decode)
     uint32_t y_stride;  // token-major: >= rows of that weight; row-major: >= n
     uint32_t rows_per_wave;
-    uint32_t wave_end[kMaxGemvBatch];  // running total of waves (workgroups) per weight: a wave never straddles weights
+    uint32_t total_waves;
     int y_row_major;
     int accumulate;
+    uint32_t wave_end[kMaxGemvBatch];  // running total of waves per weight (a wave never straddles weights); UINT32_MAX past the batch
 };
 
 template <int TYPE, int NT>
@@ -78,24 +79,61 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     const uint32_t nb = a.k >> 5;
     const uint32_t tok0 = blockIdx.y * NT;
 
-    // Which weight of the batch this wave works on: scalar, once per wave, and
-    // branch-free so that all kernel arguments arrive in one scalar-load round trip.
     const uint32_t gwave =
         FUSEQ ? blockIdx.x * kFusedWaves + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) : blockIdx.x;
-    const uint32_t cnt = MULTI ? a.batch.count : 1u;
+    // The f32 activations are requested first of all (fused variant): they need only two
+    // scalars of the argument block, and everything below overlaps with their latency.
+    constexpr int kQuadRounds = kFusedMaxK / 4 / (64 * kFusedWaves);  // 8
+    float4 xv[FUSEQ ? kQuadRounds : 1];
+    if constexpr (FUSEQ) {
+        const uint32_t quads = a.k >> 2;
+#pragma unroll
+        for (int i = 0; i < kQuadRounds; i++) {
+            const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
+            xv[i] = reinterpret_cast<const float4*>(a.xf)[min(quad, quads - 1)];  // clamped, unconditional
+        }
+        // keep the compiler from moving the weight loads in front of these
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // Which weight of the batch this wave works on.  Every per-weight field is copied out of
+    // the argument block first (one scalar-load round trip for all of them; the empty asm
+    // keeps the compiler from sinking the loads into the selection below, which would make
+    // them a second, dependent round trip) and then picked with scalar selects.
+    // wave_end[] entries past the batch are UINT32_MAX (set_wave_ends).
     uint32_t widx = 0;
-    if constexpr (MULTI)
-        widx = (uint32_t)(cnt > 1 && gwave >= a.wave_end[0]) + (uint32_t)(cnt > 2 && gwave >= a.wave_end[1]) +
-               (uint32_t)(cnt > 3 && gwave >= a.wave_end[2]);
-    // widx is wave-uniform: these are scalar loads from the argument block at a computed
-    // offset (a second round trip, which single-weight launches do not pay).
-    const uint8_t* wbase = a.batch.w[widx];
-    float* ybase = a.batch.y[widx];
-    const uint32_t rows = a.batch.row_end[widx] - (widx ? a.batch.row_end[widx - 1] : 0u);
-    const uint32_t wave = gwave - (widx ? a.wave_end[widx - 1] : 0u);
+    const uint8_t* wbase = a.batch.w[0];
+    float* ybase = a.batch.y[0];
+    uint32_t row_hi = a.batch.row_end[0], row_lo = 0, wave_lo = 0;
+    if constexpr (MULTI) {
+        uint64_t w0 = (uint64_t)a.batch.w[0], w1 = (uint64_t)a.batch.w[1], w2 = (uint64_t)a.batch.w[2], w3 = (uint64_t)a.batch.w[3];
+        uint64_t y0 = (uint64_t)a.batch.y[0], y1 = (uint64_t)a.batch.y[1], y2 = (uint64_t)a.batch.y[2], y3 = (uint64_t)a.batch.y[3];
+        uint32_t r0 = a.batch.row_end[0], r1 = a.batch.row_end[1], r2 = a.batch.row_end[2], r3 = a.batch.row_end[3];
+        uint32_t e0 = a.wave_end[0], e1 = a.wave_end[1], e2 = a.wave_end[2], cnt = a.batch.count;
+        // (the inputs only pull the remaining fields into the same round trip)
+        asm(""
+            : "+s"(w0), "+s"(w1), "+s"(w2), "+s"(w3), "+s"(y0), "+s"(y1), "+s"(y2), "+s"(y3), "+s"(r0), "+s"(r1), "+s"(r2),
+              "+s"(r3), "+s"(e0), "+s"(e1), "+s"(e2), "+s"(cnt)
+            : "s"(a.xq), "s"(a.xs), "s"(a.total_waves), "s"(a.accumulate), "s"(a.rows_per_wave));
+        widx = min((uint32_t)(gwave >= e0) + (uint32_t)(gwave >= e1) + (uint32_t)(gwave >= e2), cnt - 1u);
+        // Masks instead of ?: -- the compiler turns a chain of scalar selects into a chain of
+        // branches, and a taken scalar branch costs more than all of this arithmetic.
+        const uint64_t m0 = 0ull - (uint64_t)(widx == 0), m1 = 0ull - (uint64_t)(widx == 1), m2 = 0ull - (uint64_t)(widx == 2),
+                       m3 = 0ull - (uint64_t)(widx == 3);
+        auto pick = [&](uint64_t v0, uint64_t v1, uint64_t v2, uint64_t v3) { return (v0 & m0) | (v1 & m1) | (v2 & m2) | (v3 & m3); };
+        // (the integers came out of an asm: say again that these are global addresses)
+        wbase = (const uint8_t*)(const uint8_t __attribute__((address_space(1)))*)pick(w0, w1, w2, w3);
+        ybase = (float*)(float __attribute__((address_space(1)))*)pick(y0, y1, y2, y3);
+        row_hi = (uint32_t)pick(r0, r1, r2, r3);
+        row_lo = (uint32_t)pick(0u, r0, r1, r2);
+        wave_lo = (uint32_t)pick(0u, e0, e1, e2);
+    }
+    const uint32_t rows = row_hi - row_lo;
+    const uint32_t wave = gwave - wave_lo;
     // Waves past the end of the batch (last workgroup of a fused launch) get an empty row
     // range but still take part in the cooperative quantization and its barrier.
-    const bool live_wave = gwave < a.wave_end[cnt - 1];
+    const bool live_wave = gwave < a.total_waves;
     const uint32_t wave_row0 = live_wave ? wave * a.rows_per_wave : 0;
     const uint32_t wave_row1 = live_wave ? min(wave_row0 + a.rows_per_wave, rows) : 0;
 
@@ -175,20 +213,6 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     //   3. wait for (1) only, quantize into LDS, barrier -- all under the latency of (2).
     __shared__ __align__(16) uint32_t fq[FUSEQ ? kFusedMaxK / 4 : 4];
     __shared__ float fs[FUSEQ ? kFusedMaxK / 32 : 1];
-    constexpr int kQuadRounds = kFusedMaxK / 4 / (64 * kFusedWaves);  // 8
-    float4 xv[FUSEQ ? kQuadRounds : 1];
-    if constexpr (FUSEQ) {
-        const uint32_t quads = a.k >> 2;
-#pragma unroll
-        for (int i = 0; i < kQuadRounds; i++) {
-            const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
-            xv[i] = reinterpret_cast<const float4*>(a.xf)[min(quad, quads - 1)];  // clamped, unconditional
-        }
-        // keep the compiler from moving the weight loads in front of these
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-    }
-
     issue_pass(wave_row0);
     if constexpr (FUSEQ) {
         asm volatile("" ::: "memory");
@@ -206,9 +230,7 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
             if (i * 64 * kFusedWaves < quads) {  // uniform: whole rounds only differ in their tail
                 const float4 v = xv[i];
                 float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-                amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-                amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-                amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+                amax = group_max8(amax);
                 float id;
                 const float scale = q8_scale_and_inverse(amax, id);
                 if (quad < quads) {
@@ -362,6 +384,8 @@ inline uint32_t set_wave_ends(GemvArgs& a) {
         waves += (rows + a.rows_per_wave - 1) / a.rows_per_wave;
         a.wave_end[i] = waves;
     }
+    for (uint32_t i = a.batch.count; i < kMaxGemvBatch; i++) a.wave_end[i] = UINT32_MAX;
+    a.total_waves = waves;
     return waves;
 }
 

@@ -38,9 +38,7 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float* __restr
     }
 
     float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    amax = group_max8(amax);
 
     float id;
     const float scale = q8_scale_and_inverse(amax, id);

@@ -168,6 +168,15 @@ __device__ __forceinline__ float dpp_add(float v) {
     return v + __builtin_bit_cast(float, moved);
 }
 
+// Maximum over groups of 8 consecutive lanes (the eight lanes that share one 32-element
+// activation block in the quantizers), same three DPP steps, no LDS crossbar.
+__device__ __forceinline__ float group_max8(float v) {
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false)));
+    return v;
+}
+
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v) {
     if constexpr (WIDTH >= 2) v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
