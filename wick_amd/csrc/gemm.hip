@@ -60,7 +60,7 @@ constexpr float kBias = 12582912.0f;
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
-typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 struct GemmArgs {
     const uint8_t* w;
@@ -83,7 +83,7 @@ struct Stage {
     uint4 wt[2][KB][BM + 2];    // [khalf][block][row]  int8 weights (Q4_0: x16)
     uint4 xt[KB][2][BN + 1];    // [block][khalf][token] int8 activations
     float2 dws[KB][BM + 2];     // {dw, -12582912*dw} per block and row (dw x 1/16 for Q4_0)
-    h8 dxh[KB][BN / 32][2][2];  // [block][token tile][lane half][2 x 8 halves]: token scales in lane order
+    float4 dxf[KB][BN / 32][2][4];  // [block][token tile][lane half][16 floats]: token scales in the order a lane consumes them
 };
 
 struct Smem {
@@ -171,12 +171,88 @@ __device__ __forceinline__ void store_stage(Stage& s, const StageRegs<TYPE>& r) 
     if (t < BN) {
         // token t of the tile sits at MFMA row t % 32 = 8*gq + 4*g + e -> lane half g, slot 4*gq + e
         const uint32_t tile = t >> 5, g = (t >> 2) & 1u, slot = ((t >> 3) & 3u) * 4 + (t & 3u);
-        _Float16* base = reinterpret_cast<_Float16*>(&s.dxh[0][tile][g][0]) + slot;
-        constexpr int kBlockStride = sizeof(s.dxh[0]) / sizeof(_Float16);
-        base[0 * kBlockStride] = (_Float16)r.dx.x;  // exact: the scales are f16 values
-        base[1 * kBlockStride] = (_Float16)r.dx.y;
-        base[2 * kBlockStride] = (_Float16)r.dx.z;
-        base[3 * kBlockStride] = (_Float16)r.dx.w;
+        float* base = reinterpret_cast<float*>(&s.dxf[0][tile][g][0]) + slot;
+        constexpr int kBlockStride = sizeof(s.dxf[0]) / sizeof(float);
+        base[0 * kBlockStride] = r.dx.x;
+        base[1 * kBlockStride] = r.dx.y;
+        base[2 * kBlockStride] = r.dx.z;
+        base[3 * kBlockStride] = r.dx.w;
+    }
+}
+
+// Per-block operands of a wave's 2 x 2 MFMA tiles.
+struct Mats {
+    v4i av[2], bv[2];  // [token tile], [row tile]: 16 K-bytes of this lane's operand row
+};
+struct RowScales {
+    float2 dw[2];  // {dw, -12582912*dw} of this lane's weight row, per row tile
+};
+struct TokScales {
+    v4f dx[4];  // the 16 token scales of one token tile, in result-register order
+};
+
+// All LDS reads of the main loop are inline assembly on purpose.  While direct-to-LDS
+// copies (of the NEXT stage, into the other buffer) are in flight, the compiler makes
+// every LDS read it can see wait for all of them, which would put the whole global-memory
+// latency at the start of each stage.  These reads touch only the current buffer; the
+// copies are waited for explicitly before the barrier that ends the stage.  Data arrives
+// in issue order; the *_ready functions are the matching waits (at most N later LDS reads
+// still outstanding) and tie the registers, so nothing can use them earlier.
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
+}
+__device__ __forceinline__ void load_mats(const Stage& s, int b, uint32_t g, uint32_t l32, uint32_t wrow0, uint32_t wtok0, Mats& m) {
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++) asm volatile("ds_read_b128 %0, %1" : "=v"(m.av[tt]) : "v"(lds_addr(&s.xt[b][g][wtok0 + tt * 32 + l32])));
+#pragma unroll
+    for (int rt = 0; rt < 2; rt++) asm volatile("ds_read_b128 %0, %1" : "=v"(m.bv[rt]) : "v"(lds_addr(&s.wt[g][b][wrow0 + rt * 32 + l32])));
+}
+__device__ __forceinline__ void load_row_scales(const Stage& s, int b, uint32_t l32, uint32_t wrow0, RowScales& r) {
+#pragma unroll
+    for (int rt = 0; rt < 2; rt++) asm volatile("ds_read_b64 %0, %1" : "=v"(r.dw[rt]) : "v"(lds_addr(&s.dws[b][wrow0 + rt * 32 + l32])));
+}
+__device__ __forceinline__ void load_tok_scales(const Stage& s, int b, int tt, uint32_t g, uint32_t wtok0, TokScales& t) {
+    const uint32_t addr = lds_addr(&s.dxf[b][(wtok0 >> 5) + tt][g][0]);
+    asm volatile("ds_read_b128 %0, %1" : "=v"(t.dx[0]) : "v"(addr));
+    asm volatile("ds_read_b128 %0, %1 offset:16" : "=v"(t.dx[1]) : "v"(addr));
+    asm volatile("ds_read_b128 %0, %1 offset:32" : "=v"(t.dx[2]) : "v"(addr));
+    asm volatile("ds_read_b128 %0, %1 offset:48" : "=v"(t.dx[3]) : "v"(addr));
+}
+template <int N>
+__device__ __forceinline__ void mats_ready(Mats& m, RowScales& r) {
+    asm volatile("s_waitcnt lgkmcnt(%6)"
+                 : "+v"(m.av[0]), "+v"(m.av[1]), "+v"(m.bv[0]), "+v"(m.bv[1]), "+v"(r.dw[0]), "+v"(r.dw[1])
+                 : "n"(N)
+                 : "memory");
+}
+template <int N>
+__device__ __forceinline__ void tok_scales_ready(TokScales& t) {
+    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(t.dx[0]), "+v"(t.dx[1]), "+v"(t.dx[2]), "+v"(t.dx[3]) : "n"(N) : "memory");
+}
+
+// Scales one 32 x 32 MFMA result into the f32 accumulators: two full-rate v_fma_f32 per
+// value (a v_fma_mix_f32 with an f16 scale operand would save registers but issues at half
+// the rate, and this kernel is bound by exactly these instructions).
+__device__ __forceinline__ void scale_tile(const v16i& d, const float2 dw, const TokScales& t, float (&acc)[16]) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const float v = __builtin_fmaf(__int_as_float(d[r]), dw.x, dw.y);
+        acc[r] = __builtin_fmaf(v, t.dx[r >> 2][r & 3], acc[r]);
+    }
+}
+
+// Parity hook: the raw i32 block dots of one MFMA result.
+template <int TYPE>
+__device__ __forceinline__ void dump_tile(const GemmArgs& a, const v16i& d, uint32_t row, uint32_t tok_base, uint32_t g, uint32_t nb,
+                                          uint32_t block) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const uint32_t tok = tok_base + 8 * (r >> 2) + 4 * g + (r & 3);
+        if (row < a.m && tok < a.n) {
+            int v = d[r] - (int)kBiasBits;
+            if (TYPE == 2) v >>= 4;  // weights were stored x16; exact
+            a.dots[((size_t)tok * a.m + row) * nb + block] = v;
+        }
     }
 }
 
@@ -253,55 +329,55 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
             load_stage<TYPE>(a, row0, tok0, (st + 1) * KB, regs);
         }
 
-        // 16 MFMA tiles per stage.  Within a wave each MFMA is followed by its 32 FMAs;
-        // the matrix core of a SIMD is kept busy by the other resident wave(s), whose FMA
-        // phases fall into this wave's MFMA latency and vice versa.  The block loop is kept
-        // rolled on purpose: unrolled, the compiler issues all 16 MFMAs of the stage up
-        // front and spills their results.
+        // 16 MFMA tiles per stage, software-pipelined at MFMA granularity: the matrix core
+        // works on tile i+1 while the vector ALU scales tile i (two result buffers), and the
+        // operands of block b+1 are fetched from LDS into registers as soon as block b has
+        // released them, so neither LDS nor MFMA latency sits in the wave's dependency chain.
+        // The scheduling barriers pin that order; the block loop stays rolled (unrolled, the
+        // compiler issues all 16 MFMAs of the stage up front and spills their results).
+        // Tile order within a block: (token tile, row tile) = (0,0) (0,1) (1,0) (1,1).
+        Mats mt;
+        RowScales rs, rs_next;
+        TokScales ts0, ts1;
+        load_mats(s, 0, g, l32, wrow0, wtok0, mt);
+        load_row_scales(s, 0, l32, wrow0, rs);
+        load_tok_scales(s, 0, 0, g, wtok0, ts0);
+        load_tok_scales(s, 0, 1, g, wtok0, ts1);
+        mats_ready<8>(mt, rs);
+        v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[0], mt.bv[0], cbias, 0, 0, 0), d1;
+        tok_scales_ready<4>(ts0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll 1
         for (int b = 0; b < KB; b++) {
-            v4i av[2], bv[2];
-            float2 dw[2];
-            h8 dx[2][2];
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++) {
-                const uint4 t4 = s.xt[b][g][wtok0 + tt * 32 + l32];
-                av[tt] = v4i{(int)t4.x, (int)t4.y, (int)t4.z, (int)t4.w};
-                dx[tt][0] = s.dxh[b][(wtok0 >> 5) + tt][g][0];
-                dx[tt][1] = s.dxh[b][(wtok0 >> 5) + tt][g][1];
-            }
-#pragma unroll
-            for (int rt = 0; rt < 2; rt++) {
-                const uint4 t4 = s.wt[g][b][wrow0 + rt * 32 + l32];
-                bv[rt] = v4i{(int)t4.x, (int)t4.y, (int)t4.z, (int)t4.w};
-                dw[rt] = s.dws[b][wrow0 + rt * 32 + l32];
-            }
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++) {
-#pragma unroll
-                for (int rt = 0; rt < 2; rt++) {
-                    const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[tt], bv[rt], cbias, 0, 0, 0);
-                    if constexpr (DUMP) {
-                        const uint32_t row = row0 + wrow0 + rt * 32 + l32;
-#pragma unroll
-                        for (int r = 0; r < 16; r++) {
-                            const uint32_t tok = tok0 + wtok0 + tt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-                            if (row < a.m && tok < a.n) {
-                                int v = d[r] - (int)kBiasBits;
-                                if (TYPE == 2) v >>= 4;  // weights were stored x16; exact
-                                a.dots[((size_t)tok * a.m + row) * nb + st * KB + b] = v;
-                            }
-                        }
-                    } else {
-#pragma unroll
-                        for (int r = 0; r < 16; r++) {
-                            const float t = __builtin_fmaf(__int_as_float(d[r]), dw[rt].x, dw[rt].y);
-                            acc[tt][rt][r] = __builtin_fmaf(t, (float)dx[tt][r >> 3][r & 7], acc[tt][rt][r]);
-                        }
-                    }
-                }
-            }
+            const int bn = b + 1 < KB ? b + 1 : b;  // last iteration: harmless re-read of its own block
+            const uint32_t row = row0 + wrow0 + l32, tokb = tok0 + wtok0, blk = st * KB + b;
+            d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[0], mt.bv[1], cbias, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (DUMP) dump_tile<TYPE>(a, d0, row, tokb, g, nb, blk); else scale_tile(d0, rs.dw[0], ts0, acc[0][0]);
+            __builtin_amdgcn_sched_barrier(0);
+            d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[1], mt.bv[0], cbias, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (DUMP) dump_tile<TYPE>(a, d1, row + 32, tokb, g, nb, blk); else scale_tile(d1, rs.dw[1], ts0, acc[0][1]);
+            __builtin_amdgcn_sched_barrier(0);
+            d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[1], mt.bv[1], cbias, 0, 0, 0);
+            // block b needs its matrices and the scales of token tile 0 no longer: fetch block b+1's
+            load_tok_scales(s, bn, 0, g, wtok0, ts0);       // 4 reads (ts1 of this block arrived long ago)
+            load_mats(s, bn, g, l32, wrow0, wtok0, mt);     // 4 reads
+            load_row_scales(s, bn, l32, wrow0, rs_next);    // 2 reads
+            tok_scales_ready<10>(ts1);  // issued at the end of the previous iteration, before the ten reads above
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (DUMP) dump_tile<TYPE>(a, d0, row, tokb + 32, g, nb, blk); else scale_tile(d0, rs.dw[0], ts1, acc[1][0]);
+            __builtin_amdgcn_sched_barrier(0);
+            mats_ready<0>(mt, rs_next);
+            tok_scales_ready<0>(ts0);
+            d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[0], mt.bv[0], cbias, 0, 0, 0);  // first tile of block b+1
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (DUMP) dump_tile<TYPE>(a, d1, row + 32, tokb + 32, g, nb, blk); else scale_tile(d1, rs.dw[1], ts1, acc[1][1]);
+            __builtin_amdgcn_sched_barrier(0);
+            load_tok_scales(s, bn, 1, g, wtok0, ts1);       // waited for by the next iteration's lgkmcnt(0)
+            rs = rs_next;
         }
+        tok_scales_ready<0>(ts1);  // nothing of this stage's buffer is read past this point
 
         // The other buffer was last read in stage st-1; every wave has passed the barrier
         // that ended that stage, so it is free to be refilled now.
