@@ -201,22 +201,50 @@ struct TokScales {
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
     return (uint32_t)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
 }
-__device__ __forceinline__ void load_mats(const Stage& s, int b, uint32_t g, uint32_t l32, uint32_t wrow0, uint32_t wtok0, Mats& m) {
-#pragma unroll
-    for (int tt = 0; tt < 2; tt++) asm volatile("ds_read_b128 %0, %1" : "=v"(m.av[tt]) : "v"(lds_addr(&s.xt[b][g][wtok0 + tt * 32 + l32])));
-#pragma unroll
-    for (int rt = 0; rt < 2; rt++) asm volatile("ds_read_b128 %0, %1" : "=v"(m.bv[rt]) : "v"(lds_addr(&s.wt[g][b][wrow0 + rt * 32 + l32])));
+// A lane's four LDS read addresses (its rows of xt / wt / dws / dxf for the block being
+// fetched).  Token tile, row tile and the pieces of a scale row are immediate offsets, so
+// moving to the next block costs four additions instead of one per read.
+struct LaneAddr {
+    uint32_t xt, wt, dws, dxf;
+};
+constexpr int kOffXt = sizeof(uint4) * 2 * (BN + 1);         // one block of xt
+constexpr int kOffWt = sizeof(uint4) * (BM + 2);             // one block of wt (within a khalf plane)
+constexpr int kOffDws = sizeof(float2) * (BM + 2);           // one block of dws
+constexpr int kOffDxf = sizeof(float4) * (BN / 32) * 2 * 4;  // one block of dxf
+__device__ __forceinline__ void next_block(LaneAddr& la, bool advance) {
+    la.xt += advance ? kOffXt : 0;
+    la.wt += advance ? kOffWt : 0;
+    la.dws += advance ? kOffDws : 0;
+    la.dxf += advance ? kOffDxf : 0;
 }
-__device__ __forceinline__ void load_row_scales(const Stage& s, int b, uint32_t l32, uint32_t wrow0, RowScales& r) {
-#pragma unroll
-    for (int rt = 0; rt < 2; rt++) asm volatile("ds_read_b64 %0, %1" : "=v"(r.dw[rt]) : "v"(lds_addr(&s.dws[b][wrow0 + rt * 32 + l32])));
+template <int OFF>
+__device__ __forceinline__ void lds_read16(uint32_t addr, v4i& dst) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
-__device__ __forceinline__ void load_tok_scales(const Stage& s, int b, int tt, uint32_t g, uint32_t wtok0, TokScales& t) {
-    const uint32_t addr = lds_addr(&s.dxf[b][(wtok0 >> 5) + tt][g][0]);
-    asm volatile("ds_read_b128 %0, %1" : "=v"(t.dx[0]) : "v"(addr));
-    asm volatile("ds_read_b128 %0, %1 offset:16" : "=v"(t.dx[1]) : "v"(addr));
-    asm volatile("ds_read_b128 %0, %1 offset:32" : "=v"(t.dx[2]) : "v"(addr));
-    asm volatile("ds_read_b128 %0, %1 offset:48" : "=v"(t.dx[3]) : "v"(addr));
+template <int OFF>
+__device__ __forceinline__ void lds_read16(uint32_t addr, v4f& dst) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF>
+__device__ __forceinline__ void lds_read8(uint32_t addr, float2& dst) {
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+__device__ __forceinline__ void load_mats(const LaneAddr& la, Mats& m) {
+    lds_read16<0>(la.xt, m.av[0]);
+    lds_read16<32 * 16>(la.xt, m.av[1]);
+    lds_read16<0>(la.wt, m.bv[0]);
+    lds_read16<32 * 16>(la.wt, m.bv[1]);
+}
+__device__ __forceinline__ void load_row_scales(const LaneAddr& la, RowScales& r) {
+    lds_read8<0>(la.dws, r.dw[0]);
+    lds_read8<32 * 8>(la.dws, r.dw[1]);
+}
+template <int TT>
+__device__ __forceinline__ void load_tok_scales(const LaneAddr& la, TokScales& t) {
+    lds_read16<TT * 128 + 0>(la.dxf, t.dx[0]);
+    lds_read16<TT * 128 + 16>(la.dxf, t.dx[1]);
+    lds_read16<TT * 128 + 32>(la.dxf, t.dx[2]);
+    lds_read16<TT * 128 + 48>(la.dxf, t.dx[3]);
 }
 template <int N>
 __device__ __forceinline__ void mats_ready(Mats& m, RowScales& r) {
@@ -312,6 +340,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
     v16i cbias;
 #pragma unroll
     for (int r = 0; r < 16; r++) cbias[r] = (int)kBiasBits;
+    asm volatile("" : "+v"(cbias));  // keep it in registers: left alone, the compiler rebuilds all 16 before every MFMA group
 
     StageRegs<TYPE> regs;
     dma_activations(a, sm.st[0], tok0, 0);
@@ -339,17 +368,22 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
         Mats mt;
         RowScales rs, rs_next;
         TokScales ts0, ts1;
-        load_mats(s, 0, g, l32, wrow0, wtok0, mt);
-        load_row_scales(s, 0, l32, wrow0, rs);
-        load_tok_scales(s, 0, 0, g, wtok0, ts0);
-        load_tok_scales(s, 0, 1, g, wtok0, ts1);
+        LaneAddr la;  // block 0 of this stage's buffer
+        la.xt = lds_addr(&s.xt[0][g][wtok0 + l32]);
+        la.wt = lds_addr(&s.wt[g][0][wrow0 + l32]);
+        la.dws = lds_addr(&s.dws[0][wrow0 + l32]);
+        la.dxf = lds_addr(&s.dxf[0][wtok0 >> 5][g][0]);
+        load_mats(la, mt);
+        load_row_scales(la, rs);
+        load_tok_scales<0>(la, ts0);
+        load_tok_scales<1>(la, ts1);
         mats_ready<8>(mt, rs);
         v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[0], mt.bv[0], cbias, 0, 0, 0), d1;
         tok_scales_ready<4>(ts0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll 1
         for (int b = 0; b < KB; b++) {
-            const int bn = b + 1 < KB ? b + 1 : b;  // last iteration: harmless re-read of its own block
+            next_block(la, b + 1 < KB);  // last iteration: harmless re-read of its own block
             const uint32_t row = row0 + wrow0 + l32, tokb = tok0 + wtok0, blk = st * KB + b;
             d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[0], mt.bv[1], cbias, 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
@@ -361,9 +395,9 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
             __builtin_amdgcn_sched_barrier(0);
             d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[1], mt.bv[1], cbias, 0, 0, 0);
             // block b needs its matrices and the scales of token tile 0 no longer: fetch block b+1's
-            load_tok_scales(s, bn, 0, g, wtok0, ts0);       // 4 reads (ts1 of this block arrived long ago)
-            load_mats(s, bn, g, l32, wrow0, wtok0, mt);     // 4 reads
-            load_row_scales(s, bn, l32, wrow0, rs_next);    // 2 reads
+            load_tok_scales<0>(la, ts0);    // 4 reads (ts1 of this block arrived long ago)
+            load_mats(la, mt);              // 4 reads
+            load_row_scales(la, rs_next);   // 2 reads
             tok_scales_ready<10>(ts1);  // issued at the end of the previous iteration, before the ten reads above
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (DUMP) dump_tile<TYPE>(a, d0, row, tokb + 32, g, nb, blk); else scale_tile(d0, rs.dw[0], ts1, acc[1][0]);
@@ -374,7 +408,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (DUMP) dump_tile<TYPE>(a, d1, row + 32, tokb + 32, g, nb, blk); else scale_tile(d1, rs.dw[1], ts1, acc[1][1]);
             __builtin_amdgcn_sched_barrier(0);
-            load_tok_scales(s, bn, 1, g, wtok0, ts1);       // waited for by the next iteration's lgkmcnt(0)
+            load_tok_scales<1>(la, ts1);    // waited for by the next iteration's lgkmcnt(0)
             rs = rs_next;
         }
         tok_scales_ready<0>(ts1);  // nothing of this stage's buffer is read past this point
