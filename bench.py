@@ -410,12 +410,12 @@ def main():
             "unit": "GB/s",
             "frac": dec["gemv_kernel_GBps"] / HBM_PEAK_GBS,
             # HBM bytes per launch (average over the 65 launches of a step) from the calibrated FETCH_SIZE / WRITE_SIZE passes
-            # recorded in profiles/decode_step_lfm2_350m_q4_0.txt: (22*4.29 + 16*2.93 + 37.88 + 26*1.15 MB read + ~1.2 MB written) / 65
-            "traffic": 3.24e6,
+            # recorded in profiles/decode_step_lfm2_350m_q4_0.txt: mean over all GEMV dispatches of the step, 3.21 MB read + 0.02 MB written
+            "traffic": 3.23e6,
             "traffic_source": "profiles/decode_step_lfm2_350m_q4_0.txt (rocprofv3 --pmc FETCH_SIZE x2.0, WRITE_SIZE x1.0; copy-calibrated)",
             "bytes_per_launch_avg": dec["gemv_bytes_per_step"] / dec["gemv_launches_per_step"],
             "avg_launch_us": dec["gemv_kernel_avg_us"],
-            "note": "per-dispatch timestamps include ~4 us of fixed dispatch cost per launch; in the graph the same launches average "
+            "note": "per-dispatch timestamps include a fixed dispatch cost per launch; in the graph the same launches average "
                     f"{dec['us_per_launch_in_graph']:.2f} us each",
         },
         "decode_step": dec,
@@ -426,8 +426,8 @@ def main():
         g = bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048)
         g["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma_kernel<Q4_0>", "achieved": g["gemm_kernel_TOPS"], "peak": INT8_PEAK_TOPS,
                          "unit": "TOP/s", "frac": g["gemm_kernel_TOPS"] / INT8_PEAK_TOPS,
-                         # 84.84 MB read + 60.04 MB written per launch (algorithmic 12.57 + 55.35 MB), profiles/gemm_q4_0_6912x2002x2048.txt
-                         "traffic": 144.9e6, "traffic_source": "profiles/gemm_q4_0_6912x2002x2048.txt"}
+                         # 79.20 MB read + 55.35 MB written per launch (algorithmic 12.57 + 55.35 MB), profiles/gemm_q4_0_6912x2002x2048.txt
+                         "traffic": 134.6e6, "traffic_source": "profiles/gemm_q4_0_6912x2002x2048.txt"}
         out["gemm"] = g
         del host_weights  # the CPU leg regenerates what it needs; keep host memory low
         dq = bench_decode(ctx, W, O, W.Q8_0, max(10, args.steps // 2), args.warmup, synth_decode_weights(O, W.Q8_0), with_unfused=False)
