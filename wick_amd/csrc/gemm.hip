@@ -8,30 +8,36 @@
 // blocks: every v_mfma_i32_32x32x32_i8 covers exactly one block (K = 32) and its
 // 32x32 i32 result is scaled into f32 accumulators on the vector ALU.
 //
-// Workgroup = 256 threads = 4 waves, tile = 128 weight rows x 128 tokens, each
-// wave owns 64 x 64 (2 x 2 MFMA tiles).  One stage = 4 blocks (128 elements of K):
-//   * weights: each thread reads one 36/68-byte block pair with dword-aligned wide
-//     loads, unpacks nibbles to int8 and writes 16-byte operand rows to LDS;
+// Workgroup = 512 threads = 8 waves, tile = 128 weight rows x 128 tokens, each wave
+// owns 64 rows x 32 tokens = 4 x 2 tiles of v_mfma_i32_16x16x32_i8.  The small MFMA
+// shape is chosen for its register footprint: 4 result registers per tile (16 for the
+// 32x32 shape), a 4-register bias and 4 token scales per tile keep the kernel under 128
+// VGPRs, so FOUR waves share a SIMD.  That matters more than the matrix rate (the 16x16x32
+// instruction runs at half the 32x32x32 rate, 1.9 vs 3.8 POP/s measured): a wave can issue
+// a vector-ALU instruction only every ~4.7 cycles while a SIMD retires one every ~2.2, and
+// the kernel is bound by the two scaling FMAs per result.
+// One stage = 4 blocks (128 elements of K):
+//   * weights: threads 0-255 read one 36/68-byte block pair each with dword-aligned wide
+//     loads, unpack nibbles to int8 and write 16-byte operand rows to LDS;
 //   * activations: copied global -> LDS directly (global_load_lds_dwordx4, asynchronous,
-//     no registers); token scales through registers (f32 -> f16, lane order).
-// LDS holds two stages.  The global loads of stage s+1 are issued before stage s is
-// computed and written to the other LDS buffer after it, so there is one barrier
-// per stage and the load latency hides behind the stage's ALU work.
+//     no registers); token scales through registers.
+// LDS holds two stages (77 KB, two workgroups per CU).  The global loads of stage s+1 are
+// issued before stage s is computed and written to the other LDS buffer after it, so there
+// is one barrier per stage and the load latency hides behind the stage's ALU work.
 //
-// LDS operand layout: [block][khalf][row][16 bytes].  An MFMA lane supplies 16
-// consecutive K-bytes of one operand row, lanes 0-31 the first half of the block
-// and lanes 32-63 the second, so 32 consecutive lanes read 512 consecutive bytes:
-// conflict-free.  For Q4_0 the low nibbles of a block ARE its first 16 elements and
-// the high nibbles its last 16 (wick/src/quant.rs:82-88), so the two halves fall
-// out of one and / shift each.  (The K order inside an MFMA is irrelevant as long
-// as both operands use the same one.)
+// LDS operand layout: [block][khalf][row][16 bytes] (weights: [khalf][block][row]).  An
+// MFMA lane supplies 8 consecutive K-bytes of operand row lane % 16, K-quarter lane / 16,
+// so 32 consecutive lanes read 256 consecutive bytes (the two 8-byte halves of 16 rows):
+// conflict-free.  For Q4_0 the low nibbles of a block ARE its first 16 elements and the
+// high nibbles its last 16 (wick/src/quant.rs:82-88), so the two halves fall out of one
+// and / shift each.  (The K order inside an MFMA is irrelevant as long as both operands
+// use the same one.)
 //
-// Roles: tokens are the MFMA "A" (M) operand, weight rows the "B" (N) operand, so
-// in the 32x32 result a lane holds ONE weight row (n = lane % 32) and 16 tokens
-// (m = 8*(r/4) + 4*(lane/32) + r%4).  Its weight scale is one register per block;
-// the 16 token scales are kept as f16 in LDS, stored in the order a lane consumes
-// them (32 contiguous bytes per lane half, tile and block) and fed to the FMA as
-// f16 operands (v_fma_mix_f32), which is exact because they ARE f16 values.
+// Roles: tokens are the MFMA "A" (M) operand, weight rows the "B" (N) operand, so in the
+// 16x16 result a lane holds ONE weight row (n = lane % 16) and 4 consecutive tokens
+// (m = 4*(lane/16) + r).  Its weight scale is one register pair per block and row tile;
+// the token scales sit in LDS as f32, token-major, and a lane reads its four with one
+// 16-byte read (a broadcast within each group of 16 lanes).
 //
 // Scaling is what bounds this kernel (vector ALU, not the matrix core), so it is
 // cut to two FMAs per result:
@@ -43,7 +49,8 @@
 //     gives exactly the f32 12582912 + v, so the i32 -> f32 conversion is free.
 //   * t = fma(D_as_f32, dw, -12582912*dw) = round(v * dw) exactly (single rounding;
 //     12582912*dw is exact because dw has an 11-bit significand);
-//     acc = fma(t, dx, acc).
+//     acc = fma(t, dx, acc), both plain v_fma_f32 (v_fma_mix_f32 with an f16 scale
+//     operand would save registers but issues at half the rate).
 #include "wick_rocm_device.h"
 #include "wick_rocm_internal.h"
 
@@ -54,12 +61,13 @@ namespace {
 constexpr int BM = 128;       // weight rows per workgroup
 constexpr int BN = 128;       // tokens per workgroup
 constexpr int KB = 4;         // blocks per stage
-constexpr int THREADS = 256;  // 4 waves: 2 (rows) x 2 (tokens)
+constexpr int THREADS = 512;  // 8 waves: 2 (rows) x 4 (tokens)
+constexpr int TT = 2;          // 16-token MFMA tiles per wave
+constexpr int RT = 4;          // 16-row MFMA tiles per wave
 constexpr uint32_t kBiasBits = 0x4B400000u;  // 12582912.0f
 constexpr float kBias = 12582912.0f;
 
 typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 struct GemmArgs {
@@ -81,9 +89,9 @@ struct GemmArgs {
 // walk consecutive rows of one plane.
 struct Stage {
     uint4 wt[2][KB][BM + 2];    // [khalf][block][row]  int8 weights (Q4_0: x16)
-    uint4 xt[KB][2][BN + 1];    // [block][khalf][token] int8 activations
+    uint4 xt[BN][2 * KB];       // [token][16-byte K-chunk, swizzled] int8 activations, see dma_activations
     float2 dws[KB][BM + 2];     // {dw, -12582912*dw} per block and row (dw x 1/16 for Q4_0)
-    float4 dxf[KB][BN / 32][2][4];  // [block][token tile][lane half][16 floats]: token scales in the order a lane consumes them
+    float dxf[KB][BN];          // token scales
 };
 
 struct Smem {
@@ -102,41 +110,46 @@ struct StageRegs {
 
 // Activation tiles go global -> LDS directly (global_load_lds_dwordx4): no staging
 // registers, no unpack, no ds_write, and the copy runs asynchronously under the stage's
-// ALU work.  One wave instruction fills 64 consecutive tokens of one [block][khalf]
-// plane (lane l -> token l, 16 bytes each, contiguous 1 KB in LDS); a stage has
-// 8 planes x 2 token halves = 16 such instructions, four per wave.
+// ALU work.  A token's 128 K-bytes of the stage are exactly one cache line, so one wave
+// instruction fetches 8 tokens x 8 16-byte chunks = 8 whole lines (lane l -> token l / 8,
+// position l % 8; the address unit works per line touched, and a chunk-major split would
+// touch 64 lines per instruction).  Direct-to-LDS data lands lane-contiguous, i.e. as
+// [token][8 positions] rows of 128 bytes, which an MFMA operand read (16 tokens, same
+// chunk) would hit with an 8-way bank conflict.  So position p of token t holds K-chunk
+// p ^ ((t >> 1) & 7): the lane picks its GLOBAL chunk accordingly, and 16 consecutive
+// tokens reading one chunk then spread over all banks.  16 instructions per stage, two
+// per wave.
+__device__ __forceinline__ uint32_t xt_swizzle(uint32_t token_in_tile) { return (token_in_tile >> 1) & 7u; }
 __device__ __forceinline__ void dma_activations(const GemmArgs& a, Stage& s, uint32_t tok0, uint32_t kb0) {
     const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // = block of the stage
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 #pragma unroll
-    for (int half = 0; half < 2; half++) {
-        const uint32_t tok = min(tok0 + 64u * half + lane, a.n - 1);
-        const int8_t* src = a.xq + (size_t)tok * a.k + (size_t)(kb0 + wave) * 32;
-#pragma unroll
-        for (int kh = 0; kh < 2; kh++) {
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(src + 16 * kh),
-                                             (void __attribute__((address_space(3)))*)&s.xt[wave][kh][64 * half], 16, 0, 0);
-        }
+    for (int j = 0; j < 2; j++) {
+        const uint32_t t = 8u * (2u * wave + j) + (lane >> 3);  // token within the tile
+        const uint32_t chunk = (lane & 7u) ^ xt_swizzle(t);
+        const uint32_t tok = min(tok0 + t, a.n - 1);
+        const int8_t* src = a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + 16u * chunk;
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+                                         (void __attribute__((address_space(3)))*)&s.xt[8u * (2u * wave + j)][0], 16, 0, 0);
     }
 }
 
 // Thread -> work of one stage:
-//   weights      256 pairs   = 128 rows x 2 pairs             : row = t >> 1, pair = t & 1
+//   weights      256 pairs   = 128 rows x 2 pairs             : threads 0..255, row = t >> 1, pair = t & 1
 //   activations  direct-to-LDS, see dma_activations
-//   token scales 128 tokens x 4 blocks (one float4)           : threads 0..127, token = t
+//   token scales 128 tokens x 4 blocks (one float4)           : threads 256..383, token = t - 256
 template <int TYPE>
 __device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uint32_t tok0, uint32_t kb0,
                                            StageRegs<TYPE>& r) {
     using PT = PairTraits<TYPE>;
     const uint32_t t = threadIdx.x;
     const uint32_t nb = a.k >> 5;
-    {
+    if (t < 2 * BM) {
         const uint32_t row = min(row0 + (t >> 1), a.m - 1);
         const uint8_t* p = a.w + ((size_t)row * nb + kb0 + 2 * (t & 1u)) * (PT::BYTES / 2);
         load_pair<PT::DWORDS>(p, r.w);
-    }
-    if (t < BN && a.xs) {  // xs is null only for the parity hook, which never scales
-        const uint32_t tok = min(tok0 + t, a.n - 1);
+    } else if (t < 2 * BM + BN && a.xs) {  // xs is null only for the parity hook, which never scales
+        const uint32_t tok = min(tok0 + (t - 2 * BM), a.n - 1);
         r.dx = *reinterpret_cast<const float4*>(a.xs + (size_t)tok * nb + kb0);
     } else {
         r.dx = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -147,7 +160,7 @@ template <int TYPE>
 __device__ __forceinline__ void store_stage(Stage& s, const StageRegs<TYPE>& r) {
     using PT = PairTraits<TYPE>;
     const uint32_t t = threadIdx.x;
-    {
+    if (t < 2 * BM) {
         const uint32_t row = t >> 1;
         const uint32_t b0 = 2 * (t & 1u);
         uint32_t d0, d1, q0[PT::NQ], q1[PT::NQ];
@@ -168,27 +181,22 @@ __device__ __forceinline__ void store_stage(Stage& s, const StageRegs<TYPE>& r) 
             s.wt[1][b0 + 1][row] = make_uint4(q1[4], q1[5], q1[6], q1[7]);
         }
     }
-    if (t < BN) {
-        // token t of the tile sits at MFMA row t % 32 = 8*gq + 4*g + e -> lane half g, slot 4*gq + e
-        const uint32_t tile = t >> 5, g = (t >> 2) & 1u, slot = ((t >> 3) & 3u) * 4 + (t & 3u);
-        float* base = reinterpret_cast<float*>(&s.dxf[0][tile][g][0]) + slot;
-        constexpr int kBlockStride = sizeof(s.dxf[0]) / sizeof(float);
-        base[0 * kBlockStride] = r.dx.x;
-        base[1 * kBlockStride] = r.dx.y;
-        base[2 * kBlockStride] = r.dx.z;
-        base[3 * kBlockStride] = r.dx.w;
+    if (t >= 2 * BM && t < 2 * BM + BN) {
+        const uint32_t u = t - 2 * BM;
+        s.dxf[0][u] = r.dx.x;
+        s.dxf[1][u] = r.dx.y;
+        s.dxf[2][u] = r.dx.z;
+        s.dxf[3][u] = r.dx.w;
     }
 }
 
-// Per-block operands of a wave's 2 x 2 MFMA tiles.
+// Per-block operands of a wave's TT x RT MFMA tiles: 8 K-bytes of this lane's operand row.
 struct Mats {
-    v4i av[2], bv[2];  // [token tile], [row tile]: 16 K-bytes of this lane's operand row
+    long av[TT], bv[RT];
 };
-struct RowScales {
-    float2 dw[2];  // {dw, -12582912*dw} of this lane's weight row, per row tile
-};
-struct TokScales {
-    v4f dx[4];  // the 16 token scales of one token tile, in result-register order
+struct Scales {
+    float2 dw[RT];  // {dw, -12582912*dw} of this lane's weight row, per row tile
+    v4f dx[TT];     // scales of this lane's four tokens, per token tile
 };
 
 // All LDS reads of the main loop are inline assembly on purpose.  While direct-to-LDS
@@ -196,90 +204,93 @@ struct TokScales {
 // every LDS read it can see wait for all of them, which would put the whole global-memory
 // latency at the start of each stage.  These reads touch only the current buffer; the
 // copies are waited for explicitly before the barrier that ends the stage.  Data arrives
-// in issue order; the *_ready functions are the matching waits (at most N later LDS reads
-// still outstanding) and tie the registers, so nothing can use them earlier.
+// in issue order; lds_wait<N> is the matching wait (at most N later LDS reads still
+// outstanding) and ties the registers, so nothing can use them earlier.
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
     return (uint32_t)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
 }
-// A lane's four LDS read addresses (its rows of xt / wt / dws / dxf for the block being
-// fetched).  Token tile, row tile and the pieces of a scale row are immediate offsets, so
-// moving to the next block costs four additions instead of one per read.
+// A lane's four LDS read addresses (its rows of xt / wt / dws and its tokens of dxf for the
+// block being fetched).  Tile indices are immediate offsets; moving to the next block costs
+// three additions and, for the swizzled activation tile, one xor + shift-add:
+// xt = xbase + ((block ^ xsh) << 5).
 struct LaneAddr {
     uint32_t xt, wt, dws, dxf;
+    uint32_t xbase, xsh;
 };
-constexpr int kOffXt = sizeof(uint4) * 2 * (BN + 1);         // one block of xt
-constexpr int kOffWt = sizeof(uint4) * (BM + 2);             // one block of wt (within a khalf plane)
-constexpr int kOffDws = sizeof(float2) * (BM + 2);           // one block of dws
-constexpr int kOffDxf = sizeof(float4) * (BN / 32) * 2 * 4;  // one block of dxf
-__device__ __forceinline__ void next_block(LaneAddr& la, bool advance) {
-    la.xt += advance ? kOffXt : 0;
+constexpr int kOffWt = sizeof(uint4) * (BM + 2);      // one block of wt (within a khalf plane)
+constexpr int kOffDws = sizeof(float2) * (BM + 2);    // one block of dws
+constexpr int kOffDxf = sizeof(float) * BN;           // one block of dxf
+__device__ __forceinline__ void next_block(LaneAddr& la, uint32_t block, bool advance) {
+    la.xt = la.xbase + (((advance ? block + 1 : block) ^ la.xsh) << 5);
     la.wt += advance ? kOffWt : 0;
     la.dws += advance ? kOffDws : 0;
     la.dxf += advance ? kOffDxf : 0;
-}
-template <int OFF>
-__device__ __forceinline__ void lds_read16(uint32_t addr, v4i& dst) {
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
 template <int OFF>
 __device__ __forceinline__ void lds_read16(uint32_t addr, v4f& dst) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
 template <int OFF>
+__device__ __forceinline__ void lds_read8(uint32_t addr, long& dst) {
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF>
 __device__ __forceinline__ void lds_read8(uint32_t addr, float2& dst) {
     asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
-__device__ __forceinline__ void load_mats(const LaneAddr& la, Mats& m) {
-    lds_read16<0>(la.xt, m.av[0]);
-    lds_read16<32 * 16>(la.xt, m.av[1]);
-    lds_read16<0>(la.wt, m.bv[0]);
-    lds_read16<32 * 16>(la.wt, m.bv[1]);
+__device__ __forceinline__ void load_mats(const LaneAddr& la, Mats& m) {  // TT + RT = 6 reads
+    lds_read8<0 * 16 * 128>(la.xt, m.av[0]);  // 16 tokens further: same swizzle
+    lds_read8<1 * 16 * 128>(la.xt, m.av[1]);
+    lds_read8<0 * 256>(la.wt, m.bv[0]);
+    lds_read8<1 * 256>(la.wt, m.bv[1]);
+    lds_read8<2 * 256>(la.wt, m.bv[2]);
+    lds_read8<3 * 256>(la.wt, m.bv[3]);
 }
-__device__ __forceinline__ void load_row_scales(const LaneAddr& la, RowScales& r) {
-    lds_read8<0>(la.dws, r.dw[0]);
-    lds_read8<32 * 8>(la.dws, r.dw[1]);
+__device__ __forceinline__ void load_row_scales(const LaneAddr& la, Scales& s) {  // RT = 4 reads
+    lds_read8<0 * 128>(la.dws, s.dw[0]);
+    lds_read8<1 * 128>(la.dws, s.dw[1]);
+    lds_read8<2 * 128>(la.dws, s.dw[2]);
+    lds_read8<3 * 128>(la.dws, s.dw[3]);
 }
-template <int TT>
-__device__ __forceinline__ void load_tok_scales(const LaneAddr& la, TokScales& t) {
-    lds_read16<TT * 128 + 0>(la.dxf, t.dx[0]);
-    lds_read16<TT * 128 + 16>(la.dxf, t.dx[1]);
-    lds_read16<TT * 128 + 32>(la.dxf, t.dx[2]);
-    lds_read16<TT * 128 + 48>(la.dxf, t.dx[3]);
+template <int T>
+__device__ __forceinline__ void load_tok_scales(const LaneAddr& la, Scales& s) {  // 1 read
+    lds_read16<T * 64>(la.dxf, s.dx[T]);
 }
 template <int N>
-__device__ __forceinline__ void mats_ready(Mats& m, RowScales& r) {
+__device__ __forceinline__ void lds_wait(Mats& m) {
     asm volatile("s_waitcnt lgkmcnt(%6)"
-                 : "+v"(m.av[0]), "+v"(m.av[1]), "+v"(m.bv[0]), "+v"(m.bv[1]), "+v"(r.dw[0]), "+v"(r.dw[1])
+                 : "+v"(m.av[0]), "+v"(m.av[1]), "+v"(m.bv[0]), "+v"(m.bv[1]), "+v"(m.bv[2]), "+v"(m.bv[3])
                  : "n"(N)
                  : "memory");
 }
 template <int N>
-__device__ __forceinline__ void tok_scales_ready(TokScales& t) {
-    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(t.dx[0]), "+v"(t.dx[1]), "+v"(t.dx[2]), "+v"(t.dx[3]) : "n"(N) : "memory");
+__device__ __forceinline__ void lds_wait(Scales& s) {
+    asm volatile("s_waitcnt lgkmcnt(%6)"
+                 : "+v"(s.dw[0]), "+v"(s.dw[1]), "+v"(s.dw[2]), "+v"(s.dw[3]), "+v"(s.dx[0]), "+v"(s.dx[1])
+                 : "n"(N)
+                 : "memory");
 }
 
-// Scales one 32 x 32 MFMA result into the f32 accumulators: two full-rate v_fma_f32 per
-// value (a v_fma_mix_f32 with an f16 scale operand would save registers but issues at half
-// the rate, and this kernel is bound by exactly these instructions).
-__device__ __forceinline__ void scale_tile(const v16i& d, const float2 dw, const TokScales& t, float (&acc)[16]) {
+// Scales one 16 x 16 MFMA result (4 values per lane) into the f32 accumulators: two
+// full-rate v_fma_f32 per value.
+__device__ __forceinline__ void scale_tile(const v4i& d, const float2 dw, const v4f& dx, float (&acc)[4]) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
+    for (int r = 0; r < 4; r++) {
         const float v = __builtin_fmaf(__int_as_float(d[r]), dw.x, dw.y);
-        acc[r] = __builtin_fmaf(v, t.dx[r >> 2][r & 3], acc[r]);
+        acc[r] = __builtin_fmaf(v, dx[r], acc[r]);
     }
 }
 
-// Parity hook: the raw i32 block dots of one MFMA result.
+// Parity hook: the raw i32 block dots of one MFMA result.  row = this lane's weight row,
+// tok = the first of its four tokens.
 template <int TYPE>
-__device__ __forceinline__ void dump_tile(const GemmArgs& a, const v16i& d, uint32_t row, uint32_t tok_base, uint32_t g, uint32_t nb,
-                                          uint32_t block) {
+__device__ __forceinline__ void dump_tile(const GemmArgs& a, const v4i& d, uint32_t row, uint32_t tok, uint32_t nb, uint32_t block) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const uint32_t tok = tok_base + 8 * (r >> 2) + 4 * g + (r & 3);
-        if (row < a.m && tok < a.n) {
+    for (int r = 0; r < 4; r++) {
+        if (row < a.m && tok + r < a.n) {
             int v = d[r] - (int)kBiasBits;
             if (TYPE == 2) v >>= 4;  // weights were stored x16; exact
-            a.dots[((size_t)tok * a.m + row) * nb + block] = v;
+            a.dots[((size_t)(tok + r) * a.m + row) * nb + block] = v;
         }
     }
 }
@@ -311,7 +322,7 @@ __device__ __forceinline__ void tile_of_block(uint32_t bid, uint32_t row_tiles, 
 }
 
 template <int TYPE, bool DUMP>
-__global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
+__global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
     __shared__ Smem sm;
     uint32_t row_tile, tok_tile;
     bool valid_tile;
@@ -322,25 +333,23 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t l32 = lane & 31u;
-    const uint32_t g = lane >> 5;             // which 16-byte half of the block this lane feeds
-    const uint32_t wrow0 = (wave >> 1) * 64;  // wave's rows within the tile
-    const uint32_t wtok0 = (wave & 1u) * 64;
+    const uint32_t l16 = lane & 15u;
+    const uint32_t kq = lane >> 4;            // which 8-byte quarter of the block this lane feeds
+    const uint32_t wrow0 = (wave >> 2) * 64;  // wave's rows within the tile
+    const uint32_t wtok0 = (wave & 3u) * 32;  // wave's tokens within the tile
     const uint32_t nb = a.k >> 5;
     const uint32_t stages = nb / KB;
 
-    float acc[2][2][16];
+    float acc[TT][RT][4];
 #pragma unroll
-    for (int tt = 0; tt < 2; tt++)
+    for (int tt = 0; tt < TT; tt++)
 #pragma unroll
-        for (int rt = 0; rt < 2; rt++)
+        for (int rt = 0; rt < RT; rt++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[tt][rt][r] = 0.0f;
+            for (int r = 0; r < 4; r++) acc[tt][rt][r] = 0.0f;
 
-    v16i cbias;
-#pragma unroll
-    for (int r = 0; r < 16; r++) cbias[r] = (int)kBiasBits;
-    asm volatile("" : "+v"(cbias));  // keep it in registers: left alone, the compiler rebuilds all 16 before every MFMA group
+    v4i cbias = {(int)kBiasBits, (int)kBiasBits, (int)kBiasBits, (int)kBiasBits};
+    asm volatile("" : "+v"(cbias));  // keep it in registers (left alone, the compiler rebuilds it before every MFMA)
 
     StageRegs<TYPE> regs;
     dma_activations(a, sm.st[0], tok0, 0);
@@ -358,60 +367,55 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
             load_stage<TYPE>(a, row0, tok0, (st + 1) * KB, regs);
         }
 
-        // 16 MFMA tiles per stage, software-pipelined at MFMA granularity: the matrix core
-        // works on tile i+1 while the vector ALU scales tile i (two result buffers), and the
-        // operands of block b+1 are fetched from LDS into registers as soon as block b has
-        // released them, so neither LDS nor MFMA latency sits in the wave's dependency chain.
-        // The scheduling barriers pin that order; the block loop stays rolled (unrolled, the
-        // compiler issues all 16 MFMAs of the stage up front and spills their results).
-        // Tile order within a block: (token tile, row tile) = (0,0) (0,1) (1,0) (1,1).
-        Mats mt;
-        RowScales rs, rs_next;
-        TokScales ts0, ts1;
+        // 8 MFMA tiles per block, software-pipelined by hand: four result buffers, the matrix
+        // core runs up to four tiles ahead of the vector ALU, and every operand register is
+        // refilled from LDS (for block b+1) as soon as its last use in block b has been
+        // issued, so LDS latency stays out of the wave's dependency chain.  The scheduling
+        // barriers pin that order; the block loop stays rolled.
+        // Tile order: t = 4 * token tile + row tile.
         LaneAddr la;  // block 0 of this stage's buffer
-        la.xt = lds_addr(&s.xt[0][g][wtok0 + l32]);
-        la.wt = lds_addr(&s.wt[g][0][wrow0 + l32]);
-        la.dws = lds_addr(&s.dws[0][wrow0 + l32]);
-        la.dxf = lds_addr(&s.dxf[0][wtok0 >> 5][g][0]);
-        load_mats(la, mt);
-        load_row_scales(la, rs);
-        load_tok_scales<0>(la, ts0);
-        load_tok_scales<1>(la, ts1);
-        mats_ready<8>(mt, rs);
-        v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[0], mt.bv[0], cbias, 0, 0, 0), d1;
-        tok_scales_ready<4>(ts0);
-        __builtin_amdgcn_sched_barrier(0);
+        // this lane's token row; K-chunk 2*block + (kq >> 1) sits at position chunk ^ swizzle
+        la.xsh = xt_swizzle(wtok0 + l16) >> 1;
+        la.xbase = lds_addr(&s.xt[wtok0 + l16][0]) + ((((kq >> 1) ^ xt_swizzle(wtok0 + l16)) & 1u) << 4) + 8 * (kq & 1u);
+        la.xt = la.xbase + (la.xsh << 5);
+        la.wt = lds_addr(&s.wt[kq >> 1][0][wrow0 + l16]) + 8 * (kq & 1u);
+        la.dws = lds_addr(&s.dws[0][wrow0 + l16]);
+        la.dxf = lds_addr(&s.dxf[0][wtok0 + 4 * kq]);
+        Mats mt;
+        Scales sc;
+        load_mats(la, mt);              // 6 reads
+        load_tok_scales<0>(la, sc);     // 1
+        load_tok_scales<1>(la, sc);     // 1
+        load_row_scales(la, sc);        // 4
 #pragma unroll 1
         for (int b = 0; b < KB; b++) {
-            next_block(la, b + 1 < KB);  // last iteration: harmless re-read of its own block
-            const uint32_t row = row0 + wrow0 + l32, tokb = tok0 + wtok0, blk = st * KB + b;
-            d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[0], mt.bv[1], cbias, 0, 0, 0);
+            next_block(la, (uint32_t)b, b + 1 < KB);  // last iteration: harmless re-read of its own block
+            const uint32_t row = row0 + wrow0 + l16, tok = tok0 + wtok0 + 4 * kq, blk = st * KB + b;
+            v4i d[4];
+            lds_wait<6>(mt);  // the six reads issued after the matrices may still be in flight
+#pragma unroll
+            for (int t = 0; t < 4; t++) d[t] = __builtin_amdgcn_mfma_i32_16x16x32_i8(mt.av[0], mt.bv[t], cbias, 0, 0, 0);
+            lds_wait<0>(sc);
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (DUMP) dump_tile<TYPE>(a, d0, row, tokb, g, nb, blk); else scale_tile(d0, rs.dw[0], ts0, acc[0][0]);
-            __builtin_amdgcn_sched_barrier(0);
-            d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[1], mt.bv[0], cbias, 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (DUMP) dump_tile<TYPE>(a, d1, row + 32, tokb, g, nb, blk); else scale_tile(d1, rs.dw[1], ts0, acc[0][1]);
-            __builtin_amdgcn_sched_barrier(0);
-            d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[1], mt.bv[1], cbias, 0, 0, 0);
-            // block b needs its matrices and the scales of token tile 0 no longer: fetch block b+1's
-            load_tok_scales<0>(la, ts0);    // 4 reads (ts1 of this block arrived long ago)
-            load_mats(la, mt);              // 4 reads
-            load_row_scales(la, rs_next);   // 2 reads
-            tok_scales_ready<10>(ts1);  // issued at the end of the previous iteration, before the ten reads above
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (DUMP) dump_tile<TYPE>(a, d0, row, tokb + 32, g, nb, blk); else scale_tile(d0, rs.dw[0], ts1, acc[1][0]);
-            __builtin_amdgcn_sched_barrier(0);
-            mats_ready<0>(mt, rs_next);
-            tok_scales_ready<0>(ts0);
-            d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.av[0], mt.bv[0], cbias, 0, 0, 0);  // first tile of block b+1
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (DUMP) dump_tile<TYPE>(a, d1, row + 32, tokb + 32, g, nb, blk); else scale_tile(d1, rs.dw[1], ts1, acc[1][1]);
-            __builtin_amdgcn_sched_barrier(0);
-            load_tok_scales<1>(la, ts1);    // waited for by the next iteration's lgkmcnt(0)
-            rs = rs_next;
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const int tt = t >> 2, rt = t & 3;
+                if constexpr (DUMP) dump_tile<TYPE>(a, d[t & 3], row + 16 * rt, tok + 16 * tt, nb, blk);
+                else scale_tile(d[t & 3], sc.dw[rt], sc.dx[tt], acc[tt][rt]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (t < 4) {
+                    d[t & 3] = __builtin_amdgcn_mfma_i32_16x16x32_i8(mt.av[1], mt.bv[t], cbias, 0, 0, 0);
+                    if (t == 3) {
+                        load_mats(la, mt);           // all eight MFMAs of this block have been issued
+                        load_tok_scales<0>(la, sc);  // token tile 0 is done
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            load_tok_scales<1>(la, sc);
+            load_row_scales(la, sc);
         }
-        tok_scales_ready<0>(ts1);  // nothing of this stage's buffer is read past this point
+        lds_wait<0>(sc);  // nothing of this stage's buffer is read past this point
 
         // The other buffer was last read in stage st-1; every wave has passed the barrier
         // that ended that stage, so it is free to be refilled now.
@@ -422,13 +426,13 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_mfma_kernel(GemmArgs a) {
 
     if constexpr (!DUMP) {
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++)
+        for (int tt = 0; tt < TT; tt++)
 #pragma unroll
-            for (int rt = 0; rt < 2; rt++) {
-                const uint32_t row = row0 + wrow0 + rt * 32 + l32;
+            for (int rt = 0; rt < RT; rt++) {
+                const uint32_t row = row0 + wrow0 + 16 * rt + l16;
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const uint32_t tok = tok0 + wtok0 + tt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+                for (int r = 0; r < 4; r++) {
+                    const uint32_t tok = tok0 + wtok0 + 16 * tt + 4 * kq + r;
                     if (row < a.m && tok < a.n) {
                         float* dst = a.y_row_major ? a.y + (size_t)row * a.y_stride + tok : a.y + (size_t)tok * a.y_stride + row;
                         *dst = a.accumulate ? *dst + acc[tt][rt][r] : acc[tt][rt][r];
