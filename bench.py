@@ -300,6 +300,22 @@ def bench_lm_head_sweep(ctx, W, O, dtype=8, m=65536, k=2048, ns=(1, 4, 16, 64)):
     return {"dtype": dtype, "m": m, "k": k, "rows": rows, "first_n_where_mfma_wins": crossover, "library_hand_off_n": W.GEMM_MIN_N}
 
 
+def bench_probe(ctx, iters=20000):
+    """Register-only ceilings of this GPU for the GEMM's two bounds (no memory traffic)."""
+    out = {}
+    for shape, name, unit in [(0, "mfma_i32_32x32x32_i8", "TOP/s"), (1, "mfma_i32_16x16x32_i8", "TOP/s"), (2, "v_fma_f32", "TFLOP/s")]:
+        ctx.probe_rate(shape, iters)
+        ctx.sync()
+        e0, e1 = ctx.event(), ctx.event()
+        ctx.record(e0)
+        ops = ctx.probe_rate(shape, iters)
+        ctx.record(e1)
+        ms = ctx.elapsed_ms(e0, e1)
+        ctx.event_destroy(e0), ctx.event_destroy(e1)
+        out[name] = {"value": ops / ms / 1e9, "unit": unit, "ms": ms}
+    return out
+
+
 def bench_copy(ctx, nbytes=256 << 20, reps=10):
     """Device-to-device copy of a known size: calibration of the FETCH_SIZE / WRITE_SIZE counters."""
     a, b = ctx.alloc(nbytes), ctx.alloc(nbytes)
@@ -348,7 +364,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline decode step (+ CPU baseline)")
-    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | copy | cpu")
+    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | copy | probe | cpu")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -371,6 +387,7 @@ def main():
             "prefill_sites": lambda: bench_prefill_sites(ctx, W, O),
             "lm_head": lambda: bench_lm_head_sweep(ctx, W, O),
             "copy": lambda: bench_copy(ctx),
+            "probe": lambda: bench_probe(ctx),
         }
         if leg not in one:
             print(f"bench.py: unknown leg {leg}", file=sys.stderr)
@@ -426,9 +443,11 @@ def main():
         g = bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048)
         g["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma_kernel<Q4_0>", "achieved": g["gemm_kernel_TOPS"], "peak": INT8_PEAK_TOPS,
                          "unit": "TOP/s", "frac": g["gemm_kernel_TOPS"] / INT8_PEAK_TOPS,
-                         # 79.20 MB read + 55.35 MB written per launch (algorithmic 12.57 + 55.35 MB), profiles/gemm_q4_0_6912x2002x2048.txt
-                         "traffic": 134.6e6, "traffic_source": "profiles/gemm_q4_0_6912x2002x2048.txt"}
+                         # 88.97 MB read + 55.39 MB written per launch (algorithmic 12.57 + 55.35 MB), profiles/gemm_q4_0_6912x2002x2048.txt
+                         "traffic": 144.4e6, "traffic_source": "profiles/gemm_q4_0_6912x2002x2048.txt"}
         out["gemm"] = g
+        out["measured_ceilings"] = bench_probe(ctx)
+        g["roofline"]["frac_of_measured_mfma_ceiling"] = g["gemm_kernel_TOPS"] / out["measured_ceilings"]["mfma_i32_32x32x32_i8"]["value"]
         del host_weights  # the CPU leg regenerates what it needs; keep host memory low
         dq = bench_decode(ctx, W, O, W.Q8_0, max(10, args.steps // 2), args.warmup, synth_decode_weights(O, W.Q8_0), with_unfused=False)
         out["decode_step_q8_0"] = dq

@@ -88,6 +88,13 @@ int wick_rocm_buffer_free(wick_rocm_ctx *ctx, void *d_ptr);
 int wick_rocm_upload(wick_rocm_ctx *ctx, void *d_dst, const void *src, size_t nbytes);   /* H2D, ordered on the stream */
 int wick_rocm_download(wick_rocm_ctx *ctx, void *dst, const void *d_src, size_t nbytes); /* D2H, waits for the stream */
 int wick_rocm_sync(wick_rocm_ctx *ctx);
+/* Measurement aid with no counterpart in the reference: enqueues a register-only kernel that
+ * does nothing but issue one instruction (shape 0 = v_mfma_i32_32x32x32_i8, 1 =
+ * v_mfma_i32_16x16x32_i8, 2 = v_fma_f32) `iters` x 4 times per wave on every SIMD, and returns
+ * the number of operations it performs (int8 ops / flops).  Timed by the caller (events or
+ * kernel timing, family 3), it gives this GPU's own ceiling for the prefill GEMM's two bounds. */
+int wick_rocm_probe_rate(wick_rocm_ctx *ctx, int shape, uint32_t iters, double *ops);
+
 /* Device-to-device copy enqueued on the context's stream (the counterpart of a Metal
  * blit between the reference's scratch buffers). */
 int wick_rocm_copy(wick_rocm_ctx *ctx, void *d_dst, const void *d_src, size_t nbytes);

@@ -155,3 +155,16 @@ def test_cpp_host_mirror_selftest():
     assert os.path.exists(exe), "host_selftest has not been built (make -C wick_amd/csrc)"
     out = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     assert out.returncode == 0 and "selftest OK" in out.stdout, out.stdout + out.stderr
+
+
+def test_rate_probes(ctx):
+    """The register-only instruction-rate probes launch, report their operation counts and
+    reject bad arguments (they are measurement aids; nothing is checked about their speed)."""
+    for shape, per_iter in [(0, 4 * 65536.0), (1, 4 * 16384.0), (2, 4 * 4 * 64 * 2.0)]:
+        ops = ctx.probe_rate(shape, 10)
+        assert ops > 0 and ops % (per_iter * 10) == 0
+    ctx.sync()
+    with pytest.raises(W.RocmError):
+        ctx.probe_rate(3, 10)
+    with pytest.raises(W.RocmError):
+        ctx.probe_rate(0, 0)

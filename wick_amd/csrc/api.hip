@@ -32,6 +32,7 @@ struct wick_rocm_ctx {
     uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
     KernelTimer timer;
     int64_t gemv_direct_max_bytes = -1;
+    void* probe_sink = nullptr;  // 64 bytes the rate probes may (never do) write to
     Launch launch() { return Launch{stream, &timer, gemv_direct_max_bytes}; }
 };
 
@@ -182,6 +183,7 @@ void wick_rocm_ctx_destroy(wick_rocm_ctx* ctx) {
         }
         if (ctx->scratch_q) (void)hipFree(ctx->scratch_q);
         if (ctx->scratch_s) (void)hipFree(ctx->scratch_s);
+        if (ctx->probe_sink) (void)hipFree(ctx->probe_sink);
         for (auto* v : {&ctx->timer.recs, &ctx->timer.spares})
             for (KernelTimer::Rec& r : *v) {
                 (void)hipEventDestroy(r.start);
@@ -252,6 +254,17 @@ int wick_rocm_copy(wick_rocm_ctx* ctx, void* d_dst, const void* d_src, size_t nb
     if (nbytes == 0) return WICK_ROCM_OK;
     if (!d_dst || !d_src) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "copy: null pointer");
     WR_HIP(ctx, hipMemcpyAsync(d_dst, d_src, nbytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_probe_rate(wick_rocm_ctx* ctx, int shape, uint32_t iters, double* ops) {
+    WR_ENTER(ctx);
+    if (!ops || shape < 0 || shape > 2 || iters == 0) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "probe_rate: shape must be 0..2, iters > 0");
+    if (!ctx->probe_sink) {
+        if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "probe_rate: first call must be outside graph capture");
+        WR_HIP(ctx, hipMalloc(&ctx->probe_sink, 64));
+    }
+    WR_HIP(ctx, launch_probe(shape, iters, ctx->num_cus, reinterpret_cast<int*>(ctx->probe_sink), ops, ctx->launch()));
     return WICK_ROCM_OK;
 }
 

@@ -101,6 +101,10 @@ hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k
 
 // Per-block i32 dots, out[(j*m + i)*nb + b], through the same unpack + v_dot4 code
 // as the GEMV, or through the GEMM's loads / LDS layout / MFMA (k % 256 == 0).
+// Register-only instruction-rate probes (probe.hip): shape 0 = v_mfma_i32_32x32x32_i8, 1 = v_mfma_i32_16x16x32_i8,
+// 2 = v_fma_f32.
+hipError_t launch_probe(int shape, uint32_t iters, int num_cus, int* d_sink, double* ops, const Launch& L);
+
 hipError_t launch_block_dots_dot4(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,
                                   int32_t* d_out, const Launch& L);
 hipError_t launch_block_dots_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,

@@ -73,6 +73,7 @@ _SIGNATURES = {
     "wick_rocm_copy": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_set_gemm_min_n": (C.c_int, [_P, C.c_uint32]),
     "wick_rocm_set_gemv_policy": (C.c_int, [_P, C.c_int64]),
+    "wick_rocm_probe_rate": (C.c_int, [_P, C.c_int, C.c_uint32, C.POINTER(C.c_double)]),
     "wick_rocm_weight_upload": (C.c_int, [_P, _P, C.c_size_t, C.c_int, C.c_uint32, C.c_uint32, C.POINTER(_P)]),
     "wick_rocm_weight_free": (C.c_int, [_P, _P]),
     "wick_rocm_weight_info": (C.c_int, [_P, C.POINTER(C.c_int), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_size_t)]),
@@ -215,6 +216,12 @@ class RocmContext:
 
     def copy(self, dst, src, nbytes: int) -> None:
         self._check(self._lib.wick_rocm_copy(self._h, _ptr(dst), _ptr(src), nbytes))
+
+    def probe_rate(self, shape: int, iters: int) -> float:
+        """Enqueues a register-only instruction-rate probe; returns the operations it performs."""
+        ops = C.c_double()
+        self._check(self._lib.wick_rocm_probe_rate(self._h, shape, iters, C.byref(ops)))
+        return ops.value
 
     def set_gemv_policy(self, direct_max_bytes: int = -1) -> None:
         """Weight-fetch threshold of the n = 1 GEMV (negative = default); results do not depend on it."""
