@@ -68,15 +68,25 @@ constexpr int kFusedMaxK = 8192;
 //              slot and LDS operations of a wave execute in order, so no barrier is involved.
 enum { kDirect = 0, kDirectNT = 1, kSpan = 2 };
 
+// The leading scalar parameters repeat fields of `a` (x = a.xf for the fused variant, a.xq
+// otherwise; w0 / y0 / rows0 = weight 0 of the batch).  Passed on their own, at the front,
+// they are the kernel arguments the hardware preloads into SGPRs at wave launch (the build
+// asks for that, -amdgpu-kernarg-preload-count): everything needed to issue the activation
+// and weight loads of a single-weight launch is there at the first instruction, instead of
+// after one or two scalar-load round trips (~0.15 us each, on the critical path of a
+// 2-3 us launch).  The rest of `a` is still fetched the ordinary way, under those loads.
 template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI, int MODE>
-__global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kernel(GemvArgs a) {
+__global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kernel(const void* p_x, const uint8_t* p_w0, float* p_y0,
+                                                                                  uint32_t p_k, uint32_t p_rows0,
+                                                                                  uint32_t p_rows_per_wave, uint32_t p_total_waves,
+                                                                                  int p_accumulate, GemvArgs a) {
     using PT = PairTraits<TYPE>;
     constexpr int RPW = 64 / LPR;  // rows per wave pass
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t sub = lane % LPR;
     const uint32_t rsel = lane / LPR;
-    const uint32_t ppr = a.k >> 6;  // pairs per row
-    const uint32_t nb = a.k >> 5;
+    const uint32_t ppr = p_k >> 6;  // pairs per row
+    const uint32_t nb = p_k >> 5;
     const uint32_t tok0 = blockIdx.y * NT;
 
     const uint32_t gwave =
@@ -86,11 +96,11 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     constexpr int kQuadRounds = kFusedMaxK / 4 / (64 * kFusedWaves);  // 8
     float4 xv[FUSEQ ? kQuadRounds : 1];
     if constexpr (FUSEQ) {
-        const uint32_t quads = a.k >> 2;
+        const uint32_t quads = p_k >> 2;
 #pragma unroll
         for (int i = 0; i < kQuadRounds; i++) {
             const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
-            xv[i] = reinterpret_cast<const float4*>(a.xf)[min(quad, quads - 1)];  // clamped, unconditional
+            xv[i] = reinterpret_cast<const float4*>(p_x)[min(quad, quads - 1)];  // clamped, unconditional
         }
         // keep the compiler from moving the weight loads in front of these
         asm volatile("" ::: "memory");
@@ -103,9 +113,9 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     // them a second, dependent round trip) and then picked with scalar selects.
     // wave_end[] entries past the batch are UINT32_MAX (set_wave_ends).
     uint32_t widx = 0;
-    const uint8_t* wbase = a.batch.w[0];
-    float* ybase = a.batch.y[0];
-    uint32_t row_hi = a.batch.row_end[0], row_lo = 0, wave_lo = 0;
+    const uint8_t* wbase = p_w0;
+    float* ybase = p_y0;
+    uint32_t row_hi = p_rows0, row_lo = 0, wave_lo = 0;
     if constexpr (MULTI) {
         uint64_t w0 = (uint64_t)a.batch.w[0], w1 = (uint64_t)a.batch.w[1], w2 = (uint64_t)a.batch.w[2], w3 = (uint64_t)a.batch.w[3];
         uint64_t y0 = (uint64_t)a.batch.y[0], y1 = (uint64_t)a.batch.y[1], y2 = (uint64_t)a.batch.y[2], y3 = (uint64_t)a.batch.y[3];
@@ -115,7 +125,7 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
         asm(""
             : "+s"(w0), "+s"(w1), "+s"(w2), "+s"(w3), "+s"(y0), "+s"(y1), "+s"(y2), "+s"(y3), "+s"(r0), "+s"(r1), "+s"(r2),
               "+s"(r3), "+s"(e0), "+s"(e1), "+s"(e2), "+s"(cnt)
-            : "s"(a.xq), "s"(a.xs), "s"(a.total_waves), "s"(a.accumulate), "s"(a.rows_per_wave));
+            : "s"(a.xs));
         widx = min((uint32_t)(gwave >= e0) + (uint32_t)(gwave >= e1) + (uint32_t)(gwave >= e2), cnt - 1u);
         // Masks instead of ?: -- the compiler turns a chain of scalar selects into a chain of
         // branches, and a taken scalar branch costs more than all of this arithmetic.
@@ -133,9 +143,9 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     const uint32_t wave = gwave - wave_lo;
     // Waves past the end of the batch (last workgroup of a fused launch) get an empty row
     // range but still take part in the cooperative quantization and its barrier.
-    const bool live_wave = gwave < a.total_waves;
-    const uint32_t wave_row0 = live_wave ? wave * a.rows_per_wave : 0;
-    const uint32_t wave_row1 = live_wave ? min(wave_row0 + a.rows_per_wave, rows) : 0;
+    const bool live_wave = gwave < p_total_waves;
+    const uint32_t wave_row0 = live_wave ? wave * p_rows_per_wave : 0;
+    const uint32_t wave_row1 = live_wave ? min(wave_row0 + p_rows_per_wave, rows) : 0;
 
     bool pvalid[NCHUNK];
 #pragma unroll
@@ -223,7 +233,7 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     // into LDS (eight lanes per 32-element block, exactly like the stand-alone quantizer
     // kernel), instead of every wave redoing it.  Only n = 1 uses this variant.
     if constexpr (FUSEQ) {
-        const uint32_t quads = a.k >> 2;
+        const uint32_t quads = p_k >> 2;
 #pragma unroll
         for (int i = 0; i < kQuadRounds; i++) {
             const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
@@ -266,7 +276,7 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
                     act[c].s[t][h] = ok ? fs[2 * pp + h] : 0.0f;
                 }
             } else {
-                const uint4* src = reinterpret_cast<const uint4*>(a.xq + (size_t)tok * a.k + (size_t)pp * 64);
+                const uint4* src = reinterpret_cast<const uint4*>(static_cast<const int8_t*>(p_x) + (size_t)tok * p_k + (size_t)pp * 64);
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
                     uint4 lo = src[2 * h], hi = src[2 * h + 1];
@@ -309,7 +319,7 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
                 if (sub == 0 && rvalid[u] && tok0 + t < a.n) {
                     float* dst = a.y_row_major ? ybase + (size_t)lrow[u] * a.y_stride + (tok0 + t)
                                                : ybase + (size_t)(tok0 + t) * a.y_stride + lrow[u];
-                    *dst = a.accumulate ? *dst + tot : tot;
+                    *dst = p_accumulate ? *dst + tot : tot;
                 }
             }
         }
@@ -418,18 +428,19 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
     const uint64_t direct_max = L.gemv_direct_max_bytes >= 0 ? (uint64_t)L.gemv_direct_max_bytes : (TYPE == 2 ? kDirectMaxBytesQ4 : kDirectMaxBytesQ8);
     const int mode = NT > 1 ? kDirect : (bytes < direct_max ? kSmall : kSpan);
     const bool multi = a.batch.count > 1;
+    // hot scalars first (preloaded into SGPRs), then the whole argument block
+    auto go = [&](auto kernel) {
+        return launch_kernel(L, kFamGemv, kernel, grid, block, FUSEQ ? static_cast<const void*>(a.xf) : static_cast<const void*>(a.xq),
+                             a.batch.w[0], a.batch.y[0], a.k, a.batch.row_end[0], a.rows_per_wave, a.total_waves, a.accumulate, a);
+    };
     if constexpr (NT == 1) {
-        if (mode == kSpan && multi)
-            return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSpan>, grid, block, a);
-        if (mode == kSpan)
-            return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan>, grid, block, a);
-        if (multi)
-            return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSmall>, grid, block, a);
-        return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall>, grid, block, a);
+        if (mode == kSpan && multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSpan>);
+        if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan>);
+        if (multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSmall>);
+        return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall>);
     } else {
-        if (multi)
-            return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kDirect>, grid, block, a);
-        return launch_kernel(L, kFamGemv, gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kDirect>, grid, block, a);
+        if (multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kDirect>);
+        return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kDirect>);
     }
 }
 
