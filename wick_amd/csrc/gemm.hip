@@ -60,6 +60,7 @@ namespace {
 
 constexpr int BM = 128;       // weight rows per workgroup
 constexpr int BN = 128;       // tokens per workgroup
+constexpr int BN_NARROW = 64;  // ... of the narrow kernel (n <= 64)
 constexpr int KB = 4;         // blocks per stage
 constexpr int THREADS = 512;  // 8 waves: 2 (rows) x 4 (tokens)
 constexpr int TT = 2;          // 16-token MFMA tiles per wave
@@ -87,16 +88,20 @@ struct GemmArgs {
 // plane, two float2 per scale row) so that the stage WRITES, where neighbouring
 // lanes hit different planes of the same row, spread over the LDS banks; reads
 // walk consecutive rows of one plane.
-struct Stage {
+template <int NTOK>  // tokens per workgroup tile: BN, or BN_NARROW for the narrow kernel
+struct StageT {
     uint4 wt[2][KB][BM + 2];    // [khalf][block][row]  int8 weights (Q4_0: x16)
-    uint4 xt[BN][2 * KB];       // [token][16-byte K-chunk, swizzled] int8 activations, see dma_activations
+    uint4 xt[NTOK][2 * KB];     // [token][16-byte K-chunk, swizzled] int8 activations, see dma_activations
     float2 dws[KB][BM + 2];     // {dw, -12582912*dw} per block and row (dw x 1/16 for Q4_0)
-    float dxf[KB][BN];          // token scales
+    float dxf[KB][NTOK];        // token scales
 };
+using Stage = StageT<BN>;
 
-struct Smem {
-    Stage st[2];
+template <int NTOK>
+struct SmemT {
+    StageT<NTOK> st[2];
 };
+using Smem = SmemT<BN>;
 
 // 16*(nibble-8) for the four low / four high nibbles of each byte of q.
 __device__ __forceinline__ uint32_t q4_lo_x16(uint32_t q) { return ((q << 4) & 0xf0f0f0f0u) ^ 0x80808080u; }
@@ -120,25 +125,27 @@ struct StageRegs {
 // tokens reading one chunk then spread over all banks.  16 instructions per stage, two
 // per wave.
 __device__ __forceinline__ uint32_t xt_swizzle(uint32_t token_in_tile) { return (token_in_tile >> 1) & 7u; }
-__device__ __forceinline__ void dma_activations(const GemmArgs& a, Stage& s, uint32_t tok0, uint32_t kb0) {
+template <int NTOK>
+__device__ __forceinline__ void dma_activations(const GemmArgs& a, StageT<NTOK>& s, uint32_t tok0, uint32_t kb0) {
+    constexpr int PER_WAVE = NTOK / 8 / (THREADS / 64);  // instructions per wave and stage
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const uint32_t t = 8u * (2u * wave + j) + (lane >> 3);  // token within the tile
+    for (int j = 0; j < PER_WAVE; j++) {
+        const uint32_t t = 8u * (PER_WAVE * wave + j) + (lane >> 3);  // token within the tile
         const uint32_t chunk = (lane & 7u) ^ xt_swizzle(t);
         const uint32_t tok = min(tok0 + t, a.n - 1);
         const int8_t* src = a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + 16u * chunk;
         __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
-                                         (void __attribute__((address_space(3)))*)&s.xt[8u * (2u * wave + j)][0], 16, 0, 0);
+                                         (void __attribute__((address_space(3)))*)&s.xt[8u * (PER_WAVE * wave + j)][0], 16, 0, 0);
     }
 }
 
 // Thread -> work of one stage:
 //   weights      256 pairs   = 128 rows x 2 pairs             : threads 0..255, row = t >> 1, pair = t & 1
 //   activations  direct-to-LDS, see dma_activations
-//   token scales 128 tokens x 4 blocks (one float4)           : threads 256..383, token = t - 256
-template <int TYPE>
+//   token scales one float4 (4 blocks) per token               : threads 256..256+NTOK-1, token = t - 256
+template <int TYPE, int NTOK>
 __device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uint32_t tok0, uint32_t kb0,
                                            StageRegs<TYPE>& r) {
     using PT = PairTraits<TYPE>;
@@ -148,7 +155,7 @@ __device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uin
         const uint32_t row = min(row0 + (t >> 1), a.m - 1);
         const uint8_t* p = a.w + ((size_t)row * nb + kb0 + 2 * (t & 1u)) * (PT::BYTES / 2);
         load_pair<PT::DWORDS>(p, r.w);
-    } else if (t < 2 * BM + BN && a.xs) {  // xs is null only for the parity hook, which never scales
+    } else if (t < 2 * BM + NTOK && a.xs) {  // xs is null only for the parity hook, which never scales
         const uint32_t tok = min(tok0 + (t - 2 * BM), a.n - 1);
         r.dx = *reinterpret_cast<const float4*>(a.xs + (size_t)tok * nb + kb0);
     } else {
@@ -156,8 +163,8 @@ __device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uin
     }
 }
 
-template <int TYPE>
-__device__ __forceinline__ void store_stage(Stage& s, const StageRegs<TYPE>& r) {
+template <int TYPE, int NTOK>
+__device__ __forceinline__ void store_stage(StageT<NTOK>& s, const StageRegs<TYPE>& r) {
     using PT = PairTraits<TYPE>;
     const uint32_t t = threadIdx.x;
     if (t < 2 * BM) {
@@ -181,7 +188,7 @@ __device__ __forceinline__ void store_stage(Stage& s, const StageRegs<TYPE>& r) 
             s.wt[1][b0 + 1][row] = make_uint4(q1[4], q1[5], q1[6], q1[7]);
         }
     }
-    if (t >= 2 * BM && t < 2 * BM + BN) {
+    if (t >= 2 * BM && t < 2 * BM + NTOK) {
         const uint32_t u = t - 2 * BM;
         s.dxf[0][u] = r.dx.x;
         s.dxf[1][u] = r.dx.y;
@@ -353,8 +360,8 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
 
     StageRegs<TYPE> regs;
     dma_activations(a, sm.st[0], tok0, 0);
-    load_stage<TYPE>(a, row0, tok0, 0, regs);
-    store_stage<TYPE>(sm.st[0], regs);
+    load_stage<TYPE, BN>(a, row0, tok0, 0, regs);
+    store_stage<TYPE, BN>(sm.st[0], regs);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
     __syncthreads();
 
@@ -364,7 +371,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
             // the other LDS stage was last read in stage st-1 and every wave has passed the
             // barrier that ended it, so it can be refilled from here on
             dma_activations(a, sm.st[(st + 1) & 1u], tok0, (st + 1) * KB);
-            load_stage<TYPE>(a, row0, tok0, (st + 1) * KB, regs);
+            load_stage<TYPE, BN>(a, row0, tok0, (st + 1) * KB, regs);
         }
 
         // 8 MFMA tiles per block, software-pipelined by hand: four result buffers, the matrix
@@ -419,7 +426,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
 
         // The other buffer was last read in stage st-1; every wave has passed the barrier
         // that ended that stage, so it is free to be refilled now.
-        if (st + 1 < stages) store_stage<TYPE>(sm.st[(st + 1) & 1u], regs);
+        if (st + 1 < stages) store_stage<TYPE, BN>(sm.st[(st + 1) & 1u], regs);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS copies of the next stage have landed
         __syncthreads();
     }
@@ -442,13 +449,154 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Narrow variant for 16 <= n <= 64 (an LM head or a projection over a short prompt): tile =
+// 128 weight rows x 64 tokens, every one of the 8 waves owns 16 rows x all 64 tokens (one
+// row tile x four token tiles), so no matrix or scaling work is spent on token columns that
+// do not exist beyond the 64, and the weights -- the only large operand -- are streamed
+// exactly once.  Same staging, LDS layouts and arithmetic as the wide kernel; 60 KB of LDS,
+// two workgroups per CU.
+struct NarrowMats {
+    long av[4], bv;
+};
+struct NarrowScales {
+    float2 dw;
+    v4f dx[4];
+};
+constexpr int kOffDxfNarrow = sizeof(float) * BN_NARROW;
+__device__ __forceinline__ void load_mats(const LaneAddr& la, NarrowMats& m) {  // 5 reads
+    lds_read8<0 * 16 * 128>(la.xt, m.av[0]);
+    lds_read8<1 * 16 * 128>(la.xt, m.av[1]);
+    lds_read8<2 * 16 * 128>(la.xt, m.av[2]);
+    lds_read8<3 * 16 * 128>(la.xt, m.av[3]);
+    lds_read8<0>(la.wt, m.bv);
+}
+__device__ __forceinline__ void load_scales(const LaneAddr& la, NarrowScales& s) {  // 5 reads
+    lds_read8<0>(la.dws, s.dw);
+    lds_read16<0 * 64>(la.dxf, s.dx[0]);
+    lds_read16<1 * 64>(la.dxf, s.dx[1]);
+    lds_read16<2 * 64>(la.dxf, s.dx[2]);
+    lds_read16<3 * 64>(la.dxf, s.dx[3]);
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(NarrowMats& m) {
+    asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(m.av[0]), "+v"(m.av[1]), "+v"(m.av[2]), "+v"(m.av[3]), "+v"(m.bv) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(NarrowScales& s) {
+    asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(s.dw), "+v"(s.dx[0]), "+v"(s.dx[1]), "+v"(s.dx[2]), "+v"(s.dx[3]) : "n"(N) : "memory");
+}
+
+template <int TYPE, bool DUMP>
+__global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
+    __shared__ SmemT<BN_NARROW> sm;
+    uint32_t row_tile, tok_tile;
+    bool valid_tile;
+    tile_of_block(blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
+    if (!valid_tile) return;  // whole workgroup leaves together
+    const uint32_t row0 = row_tile * BM;
+    const uint32_t tok0 = tok_tile * BN_NARROW;
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t l16 = lane & 15u;
+    const uint32_t kq = lane >> 4;      // which 8-byte quarter of the block this lane feeds
+    const uint32_t wrow0 = wave * 16;   // wave's rows within the tile
+    const uint32_t nb = a.k >> 5;
+    const uint32_t stages = nb / KB;
+
+    float acc[4][4];
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[tt][r] = 0.0f;
+
+    v4i cbias = {(int)kBiasBits, (int)kBiasBits, (int)kBiasBits, (int)kBiasBits};
+    asm volatile("" : "+v"(cbias));
+
+    StageRegs<TYPE> regs;
+    dma_activations(a, sm.st[0], tok0, 0);
+    load_stage<TYPE, BN_NARROW>(a, row0, tok0, 0, regs);
+    store_stage<TYPE, BN_NARROW>(sm.st[0], regs);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
+    __syncthreads();
+
+    for (uint32_t st = 0; st < stages; st++) {
+        const StageT<BN_NARROW>& s = sm.st[st & 1u];
+        if (st + 1 < stages) {
+            dma_activations(a, sm.st[(st + 1) & 1u], tok0, (st + 1) * KB);
+            load_stage<TYPE, BN_NARROW>(a, row0, tok0, (st + 1) * KB, regs);
+        }
+
+        LaneAddr la;  // block 0 of this stage's buffer
+        la.xsh = xt_swizzle(l16) >> 1;
+        la.xbase = lds_addr(&s.xt[l16][0]) + ((((kq >> 1) ^ xt_swizzle(l16)) & 1u) << 4) + 8 * (kq & 1u);
+        la.xt = la.xbase + (la.xsh << 5);
+        la.wt = lds_addr(&s.wt[kq >> 1][0][wrow0 + l16]) + 8 * (kq & 1u);
+        la.dws = lds_addr(&s.dws[0][wrow0 + l16]);
+        la.dxf = lds_addr(&s.dxf[0][4 * kq]);
+        NarrowMats mt;
+        NarrowScales sc;
+        load_mats(la, mt);    // 5 reads
+        load_scales(la, sc);  // 5 reads
+#pragma unroll 1
+        for (int b = 0; b < KB; b++) {
+            // addresses of block b+1 (last iteration: harmless re-read of its own block)
+            const bool adv = b + 1 < KB;
+            la.xt = la.xbase + ((((uint32_t)(adv ? b + 1 : b)) ^ la.xsh) << 5);
+            la.wt += adv ? kOffWt : 0;
+            la.dws += adv ? kOffDws : 0;
+            la.dxf += adv ? kOffDxfNarrow : 0;
+            const uint32_t row = row0 + wrow0 + l16, tok = tok0 + 4 * kq, blk = st * KB + b;
+            v4i d[4];
+            lds_wait<5>(mt);  // the five scale reads issued after the matrices may still be in flight
+#pragma unroll
+            for (int tt = 0; tt < 4; tt++) d[tt] = __builtin_amdgcn_mfma_i32_16x16x32_i8(mt.av[tt], mt.bv, cbias, 0, 0, 0);
+            load_mats(la, mt);  // in place: the MFMAs that read block b's operands have been issued
+            lds_wait<5>(sc);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int tt = 0; tt < 4; tt++) {
+                if constexpr (DUMP) dump_tile<TYPE>(a, d[tt], row, tok + 16 * tt, nb, blk);
+                else scale_tile(d[tt], sc.dw, sc.dx[tt], acc[tt]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            load_scales(la, sc);
+        }
+        lds_wait<0>(sc);  // nothing of this stage's buffer is read past this point
+
+        if (st + 1 < stages) store_stage<TYPE, BN_NARROW>(sm.st[(st + 1) & 1u], regs);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS copies of the next stage have landed
+        __syncthreads();
+    }
+
+    if constexpr (!DUMP) {
+        const uint32_t row = row0 + wrow0 + l16;
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t tok = tok0 + 16 * tt + 4 * kq + r;
+                if (row < a.m && tok < a.n) {
+                    float* dst = a.y_row_major ? a.y + (size_t)row * a.y_stride + tok : a.y + (size_t)tok * a.y_stride + row;
+                    *dst = a.accumulate ? *dst + acc[tt][r] : acc[tt][r];
+                }
+            }
+    }
+}
+
 template <bool DUMP>
 hipError_t launch(int type, GemmArgs& a, const Launch& L) {
     if (a.m == 0 || a.n == 0) return hipSuccess;
     a.row_tiles = (a.m + BM - 1) / BM;
-    a.tok_tiles = (a.n + BN - 1) / BN;
+    const bool narrow = a.n <= BN_NARROW;
+    a.tok_tiles = narrow ? 1 : (a.n + BN - 1) / BN;
     const uint32_t tiles = a.row_tiles * a.tok_tiles;
     const uint32_t blocks = ((tiles + 7u) / 8u) * 8u;  // every XCD gets the same number of slots
+    if (narrow) {
+        if (type == kTypeQ4_0) return launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
+        return launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
+    }
     if (type == kTypeQ4_0)
         return launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
     return launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
