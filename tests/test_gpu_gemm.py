@@ -18,6 +18,7 @@ SHAPES = [
     (64, 2, 256), (100, 15, 512),                                                # multi-token GEMV
     (128, 16, 256), (128, 128, 256), (1, 16, 256), (130, 129, 512), (200, 50, 512), (256, 300, 1024),
     (512, 100, 2048), (1000, 257, 4608), (300, 64, 6912),                        # MFMA, ragged tiles
+    (129, 17, 128), (16, 33, 256), (250, 63, 384), (131, 64, 1024), (257, 65, 512),  # narrow kernel (n <= 64) and its hand-off
 ]
 
 
