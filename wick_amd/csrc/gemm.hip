@@ -589,8 +589,10 @@ template <bool DUMP>
 hipError_t launch(int type, GemmArgs& a, const Launch& L) {
     if (a.m == 0 || a.n == 0) return hipSuccess;
     a.row_tiles = (a.m + BM - 1) / BM;
-    const bool narrow = a.n <= BN_NARROW;
-    a.tok_tiles = narrow ? 1 : (a.n + BN - 1) / BN;
+    // The narrow tile also serves small problems that would leave more than half of the
+    // 512 resident workgroup slots (2 per CU) empty with the wide tile: twice the tiles.
+    const bool narrow = a.n <= BN_NARROW || a.row_tiles * ((a.n + BN - 1) / BN) <= 256;
+    a.tok_tiles = narrow ? (a.n + BN_NARROW - 1) / BN_NARROW : (a.n + BN - 1) / BN;
     const uint32_t tiles = a.row_tiles * a.tok_tiles;
     const uint32_t blocks = ((tiles + 7u) / 8u) * 8u;  // every XCD gets the same number of slots
     if (narrow) {
