@@ -100,7 +100,10 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
 #pragma unroll
         for (int i = 0; i < kQuadRounds; i++) {
             const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
-            xv[i] = reinterpret_cast<const float4*>(p_x)[min(quad, quads - 1)];  // clamped, unconditional
+            // whole rounds past the end of the vector are skipped (uniform, one taken branch);
+            // within a round: clamped
+            if (i > 0 && i * 64 * kFusedWaves >= quads) break;
+            xv[i] = reinterpret_cast<const float4*>(p_x)[min(quad, quads - 1)];
         }
         // keep the compiler from moving the weight loads in front of these
         asm volatile("" ::: "memory");
