@@ -46,7 +46,8 @@ BW = {2: 18, 8: 34}
 def gemv_bytes(dtype: int, m: int, k: int, n: int = 1) -> int:
     """Algorithmic bytes of one GEMV: weights once + Q8_0 activations (34 B / block) + f32 output."""
     nb = k // 32
-    return m * nb * BW[dtype] + nb * 34 * n + 4 * m * n
+    wbytes = m * (k // 256) * 210 if dtype == 14 else m * nb * BW[dtype]  # 14 = Q6_K
+    return wbytes + nb * 34 * n + 4 * m * n
 
 
 def quant_bytes(n: int, k: int) -> int:
@@ -386,6 +387,7 @@ def main():
             "gemm": lambda: bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048),
             "prefill_sites": lambda: bench_prefill_sites(ctx, W, O),
             "lm_head": lambda: bench_lm_head_sweep(ctx, W, O),
+            "lm_head_q6k": lambda: bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024),
             "copy": lambda: bench_copy(ctx),
             "probe": lambda: bench_probe(ctx),
         }
@@ -453,6 +455,8 @@ def main():
         out["decode_step_q8_0"] = dq
         out["prefill_sites"] = bench_prefill_sites(ctx, W, O)
         out["lm_head_sweep"] = bench_lm_head_sweep(ctx, W, O)
+        # shipped LFM2 Q4_0 files keep the tied embedding / LM head in Q6_K (wick/src/model/metal_lfm2.rs:175-180)
+        out["lm_head_q6_k_65536x1024"] = bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024)
         host_weights = None
     ctx.close()
     if not args.skip_cpu:

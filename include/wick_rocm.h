@@ -23,6 +23,11 @@
  *   - Weight bytes keep the GGUF block layout verbatim (wick/src/quant.rs:13-34):
  *     row-major, m rows of k/32 blocks; Q4_0 block = {f16 d; u8 qs[16]} (18 B),
  *     Q8_0 block = {f16 d; i8 qs[32]} (34 B).  Nothing is repacked.
+ *   - Q6_K weights (wick/src/quant.rs:54-70: {u8 ql[128]; u8 qh[64]; i8 scales[16];
+ *     f16 d}, 210 B per 256 weights, k % 256 == 0, k <= 8192) take the decode path
+ *     only: the integer Q6_K x Q8_0 GEMV of wick/src/backend/simd.rs:547-640
+ *     (one f32 scale product per 16-weight group).  Batched calls run that GEMV once
+ *     per token; their quants must be 16-byte aligned.
  *   - Quantized activations use the reference's split layout
  *     (wick/src/kv_cache.rs:103-106, wick/src/backend/simd.rs:683-685):
  *     scales f32 [n][k/32] (values are f16-representable), quants i8 [n][k].
@@ -40,15 +45,15 @@ extern "C" {
 typedef enum wick_rocm_status {
     WICK_ROCM_OK = 0,
     WICK_ROCM_ERR_INVALID_ARG = -1, /* null pointer, zero size, bad stride or alignment */
-    WICK_ROCM_ERR_UNSUPPORTED_DTYPE = -2, /* ggml type other than Q4_0 (2) / Q8_0 (8) */
-    WICK_ROCM_ERR_BAD_SHAPE = -3,   /* k % 32 != 0, byte count != m * (k/32) * block bytes */
+    WICK_ROCM_ERR_UNSUPPORTED_DTYPE = -2, /* ggml type other than Q4_0 (2) / Q8_0 (8) / Q6_K (14) */
+    WICK_ROCM_ERR_BAD_SHAPE = -3,   /* k % 32 != 0 (Q6_K: k % 256, k > 8192), byte count != rows * row bytes */
     WICK_ROCM_ERR_HIP = -4,         /* a HIP runtime call failed (message has the HIP error) */
     WICK_ROCM_ERR_NO_DEVICE = -5,   /* no gfx950 device with that index */
     WICK_ROCM_ERR_STATE = -6        /* capture begun twice, graph launched while capturing, ... */
 } wick_rocm_status;
 
 /* ggml tensor type ids, wick/src/gguf.rs:36-51 */
-enum { WICK_ROCM_TYPE_Q4_0 = 2, WICK_ROCM_TYPE_Q8_0 = 8 };
+enum { WICK_ROCM_TYPE_Q4_0 = 2, WICK_ROCM_TYPE_Q8_0 = 8, WICK_ROCM_TYPE_Q6_K = 14 };
 
 /* Output layouts of the batched GEMM. */
 enum {
@@ -103,7 +108,7 @@ int wick_rocm_copy(wick_rocm_ctx *ctx, void *d_dst, const void *d_src, size_t nb
  * Stands in for MetalWeight {mmap_offset, dtype, m, k} (wick/src/model/metal_lfm2.rs:28-36,
  * 409-421).  A discrete GPU cannot wrap the GGUF mmap in place, so the block
  * bytes are copied once, verbatim, into HBM.  `nbytes` must equal
- * m * (k/32) * block_bytes(ggml_type).  The handle stays valid until
+ * m * (k/32) * block_bytes(ggml_type), for Q6_K m * (k/256) * 210.  The handle stays valid until
  * wick_rocm_weight_free or context destruction. */
 int wick_rocm_weight_upload(wick_rocm_ctx *ctx, const void *host_blocks, size_t nbytes, int ggml_type,
                             uint32_t m, uint32_t k, wick_rocm_weight **out);
@@ -187,7 +192,9 @@ int wick_rocm_reserve_scratch(wick_rocm_ctx *ctx, uint32_t max_n, uint32_t max_k
 
 /* ---- parity hook ----------------------------------------------------------
  * The exact per-block i32 dots the kernels scale and accumulate
- * (wick/src/backend/simd.rs:369-383, 478-492): d_out[(j*m + i)*(k/32) + b]. */
+ * (wick/src/backend/simd.rs:369-383, 478-492): d_out[(j*m + i)*(k/32) + b].
+ * For Q6_K weights: the i32 dot of every 16-weight group (wick/src/backend/simd.rs:583-630),
+ * d_out[(j*m + i)*(k/16) + g]. */
 int wick_rocm_block_dots_i32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_t *d_quants, uint32_t n,
                              int32_t *d_out);
 

@@ -53,6 +53,8 @@ def lib() -> C.CDLL:
         L.orc_f32_to_f16_bits.restype = C.c_uint16
         L.orc_f32_to_f16_bits.argtypes = [C.c_float]
         L.orc_quantize_q8_0.restype = C.c_int64
+        for f in ("orc_q6k_group_dots_i32", "orc_gemv_q6k_q8", "orc_gemv_q6k_q8_f64"):
+            getattr(L, f).restype = C.c_int
         for f in ("orc_block_dots_i32", "orc_gemv_q8", "orc_gemv_q8_f64", "orc_gemm_q8", "orc_gemm_q8_f64"):
             getattr(L, f).restype = C.c_int
         _lib = L
@@ -163,6 +165,47 @@ def build_matrix(ggml_type: int, values: np.ndarray, m: int, k: int) -> np.ndarr
     return out
 
 
+# ---- Q6_K (the LM head of shipped LFM2 Q4_0 files) ---------------------------
+
+Q6_K = 14
+Q6K_BLOCK_BYTES = 210
+
+
+def dequant_q6_k(a: np.ndarray, m: int, k: int) -> np.ndarray:
+    src = _c(a, np.uint8)
+    assert k % 256 == 0 and src.size == m * (k // 256) * Q6K_BLOCK_BYTES
+    dst = np.empty(m * k, np.float32)
+    lib().orc_dequant_q6_k_row(_p(src), C.c_int64(m * (k // 256)), _p(dst))
+    return dst.reshape(m, k)
+
+
+def q6k_group_dots_i32(a, quants, m: int, k: int) -> np.ndarray:
+    """Exact i32 dots of every 16-weight group with its activation quants, shape [m, k/16]."""
+    a = _c(a, np.uint8)
+    q = _c(quants, np.int8)
+    out = np.empty((m, k // 16), np.int32)
+    assert lib().orc_q6k_group_dots_i32(_p(a), _p(q), C.c_int64(m), C.c_int64(k), _p(out)) == 0
+    return out
+
+
+def gemv_q6k_q8(a, scales, quants, m: int, k: int, f64: bool = False) -> np.ndarray:
+    a = _c(a, np.uint8)
+    s = _c(scales, np.float32)
+    q = _c(quants, np.int8)
+    y = np.empty(m, np.float64 if f64 else np.float32)
+    fn = lib().orc_gemv_q6k_q8_f64 if f64 else lib().orc_gemv_q6k_q8
+    assert fn(_p(a), _p(s), _p(q), _p(y), C.c_int64(m), C.c_int64(k)) == 0
+    return y
+
+
+def build_q6_k(values: np.ndarray, m: int, k: int) -> np.ndarray:
+    v = _c(values, np.float32).ravel()
+    assert v.size == m * k and k % 256 == 0
+    out = np.empty(m * (k // 256) * Q6K_BLOCK_BYTES, np.uint8)
+    lib().orc_build_q6_k_matrix(_p(v), C.c_int64(m), C.c_int64(k), _p(out))
+    return out
+
+
 def fill_normal(seed: int, sigma: float, n: int) -> np.ndarray:
     out = np.empty(n, np.float32)
     lib().orc_fill_normal(C.c_uint64(seed), C.c_float(sigma), C.c_int64(n), _p(out))
@@ -171,6 +214,8 @@ def fill_normal(seed: int, sigma: float, n: int) -> np.ndarray:
 
 def synth_weight(ggml_type: int, m: int, k: int, seed: int, sigma: float = 0.02) -> np.ndarray:
     """Seeded N(0, sigma^2) weights quantized to raw GGUF blocks."""
+    if ggml_type == Q6_K:
+        return build_q6_k(fill_normal(seed, sigma, m * k), m, k)
     return build_matrix(ggml_type, fill_normal(seed, sigma, m * k), m, k)
 
 

@@ -23,6 +23,13 @@
  *                                               the reference's own shapes (simd.rs:1440-1623),
  *                                               Q8_0 closed form -16/(row+1) (bench_perf.rs:852-971)
  *   orc_build_q4_0_matrix / orc_build_q8_0_matrix   input generators only; numpy restatement
+ *   orc_dequant_q6_k_row                        the reference's closed-form block (all quants 32 -> 0,
+ *                                               quant.rs:819-846) + an independent numpy bit-twiddling
+ *                                               restatement of quant.rs:380-412 on random bytes
+ *   orc_q6k_group_dots_i32, orc_gemv_q6k_q8     python-integer brute force; f64 dequantize-then-dot;
+ *                                               the reference's varied block (quant.rs:849-880) dotted
+ *                                               both ways
+ *   orc_build_q6_k_matrix                       input generator only (round trip error bound)
  */
 #include <math.h>
 #include <stdint.h>
@@ -356,6 +363,146 @@ ORC_API void orc_build_q8_0_matrix(const float *values, int64_t m, int64_t k, ui
                 if (q < -128.0f) q = -128.0f;
                 if (q > 127.0f) q = 127.0f;
                 o[2 + i] = (uint8_t)(int8_t)q;
+            }
+        }
+}
+
+/* ------------------------------------------------------------------ Q6_K
+ * BlockQ6K (wick/src/quant.rs:60-70): 256 weights in 210 bytes
+ *   ql[128]  low 4 bits, qh[64]  high 2 bits, scales[16] int8 (one per 16 weights), d f16.
+ * Element e = 128 n + 32 j + l  (n < 2, j < 4, l < 32), from dequantize_q6_k_block
+ * (quant.rs:380-412):
+ *   q = ((ql[64 n + 32 (j & 1) + l] >> 4 (j >> 1)) & 15) | (((qh[32 n + l] >> 2 j) & 3) << 4)
+ *   w = f32(d) * scales[e / 16] * (q - 32)
+ * (the reference indexes scales as 8 n + l / 16 + 2 j, which is e / 16). */
+#define Q6K_BLOCK_BYTES 210
+#define Q6K_SUPER 256
+
+static inline int q6k_quant(const uint8_t *blk, int e) {
+    int n = e >> 7, j = (e >> 5) & 3, l = e & 31;
+    int lo = (blk[64 * n + 32 * (j & 1) + l] >> (4 * (j >> 1))) & 15;
+    int hi = (blk[128 + 32 * n + l] >> (2 * j)) & 3;
+    return (lo | (hi << 4)) - 32;
+}
+
+ORC_API void orc_dequant_q6_k_row(const uint8_t *src, int64_t n_blocks, float *dst) {
+    for (int64_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = src + b * Q6K_BLOCK_BYTES;
+        const int8_t *sc = (const int8_t *)(blk + 192);
+        float d = orc_f16_bits_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+        for (int e = 0; e < Q6K_SUPER; e++) {
+            /* d * sc * q, left to right, like quant.rs:400-403 */
+            volatile float ds = d * (float)sc[e >> 4];
+            dst[b * Q6K_SUPER + e] = ds * (float)q6k_quant(blk, e);
+        }
+    }
+}
+
+/* Exact i32 dot of every 16-weight group with its 16 activation quants:
+ * out[(i * (k/16)) + g]  (one token; what gemv_q6k_q8_0_neon feeds to vaddvq_s32). */
+ORC_API int orc_q6k_group_dots_i32(const uint8_t *a, const int8_t *xq, int64_t m, int64_t k, int32_t *out) {
+    if (k % Q6K_SUPER) return -1;
+    int64_t nbk = k / Q6K_SUPER;
+    for (int64_t i = 0; i < m; i++)
+        for (int64_t b = 0; b < nbk; b++) {
+            const uint8_t *blk = a + (i * nbk + b) * Q6K_BLOCK_BYTES;
+            for (int g = 0; g < 16; g++) {
+                int32_t s = 0;
+                for (int t = 0; t < 16; t++) s += q6k_quant(blk, 16 * g + t) * (int32_t)xq[b * Q6K_SUPER + 16 * g + t];
+                out[(i * nbk + b) * 16 + g] = s;
+            }
+        }
+    return 0;
+}
+
+/* gemv_q6k_q8_0_neon (wick/src/backend/simd.rs:552-679): per row one f32 accumulator;
+ * per block, passes n = 0, 1; halves h = 0, 1; then the four groups j = 0..3 of
+ * elements 128 n + 32 j + 16 h .. + 15:
+ *   dj   = (d * f32(scales[8 n + h + 2 j])) * xs[(256 b + 128 n + 32 j + 16 h) / 32]
+ *   sumf = sumf + dj * f32(idot)            (separate multiply and add) */
+ORC_API int orc_gemv_q6k_q8(const uint8_t *a, const float *x_scales, const int8_t *x_quants, float *y,
+                            int64_t m, int64_t k) {
+    if (k % Q6K_SUPER) return -1;
+    int64_t nbk = k / Q6K_SUPER;
+    for (int64_t i = 0; i < m; i++) {
+        volatile float sumf = 0.0f;
+        for (int64_t b = 0; b < nbk; b++) {
+            const uint8_t *blk = a + (i * nbk + b) * Q6K_BLOCK_BYTES;
+            const int8_t *sc = (const int8_t *)(blk + 192);
+            float d = orc_f16_bits_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+            for (int n = 0; n < 2; n++)
+                for (int h = 0; h < 2; h++)
+                    for (int j = 0; j < 4; j++) {
+                        int e0 = 128 * n + 32 * j + 16 * h;
+                        int32_t idot = 0;
+                        for (int t = 0; t < 16; t++) idot += q6k_quant(blk, e0 + t) * (int32_t)x_quants[b * Q6K_SUPER + e0 + t];
+                        volatile float ds = d * (float)sc[8 * n + h + 2 * j];
+                        volatile float dj = ds * x_scales[(b * Q6K_SUPER + e0) / 32];
+                        volatile float prod = dj * (float)idot;
+                        sumf = sumf + prod;
+                    }
+        }
+        y[i] = sumf;
+    }
+    return 0;
+}
+
+ORC_API int orc_gemv_q6k_q8_f64(const uint8_t *a, const float *x_scales, const int8_t *x_quants, double *y,
+                                int64_t m, int64_t k) {
+    if (k % Q6K_SUPER) return -1;
+    int64_t nbk = k / Q6K_SUPER;
+    for (int64_t i = 0; i < m; i++) {
+        double acc = 0.0;
+        for (int64_t b = 0; b < nbk; b++) {
+            const uint8_t *blk = a + (i * nbk + b) * Q6K_BLOCK_BYTES;
+            const int8_t *sc = (const int8_t *)(blk + 192);
+            double d = (double)orc_f16_bits_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+            for (int e = 0; e < Q6K_SUPER; e++)
+                acc += d * (double)sc[e >> 4] * (double)q6k_quant(blk, e) * (double)x_scales[(b * Q6K_SUPER + e) / 32] *
+                       (double)x_quants[b * Q6K_SUPER + e];
+        }
+        y[i] = acc;
+    }
+    return 0;
+}
+
+/* Input generator only (the reference has no Q6_K quantizer; real files come from
+ * llama.cpp): a plain round-to-nearest Q6_K encoder.  Per 16 weights s = amax / 31; the
+ * super-block scale d = max(s) / 127 (stored as f16); scales[g] = round(s_g / d);
+ * q = clamp(round(w / (d * scales[g])), -32, 31) + 32. */
+ORC_API void orc_build_q6_k_matrix(const float *values, int64_t m, int64_t k, uint8_t *bytes) {
+    int64_t nbk = k / Q6K_SUPER;
+    for (int64_t i = 0; i < m; i++)
+        for (int64_t b = 0; b < nbk; b++) {
+            const float *w = values + i * k + b * Q6K_SUPER;
+            uint8_t *blk = bytes + (i * nbk + b) * Q6K_BLOCK_BYTES;
+            memset(blk, 0, Q6K_BLOCK_BYTES);
+            float smax = 0.0f, s[16];
+            for (int g = 0; g < 16; g++) {
+                float amax = 0.0f;
+                for (int t = 0; t < 16; t++) amax = fmaxf(amax, fabsf(w[16 * g + t]));
+                s[g] = amax / 31.0f;
+                smax = fmaxf(smax, s[g]);
+            }
+            uint16_t dh = orc_f32_to_f16_bits(smax / 127.0f);
+            float d = orc_f16_bits_to_f32(dh);
+            blk[208] = (uint8_t)(dh & 0xff);
+            blk[209] = (uint8_t)(dh >> 8);
+            for (int g = 0; g < 16; g++) {
+                int sc = d > 0.0f ? (int)lrintf(s[g] / d) : 0;
+                if (sc > 127) sc = 127;
+                ((int8_t *)(blk + 192))[g] = (int8_t)sc;
+                float step = d * (float)sc;
+                for (int t = 0; t < 16; t++) {
+                    int e = 16 * g + t;
+                    int q = step > 0.0f ? (int)lrintf(w[e] / step) : 0;
+                    if (q < -32) q = -32;
+                    if (q > 31) q = 31;
+                    q += 32;
+                    int n = e >> 7, j = (e >> 5) & 3, l = e & 31;
+                    blk[64 * n + 32 * (j & 1) + l] |= (uint8_t)((q & 15) << (4 * (j >> 1)));
+                    blk[128 + 32 * n + l] |= (uint8_t)((q >> 4) << (2 * j));
+                }
             }
         }
 }

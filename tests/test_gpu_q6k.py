@@ -1,0 +1,100 @@
+"""Q6_K decode GEMV on the GPU against the oracle (wick/src/backend/simd.rs:547-640):
+the i32 dot of every 16-weight group BIT-EXACT, f32 outputs within rel-L2 1e-5 /
+max-abs 1e-4 x RMS."""
+import numpy as np
+import pytest
+
+import wick_amd as W
+from conftest import assert_f32_parity
+from gpu_util import Problem, fetch_gemm
+
+pytestmark = pytest.mark.gpu
+
+# (m, k): every lanes-per-row tier (k/128 half blocks per row, padded to a power of two),
+# m below / above one wave pass and ragged against rows-per-wave, the LFM2 LM head width.
+SHAPES = [(1, 256), (3, 256), (33, 256), (7, 512), (130, 512), (65, 768), (257, 1024), (4099, 1024), (19, 1536), (300, 2048),
+          (1025, 2048), (31, 2560), (64, 4096), (9, 6144), (17, 8192), (65536, 1024)]
+
+
+@pytest.mark.parametrize("m,k", SHAPES)
+def test_q6k_gemv_parity(ctx, oracle, m, k):
+    with Problem(ctx, oracle, W.Q6_K, m, k, seed=m + 3 * k) as p:
+        d_y = p.alloc(m * 4)
+        ctx.gemv_with_preq(p.w, p.d_s, p.d_q, d_y)
+        assert_f32_parity(d_y.download(np.float32, m), oracle.gemv_q6k_q8(p.wb, p.s[0], p.q[0], m, k), f"q6k gemv {m}x{k}")
+        d_d = p.alloc(m * (k // 16) * 4)
+        ctx.block_dots_i32(p.w, p.d_q, 1, d_d)
+        dots = d_d.download(np.int32, m * (k // 16)).reshape(m, k // 16)
+        assert np.array_equal(dots, oracle.q6k_group_dots_i32(p.wb, p.q[0], m, k))
+
+
+def test_q6k_extreme_blocks(ctx, oracle):
+    """Random BYTES as blocks (every 6-bit value, every int8 group scale, arbitrary finite
+    f16 super-scales) against saturated activations: the integer path must stay exact."""
+    rng = np.random.default_rng(1406)
+    m, k = 96, 1024
+    wb = rng.integers(0, 256, m * (k // 256) * 210).astype(np.uint8).reshape(-1, 210)
+    wb[:, 209] &= 0x3B  # clear the top exponent bits of d: finite and modest
+    wb = wb.reshape(-1)
+    with Problem(ctx, oracle, W.Q6_K, m, k, seed=3, weight_bytes=wb) as p:
+        q = rng.choice(np.array([-127, 127, -1, 0, 1, 126], np.int8), size=k).astype(np.int8)
+        d_q = p.to_device(q)
+        d_y, d_d = p.alloc(m * 4), p.alloc(m * (k // 16) * 4)
+        ctx.gemv_with_preq(p.w, p.d_s, d_q, d_y)
+        ctx.block_dots_i32(p.w, d_q, 1, d_d)
+        assert np.array_equal(d_d.download(np.int32, m * (k // 16)).reshape(m, -1), oracle.q6k_group_dots_i32(wb, q, m, k))
+        assert_f32_parity(d_y.download(np.float32, m), oracle.gemv_q6k_q8(wb, p.s[0], q, m, k), "q6k extreme blocks")
+
+
+def test_q6k_accumulate_and_multi(ctx, oracle):
+    """y += W x, and two weights behind one call."""
+    m, k = 777, 1024
+    with Problem(ctx, oracle, W.Q6_K, m, k, seed=21) as p:
+        y0 = oracle.fill_normal(77, 1.0, m)
+        d_y = p.to_device(y0)
+        ctx.gemv_with_preq(p.w, p.d_s, p.d_q, d_y, accumulate=True)
+        ref = oracle.gemv_q6k_q8(p.wb, p.s[0], p.q[0], m, k)
+        assert_f32_parity(d_y.download(np.float32, m), y0 + ref, "q6k accumulate")
+        wb2 = oracle.synth_weight(W.Q6_K, 50, k, 5)
+        w2 = ctx.upload_weight(wb2, W.Q6_K, 50, k)
+        d_a, d_b = p.alloc(m * 4), p.alloc(50 * 4)
+        ctx.gemv_with_preq_multi([p.w, w2], p.d_s, p.d_q, [d_a, d_b])
+        assert_f32_parity(d_a.download(np.float32, m), ref, "q6k multi[0]")
+        assert_f32_parity(d_b.download(np.float32, 50), oracle.gemv_q6k_q8(wb2, p.s[0], p.q[0], 50, k), "q6k multi[1]")
+        w2.free()
+
+
+def test_q6k_f32_call_site(ctx, oracle):
+    """The reference's call-site form (f32 in, f32 out; wick/src/backend/cpu.rs:423-470 quantizes x
+    to Q8_0 first) equals quantize + pre-quantized GEMV bit for bit."""
+    m, k = 1030, 2048
+    with Problem(ctx, oracle, W.Q6_K, m, k, seed=8) as p:
+        d_x = p.to_device(p.x)
+        d_y, d_z = p.alloc(m * 4), p.alloc(m * 4)
+        ctx.encode_gemv(p.w, d_x, 0, d_y, 0)
+        ctx.gemv_with_preq(p.w, p.d_s, p.d_q, d_z)
+        y, z = d_y.download(np.float32, m), d_z.download(np.float32, m)
+        assert np.array_equal(y.view(np.uint32), z.view(np.uint32))
+        ctx.encode_gemv_fused([p.w], d_x, 0, [d_y])
+        assert np.array_equal(d_y.download(np.float32, m).view(np.uint32), z.view(np.uint32))
+
+
+@pytest.mark.parametrize("layout", [W.LAYOUT_ROW_MAJOR, W.LAYOUT_TOKEN_MAJOR])
+def test_q6k_batched(ctx, oracle, layout):
+    """Batched calls on a Q6_K weight run the GEMV per token: every column equals the oracle's GEMV."""
+    m, k, n = 203, 512, 5
+    with Problem(ctx, oracle, W.Q6_K, m, k, n=n, seed=4) as p:
+        stride = (n + 3) if layout == W.LAYOUT_ROW_MAJOR else (m + 5)
+        d_y = p.alloc(max(m, n) * stride * 4)
+        ctx.gemm_preq(p.w, p.d_s, p.d_q, n, d_y, stride, layout)
+        y = fetch_gemm(d_y, m, n, stride, layout)
+        for j in range(n):
+            assert_f32_parity(y[:, j], oracle.gemv_q6k_q8(p.wb, p.s[j], p.q[j], m, k), f"q6k batched col {j}")
+
+
+def test_q6k_rejects(ctx, oracle):
+    wb = oracle.synth_weight(W.Q6_K, 4, 256, 1)
+    with pytest.raises(W.RocmError):
+        ctx.upload_weight(wb[:-1], W.Q6_K, 4, 256)
+    with pytest.raises(W.RocmError):
+        ctx.upload_weight(np.zeros(4 * 210 // 2, np.uint8), W.Q6_K, 4, 128)

@@ -11,6 +11,7 @@ from .rocm import (  # noqa: F401
     LAYOUT_ROW_MAJOR,
     LAYOUT_TOKEN_MAJOR,
     Q4_0,
+    Q6_K,
     Q8_0,
     DeviceBuffer,
     RocmContext,

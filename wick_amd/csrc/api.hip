@@ -118,6 +118,16 @@ int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q
         return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "unknown output layout");
     if (y_layout == WICK_ROCM_LAYOUT_TOKEN_MAJOR ? (y_stride < w->m && n > 1) : (y_stride < n))
         return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "y_stride smaller than the output extent");
+    if (w->type == kTypeQ6_K) {  // no batched kernel for Q6_K: one GEMV per token (the LM head sees one or a few)
+        if (reinterpret_cast<uintptr_t>(d_q) % 16u != 0) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "Q6_K gemm: quants must be 16-byte aligned");
+        const bool tm = y_layout == WICK_ROCM_LAYOUT_TOKEN_MAJOR;
+        for (uint32_t j = 0; j < n; j++) {
+            hipError_t e = launch_gemv_q6k(static_cast<const uint8_t*>(w->d), w->m, w->k, d_q + (size_t)j * w->k, d_s + (size_t)j * (w->k / 32u),
+                                           tm ? d_y + (size_t)j * y_stride : d_y + j, tm ? 1u : y_stride, accumulate, ctx->num_cus, ctx->launch());
+            if (e != hipSuccess) return fail_hip(ctx, e, "Q6_K gemv launch");
+        }
+        return WICK_ROCM_OK;
+    }
     const bool mfma_ok = (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_q) % 16u == 0) &&
                          (reinterpret_cast<uintptr_t>(d_s) % 16u == 0);
     hipError_t e;
@@ -293,15 +303,24 @@ int wick_rocm_weight_upload(wick_rocm_ctx* ctx, const void* host_blocks, size_t 
     if (!out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "weight_upload: null out pointer");
     *out = nullptr;
     if (!host_blocks) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "weight_upload: null host pointer");
-    const int bb = block_bytes(ggml_type);
-    if (bb == 0) return fail(ctx, WICK_ROCM_ERR_UNSUPPORTED_DTYPE, "weight_upload: only Q4_0 (2) and Q8_0 (8) are supported");
-    if (m == 0 || k == 0 || k % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "weight_upload: m, k must be > 0 and k % 32 == 0");
-    if (nbytes != (size_t)m * (k / 32u) * (size_t)bb)
-        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "weight_upload: nbytes != m * (k/32) * block_bytes");
+    if (ggml_type == kTypeQ6_K) {
+        if (m == 0 || k == 0 || k % 256u != 0 || k > 8192u)
+            return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "weight_upload: Q6_K needs m > 0 and k a multiple of 256, at most 8192");
+        if (nbytes != (size_t)m * (k / 256u) * (size_t)kQ6KBlockBytes)
+            return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "weight_upload: nbytes != m * (k/256) * 210");
+    } else {
+        const int bb = block_bytes(ggml_type);
+        if (bb == 0)
+            return fail(ctx, WICK_ROCM_ERR_UNSUPPORTED_DTYPE, "weight_upload: only Q4_0 (2), Q8_0 (8) and Q6_K (14) are supported");
+        if (m == 0 || k == 0 || k % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "weight_upload: m, k must be > 0 and k % 32 == 0");
+        if (nbytes != (size_t)m * (k / 32u) * (size_t)bb)
+            return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "weight_upload: nbytes != m * (k/32) * block_bytes");
+    }
     if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "weight_upload during graph capture");
     wick_rocm_weight* w = new (std::nothrow) wick_rocm_weight();
     if (!w) return fail(ctx, WICK_ROCM_ERR_HIP, "out of host memory");
-    hipError_t e = hipMalloc(&w->d, nbytes);
+    // (+64: the Q6_K kernel reads its last 16-byte piece whole)
+    hipError_t e = hipMalloc(&w->d, nbytes + 64);
     if (e == hipSuccess) e = hipMemcpyAsync(w->d, host_blocks, nbytes, hipMemcpyHostToDevice, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
@@ -372,6 +391,18 @@ int make_batch(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* con
     return WICK_ROCM_OK;
 }
 
+// Q6_K weights (the LM head of shipped LFM2 Q4_0 files): one GEMV launch per weight.
+int q6k_gemv_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count,
+                    const int8_t* d_q, const float* d_s, int accumulate) {
+    if (reinterpret_cast<uintptr_t>(d_q) % 16u != 0) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "Q6_K gemv: quants must be 16-byte aligned");
+    for (uint32_t i = 0; i < count; i++) {
+        hipError_t e = launch_gemv_q6k(static_cast<const uint8_t*>(ws[i]->d), ws[i]->m, ws[i]->k, d_q, d_s, d_ys[i], 1, accumulate,
+                                       ctx->num_cus, ctx->launch());
+        if (e != hipSuccess) return fail_hip(ctx, e, "Q6_K gemv launch");
+    }
+    return WICK_ROCM_OK;
+}
+
 // f32 activations -> y for a group of weights (lock held): fused quantize+GEMV when
 // the pair kernel takes the shape, otherwise quantize into scratch, then GEMV.
 int gemv_f32_locked(wick_rocm_ctx* ctx, const GemvBatch& b, int type, uint32_t k, const float* x, int accumulate) {
@@ -396,6 +427,7 @@ int wick_rocm_gemv_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* w
     if (!d_quants || !d_scales) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv: null pointer");
     GemvBatch b{};
     if (int rc = make_batch(ctx, ws, d_ys, count, b)) return rc;
+    if (ws[0]->type == kTypeQ6_K) return q6k_gemv_locked(ctx, ws, d_ys, count, d_quants, d_scales, accumulate);
     hipError_t e = launch_gemv(ws[0]->type, b, ws[0]->k, d_quants, d_scales, accumulate, ctx->num_cus, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "gemv launch");
     return WICK_ROCM_OK;
@@ -409,6 +441,13 @@ int wick_rocm_gemv_f32_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* 
     GemvBatch b{};
     if (int rc = make_batch(ctx, ws, d_ys, count, b)) return rc;
     const float* x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes);
+    if (ws[0]->type == kTypeQ6_K) {  // quantize into scratch, then one launch per weight
+        const uint32_t k = ws[0]->k;
+        if (int rc = ensure_scratch(ctx, k, k / 32u)) return rc;
+        hipError_t e = launch_quantize_q8_0(x, 1, k, k, ctx->scratch_q, ctx->scratch_s, ctx->launch());
+        if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
+        return q6k_gemv_locked(ctx, ws, d_ys, count, ctx->scratch_q, ctx->scratch_s, accumulate);
+    }
     return gemv_f32_locked(ctx, b, ws[0]->type, ws[0]->k, x, accumulate);
 }
 
@@ -443,7 +482,7 @@ int wick_rocm_matmul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const fl
         return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "matmul_f32: stride smaller than the vector length");
     const float* x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes);
     float* y = reinterpret_cast<float*>(reinterpret_cast<char*>(d_y) + y_off_bytes);
-    if (n == 1) {
+    if (n == 1 && w->type != kTypeQ6_K) {
         GemvBatch b{};
         b.w[0] = static_cast<const uint8_t*>(w->d), b.y[0] = y, b.row_end[0] = w->m, b.count = 1;
         return gemv_f32_locked(ctx, b, w->type, w->k, x, accumulate);
@@ -461,6 +500,15 @@ int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, cons
     if (int rc = check_weight(ctx, w)) return rc;
     if (!d_quants || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "block_dots: null device pointer");
     if (n == 0) return WICK_ROCM_OK;
+    if (w->type == kTypeQ6_K) {  // 16-weight groups: out[(j*m + i) * (k/16) + g]
+        if (reinterpret_cast<uintptr_t>(d_quants) % 16u != 0) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "block_dots: quants must be 16-byte aligned");
+        for (uint32_t j = 0; j < n; j++) {
+            hipError_t e = launch_group_dots_q6k(static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants + (size_t)j * w->k,
+                                                 d_out + (size_t)j * w->m * (w->k / 16u), ctx->num_cus, ctx->launch());
+            if (e != hipSuccess) return fail_hip(ctx, e, "block_dots launch");
+        }
+        return WICK_ROCM_OK;
+    }
     const bool mfma = n >= ctx->gemm_min_n && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
     hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch())
                         : launch_block_dots_dot4(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch());

@@ -89,6 +89,15 @@ bool pairs_kernel_applies(const GemvBatch& batch, uint32_t k);
 hipError_t launch_gemv_f32(int type, const GemvBatch& batch, uint32_t k, const float* d_x, int accumulate, int num_cus,
                            const Launch& L);
 
+// Q6_K decode GEMV, one token (gemv_q6k.hip).  k % 256 == 0, k <= 8192; the weight allocation is padded by
+// 16 bytes; y[row * y_row_stride].  launch_group_dots_q6k is its parity hook: out[i * (k/16) + g] = exact i32 dot of 16-weight group g.
+constexpr int kTypeQ6_K = 14;  // ggml id, wick/src/gguf.rs:36-51
+constexpr int kQ6KBlockBytes = 210;
+hipError_t launch_gemv_q6k(const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, const float* d_scales, float* d_y,
+                           uint32_t y_row_stride, int accumulate, int num_cus, const Launch& L);
+hipError_t launch_group_dots_q6k(const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, int32_t* d_out, int num_cus,
+                                 const Launch& L);
+
 // Small-n GEMM done as a multi-token GEMV (weights streamed once per 1..kGemvTokens tokens).
 hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                               const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,

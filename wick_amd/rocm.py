@@ -25,6 +25,7 @@ import numpy as np
 
 Q4_0 = 2  # ggml type ids, wick/src/gguf.rs:36-51
 Q8_0 = 8
+Q6_K = 14  # decode GEMV only; 210-byte blocks of 256 weights (wick/src/quant.rs:54-70)
 BLOCK_BYTES = {Q4_0: 18, Q8_0: 34}
 LAYOUT_TOKEN_MAJOR = 0
 LAYOUT_ROW_MAJOR = 1
