@@ -112,6 +112,11 @@ int wick_rocm_copy(wick_rocm_ctx *ctx, void *d_dst, const void *d_src, size_t nb
  * wick_rocm_weight_free or context destruction. */
 int wick_rocm_weight_upload(wick_rocm_ctx *ctx, const void *host_blocks, size_t nbytes, int ggml_type,
                             uint32_t m, uint32_t k, wick_rocm_weight **out);
+/* resolve_weight + upload (wick/src/model/lfm2.rs:310-338, wick/src/model/metal_lfm2.rs:409-421): looks the
+ * tensor up in an open GGUF file (include/wick_gguf.h), takes k = ne0 and m = ne1 (m = 1 for rank 1)
+ * and uploads its bytes.  Fails like wick_rocm_weight_upload for types / shapes the kernels do not take. */
+struct wick_gguf;
+int wick_rocm_weight_from_gguf(wick_rocm_ctx *ctx, const struct wick_gguf *gguf, const char *tensor_name, wick_rocm_weight **out);
 int wick_rocm_weight_free(wick_rocm_ctx *ctx, wick_rocm_weight *w);
 int wick_rocm_weight_info(const wick_rocm_weight *w, int *ggml_type, uint32_t *m, uint32_t *k, size_t *nbytes);
 const void *wick_rocm_weight_device_ptr(const wick_rocm_weight *w);

@@ -12,10 +12,10 @@ import wick_amd
 from wick_amd import rocm
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "wick_rocm.h")).read()
+def declared_symbols(header="wick_rocm.h", prefix="wick_rocm_"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(wick_rocm_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(" + prefix + r"[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_declares_the_path():
@@ -33,6 +33,16 @@ def test_library_exports_every_declared_symbol():
 
 def test_python_mirror_binds_every_declared_symbol():
     assert sorted(rocm._SIGNATURES) == declared_symbols()
+
+
+def test_gguf_reader_symbols_are_exported_and_bound():
+    from wick_amd import gguf
+
+    names = declared_symbols("wick_gguf.h", "wick_gguf_")
+    lib = wick_amd.load_library()
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in wick_gguf.h but not exported"
+    assert sorted(gguf._SIGNATURES) == names
 
 
 def test_static_library_is_built_too():

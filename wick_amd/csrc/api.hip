@@ -12,6 +12,7 @@
 #include <string>
 
 #include "wick_rocm_internal.h"
+#include "../../include/wick_gguf.h"
 
 using namespace wick_rocm;
 
@@ -331,6 +332,20 @@ int wick_rocm_weight_upload(wick_rocm_ctx* ctx, const void* host_blocks, size_t 
     w->nbytes = nbytes, w->type = ggml_type, w->m = m, w->k = k;
     *out = w;
     return WICK_ROCM_OK;
+}
+
+int wick_rocm_weight_from_gguf(wick_rocm_ctx* ctx, const wick_gguf* gguf, const char* tensor_name, wick_rocm_weight** out) {
+    if (!ctx) return WICK_ROCM_ERR_INVALID_ARG;
+    if (!gguf || !tensor_name || !out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "weight_from_gguf: null argument");
+    uint64_t offset = 0, rows = 0, cols = 0;
+    int type = 0;
+    const void* bytes = nullptr;
+    size_t nbytes = 0;
+    if (wick_gguf_tensor_meta(gguf, tensor_name, &offset, &rows, &cols, &type) != 0 ||
+        wick_gguf_tensor_data(gguf, tensor_name, &bytes, &nbytes) != 0)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, (std::string("weight_from_gguf: ") + wick_gguf_last_error()).c_str());
+    if (rows > UINT32_MAX || cols > UINT32_MAX) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "weight_from_gguf: dimension exceeds 32 bits");
+    return wick_rocm_weight_upload(ctx, bytes, nbytes, type, (uint32_t)rows, (uint32_t)cols, out);
 }
 
 int wick_rocm_weight_free(wick_rocm_ctx* ctx, wick_rocm_weight* w) {

@@ -175,7 +175,7 @@ template <int LPR, bool DUMP>
 hipError_t launch_lpr(Q6kArgs& a, int num_cus, const Launch& L) {
     constexpr uint32_t RPW = 64 / LPR;
     const uint32_t passes = (a.m + RPW - 1) / RPW;
-    const uint32_t max_waves = (uint32_t)num_cus * 16u;
+    const uint32_t max_waves = (uint32_t)num_cus * 12u;  // measured best on the 65536 x 1024 LM head (8..16 within 7 %)
     uint32_t ppw = (passes + max_waves - 1) / max_waves;
     if (ppw == 0) ppw = 1;
     a.rows_per_wave = ppw * RPW;

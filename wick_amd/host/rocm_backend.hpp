@@ -19,11 +19,12 @@
 #include <string>
 #include <vector>
 
+#include "../../include/wick_gguf.h"
 #include "../../include/wick_rocm.h"
 
 namespace wick {
 
-enum class DType : int { Q4_0 = WICK_ROCM_TYPE_Q4_0, Q8_0 = WICK_ROCM_TYPE_Q8_0 };
+enum class DType : int { Q4_0 = WICK_ROCM_TYPE_Q4_0, Q8_0 = WICK_ROCM_TYPE_Q8_0, Q6_K = WICK_ROCM_TYPE_Q6_K };
 
 struct BackendError : std::runtime_error {
     int status;
@@ -31,6 +32,22 @@ struct BackendError : std::runtime_error {
 };
 
 class RocmContext;
+
+// An open GGUF file (GgufFile::open, wick/src/gguf.rs:331-341).
+class GgufFile {
+public:
+    explicit GgufFile(const std::string& path) {
+        const int rc = wick_gguf_open(path.c_str(), &g_);
+        if (rc != 0) throw BackendError(rc, wick_gguf_last_error());
+    }
+    ~GgufFile() { wick_gguf_close(g_); }
+    GgufFile(const GgufFile&) = delete;
+    GgufFile& operator=(const GgufFile&) = delete;
+    const wick_gguf* raw() const { return g_; }
+
+private:
+    wick_gguf* g_ = nullptr;
+};
 
 // Device-resident weight: GGUF block bytes verbatim.
 struct RocmWeight {
@@ -82,6 +99,16 @@ public:
         RocmWeight w;
         w.dtype = dtype, w.m = m, w.k = k;
         check(wick_rocm_weight_upload(ctx_, blocks, nbytes, static_cast<int>(dtype), m, k, &w.handle));
+        return w;
+    }
+    // resolve_weight (wick/src/model/lfm2.rs:310-338) + upload: k = ne0, m = ne1.
+    RocmWeight weight_from_gguf(const GgufFile& gguf, const std::string& tensor_name) {
+        RocmWeight w;
+        check(wick_rocm_weight_from_gguf(ctx_, gguf.raw(), tensor_name.c_str(), &w.handle));
+        int type = 0;
+        size_t nbytes = 0;
+        check(wick_rocm_weight_info(w.handle, &type, &w.m, &w.k, &nbytes));
+        w.dtype = static_cast<DType>(type);
         return w;
     }
     void free_weight(RocmWeight& w) {

@@ -76,6 +76,7 @@ _SIGNATURES = {
     "wick_rocm_set_gemv_policy": (C.c_int, [_P, C.c_int64]),
     "wick_rocm_probe_rate": (C.c_int, [_P, C.c_int, C.c_uint32, C.POINTER(C.c_double)]),
     "wick_rocm_weight_upload": (C.c_int, [_P, _P, C.c_size_t, C.c_int, C.c_uint32, C.c_uint32, C.POINTER(_P)]),
+    "wick_rocm_weight_from_gguf": (C.c_int, [_P, _P, C.c_char_p, C.POINTER(_P)]),
     "wick_rocm_weight_free": (C.c_int, [_P, _P]),
     "wick_rocm_weight_info": (C.c_int, [_P, C.POINTER(C.c_int), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_size_t)]),
     "wick_rocm_weight_device_ptr": (_P, [_P]),
@@ -244,6 +245,14 @@ class RocmContext:
         h = _P()
         self._check(self._lib.wick_rocm_weight_upload(self._h, a.ctypes.data, a.nbytes, dtype, m, k, C.byref(h)))
         return RocmWeight(self, h.value, dtype, m, k, a.nbytes)
+
+    def weight_from_gguf(self, gguf, tensor_name: str) -> RocmWeight:
+        """resolve_weight + upload (wick/src/model/lfm2.rs:310-338): `gguf` is a wick_amd.gguf.GgufFile."""
+        h = _P()
+        self._check(self._lib.wick_rocm_weight_from_gguf(self._h, gguf.handle, tensor_name.encode(), C.byref(h)))
+        t, m, k, nb = C.c_int(), C.c_uint32(), C.c_uint32(), C.c_size_t()
+        self._check(self._lib.wick_rocm_weight_info(h.value, C.byref(t), C.byref(m), C.byref(k), C.byref(nb)))
+        return RocmWeight(self, h.value, t.value, m.value, k.value, nb.value)
 
     # -- hot path on pre-quantized activations ------------------------------
     def quantize_q8_0(self, x, n: int, k: int, x_stride: int, quants, scales) -> None:
