@@ -1,0 +1,191 @@
+"""CPU oracle of wick's LFM2 decode step (TEST INFRASTRUCTURE, not product code).
+
+Only tests, ``__graft_entry__.smoke()`` and ``bench.py``'s cpu-baseline leg may import this
+module.  The per-operation functions wrap ``oracle/wick_oracle_ops.c`` one to one; the
+step itself (``Lfm2Oracle.forward``) is the aarch64 branch of the reference's CPU model:
+every GEMV runs on Q8_0-quantized activations (wick/src/model/lfm2.rs:1020-1124 run_layers,
+:646-730 conv block, :733-1017 attention block, :2258-2289 forward).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import oracle as O
+
+F32 = 0  # ggml type id
+
+_ops = None
+
+
+def ops() -> C.CDLL:
+    global _ops
+    if _ops is None:
+        L = O._load("libwick_oracle_ops.so")
+        L.orc_ggml_expf.restype = C.c_float
+        L.orc_ggml_expf.argtypes = [C.c_float]
+        L.orc_rope_theta_scale.restype = C.c_float
+        L.orc_rope_theta_scale.argtypes = [C.c_int64, C.c_float]
+        L.orc_argmax.restype = C.c_int64
+        _ops = L
+    return _ops
+
+
+_p, _c = O._p, O._c
+
+
+def ggml_expf(x: float) -> float:
+    return float(ops().orc_ggml_expf(C.c_float(float(x))))
+
+
+def rmsnorm(x, weight, eps: float) -> np.ndarray:
+    y = _c(x, np.float32).copy()
+    ops().orc_rmsnorm(_p(y), _p(_c(weight, np.float32)), C.c_int64(y.size), C.c_float(eps))
+    return y
+
+
+def silu_mul(gate, up) -> np.ndarray:
+    g = _c(gate, np.float32).copy()
+    ops().orc_silu_mul(_p(g), _p(_c(up, np.float32)), C.c_int64(g.size))
+    return g
+
+
+def softmax(x) -> np.ndarray:
+    y = _c(x, np.float32).copy()
+    ops().orc_softmax(_p(y), C.c_int64(y.size))
+    return y
+
+
+def rope(q, k, pos: int, n_heads: int, n_kv_heads: int, head_dim: int, freq_base: float):
+    q2, k2 = _c(q, np.float32).copy(), _c(k, np.float32).copy()
+    ops().orc_rope(_p(q2), _p(k2), C.c_int64(pos), C.c_int64(n_heads), C.c_int64(n_kv_heads), C.c_int64(head_dim), C.c_float(freq_base))
+    return q2, k2
+
+
+def rope_theta_scale(head_dim: int, freq_base: float) -> float:
+    return float(ops().orc_rope_theta_scale(head_dim, C.c_float(freq_base)))
+
+
+def attn_scores(q_head, k_cache, kv_dim: int, kv_h_offset: int, head_dim: int, scale: float, seq_len: int) -> np.ndarray:
+    out = np.zeros(seq_len, np.float32)
+    ops().orc_attn_scores(_p(_c(q_head, np.float32)), _p(_c(k_cache, np.float32)), _p(out), C.c_int64(kv_dim), C.c_int64(kv_h_offset),
+                          C.c_int64(head_dim), C.c_float(scale), C.c_int64(seq_len))
+    return out
+
+
+def attn_values(scores, v_cache, kv_dim: int, kv_h_offset: int, head_dim: int, seq_len: int) -> np.ndarray:
+    out = np.zeros(head_dim, np.float32)
+    ops().orc_attn_values(_p(_c(scores, np.float32)), _p(_c(v_cache, np.float32)), _p(out), C.c_int64(kv_dim), C.c_int64(kv_h_offset),
+                          C.c_int64(head_dim), C.c_int64(seq_len))
+    return out
+
+
+def attention(q, k_cache, v_cache, n_heads: int, n_kv_heads: int, head_dim: int, seq_len: int) -> np.ndarray:
+    """All heads of one decode position (wick/src/model/lfm2.rs:984-1006): [n_heads * head_dim]."""
+    q = _c(q, np.float32)
+    kc, vc = _c(k_cache, np.float32), _c(v_cache, np.float32)
+    kv_dim, group = n_kv_heads * head_dim, n_heads // n_kv_heads
+    scale = np.float32(1.0) / np.sqrt(np.float32(head_dim))
+    out = np.zeros(n_heads * head_dim, np.float32)
+    scratch = np.zeros(max(seq_len, 1), np.float32)
+    for h in range(n_heads):
+        ops().orc_attention_head(_p(q[h * head_dim:]), _p(kc), _p(vc), _p(scratch), _p(out[h * head_dim:]), C.c_int64(kv_dim),
+                                 C.c_int64((h // group) * head_dim), C.c_int64(head_dim), C.c_float(scale), C.c_int64(seq_len))
+    return out
+
+
+def shortconv_step(proj, buffer, conv_weight, hidden: int, kernel_size: int) -> np.ndarray:
+    """One decode step of the gated short convolution; `buffer` ([(kernel-1) * hidden] f32) is updated in place."""
+    assert buffer.dtype == np.float32 and buffer.flags.c_contiguous and buffer.size == (kernel_size - 1) * hidden
+    out = np.empty(hidden, np.float32)
+    ops().orc_shortconv_step(_p(_c(proj, np.float32)), _p(buffer), _p(_c(conv_weight, np.float32)), _p(out), C.c_int64(hidden),
+                             C.c_int64(kernel_size))
+    return out
+
+
+def argmax(x) -> int:
+    x = _c(x, np.float32)
+    return int(ops().orc_argmax(_p(x), C.c_int64(x.size))) if x.size else 0
+
+
+def embed_row(ggml_type: int, data: np.ndarray, row: int, k: int) -> np.ndarray:
+    """dequantize_row_into, wick/src/model/lfm2.rs:621-643."""
+    if ggml_type == F32:
+        return data.view(np.float32)[row * k:(row + 1) * k].copy()
+    if ggml_type == O.Q6_K:
+        rb = k // 256 * 210
+        return O.dequant_q6_k(data[row * rb:(row + 1) * rb], 1, k)[0]
+    rb = k // 32 * O.BLOCK_BYTES[ggml_type]
+    return O.dequant_row(ggml_type, data[row * rb:(row + 1) * rb])
+
+
+def gemv(ggml_type: int, data: np.ndarray, x: np.ndarray, m: int, k: int) -> np.ndarray:
+    """The aarch64 GEMV dispatch: quantize x to Q8_0, integer dots (wick/src/backend/cpu.rs:334-354, 423-470)."""
+    s, q = O.quantize_q8_0(x)
+    if ggml_type == O.Q6_K:
+        return O.gemv_q6k_q8(data, s, q, m, k)
+    return O.gemv_q8(ggml_type, data, s, q, m, k)
+
+
+class Lfm2Oracle:
+    """`cfg`: n_layers, hidden_size, intermediate_size, n_heads, vocab_size, rope_theta, rms_norm_eps,
+    conv_kernel_size, kv_heads_per_layer (0 = gated-conv layer).  `tensors`: GGUF name -> (ggml_type, dims, array),
+    quantized weights as raw block bytes (dims [k, m]), norms / conv kernels as float32."""
+
+    def __init__(self, cfg: dict, tensors: dict):
+        self.cfg, self.t = cfg, tensors
+
+    def new_state(self) -> dict:
+        c = self.cfg
+        hs, dconv = c["hidden_size"], c["conv_kernel_size"] - 1
+        st = {"seq_len": 0, "layers": []}
+        for n_kv in c["kv_heads_per_layer"]:
+            st["layers"].append({"k": [], "v": []} if n_kv else {"buf": np.zeros(dconv * hs, np.float32)})
+        return st
+
+    def _f32(self, name):
+        return self.t[name][2].view(np.float32).ravel()
+
+    def _gemv(self, name, x):
+        gt, dims, data = self.t[name]
+        return gemv(gt, data, x, dims[1], dims[0])
+
+    def hidden_after_layers(self, token: int, pos: int, state: dict) -> np.ndarray:
+        c = self.cfg
+        hs, eps = c["hidden_size"], c["rms_norm_eps"]
+        gt, dims, data = self.t["token_embd.weight"]
+        hidden = embed_row(gt, data, token, dims[0])
+        for i, n_kv in enumerate(c["kv_heads_per_layer"]):
+            normed = rmsnorm(hidden, self._f32(f"blk.{i}.attn_norm.weight"), eps)
+            if n_kv == 0:
+                proj = self._gemv(f"blk.{i}.shortconv.in_proj.weight", normed)
+                gated = shortconv_step(proj, state["layers"][i]["buf"], self._f32(f"blk.{i}.shortconv.conv.weight"), hs, c["conv_kernel_size"])
+                out = self._gemv(f"blk.{i}.shortconv.out_proj.weight", gated)
+            else:
+                hd = hs // c["n_heads"]
+                q = self._gemv(f"blk.{i}.attn_q.weight", normed)
+                k = self._gemv(f"blk.{i}.attn_k.weight", normed)
+                v = self._gemv(f"blk.{i}.attn_v.weight", normed)
+                qn, kn = self._f32(f"blk.{i}.attn_q_norm.weight"), self._f32(f"blk.{i}.attn_k_norm.weight")
+                for h in range(c["n_heads"]):
+                    q[h * hd:(h + 1) * hd] = rmsnorm(q[h * hd:(h + 1) * hd], qn, eps)
+                for h in range(n_kv):
+                    k[h * hd:(h + 1) * hd] = rmsnorm(k[h * hd:(h + 1) * hd], kn, eps)
+                q, k = rope(q, k, pos, c["n_heads"], n_kv, hd, c["rope_theta"])
+                ls = state["layers"][i]
+                ls["k"].append(k), ls["v"].append(v)
+                attn = attention(q, np.concatenate(ls["k"]), np.concatenate(ls["v"]), c["n_heads"], n_kv, hd, len(ls["k"]))
+                out = self._gemv(f"blk.{i}.attn_output.weight", attn)
+            hidden = hidden + out
+            ffn_in = rmsnorm(hidden, self._f32(f"blk.{i}.ffn_norm.weight"), eps)
+            gate = self._gemv(f"blk.{i}.ffn_gate.weight", ffn_in)
+            up = self._gemv(f"blk.{i}.ffn_up.weight", ffn_in)
+            hidden = hidden + self._gemv(f"blk.{i}.ffn_down.weight", silu_mul(gate, up))
+        state["seq_len"] += 1
+        return rmsnorm(hidden, self._f32("token_embd_norm.weight"), eps)
+
+    def forward(self, token: int, pos: int, state: dict) -> np.ndarray:
+        """Logits of one decode step (tied embedding as LM head, wick/src/model/lfm2.rs:2258-2289)."""
+        hidden = self.hidden_after_layers(token, pos, state)
+        return self._gemv("token_embd.weight", hidden)

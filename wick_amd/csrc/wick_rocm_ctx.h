@@ -1,0 +1,79 @@
+// Context, handle structs and the entry-point prologue shared by the translation units that
+// implement the C ABI (api.hip, lfm2_api.hip).  Not installed.
+#pragma once
+
+#include <mutex>
+#include <string>
+
+#include "../../include/wick_rocm.h"
+#include "wick_rocm_internal.h"
+
+using namespace wick_rocm;
+
+struct wick_rocm_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::mutex mu;  // serialises calls on this context, like the reference's infer_lock
+    std::string err;
+    std::string name;
+    int num_cus = 0;
+    size_t hbm_bytes = 0;
+    bool capturing = false;
+    // scratch for wick_rocm_matmul_f32 (quantized activations)
+    int8_t* scratch_q = nullptr;
+    float* scratch_s = nullptr;
+    size_t scratch_q_cap = 0;  // bytes
+    size_t scratch_s_cap = 0;  // floats
+    uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
+    KernelTimer timer;
+    int64_t gemv_direct_max_bytes = -1;
+    void* probe_sink = nullptr;  // 64 bytes the rate probes may (never do) write to
+    Launch launch() { return Launch{stream, &timer, gemv_direct_max_bytes}; }
+};
+
+struct wick_rocm_weight {
+    void* d = nullptr;
+    size_t nbytes = 0;
+    int type = 0;
+    uint32_t m = 0, k = 0;
+};
+
+struct wick_rocm_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+struct wick_rocm_event {
+    hipEvent_t ev = nullptr;
+};
+
+
+inline int fail(wick_rocm_ctx* ctx, int code, const char* what) {
+    if (ctx) ctx->err = what;
+    return code;
+}
+
+inline int fail_hip(wick_rocm_ctx* ctx, hipError_t e, const char* where) {
+    if (ctx) {
+        ctx->err = std::string(where) + ": " + hipGetErrorString(e);
+    }
+    return WICK_ROCM_ERR_HIP;
+}
+
+#define WR_HIP(ctx, call)                                      \
+    do {                                                       \
+        hipError_t e_ = (call);                                \
+        if (e_ != hipSuccess) return fail_hip(ctx, e_, #call); \
+    } while (0)
+
+// Takes the context lock and makes its device current for the calling thread.
+struct Guard {
+    std::unique_lock<std::mutex> lk;
+    hipError_t status;
+    explicit Guard(wick_rocm_ctx* ctx) : lk(ctx->mu), status(hipSetDevice(ctx->device)) {}
+};
+
+#define WR_ENTER(ctx)                                                   \
+    if (!(ctx)) return WICK_ROCM_ERR_INVALID_ARG;                       \
+    Guard guard_(ctx);                                                  \
+    if (guard_.status != hipSuccess) return fail_hip(ctx, guard_.status, "hipSetDevice")
