@@ -1,0 +1,115 @@
+/* wick_rocm_lfm2.h -- the LFM2 decode step around the matmul path, on one gfx950 GPU.
+ *
+ * Two layers, both on top of include/wick_rocm.h (same context, same status codes, same
+ * enqueue-only semantics, device pointers named d_*):
+ *
+ *  1. The non-matmul operations of a decode step as single calls, shaped like the reference's
+ *     GPU encoder call sites (wick/src/model/metal_lfm2.rs:1380-1990) and computing what its CPU
+ *     operations compute (wick/src/backend/cpu.rs:577-731, 1320-1401, 2113-2161).
+ *  2. A model handle that owns weights, KV caches, conv state and scratch, like the reference's
+ *     GPU models (wick/src/model/metal_lfm2.rs:254-267), with forward / forward_greedy of
+ *     `trait Model` (wick/src/model/mod.rs:72-323).  The step follows the aarch64 CPU model:
+ *     every GEMV runs on Q8_0-quantized activations, the KV cache holds f32
+ *     (wick/src/model/lfm2.rs:646-1124, 2258-2289).
+ *
+ * "pos" / "token" arguments come in pairs: a by-value number and a device pointer.  When the
+ * pointer is non-null the kernel reads it instead, so a captured graph of the step can be
+ * replayed for every token.
+ */
+#ifndef WICK_ROCM_LFM2_H
+#define WICK_ROCM_LFM2_H
+
+#include "wick_rocm.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+struct wick_gguf;
+
+/* ---- operations ---------------------------------------------------------------------- */
+
+/* Embedding lookup = dequantize_row_into (wick/src/model/lfm2.rs:621-643): row `token` (or *d_token) of a
+ * Q4_0 / Q8_0 / Q6_K weight as k floats.  A by-value token >= m is an error; a device-side one leaves d_out untouched. */
+int wick_rocm_embed_row(wick_rocm_ctx *ctx, const wick_rocm_weight *w, uint32_t token, const uint32_t *d_token, float *d_out);
+
+/* encode_rmsnorm / encode_per_head_rmsnorm (wick/src/model/metal_lfm2.rs:1380-1398, 1480-1496) = cpu::rmsnorm
+ * (wick/src/backend/cpu.rs:577-594) on `rows` vectors of `dim` floats that share one weight vector:
+ * y[r*y_stride + i] = x[r*x_stride + i] * inv_rms_r * weight[i].  d_y may equal d_x. */
+int wick_rocm_rmsnorm(wick_rocm_ctx *ctx, const float *d_x, const float *d_weight, float *d_y, uint32_t rows, uint32_t dim,
+                      uint32_t x_stride, uint32_t y_stride, float eps);
+
+/* encode_qk_norm_rope + the KV append (wick/src/model/metal_lfm2.rs:1542-1580, 4178-4193; CPU:
+ * wick/src/model/lfm2.rs:783-857, cpu::rope wick/src/backend/cpu.rs:2113-2161): per-head RMSNorm of Q and K
+ * with the layer's q_norm / k_norm weights, RoPE at `pos`, both in place; then K and V of this position are
+ * stored at row `pos` of the caches ([max_seq][n_kv_heads*head_dim] floats).  theta_scale = freq_base^(-2/head_dim)
+ * as an f32 (wick_rocm_rope_theta_scale).  head_dim even, <= 256. */
+int wick_rocm_qk_norm_rope(wick_rocm_ctx *ctx, float *d_q, float *d_k, const float *d_v, const float *d_q_norm, const float *d_k_norm,
+                           float *d_k_cache, float *d_v_cache, uint32_t pos, const uint32_t *d_pos, uint32_t max_seq, uint32_t head_dim,
+                           uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale);
+float wick_rocm_rope_theta_scale(uint32_t head_dim, float freq_base);
+
+/* encode_attention (wick/src/model/metal_lfm2.rs:1736-1867) = attn_scores + softmax_inplace + attn_values per
+ * query head (wick/src/model/lfm2.rs:984-1006) over cache rows [0, seq_len) (seq_len = *d_pos + 1 when d_pos is
+ * given), grouped-query: head h reads KV head h / (n_heads / n_kv_heads).  d_scores is scratch of
+ * n_heads * max_seq floats.  head_dim % 4 == 0, <= 256. */
+int wick_rocm_attention_decode(wick_rocm_ctx *ctx, const float *d_q, const float *d_k_cache, const float *d_v_cache, float *d_out,
+                               float *d_scores, uint32_t seq_len, const uint32_t *d_pos, uint32_t max_seq, uint32_t n_heads,
+                               uint32_t n_kv_heads, uint32_t head_dim);
+
+/* encode_conv1d_fused (wick/src/model/metal_lfm2.rs:1959-1991) = the middle of forward_conv_block
+ * (wick/src/model/lfm2.rs:694-726): d_proj = [b | c | x] (hidden floats each), d_buffer the rolling state
+ * ((kernel_size-1) * hidden floats, updated in place), d_conv_weight [hidden][kernel_size]; d_out = c * conv(b*x). */
+int wick_rocm_shortconv_step(wick_rocm_ctx *ctx, const float *d_proj, float *d_buffer, const float *d_conv_weight, float *d_out,
+                             uint32_t hidden, uint32_t kernel_size);
+
+/* encode_elementwise(silu_mul_inplace) (wick/src/model/metal_lfm2.rs:1701-1715) = cpu::silu_mul_inplace
+ * (wick/src/backend/cpu.rs:668-673): gate = silu(gate) * up. */
+int wick_rocm_silu_mul(wick_rocm_ctx *ctx, float *d_gate, const float *d_up, uint32_t n);
+
+/* argmax_f32 dispatch of forward_greedy (wick/src/model/metal_lfm2.rs:2187-2195) with the tie / NaN rules of
+ * cpu_argmax (wick/src/sampler.rs:7-19).  d_out[0] = pick; when given, *d_token = pick and *d_pos += 1. */
+int wick_rocm_argmax(wick_rocm_ctx *ctx, const float *d_logits, uint32_t n, uint32_t *d_out, uint32_t *d_token, uint32_t *d_pos);
+
+/* ---- the model --------------------------------------------------------------------------- */
+
+typedef struct wick_rocm_lfm2 wick_rocm_lfm2;
+
+/* ModelConfig (wick/src/model/mod.rs:23-70) as far as the step needs it. */
+typedef struct wick_rocm_lfm2_config {
+    uint32_t n_layers, hidden_size, intermediate_size, n_heads, n_kv_heads /* max over layers */, vocab_size, max_seq_len,
+        conv_kernel_size;
+    float rope_theta, rms_norm_eps;
+} wick_rocm_lfm2_config;
+
+/* load_model_metal's counterpart (wick/src/model/mod.rs:385-403; metadata keys, tensor names and checks of
+ * Lfm2Model::from_gguf_with_id, wick/src/model/lfm2.rs:97-300): reads the config, uploads every weight, allocates
+ * KV caches for min(context_size, lfm2.context_length) positions, conv state and scratch.  The GGUF handle is not
+ * referenced after the call returns. */
+int wick_rocm_lfm2_load(wick_rocm_ctx *ctx, const struct wick_gguf *gguf, uint32_t context_size, wick_rocm_lfm2 **out);
+int wick_rocm_lfm2_free(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model);
+int wick_rocm_lfm2_get_config(const wick_rocm_lfm2 *model, wick_rocm_lfm2_config *out);
+/* kv_heads_per_layer (0 = gated-conv layer). */
+int wick_rocm_lfm2_layer_kv_heads(const wick_rocm_lfm2 *model, uint32_t layer, uint32_t *n_kv_heads);
+/* Model::gpu_memory_bytes. */
+size_t wick_rocm_lfm2_gpu_memory_bytes(const wick_rocm_lfm2 *model);
+/* A fresh InferenceState: conv state zeroed, caches logically empty. */
+int wick_rocm_lfm2_reset(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model);
+
+/* Model::forward (wick/src/model/lfm2.rs:2258-2289): one token at position `pos` (= tokens seen so far) ->
+ * vocab_size logits copied to `logits` (host memory; may be null to leave them on the device).  Waits for the step. */
+int wick_rocm_lfm2_forward(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t token, uint32_t pos, float *logits);
+/* Model::forward_greedy (wick/src/model/metal_lfm2.rs:2151-2200): same step, the pick is made on the device. */
+int wick_rocm_lfm2_forward_greedy(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t token, uint32_t pos, uint32_t *next_token);
+/* n greedy steps starting with `token` at `pos`, without a host round trip between steps: out_tokens[i] is the
+ * pick after step i (which is also step i+1's input). */
+int wick_rocm_lfm2_generate_greedy(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t token, uint32_t pos, uint32_t n,
+                                   uint32_t *out_tokens);
+/* Device buffers of the last step, for inspection: logits [vocab_size], final normed hidden state [hidden_size]. */
+const float *wick_rocm_lfm2_logits_device(const wick_rocm_lfm2 *model);
+const float *wick_rocm_lfm2_hidden_device(const wick_rocm_lfm2 *model);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WICK_ROCM_LFM2_H */

@@ -45,6 +45,16 @@ def test_gguf_reader_symbols_are_exported_and_bound():
     assert sorted(gguf._SIGNATURES) == names
 
 
+def test_lfm2_step_symbols_are_exported_and_bound():
+    from wick_amd import lfm2
+
+    names = declared_symbols("wick_rocm_lfm2.h", "wick_rocm_")
+    lib = wick_amd.load_library()
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in wick_rocm_lfm2.h but not exported"
+    assert sorted(lfm2._SIGNATURES) == names
+
+
 def test_static_library_is_built_too():
     """What a Rust build.rs would link (cargo:rustc-link-lib=static=wick_rocm)."""
     assert os.path.exists(os.path.join(ROOT, "wick_amd", "lib", "libwick_rocm.a"))

@@ -1,0 +1,176 @@
+"""The decode step's non-matmul operations on the GPU against the oracle (wick/src/backend/cpu.rs:577-731,
+1320-1401, 2113-2161; wick/src/model/lfm2.rs:621-726).  Bit-exact where the kernel keeps the reference's
+operation order (embedding rows, SiLU gate, short conv, attention scores, argmax); within a stated
+tolerance where a sum is taken in another order or sin/cos come from the device library."""
+import numpy as np
+import pytest
+
+import wick_amd as W
+from oracle import lfm2_oracle as L
+from wick_amd.lfm2 import Lfm2Ops, rope_theta_scale
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def ops(ctx):
+    return Lfm2Ops(ctx)
+
+
+def bits(a):
+    return np.asarray(a, np.float32).view(np.uint32)
+
+
+def max_ulp(a, b):
+    a = np.asarray(a, np.float32).view(np.int32).astype(np.int64)
+    b = np.asarray(b, np.float32).view(np.int32).astype(np.int64)
+    return int(np.abs(a - b).max())
+
+
+@pytest.mark.parametrize("dtype,k", [(W.Q4_0, 256), (W.Q8_0, 1024), (W.Q6_K, 512), (W.Q6_K, 1024)])
+def test_embed_row(ctx, ops, oracle, dtype, k):
+    m = 77
+    wb = oracle.synth_weight(dtype, m, k, seed=k + dtype)
+    w = ctx.upload_weight(wb, dtype, m, k)
+    d_out, d_tok = ctx.alloc(k * 4), ctx.to_device(np.array([m - 1], np.uint32))
+    for token in (0, 13, m - 1):
+        ops.embed_row(w, d_out, token)
+        assert np.array_equal(bits(d_out.download(np.float32, k)), bits(L.embed_row(dtype, wb, token, k)))
+    ops.embed_row(w, d_out, 0, d_token=d_tok)  # device-side token wins over the by-value one
+    assert np.array_equal(bits(d_out.download(np.float32, k)), bits(L.embed_row(dtype, wb, m - 1, k)))
+    with pytest.raises(W.RocmError):
+        ops.embed_row(w, d_out, m)
+    w.free(), d_out.free(), d_tok.free()
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 4), (1, 1024), (1, 2048), (16, 64), (3, 100), (1, 5000)])
+def test_rmsnorm(ctx, ops, oracle, rows, dim):
+    x = oracle.fill_normal(rows * dim, 1.5, rows * dim)
+    w = 1.0 + 0.3 * oracle.fill_normal(dim, 1.0, dim)
+    d_x, d_w, d_y = ctx.to_device(x), ctx.to_device(w), ctx.alloc(rows * dim * 4)
+    ops.encode_rmsnorm(d_x, d_w, d_y, dim, 1e-5, rows=rows)
+    y = d_y.download(np.float32, rows * dim).reshape(rows, dim)
+    ref = np.stack([L.rmsnorm(x[r * dim:(r + 1) * dim], w, 1e-5) for r in range(rows)])
+    # the f64 sum of squares is taken in another order: inv_rms may differ in its last bit
+    assert max_ulp(y, ref) <= 2
+    ops.encode_rmsnorm(d_x, d_w, d_x, dim, 1e-5, rows=rows)  # in place
+    assert np.array_equal(d_x.download(np.float32, rows * dim).reshape(rows, dim), y)
+    for b in (d_x, d_w, d_y):
+        b.free()
+
+
+def test_rmsnorm_reference_closed_forms(ctx, ops):
+    d_x, d_w, d_y = ctx.to_device(np.array([1, 2, 3, 4], np.float32)), ctx.to_device(np.ones(4, np.float32)), ctx.alloc(16)
+    ops.encode_rmsnorm(d_x, d_w, d_y, 4, 1e-5)  # wick/src/backend/cpu.rs:2278-2295
+    assert np.allclose(d_y.download(np.float32, 4), np.array([1, 2, 3, 4]) / np.sqrt(7.5 + 1e-5), atol=1e-6)
+    for b in (d_x, d_w, d_y):
+        b.free()
+
+
+@pytest.mark.parametrize("n", [1, 255, 4608, 10000])
+def test_silu_mul_bit_exact(ctx, ops, oracle, n):
+    g = oracle.fill_normal(n + 1, 4.0, n)
+    g[: min(n, 8)] = np.array([0.0, -0.0, 90.0, -90.0, 104.0, -104.0, 1e-30, -200.0], np.float32)[: min(n, 8)]  # every range branch of expf
+    u = oracle.fill_normal(n + 2, 1.0, n)
+    d_g, d_u = ctx.to_device(g), ctx.to_device(u)
+    ops.silu_mul_inplace(d_g, d_u, n)
+    assert np.array_equal(bits(d_g.download(np.float32, n)), bits(L.silu_mul(g, u)))
+    d_g.free(), d_u.free()
+
+
+@pytest.mark.parametrize("hidden,kernel", [(96, 3), (1024, 3), (300, 4), (64, 2), (128, 1)])
+def test_shortconv_steps_bit_exact(ctx, ops, oracle, hidden, kernel):
+    w = oracle.fill_normal(kernel, 0.5, hidden * kernel)
+    buf = np.zeros(max(kernel - 1, 1) * hidden, np.float32)
+    d_w, d_buf, d_out = ctx.to_device(w), ctx.to_device(buf), ctx.alloc(hidden * 4)
+    ref_buf = np.zeros((kernel - 1) * hidden, np.float32)
+    for step in range(5):
+        proj = oracle.fill_normal(100 + step, 1.0, 3 * hidden)
+        d_proj = ctx.to_device(proj)
+        ops.encode_conv1d_fused(d_proj, d_buf, d_w, d_out, hidden, kernel)
+        ref = L.shortconv_step(proj, ref_buf, w, hidden, kernel)
+        assert np.array_equal(bits(d_out.download(np.float32, hidden)), bits(ref))
+        if kernel > 1:
+            assert np.array_equal(bits(d_buf.download(np.float32, (kernel - 1) * hidden)), bits(ref_buf))
+        d_proj.free()
+    for b in (d_w, d_buf, d_out):
+        b.free()
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,pos", [(4, 2, 64, 0), (16, 8, 64, 5), (8, 8, 32, 300), (4, 1, 128, 4095), (2, 2, 256, 17)])
+def test_qk_norm_rope_and_append(ctx, ops, oracle, n_heads, n_kv, hd, pos):
+    max_seq, eps, base = 4096, 1e-5, 1_000_000.0
+    kv_dim = n_kv * hd
+    q, k, v = oracle.fill_normal(1, 1.0, n_heads * hd), oracle.fill_normal(2, 1.0, kv_dim), oracle.fill_normal(3, 1.0, kv_dim)
+    qn, kn = 1 + 0.2 * oracle.fill_normal(4, 1.0, hd), 1 + 0.2 * oracle.fill_normal(5, 1.0, hd)
+    d = {n: ctx.to_device(a) for n, a in dict(q=q, k=k, v=v, qn=qn, kn=kn).items()}
+    d_kc, d_vc = ctx.to_device(np.full(max_seq * kv_dim, 7.0, np.float32)), ctx.to_device(np.full(max_seq * kv_dim, 7.0, np.float32))
+    ts = rope_theta_scale(hd, base)
+    assert ts == L.rope_theta_scale(hd, base)
+    ops.encode_qk_norm_rope(d["q"], d["k"], d["v"], d["qn"], d["kn"], d_kc, d_vc, pos, max_seq, hd, n_heads, n_kv, eps, ts)
+    qr = np.concatenate([L.rmsnorm(q[h * hd:(h + 1) * hd], qn, eps) for h in range(n_heads)])
+    kr = np.concatenate([L.rmsnorm(k[h * hd:(h + 1) * hd], kn, eps) for h in range(n_kv)])
+    qr, kr = L.rope(qr, kr, pos, n_heads, n_kv, hd, base)
+    got_q, got_k = d["q"].download(np.float32, n_heads * hd), d["k"].download(np.float32, kv_dim)
+    # sin/cos of the device library vs libm (an ulp or two of a value <= 1) on top of the norm's last-bit freedom
+    assert np.allclose(got_q, qr, rtol=0, atol=2e-6 * np.abs(qr).max()) and np.allclose(got_k, kr, rtol=0, atol=2e-6 * np.abs(kr).max())
+    kc = d_kc.download(np.float32, max_seq * kv_dim).reshape(max_seq, kv_dim)
+    vc = d_vc.download(np.float32, max_seq * kv_dim).reshape(max_seq, kv_dim)
+    assert np.array_equal(bits(kc[pos]), bits(got_k)) and np.array_equal(bits(vc[pos]), bits(v))
+    untouched = np.ones(max_seq, bool)
+    untouched[pos] = False
+    assert (kc[untouched] == 7.0).all() and (vc[untouched] == 7.0).all()
+    with pytest.raises(W.RocmError):
+        ops.encode_qk_norm_rope(d["q"], d["k"], d["v"], d["qn"], d["kn"], d_kc, d_vc, max_seq, max_seq, hd, n_heads, n_kv, eps, ts)
+    for b in list(d.values()) + [d_kc, d_vc]:
+        b.free()
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,seq", [(4, 2, 64, 1), (16, 8, 64, 10), (16, 8, 64, 257), (8, 2, 64, 1500), (4, 4, 32, 33), (3, 1, 96, 70),
+                                                 (2, 1, 256, 19)])
+def test_attention_decode(ctx, ops, oracle, n_heads, n_kv, hd, seq):
+    max_seq, kv_dim = seq + 3, n_kv * hd
+    q = oracle.fill_normal(seq, 1.0, n_heads * hd)
+    kc, vc = oracle.fill_normal(seq + 1, 1.0, max_seq * kv_dim), oracle.fill_normal(seq + 2, 1.0, max_seq * kv_dim)
+    d_q, d_kc, d_vc = ctx.to_device(q), ctx.to_device(kc), ctx.to_device(vc)
+    d_out, d_sc = ctx.alloc(n_heads * hd * 4), ctx.alloc(n_heads * max_seq * 4)
+    ops.encode_attention(d_q, d_kc, d_vc, d_out, d_sc, seq, max_seq, n_heads, n_kv, hd)
+    got = d_out.download(np.float32, n_heads * hd)
+    ref = L.attention(q, kc[: seq * kv_dim], vc[: seq * kv_dim], n_heads, n_kv, hd, seq)
+    # probabilities: exp bit-exact, their f64 sum in another order; values summed in four interleaved parts
+    assert np.allclose(got, ref, rtol=0, atol=4e-6 * max(np.abs(ref).max(), 1e-3))
+    # the scratch holds the unnormalised exp(score - max): bit-exact against the oracle's scores
+    sc = d_sc.download(np.float32, n_heads * max_seq).reshape(n_heads, max_seq)[:, :seq]
+    scale = np.float32(1.0) / np.sqrt(np.float32(hd))
+    for h in (0, n_heads - 1):
+        s = L.attn_scores(q[h * hd:(h + 1) * hd], kc, kv_dim, (h // (n_heads // n_kv)) * hd, hd, scale, seq)
+        e = np.array([L.ggml_expf(float(np.float32(x) - s.max())) for x in s], np.float32)
+        assert np.array_equal(bits(sc[h]), bits(e))
+    # device-side position: seq_len = *d_pos + 1
+    d_pos = ctx.to_device(np.array([seq - 1], np.uint32))
+    ops.encode_attention(d_q, d_kc, d_vc, d_out, d_sc, 0, max_seq, n_heads, n_kv, hd, d_pos=d_pos)
+    assert np.array_equal(bits(d_out.download(np.float32, n_heads * hd)), bits(got))
+    for b in (d_q, d_kc, d_vc, d_out, d_sc, d_pos):
+        b.free()
+
+
+def test_argmax_rules(ctx, ops):
+    """cpu_argmax (wick/src/sampler.rs:7-19): last of equal maxima, NaN = -inf, -0.0 < +0.0."""
+    cases = [[1.0, 3.0, 2.0], [3.0, 1.0, 3.0, 2.0], [np.nan, 1.0, np.nan], [np.nan, np.nan], [np.nan, -np.inf], [0.0, -0.0], [-0.0, 0.0, -0.0],
+             [-5.0], [-np.inf, -np.inf, -np.inf]]
+    rng = np.random.default_rng(6)
+    cases += [rng.integers(-3, 4, n).astype(np.float32) for n in (1000, 1024, 1025, 65536)]
+    cases += [rng.standard_normal(65536).astype(np.float32)]
+    d_out = ctx.alloc(4)
+    for c in cases:
+        x = np.asarray(c, np.float32)
+        d_x = ctx.to_device(x)
+        ops.argmax(d_x, x.size, d_out)
+        assert int(d_out.download(np.uint32, 1)[0]) == L.argmax(x), c if x.size < 10 else x.size
+        d_x.free()
+    d_tok, d_pos = ctx.to_device(np.array([0], np.uint32)), ctx.to_device(np.array([41], np.uint32))
+    d_x = ctx.to_device(np.array([0.5, 9.0, 1.0], np.float32))
+    ops.argmax(d_x, 3, d_out, d_token=d_tok, d_pos=d_pos)
+    assert d_tok.download(np.uint32, 1)[0] == 1 and d_pos.download(np.uint32, 1)[0] == 42
+    for b in (d_out, d_tok, d_pos, d_x):
+        b.free()

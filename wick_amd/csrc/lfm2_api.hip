@@ -1,0 +1,434 @@
+// C ABI of include/wick_rocm_lfm2.h: the decode step's non-matmul operations as entry points, and the
+// LFM2 model handle (weights, KV caches, conv state, scratch, one captured graph per kind of step).
+// Host code only.  The model is a composition of public entry points (it holds its own lock, like the
+// reference's infer_lock, and never the context's).
+#include "../../include/wick_rocm_lfm2.h"
+
+#include <cmath>
+#include <cstring>
+#include <memory>
+#include <vector>
+
+#include "../../include/wick_gguf.h"
+#include "wick_rocm_ctx.h"
+
+namespace {
+
+bool misaligned(const void* p, size_t a) { return reinterpret_cast<uintptr_t>(p) % a != 0; }
+
+}  // namespace
+
+extern "C" {
+
+int wick_rocm_embed_row(wick_rocm_ctx* ctx, const wick_rocm_weight* w, uint32_t token, const uint32_t* d_token, float* d_out) {
+    WR_ENTER(ctx);
+    if (!w || !w->d || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "embed_row: null argument");
+    if (!d_token && token >= w->m) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "embed_row: token out of range");
+    hipError_t e = launch_embed_row(static_cast<const uint8_t*>(w->d), w->type, w->m, w->k, token, d_token, d_out, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "embed_row launch");
+}
+
+int wick_rocm_rmsnorm(wick_rocm_ctx* ctx, const float* d_x, const float* d_weight, float* d_y, uint32_t rows, uint32_t dim, uint32_t x_stride,
+                      uint32_t y_stride, float eps) {
+    WR_ENTER(ctx);
+    if (!d_x || !d_weight || !d_y) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "rmsnorm: null device pointer");
+    if (dim == 0 || (rows > 1 && (x_stride < dim || y_stride < dim))) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "rmsnorm: dim 0 or stride < dim");
+    hipError_t e = launch_rmsnorm(d_x, d_weight, d_y, rows, dim, x_stride, y_stride, eps, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "rmsnorm launch");
+}
+
+float wick_rocm_rope_theta_scale(uint32_t head_dim, float freq_base) { return powf(freq_base, -2.0f / (float)head_dim); }
+
+int wick_rocm_qk_norm_rope(wick_rocm_ctx* ctx, float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
+                           float* d_k_cache, float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim,
+                           uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale) {
+    WR_ENTER(ctx);
+    if (!d_q || !d_k || !d_v || !d_q_norm || !d_k_norm || !d_k_cache || !d_v_cache)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "qk_norm_rope: null device pointer");
+    if (head_dim == 0 || head_dim % 2u != 0 || head_dim > 256u || n_heads == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "qk_norm_rope: head_dim must be even and <= 256, n_kv_heads must divide n_heads");
+    if (!d_pos && pos >= max_seq) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "qk_norm_rope: pos beyond the cache");
+    hipError_t e = launch_qk_norm_rope(d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, pos, d_pos, max_seq, head_dim, n_heads, n_kv_heads,
+                                       eps, theta_scale, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "qk_norm_rope launch");
+}
+
+int wick_rocm_attention_decode(wick_rocm_ctx* ctx, const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out,
+                               float* d_scores, uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
+                               uint32_t head_dim) {
+    WR_ENTER(ctx);
+    if (!d_q || !d_k_cache || !d_v_cache || !d_out || !d_scores) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention: null device pointer");
+    if (head_dim == 0 || head_dim % 4u != 0 || head_dim > 256u || n_heads == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "attention: head_dim must be a multiple of 4 and <= 256, n_kv_heads must divide n_heads");
+    if (misaligned(d_k_cache, 16)) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention: key cache must be 16-byte aligned");
+    if (!d_pos && seq_len > max_seq) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention: seq_len beyond the cache");
+    const float scale = 1.0f / sqrtf((float)head_dim);  // wick/src/model/lfm2.rs:862
+    hipError_t e = launch_attention_decode(d_q, d_k_cache, d_v_cache, d_out, d_scores, seq_len, d_pos, max_seq, n_heads, n_kv_heads, head_dim, scale,
+                                           ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "attention launch");
+}
+
+int wick_rocm_shortconv_step(wick_rocm_ctx* ctx, const float* d_proj, float* d_buffer, const float* d_conv_weight, float* d_out, uint32_t hidden,
+                             uint32_t kernel_size) {
+    WR_ENTER(ctx);
+    if (!d_proj || !d_conv_weight || !d_out || (!d_buffer && kernel_size > 1)) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "shortconv: null device pointer");
+    if (hidden == 0 || kernel_size == 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "shortconv: hidden and kernel_size must be > 0");
+    hipError_t e = launch_shortconv_step(d_proj, d_buffer, d_conv_weight, d_out, hidden, kernel_size, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "shortconv launch");
+}
+
+int wick_rocm_silu_mul(wick_rocm_ctx* ctx, float* d_gate, const float* d_up, uint32_t n) {
+    WR_ENTER(ctx);
+    if (!d_gate || !d_up) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "silu_mul: null device pointer");
+    hipError_t e = launch_silu_mul(d_gate, d_up, n, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "silu_mul launch");
+}
+
+int wick_rocm_argmax(wick_rocm_ctx* ctx, const float* d_logits, uint32_t n, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos) {
+    WR_ENTER(ctx);
+    if (!d_logits || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "argmax: null device pointer");
+    hipError_t e = launch_argmax(d_logits, n, d_out, d_token, d_pos, nullptr, 0, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------------------
+// The model.
+
+namespace {
+
+struct LayerWeights {
+    uint32_t n_kv = 0;  // 0: gated-conv layer
+    wick_rocm_weight *in_proj = nullptr, *out_proj = nullptr;               // conv
+    wick_rocm_weight *q = nullptr, *k = nullptr, *v = nullptr, *o = nullptr;  // attention
+    wick_rocm_weight *gate = nullptr, *up = nullptr, *down = nullptr;
+    float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr, *conv_w = nullptr;
+    float *k_cache = nullptr, *v_cache = nullptr, *conv_state = nullptr;
+};
+
+}  // namespace
+
+struct wick_rocm_lfm2 {
+    wick_rocm_lfm2_config cfg{};
+    std::vector<LayerWeights> layers;
+    wick_rocm_weight* embd = nullptr;
+    float* out_norm = nullptr;
+    std::vector<wick_rocm_weight*> weights;  // everything uploaded, for release
+    std::vector<void*> buffers;              // every device buffer, for release
+    size_t bytes = 0;
+    float theta_scale = 0.0f;
+    // step scratch (device)
+    float *hidden = nullptr, *normed = nullptr, *proj = nullptr, *gated = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr,
+          *gate = nullptr, *up = nullptr, *scores = nullptr, *final_hidden = nullptr, *logits = nullptr;
+    uint32_t *d_token = nullptr, *d_pos = nullptr, *d_pick = nullptr, *d_history = nullptr;
+    wick_rocm_graph *g_logits = nullptr, *g_greedy = nullptr;
+    std::mutex mu;
+};
+
+namespace {
+
+int ctx_fail(wick_rocm_ctx* ctx, int code, const std::string& what) {
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    return fail(ctx, code, what.c_str());
+}
+
+int alloc(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, size_t nbytes, void** out) {
+    if (int rc = wick_rocm_buffer_alloc(ctx, nbytes, out)) return rc;
+    m->buffers.push_back(*out);
+    m->bytes += nbytes;
+    return WICK_ROCM_OK;
+}
+
+template <typename T>
+int alloc_t(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, size_t count, T** out) {
+    return alloc(ctx, m, count * sizeof(T), reinterpret_cast<void**>(out));
+}
+
+// An f32 tensor of exactly `count` elements -> device buffer (the reference's get_tensor(..).to_f32_vec()).
+int upload_f32(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, const wick_gguf* g, const std::string& name, uint64_t count, float** out) {
+    int type = 0;
+    uint32_t nd = 0;
+    uint64_t dims[8], off = 0, size = 0;
+    if (wick_gguf_tensor_info(g, name.c_str(), &type, &nd, dims, &off, &size) != 0)
+        return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, std::string("lfm2_load: ") + wick_gguf_last_error());
+    if (type != 0) return ctx_fail(ctx, WICK_ROCM_ERR_UNSUPPORTED_DTYPE, "lfm2_load: " + name + " must be F32");
+    if (size != count * 4) return ctx_fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "lfm2_load: " + name + " has an unexpected element count");
+    const void* data = nullptr;
+    size_t nbytes = 0;
+    if (wick_gguf_tensor_data(g, name.c_str(), &data, &nbytes) != 0)
+        return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, std::string("lfm2_load: ") + wick_gguf_last_error());
+    if (int rc = alloc_t(ctx, m, count, out)) return rc;
+    return wick_rocm_upload(ctx, *out, data, nbytes);
+}
+
+int upload_weight(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, const wick_gguf* g, const std::string& name, uint32_t rows, uint32_t cols,
+                  wick_rocm_weight** out) {
+    if (int rc = wick_rocm_weight_from_gguf(ctx, g, name.c_str(), out)) return rc;
+    m->weights.push_back(*out);
+    m->bytes += (*out)->nbytes;
+    if ((*out)->m != rows || (*out)->k != cols)
+        return ctx_fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "lfm2_load: " + name + " has an unexpected shape");
+    return WICK_ROCM_OK;
+}
+
+void release(wick_rocm_ctx* ctx, wick_rocm_lfm2* m) {
+    wick_rocm_sync(ctx);
+    if (m->g_logits) wick_rocm_graph_destroy(ctx, m->g_logits);
+    if (m->g_greedy) wick_rocm_graph_destroy(ctx, m->g_greedy);
+    for (wick_rocm_weight* w : m->weights) wick_rocm_weight_free(ctx, w);
+    for (void* b : m->buffers) wick_rocm_buffer_free(ctx, b);
+    delete m;
+}
+
+// y (+)= W x for 1..3 weights that share x; one launch when their types agree.
+int gemv(wick_rocm_ctx* ctx, std::initializer_list<const wick_rocm_weight*> ws, std::initializer_list<float*> ys, const float* x, int accumulate) {
+    bool same = true;
+    for (const wick_rocm_weight* w : ws) same = same && w->type == (*ws.begin())->type;
+    if (same) return wick_rocm_gemv_f32_multi(ctx, ws.begin(), ys.begin(), (uint32_t)ws.size(), x, 0, accumulate);
+    auto y = ys.begin();
+    for (const wick_rocm_weight* w : ws) {
+        if (int rc = wick_rocm_matmul_f32(ctx, w, x, 0, 1, w->k, *y++, 0, w->m, accumulate)) return rc;
+    }
+    return WICK_ROCM_OK;
+}
+
+// Enqueues one decode step that reads token / pos from the device: run_layers + the tied LM head
+// (wick/src/model/lfm2.rs:1020-1124, 2258-2289), optionally the greedy pick.
+int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
+    const wick_rocm_lfm2_config& c = m->cfg;
+    const uint32_t hs = c.hidden_size, hd = hs / c.n_heads;
+    int rc = wick_rocm_embed_row(ctx, m->embd, 0, m->d_token, m->hidden);
+    for (uint32_t i = 0; rc == 0 && i < c.n_layers; i++) {
+        const LayerWeights& L = m->layers[i];
+        rc = wick_rocm_rmsnorm(ctx, m->hidden, L.attn_norm, m->normed, 1, hs, hs, hs, c.rms_norm_eps);
+        if (rc) break;
+        if (L.n_kv == 0) {
+            if ((rc = gemv(ctx, {L.in_proj}, {m->proj}, m->normed, 0))) break;
+            if ((rc = wick_rocm_shortconv_step(ctx, m->proj, L.conv_state, L.conv_w, m->gated, hs, c.conv_kernel_size))) break;
+            if ((rc = gemv(ctx, {L.out_proj}, {m->hidden}, m->gated, 1))) break;  // hidden += out_proj(gated)
+        } else {
+            if ((rc = gemv(ctx, {L.q, L.k, L.v}, {m->q, m->k, m->v}, m->normed, 0))) break;
+            if ((rc = wick_rocm_qk_norm_rope(ctx, m->q, m->k, m->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, 0, m->d_pos, c.max_seq_len, hd, c.n_heads,
+                                             L.n_kv, c.rms_norm_eps, m->theta_scale)))
+                break;
+            if ((rc = wick_rocm_attention_decode(ctx, m->q, L.k_cache, L.v_cache, m->attn, m->scores, 0, m->d_pos, c.max_seq_len, c.n_heads, L.n_kv, hd)))
+                break;
+            if ((rc = gemv(ctx, {L.o}, {m->hidden}, m->attn, 1))) break;
+        }
+        if ((rc = wick_rocm_rmsnorm(ctx, m->hidden, L.ffn_norm, m->normed, 1, hs, hs, hs, c.rms_norm_eps))) break;
+        if ((rc = gemv(ctx, {L.gate, L.up}, {m->gate, m->up}, m->normed, 0))) break;
+        if ((rc = wick_rocm_silu_mul(ctx, m->gate, m->up, c.intermediate_size))) break;
+        rc = gemv(ctx, {L.down}, {m->hidden}, m->gate, 1);
+    }
+    if (rc) return rc;
+    if ((rc = wick_rocm_rmsnorm(ctx, m->hidden, m->out_norm, m->final_hidden, 1, hs, hs, hs, c.rms_norm_eps))) return rc;
+    if ((rc = gemv(ctx, {m->embd}, {m->logits}, m->final_hidden, 0))) return rc;
+    if (!greedy) return WICK_ROCM_OK;
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    hipError_t e = launch_argmax(m->logits, c.vocab_size, m->d_pick, m->d_token, m->d_pos, m->d_history, c.max_seq_len, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
+}
+
+int step_graph(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy, wick_rocm_graph** out) {
+    wick_rocm_graph*& g = greedy ? m->g_greedy : m->g_logits;
+    if (!g) {
+        if (int rc = wick_rocm_graph_begin(ctx)) return rc;
+        const int rc = enqueue_step(ctx, m, greedy);
+        wick_rocm_graph* captured = nullptr;
+        const int rc_end = wick_rocm_graph_end(ctx, &captured);  // always end the capture
+        if (rc) {
+            if (captured) wick_rocm_graph_destroy(ctx, captured);
+            return rc;
+        }
+        if (rc_end) return rc_end;
+        g = captured;
+    }
+    *out = g;
+    return WICK_ROCM_OK;
+}
+
+int set_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t token, uint32_t pos) {
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    hipError_t e = launch_set_step(m->d_token, token, m->d_pos, pos, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "set_step launch");
+}
+
+int check_step(wick_rocm_ctx* ctx, const wick_rocm_lfm2* m, uint32_t token, uint32_t pos, uint32_t n) {
+    if (token >= m->cfg.vocab_size) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: token_id out of range");
+    if ((uint64_t)pos + n > m->cfg.max_seq_len) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: position beyond the context size");
+    return WICK_ROCM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int wick_rocm_lfm2_load(wick_rocm_ctx* ctx, const wick_gguf* g, uint32_t context_size, wick_rocm_lfm2** out) {
+    if (!ctx) return WICK_ROCM_ERR_INVALID_ARG;
+    if (!g || !out) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2_load: null argument");
+    *out = nullptr;
+    if (context_size == 0) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2_load: context_size must be > 0");
+
+    // metadata, wick/src/model/lfm2.rs:104-136
+    wick_rocm_lfm2_config c{};
+    struct Key {
+        const char* name;
+        uint32_t* dst;
+    } required[] = {{"lfm2.block_count", &c.n_layers},
+                    {"lfm2.embedding_length", &c.hidden_size},
+                    {"lfm2.feed_forward_length", &c.intermediate_size},
+                    {"lfm2.attention.head_count", &c.n_heads},
+                    {"lfm2.vocab_size", &c.vocab_size}};
+    for (const Key& k : required)
+        if (wick_gguf_get_u32(g, k.name, k.dst) != 0) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, std::string("lfm2_load: missing ") + k.name);
+    uint32_t ctx_len = 128000, l_cache = 3;
+    wick_gguf_get_u32(g, "lfm2.context_length", &ctx_len);
+    c.max_seq_len = context_size < ctx_len ? context_size : ctx_len;
+    c.rope_theta = 1000000.0f, c.rms_norm_eps = 1e-5f;
+    wick_gguf_get_f32(g, "lfm2.rope.freq_base", &c.rope_theta);
+    wick_gguf_get_f32(g, "lfm2.attention.layer_norm_rms_epsilon", &c.rms_norm_eps);
+    wick_gguf_get_u32(g, "lfm2.shortconv.l_cache", &l_cache);  // kernel size, default 3 (wick/src/model/lfm2.rs:650)
+    c.conv_kernel_size = l_cache;
+    const void* kv_data = nullptr;
+    uint64_t kv_count = 0;
+    if (wick_gguf_get_array(g, "lfm2.attention.head_count_kv", WICK_GGUF_T_I32, &kv_data, &kv_count) != 0)
+        return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2_load: missing lfm2.attention.head_count_kv");
+    if (kv_count < c.n_layers) return ctx_fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "lfm2_load: head_count_kv array shorter than block_count");
+    if (c.n_layers == 0 || c.hidden_size == 0 || c.n_heads == 0 || c.hidden_size % c.n_heads != 0 || c.vocab_size == 0 || c.conv_kernel_size == 0 ||
+        c.intermediate_size == 0)
+        return ctx_fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "lfm2_load: degenerate model dimensions");
+    const uint32_t hs = c.hidden_size, hd = hs / c.n_heads, inter = c.intermediate_size;
+    if (hd % 4u != 0 || hd > 256u) return ctx_fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "lfm2_load: head_dim must be a multiple of 4 and <= 256");
+
+    std::unique_ptr<wick_rocm_lfm2> holder(new wick_rocm_lfm2);
+    wick_rocm_lfm2* m = holder.get();
+    auto bail = [&](int rc) {
+        release(ctx, holder.release());
+        return rc;
+    };
+    m->layers.resize(c.n_layers);
+    int rc = 0;
+    // block types from tensor presence, wick/src/model/lfm2.rs:151-170
+    for (uint32_t i = 0; i < c.n_layers; i++) {
+        const std::string p = "blk." + std::to_string(i) + ".";
+        LayerWeights& L = m->layers[i];
+        const bool is_attn = wick_gguf_tensor_info(g, (p + "attn_q.weight").c_str(), nullptr, nullptr, nullptr, nullptr, nullptr) == 0;
+        if (is_attn) {
+            int32_t n_kv;
+            memcpy(&n_kv, static_cast<const uint8_t*>(kv_data) + 4 * i, 4);
+            if (n_kv <= 0 || c.n_heads % (uint32_t)n_kv != 0)
+                return bail(ctx_fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "lfm2_load: layer " + std::to_string(i) + ": n_kv_heads must be > 0 and divide n_heads"));
+            L.n_kv = (uint32_t)n_kv;
+            c.n_kv_heads = L.n_kv > c.n_kv_heads ? L.n_kv : c.n_kv_heads;
+        }
+        if ((rc = upload_f32(ctx, m, g, p + "attn_norm.weight", hs, &L.attn_norm))) return bail(rc);
+        if ((rc = upload_f32(ctx, m, g, p + "ffn_norm.weight", hs, &L.ffn_norm))) return bail(rc);
+        if (is_attn) {
+            const uint32_t kv_dim = L.n_kv * hd;
+            if ((rc = upload_f32(ctx, m, g, p + "attn_q_norm.weight", hd, &L.q_norm))) return bail(rc);
+            if ((rc = upload_f32(ctx, m, g, p + "attn_k_norm.weight", hd, &L.k_norm))) return bail(rc);
+            if ((rc = upload_weight(ctx, m, g, p + "attn_q.weight", hs, hs, &L.q))) return bail(rc);
+            if ((rc = upload_weight(ctx, m, g, p + "attn_k.weight", kv_dim, hs, &L.k))) return bail(rc);
+            if ((rc = upload_weight(ctx, m, g, p + "attn_v.weight", kv_dim, hs, &L.v))) return bail(rc);
+            if ((rc = upload_weight(ctx, m, g, p + "attn_output.weight", hs, hs, &L.o))) return bail(rc);
+            if ((rc = alloc_t(ctx, m, (size_t)c.max_seq_len * kv_dim, &L.k_cache))) return bail(rc);
+            if ((rc = alloc_t(ctx, m, (size_t)c.max_seq_len * kv_dim, &L.v_cache))) return bail(rc);
+        } else {
+            if ((rc = upload_f32(ctx, m, g, p + "shortconv.conv.weight", (uint64_t)hs * c.conv_kernel_size, &L.conv_w))) return bail(rc);
+            if ((rc = upload_weight(ctx, m, g, p + "shortconv.in_proj.weight", 3 * hs, hs, &L.in_proj))) return bail(rc);
+            if ((rc = upload_weight(ctx, m, g, p + "shortconv.out_proj.weight", hs, hs, &L.out_proj))) return bail(rc);
+            if (c.conv_kernel_size > 1 && (rc = alloc_t(ctx, m, (size_t)(c.conv_kernel_size - 1) * hs, &L.conv_state))) return bail(rc);
+        }
+        if ((rc = upload_weight(ctx, m, g, p + "ffn_gate.weight", inter, hs, &L.gate))) return bail(rc);
+        if ((rc = upload_weight(ctx, m, g, p + "ffn_up.weight", inter, hs, &L.up))) return bail(rc);
+        if ((rc = upload_weight(ctx, m, g, p + "ffn_down.weight", hs, inter, &L.down))) return bail(rc);
+    }
+    if ((rc = upload_f32(ctx, m, g, "token_embd_norm.weight", hs, &m->out_norm))) return bail(rc);
+    if ((rc = upload_weight(ctx, m, g, "token_embd.weight", c.vocab_size, hs, &m->embd))) return bail(rc);
+
+    const uint32_t kv_max = (c.n_kv_heads ? c.n_kv_heads : 1) * hd;
+    if ((rc = alloc_t(ctx, m, hs, &m->hidden)) || (rc = alloc_t(ctx, m, hs, &m->normed)) || (rc = alloc_t(ctx, m, 3 * (size_t)hs, &m->proj)) ||
+        (rc = alloc_t(ctx, m, hs, &m->gated)) || (rc = alloc_t(ctx, m, hs, &m->q)) || (rc = alloc_t(ctx, m, kv_max, &m->k)) ||
+        (rc = alloc_t(ctx, m, kv_max, &m->v)) || (rc = alloc_t(ctx, m, hs, &m->attn)) || (rc = alloc_t(ctx, m, inter, &m->gate)) ||
+        (rc = alloc_t(ctx, m, inter, &m->up)) || (rc = alloc_t(ctx, m, (size_t)c.n_heads * c.max_seq_len, &m->scores)) ||
+        (rc = alloc_t(ctx, m, hs, &m->final_hidden)) || (rc = alloc_t(ctx, m, c.vocab_size, &m->logits)) || (rc = alloc_t(ctx, m, 1, &m->d_token)) ||
+        (rc = alloc_t(ctx, m, 1, &m->d_pos)) || (rc = alloc_t(ctx, m, 1, &m->d_pick)) || (rc = alloc_t(ctx, m, c.max_seq_len, &m->d_history)))
+        return bail(rc);
+    // GEMVs that cannot take the fused-quantizer kernel quantize into the context's scratch: size it before any capture
+    if ((rc = wick_rocm_reserve_scratch(ctx, 1, hs > inter ? hs : inter))) return bail(rc);
+    m->cfg = c;
+    m->theta_scale = wick_rocm_rope_theta_scale(hd, c.rope_theta);
+    if ((rc = wick_rocm_lfm2_reset(ctx, m))) return bail(rc);
+    if ((rc = wick_rocm_sync(ctx))) return bail(rc);  // uploads read the GGUF image: done before the caller may close it
+    *out = holder.release();
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_lfm2_free(wick_rocm_ctx* ctx, wick_rocm_lfm2* model) {
+    if (!ctx) return WICK_ROCM_ERR_INVALID_ARG;
+    if (model) release(ctx, model);
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_lfm2_get_config(const wick_rocm_lfm2* model, wick_rocm_lfm2_config* out) {
+    if (!model || !out) return WICK_ROCM_ERR_INVALID_ARG;
+    *out = model->cfg;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_lfm2_layer_kv_heads(const wick_rocm_lfm2* model, uint32_t layer, uint32_t* n_kv_heads) {
+    if (!model || !n_kv_heads || layer >= model->cfg.n_layers) return WICK_ROCM_ERR_INVALID_ARG;
+    *n_kv_heads = model->layers[layer].n_kv;
+    return WICK_ROCM_OK;
+}
+
+size_t wick_rocm_lfm2_gpu_memory_bytes(const wick_rocm_lfm2* model) { return model ? model->bytes : 0; }
+
+int wick_rocm_lfm2_reset(wick_rocm_ctx* ctx, wick_rocm_lfm2* model) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lk(model->mu);
+    const size_t state_floats = (size_t)(model->cfg.conv_kernel_size - 1) * model->cfg.hidden_size;
+    if (state_floats) {
+        const std::vector<float> zeros(state_floats, 0.0f);
+        for (const LayerWeights& L : model->layers)
+            if (L.conv_state)
+                if (int rc = wick_rocm_upload(ctx, L.conv_state, zeros.data(), state_floats * sizeof(float))) return rc;
+    }
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_lfm2_forward(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t token, uint32_t pos, float* logits) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lk(model->mu);
+    if (int rc = check_step(ctx, model, token, pos, 1)) return rc;
+    wick_rocm_graph* g = nullptr;
+    if (int rc = step_graph(ctx, model, false, &g)) return rc;
+    if (int rc = set_step(ctx, model, token, pos)) return rc;
+    if (int rc = wick_rocm_graph_launch(ctx, g)) return rc;
+    if (logits) return wick_rocm_download(ctx, logits, model->logits, (size_t)model->cfg.vocab_size * sizeof(float));
+    return wick_rocm_sync(ctx);
+}
+
+int wick_rocm_lfm2_forward_greedy(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t token, uint32_t pos, uint32_t* next_token) {
+    return wick_rocm_lfm2_generate_greedy(ctx, model, token, pos, 1, next_token);
+}
+
+int wick_rocm_lfm2_generate_greedy(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t token, uint32_t pos, uint32_t n, uint32_t* out_tokens) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    if (!out_tokens) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: null output pointer");
+    if (n == 0) return WICK_ROCM_OK;
+    std::lock_guard<std::mutex> lk(model->mu);
+    if (int rc = check_step(ctx, model, token, pos, n)) return rc;
+    wick_rocm_graph* g = nullptr;
+    if (int rc = step_graph(ctx, model, true, &g)) return rc;
+    if (int rc = set_step(ctx, model, token, pos)) return rc;
+    for (uint32_t i = 0; i < n; i++)  // the pick of step i is written to the device-side token and position pos + i of the history
+        if (int rc = wick_rocm_graph_launch(ctx, g)) return rc;
+    return wick_rocm_download(ctx, out_tokens, model->d_history + pos, (size_t)n * sizeof(uint32_t));
+}
+
+const float* wick_rocm_lfm2_logits_device(const wick_rocm_lfm2* model) { return model ? model->logits : nullptr; }
+const float* wick_rocm_lfm2_hidden_device(const wick_rocm_lfm2* model) { return model ? model->final_hidden : nullptr; }
+
+}  // extern "C"

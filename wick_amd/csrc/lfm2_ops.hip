@@ -1,0 +1,390 @@
+// The non-matmul operations of one LFM2 decode step for gfx950: embedding-row dequantization,
+// RMSNorm, per-head QK-norm + RoPE + KV append, decode attention, the gated short convolution,
+// SiLU-gate and the greedy pick.  Arithmetic follows the reference's CPU operations
+// (wick/src/backend/cpu.rs:577-731, 1320-1401, 2113-2161; wick/src/model/lfm2.rs:621-726);
+// each kernel says which steps reproduce them bit for bit and which only to rounding.
+//
+// Every product / sum that the reference computes as separate f32 operations uses
+// __fmul_rn / __fadd_rn / __fsub_rn / __fdiv_rn here: the translation unit is compiled with
+// contraction on, and a fused multiply-add would round differently.
+//
+// "pos" and "token" may live in device memory (d_pos / d_token non-null): a captured graph of
+// the step can then be replayed for every token without new kernel arguments.
+#include "wick_rocm_device.h"
+#include "wick_rocm_internal.h"
+
+namespace wick_rocm {
+
+namespace {
+
+__device__ __forceinline__ float bits_f(uint32_t u) { return __uint_as_float(u); }
+
+// ggml_expf (wick/src/backend/cpu.rs:604-652), operation for operation: bit-exact.
+__device__ __forceinline__ float ggml_expf(float x) {
+    const float R = bits_f(0x4B400000u), LOG2E = bits_f(0x3FB8AA3Bu);
+    const float LN2_HI = bits_f(0x3F317200u), LN2_LO = bits_f(0x35BFBE8Eu);
+    const float C1 = bits_f(0x3F7FFFF6u), C2 = bits_f(0x3EFFFEDBu), C3 = bits_f(0x3E2AAF33u);
+    const float C4 = bits_f(0x3D2B9F17u), C5 = bits_f(0x3C072010u);
+    const float z = __fadd_rn(R, __fmul_rn(x, LOG2E));
+    const float n = __fsub_rn(z, R);
+    const float b = __fsub_rn(__fsub_rn(x, __fmul_rn(n, LN2_HI)), __fmul_rn(n, LN2_LO));
+    const uint32_t e = __float_as_uint(z) << 23;
+    const float k = bits_f(e + 0x3F800000u);
+    const float u = __fmul_rn(b, b);
+    const float inner = __fadd_rn(__fadd_rn(C2, __fmul_rn(C3, b)), __fmul_rn(__fadd_rn(C4, __fmul_rn(C5, b)), u));
+    const float j = __fadd_rn(__fmul_rn(C1, b), __fmul_rn(inner, u));
+    const float abs_n = fabsf(n);
+    if (abs_n <= 126.0f) return __fadd_rn(k, __fmul_rn(j, k));
+    if (abs_n > 192.0f) return n > 0.0f ? __builtin_inff() : 0.0f;
+    const uint32_t d = n <= 0.0f ? 0x82000000u : 0u;
+    const float s1 = bits_f(d + 0x7f000000u);
+    const float s2 = bits_f(e - d);
+    return __fmul_rn(__fadd_rn(s2, __fmul_rn(s2, j)), s1);
+}
+
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// Sum over a block of up to 16 waves; every thread gets the total.  `slots` holds 16 doubles.
+__device__ __forceinline__ double block_sum_f64(double v, double* slots) {
+    v = wave_sum_f64(v);
+    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();  // slots may still be read from an earlier call
+    if ((threadIdx.x & 63) == 0) slots[wave] = v;
+    __syncthreads();
+    double t = 0.0;
+    for (int i = 0; i < nw; i++) t += slots[i];
+    return t;
+}
+
+// ---- embedding row -------------------------------------------------------------------
+// dequantize_row_into (wick/src/model/lfm2.rs:621-643) for Q4_0 / Q8_0 (quant.rs:78-90, 154-161) and
+// Q6_K (quant.rs:380-412: d * sc * q left to right): bit-exact.
+__global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restrict__ w, int type, uint32_t m, uint32_t k, uint32_t token,
+                                                        const uint32_t* __restrict__ d_token, float* __restrict__ out) {
+    const uint32_t row = d_token ? *d_token : token;
+    if (row >= m) return;  // the host checks a by-value token; a device-side token out of range leaves `out` untouched
+    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < k; e += gridDim.x * blockDim.x) {
+        float v;
+        if (type == kTypeQ6_K) {
+            const uint8_t* blk = w + ((size_t)row * (k >> 8) + (e >> 8)) * kQ6KBlockBytes;
+            const uint32_t i = e & 255u, n = i >> 7, j = (i >> 5) & 3u, l = i & 31u;
+            const uint32_t lo = (blk[64 * n + 32 * (j & 1u) + l] >> (4 * (j >> 1))) & 15u;
+            const uint32_t hi = (blk[128 + 32 * n + l] >> (2 * j)) & 3u;
+            const int q = (int)(lo | (hi << 4)) - 32;
+            const float d = f16_bits_to_f32((uint32_t)blk[208] | ((uint32_t)blk[209] << 8));
+            const float sc = (float)(int)(int8_t)blk[192 + (i >> 4)];
+            v = __fmul_rn(__fmul_rn(d, sc), (float)q);
+        } else if (type == kTypeQ4_0) {
+            const uint8_t* blk = w + ((size_t)row * (k >> 5) + (e >> 5)) * kQ4BlockBytes;
+            const uint32_t i = e & 31u;
+            const uint32_t byte = blk[2 + (i & 15u)];
+            const int q = (int)((i < 16u) ? (byte & 15u) : (byte >> 4)) - 8;
+            v = __fmul_rn((float)q, f16_bits_to_f32((uint32_t)blk[0] | ((uint32_t)blk[1] << 8)));
+        } else {
+            const uint8_t* blk = w + ((size_t)row * (k >> 5) + (e >> 5)) * kQ8BlockBytes;
+            v = __fmul_rn((float)(int)(int8_t)blk[2 + (e & 31u)], f16_bits_to_f32((uint32_t)blk[0] | ((uint32_t)blk[1] << 8)));
+        }
+        out[e] = v;
+    }
+}
+
+// ---- RMSNorm ---------------------------------------------------------------------------
+// rmsnorm (wick/src/backend/cpu.rs:577-594): f64 sum of squares (summed in another order than the
+// reference's loop: the f64 total can differ in its last bits, inv_rms as f32 almost never), then the
+// reference's two f32 products.  One block per row; `weight` is shared by all rows.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ weight, float* __restrict__ y,
+                                                      uint32_t dim, uint32_t x_stride, uint32_t y_stride, float eps) {
+    __shared__ double slots[16];
+    const float* xr = x + (size_t)blockIdx.x * x_stride;
+    float* yr = y + (size_t)blockIdx.x * y_stride;
+    double s = 0.0;
+    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
+        const double v = (double)xr[i];
+        s += v * v;
+    }
+    const double total = block_sum_f64(s, slots);
+    const float inv_rms = (float)(1.0 / sqrt(total / (double)dim + (double)eps));
+    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) yr[i] = __fmul_rn(__fmul_rn(xr[i], inv_rms), weight[i]);
+}
+
+// ---- per-head QK-norm + RoPE + KV append ----------------------------------------------------
+// forward_attn_block's middle (wick/src/model/lfm2.rs:783-857): every Q and K head is RMS-normalised with
+// the shared per-layer weights, rotated (apply_rope_to_head, cpu.rs:2148-2161: split halves, theta
+// multiplied up in f32 -- reproduced exactly -- sin/cos from the device library, within an ulp or two
+// of libm's), and K / V of this position are appended to the caches [t][kv_dim].
+// One 64-thread block per head: blocks [0, n_heads) are Q heads, the rest K heads (which also copy V).
+struct QkNormRopeArgs {
+    float* q;               // [n_heads * head_dim], in place
+    float* k;               // [n_kv_heads * head_dim], in place
+    const float* v;         // [n_kv_heads * head_dim]
+    const float* q_norm;    // [head_dim]
+    const float* k_norm;    // [head_dim]
+    float* k_cache;         // [max_seq][kv_dim]
+    float* v_cache;
+    const uint32_t* d_pos;  // may be null
+    uint32_t pos, max_seq, head_dim, n_heads, n_kv_heads;
+    float eps, theta_scale;
+};
+
+__global__ __launch_bounds__(64) void qk_norm_rope_kernel(QkNormRopeArgs a) {
+    const uint32_t pos = a.d_pos ? *a.d_pos : a.pos;
+    const bool is_q = blockIdx.x < a.n_heads;
+    const uint32_t h = is_q ? blockIdx.x : blockIdx.x - a.n_heads;
+    const uint32_t hd = a.head_dim, half = hd >> 1, kv_dim = a.n_kv_heads * hd;
+    float* head = (is_q ? a.q : a.k) + (size_t)h * hd;
+    const float* w = is_q ? a.q_norm : a.k_norm;
+    const uint32_t lane = threadIdx.x;
+
+    double s = 0.0;
+    for (uint32_t i = lane; i < hd; i += 64) {
+        const double v = (double)head[i];
+        s += v * v;
+    }
+    const float inv_rms = (float)(1.0 / sqrt(wave_sum_f64(s) / (double)hd + (double)a.eps));
+
+    const bool store = !is_q && pos < a.max_seq;  // the host checks a by-value pos; a device-side pos past the cache is dropped
+    float* kc = a.k_cache + (size_t)pos * kv_dim + (size_t)h * hd;
+    for (uint32_t i = lane; i < half; i += 64) {
+        float theta = (float)pos;
+        for (uint32_t j = 0; j < i; j++) theta = __fmul_rn(theta, a.theta_scale);
+        float sn, cs;
+        sincosf(theta, &sn, &cs);
+        const float x0 = __fmul_rn(__fmul_rn(head[i], inv_rms), w[i]);
+        const float x1 = __fmul_rn(__fmul_rn(head[i + half], inv_rms), w[i + half]);
+        const float r0 = __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn));
+        const float r1 = __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, cs));
+        head[i] = r0, head[i + half] = r1;
+        if (store) kc[i] = r0, kc[i + half] = r1;
+    }
+    if (store) {
+        const float* vh = a.v + (size_t)h * hd;
+        float* vc = a.v_cache + (size_t)pos * kv_dim + (size_t)h * hd;
+        for (uint32_t i = lane; i < hd; i += 64) vc[i] = vh[i];
+    }
+}
+
+// ---- decode attention -----------------------------------------------------------------
+// forward_attn_block's tail (wick/src/model/lfm2.rs:984-1006) = attn_scores -> softmax_inplace -> attn_values
+// (cpu.rs:1346-1355, 715-731, 1391-1401), one 256-thread block per query head over positions [0, seq_len).
+//   scores: one thread per position, the dot summed in the reference's order: bit-exact;
+//   softmax: ggml_expf bit-exact, f64 sum in another order (inverse may differ in the last f32 bit);
+//   values: four waves take positions t = wave (mod 4), one lane per dimension, partial sums added at
+//           the end: rounding differs from the sequential loop at the 1e-7 level.
+// `scores` is scratch [n_heads][max_seq].
+struct AttentionArgs {
+    const float* q;
+    const float* k_cache;
+    const float* v_cache;
+    float* out;     // [n_heads * head_dim]
+    float* scores;  // [n_heads][max_seq]
+    const uint32_t* d_pos;  // seq_len = *d_pos + 1 when non-null
+    uint32_t seq_len, max_seq, n_heads, n_kv_heads, head_dim;
+    float scale;
+};
+
+__global__ __launch_bounds__(256) void attention_decode_kernel(AttentionArgs a) {
+    __shared__ double slots[16];
+    __shared__ float red[256];
+    __shared__ float qs[256];
+    const uint32_t h = blockIdx.x, hd = a.head_dim, kv_dim = a.n_kv_heads * hd;
+    uint32_t seq = a.d_pos ? *a.d_pos + 1u : a.seq_len;
+    if (seq > a.max_seq) seq = a.max_seq;
+    const uint32_t kvh = h / (a.n_heads / a.n_kv_heads);
+    const float* kbase = a.k_cache + (size_t)kvh * hd;
+    const float* vbase = a.v_cache + (size_t)kvh * hd;
+    float* sc = a.scores + (size_t)h * a.max_seq;
+    const uint32_t tid = threadIdx.x;
+
+    for (uint32_t i = tid; i < hd; i += 256) qs[i] = a.q[(size_t)h * hd + i];
+    __syncthreads();
+
+    float mx = -__builtin_inff();
+    for (uint32_t t = tid; t < seq; t += 256) {
+        const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)t * kv_dim);
+        float dot = 0.0f;
+        for (uint32_t d = 0; d < hd; d += 4) {
+            const float4 kv = kr[d >> 2];
+            dot = __fadd_rn(dot, __fmul_rn(qs[d], kv.x));
+            dot = __fadd_rn(dot, __fmul_rn(qs[d + 1], kv.y));
+            dot = __fadd_rn(dot, __fmul_rn(qs[d + 2], kv.z));
+            dot = __fadd_rn(dot, __fmul_rn(qs[d + 3], kv.w));
+        }
+        const float s = __fmul_rn(dot, a.scale);
+        sc[t] = s;
+        mx = fmaxf(mx, s);
+    }
+    red[tid] = mx;
+    __syncthreads();
+    for (uint32_t off = 128; off > 0; off >>= 1) {
+        if (tid < off) red[tid] = fmaxf(red[tid], red[tid + off]);
+        __syncthreads();
+    }
+    mx = red[0];
+
+    double sum = 0.0;
+    for (uint32_t t = tid; t < seq; t += 256) {  // each thread revisits the positions it wrote
+        const float e = ggml_expf(__fsub_rn(sc[t], mx));
+        sc[t] = e;
+        sum += (double)e;
+    }
+    const double total = block_sum_f64(sum, slots);  // its barriers also publish sc[] to the block
+    const float inv = (float)(1.0 / total);
+
+    // values: thread = (part, dim); parts take interleaved positions
+    const uint32_t lanes = hd < 256u ? hd : 256u;     // hd <= 256 (checked by the host)
+    const uint32_t parts = 256u / lanes;               // 4 for head_dim 64
+    const uint32_t d = tid % lanes, part = tid / lanes;
+    float acc = 0.0f;
+    if (part < parts) {
+        for (uint32_t t = part; t < seq; t += parts) acc = __fadd_rn(acc, __fmul_rn(__fmul_rn(sc[t], inv), vbase[(size_t)t * kv_dim + d]));
+    }
+    __syncthreads();
+    red[tid] = acc;
+    __syncthreads();
+    if (tid < lanes) {
+        float r = red[tid];
+        for (uint32_t p = 1; p < parts; p++) r = __fadd_rn(r, red[p * lanes + tid]);
+        a.out[(size_t)h * hd + tid] = r;
+    }
+}
+
+// ---- gated short convolution, one step ---------------------------------------------------
+// forward_conv_block's middle (wick/src/model/lfm2.rs:694-726): proj = [b | c | x]; bx = b*x;
+// out = c * (sum_k buffer[k][ch]*w[ch][k] + bx*w[ch][K-1]); the rolling buffer shifts by one slot and takes bx.
+// One thread per channel, the reference's operation order: bit-exact.
+__global__ __launch_bounds__(256) void shortconv_step_kernel(const float* __restrict__ proj, float* __restrict__ buffer,
+                                                             const float* __restrict__ conv_w, float* __restrict__ out, uint32_t hidden,
+                                                             uint32_t kernel_size) {
+    const uint32_t ch = blockIdx.x * blockDim.x + threadIdx.x;
+    if (ch >= hidden) return;
+    const uint32_t d_conv = kernel_size - 1;
+    const float bx = __fmul_rn(proj[ch], proj[2 * hidden + ch]);
+    const float* w = conv_w + (size_t)ch * kernel_size;
+    float sum = 0.0f;
+    for (uint32_t k = 0; k < d_conv; k++) {
+        const float tap = buffer[(size_t)k * hidden + ch];
+        sum = __fadd_rn(sum, __fmul_rn(tap, w[k]));
+        if (k > 0) buffer[(size_t)(k - 1) * hidden + ch] = tap;
+    }
+    sum = __fadd_rn(sum, __fmul_rn(bx, w[d_conv]));
+    if (d_conv > 0) buffer[(size_t)(d_conv - 1) * hidden + ch] = bx;
+    out[ch] = __fmul_rn(proj[hidden + ch], sum);
+}
+
+// ---- SiLU gate ------------------------------------------------------------------------
+// silu_mul_inplace (wick/src/backend/cpu.rs:668-673): g / (1 + expf(-g)) * u, bit-exact.
+__global__ __launch_bounds__(256) void silu_mul_kernel(float* __restrict__ gate, const float* __restrict__ up, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float g = gate[i];
+    gate[i] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, ggml_expf(-g))), up[i]);
+}
+
+// ---- greedy pick ----------------------------------------------------------------------
+// cpu_argmax (wick/src/sampler.rs:7-19): NaN counts as -inf, values order by f32::total_cmp, the LAST of
+// equal maxima wins; bit-exact.  One 1024-thread block.  Optionally publishes the pick as the next step's
+// token and advances the device-side position.
+__device__ __forceinline__ unsigned long long argmax_key(float f, uint32_t index) {
+    if (f != f) f = -__builtin_inff();
+    int32_t b = (int32_t)__float_as_uint(f);
+    b ^= (int32_t)(((uint32_t)(b >> 31)) >> 1);                 // total_cmp's transform: signed order
+    const uint32_t ordered = (uint32_t)b ^ 0x80000000u;          // ... as unsigned order
+    return ((unsigned long long)ordered << 32) | index;          // equal values: the larger index wins
+}
+
+__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ x, uint32_t n, uint32_t* __restrict__ out,
+                                                      uint32_t* __restrict__ d_token, uint32_t* __restrict__ d_pos,
+                                                      uint32_t* __restrict__ d_history, uint32_t history_len) {
+    __shared__ unsigned long long red[1024];
+    unsigned long long best = 0ull;  // below every real key
+    for (uint32_t i = threadIdx.x; i < n; i += 1024) {
+        const unsigned long long key = argmax_key(x[i], i);
+        best = key > best ? key : best;
+    }
+    red[threadIdx.x] = best;
+    __syncthreads();
+    for (uint32_t off = 512; off > 0; off >>= 1) {
+        if (threadIdx.x < off) red[threadIdx.x] = red[threadIdx.x] > red[threadIdx.x + off] ? red[threadIdx.x] : red[threadIdx.x + off];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const uint32_t pick = n ? (uint32_t)(red[0] & 0xffffffffull) : 0u;
+        out[0] = pick;
+        if (d_token) *d_token = pick;
+        if (d_pos) {
+            const uint32_t pos = *d_pos;
+            if (d_history && pos < history_len) d_history[pos] = pick;  // the pick made after the token at `pos`
+            *d_pos = pos + 1u;
+        }
+    }
+}
+
+// Sets the device-side token / position of the next step (either may be null).
+__global__ void set_step_kernel(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        if (d_token) *d_token = token;
+        if (d_pos) *d_pos = pos;
+    }
+}
+
+__global__ void advance_pos_kernel(uint32_t* d_pos) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *d_pos = *d_pos + 1u;
+}
+
+}  // namespace
+
+hipError_t launch_embed_row(const uint8_t* d_w, int type, uint32_t m, uint32_t k, uint32_t token, const uint32_t* d_token, float* d_out,
+                            const Launch& L) {
+    const uint32_t blocks = (k + 255u) / 256u;
+    return launch_kernel(L, kFamOther, embed_row_kernel, dim3(blocks < 64u ? blocks : 64u), dim3(256), d_w, type, m, k, token, d_token, d_out);
+}
+
+hipError_t launch_rmsnorm(const float* d_x, const float* d_weight, float* d_y, uint32_t rows, uint32_t dim, uint32_t x_stride,
+                          uint32_t y_stride, float eps, const Launch& L) {
+    if (rows == 0) return hipSuccess;
+    return launch_kernel(L, kFamOther, rmsnorm_kernel, dim3(rows), dim3(256), d_x, d_weight, d_y, dim, x_stride, y_stride, eps);
+}
+
+hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm, float* d_k_cache,
+                               float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
+                               uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L) {
+    QkNormRopeArgs a{d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, d_pos, pos, max_seq, head_dim, n_heads, n_kv_heads, eps, theta_scale};
+    return launch_kernel(L, kFamOther, qk_norm_rope_kernel, dim3(n_heads + n_kv_heads), dim3(64), a);
+}
+
+hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scores,
+                                   uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
+                                   uint32_t head_dim, float scale, const Launch& L) {
+    AttentionArgs a{d_q, d_k_cache, d_v_cache, d_out, d_scores, d_pos, seq_len, max_seq, n_heads, n_kv_heads, head_dim, scale};
+    return launch_kernel(L, kFamOther, attention_decode_kernel, dim3(n_heads), dim3(256), a);
+}
+
+hipError_t launch_shortconv_step(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
+                                 uint32_t kernel_size, const Launch& L) {
+    return launch_kernel(L, kFamOther, shortconv_step_kernel, dim3((hidden + 255u) / 256u), dim3(256), d_proj, d_buffer, d_conv_w, d_out, hidden,
+                         kernel_size);
+}
+
+hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const Launch& L) {
+    if (n == 0) return hipSuccess;
+    return launch_kernel(L, kFamOther, silu_mul_kernel, dim3((n + 255u) / 256u), dim3(256), d_gate, d_up, n);
+}
+
+hipError_t launch_argmax(const float* d_x, uint32_t n, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos, uint32_t* d_history,
+                         uint32_t history_len, const Launch& L) {
+    return launch_kernel(L, kFamOther, argmax_kernel, dim3(1), dim3(1024), d_x, n, d_out, d_token, d_pos, d_history, history_len);
+}
+
+hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L) {
+    return launch_kernel(L, kFamOther, set_step_kernel, dim3(1), dim3(64), d_token, token, d_pos, pos);
+}
+
+hipError_t launch_advance_pos(uint32_t* d_pos, const Launch& L) {
+    return launch_kernel(L, kFamOther, advance_pos_kernel, dim3(1), dim3(64), d_pos);
+}
+
+}  // namespace wick_rocm

@@ -119,6 +119,27 @@ hipError_t launch_block_dots_dot4(int type, const uint8_t* d_w, uint32_t m, uint
 hipError_t launch_block_dots_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,
                                   int32_t* d_out, const Launch& L);
 
+// The non-matmul operations of an LFM2 decode step (lfm2_ops.hip).  d_pos / d_token, when non-null, are read on the
+// device in place of the by-value pos / token.
+hipError_t launch_embed_row(const uint8_t* d_w, int type, uint32_t m, uint32_t k, uint32_t token, const uint32_t* d_token, float* d_out,
+                            const Launch& L);
+hipError_t launch_rmsnorm(const float* d_x, const float* d_weight, float* d_y, uint32_t rows, uint32_t dim, uint32_t x_stride,
+                          uint32_t y_stride, float eps, const Launch& L);
+hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm, float* d_k_cache,
+                               float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
+                               uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L);
+hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scores,
+                                   uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
+                                   uint32_t head_dim, float scale, const Launch& L);
+hipError_t launch_shortconv_step(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
+                                 uint32_t kernel_size, const Launch& L);
+hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const Launch& L);
+// d_history[pos] = pick (pos = *d_pos before it is advanced), when given.
+hipError_t launch_argmax(const float* d_x, uint32_t n, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos, uint32_t* d_history,
+                         uint32_t history_len, const Launch& L);
+hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L);
+hipError_t launch_advance_pos(uint32_t* d_pos, const Launch& L);
+
 // n at and above which gemm_q8 uses the MFMA kernel (when k % 256 == 0).
 constexpr uint32_t kGemmMinN = 16;  // cf. GEMM_MIN_N, wick/src/model/metal_lfm2.rs:18-21
 

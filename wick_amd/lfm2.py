@@ -1,0 +1,153 @@
+"""Host mirror of ``include/wick_rocm_lfm2.h``: the decode step's non-matmul operations under the
+names of the reference's encoder call sites (wick/src/model/metal_lfm2.rs:1380-1990), and the LFM2
+model handle with ``forward`` / ``forward_greedy`` of ``trait Model`` (wick/src/model/mod.rs:72-323).
+Test / bench plumbing over ctypes, like ``wick_amd.rocm``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import numpy as np
+
+from . import rocm
+from .rocm import RocmContext, RocmWeight, _ptr
+
+_P = C.c_void_p
+_U32, _F = C.c_uint32, C.c_float
+
+
+class Lfm2Config(C.Structure):
+    """wick_rocm_lfm2_config (ModelConfig, wick/src/model/mod.rs:27-46)."""
+    _fields_ = [(n, _U32) for n in ("n_layers", "hidden_size", "intermediate_size", "n_heads", "n_kv_heads", "vocab_size", "max_seq_len",
+                                    "conv_kernel_size")] + [("rope_theta", _F), ("rms_norm_eps", _F)]
+
+
+_SIGNATURES = {
+    "wick_rocm_embed_row": (C.c_int, [_P, _P, _U32, _P, _P]),
+    "wick_rocm_rmsnorm": (C.c_int, [_P, _P, _P, _P, _U32, _U32, _U32, _U32, _F]),
+    "wick_rocm_qk_norm_rope": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32, _F, _F]),
+    "wick_rocm_rope_theta_scale": (_F, [_U32, _F]),
+    "wick_rocm_attention_decode": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32]),
+    "wick_rocm_shortconv_step": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32]),
+    "wick_rocm_silu_mul": (C.c_int, [_P, _P, _P, _U32]),
+    "wick_rocm_argmax": (C.c_int, [_P, _P, _U32, _P, _P, _P]),
+    "wick_rocm_lfm2_load": (C.c_int, [_P, _P, _U32, C.POINTER(_P)]),
+    "wick_rocm_lfm2_free": (C.c_int, [_P, _P]),
+    "wick_rocm_lfm2_get_config": (C.c_int, [_P, C.POINTER(Lfm2Config)]),
+    "wick_rocm_lfm2_layer_kv_heads": (C.c_int, [_P, _U32, C.POINTER(_U32)]),
+    "wick_rocm_lfm2_gpu_memory_bytes": (C.c_size_t, [_P]),
+    "wick_rocm_lfm2_reset": (C.c_int, [_P, _P]),
+    "wick_rocm_lfm2_forward": (C.c_int, [_P, _P, _U32, _U32, _P]),
+    "wick_rocm_lfm2_forward_greedy": (C.c_int, [_P, _P, _U32, _U32, C.POINTER(_U32)]),
+    "wick_rocm_lfm2_generate_greedy": (C.c_int, [_P, _P, _U32, _U32, _U32, _P]),
+    "wick_rocm_lfm2_logits_device": (_P, [_P]),
+    "wick_rocm_lfm2_hidden_device": (_P, [_P]),
+}
+
+_bound = False
+
+
+def _lib() -> C.CDLL:
+    global _bound
+    lib = rocm.load_library()
+    if not _bound:
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _bound = True
+    return lib
+
+
+def rope_theta_scale(head_dim: int, freq_base: float) -> float:
+    return float(_lib().wick_rocm_rope_theta_scale(head_dim, freq_base))
+
+
+class Lfm2Ops:
+    """The operations as calls on a context (device buffers in, device buffers out)."""
+
+    def __init__(self, ctx: RocmContext):
+        self.ctx, self._l = ctx, _lib()
+
+    def embed_row(self, w: RocmWeight, out, token: int = 0, d_token=None) -> None:
+        self.ctx._check(self._l.wick_rocm_embed_row(self.ctx._h, w.handle, token, _ptr(d_token), _ptr(out)))
+
+    def encode_rmsnorm(self, x, weight, y, dim: int, eps: float, rows: int = 1, x_stride: Optional[int] = None,
+                       y_stride: Optional[int] = None) -> None:
+        self.ctx._check(self._l.wick_rocm_rmsnorm(self.ctx._h, _ptr(x), _ptr(weight), _ptr(y), rows, dim, x_stride or dim, y_stride or dim, eps))
+
+    def encode_qk_norm_rope(self, q, k, v, q_norm, k_norm, k_cache, v_cache, pos: int, max_seq: int, head_dim: int, n_heads: int,
+                            n_kv_heads: int, eps: float, theta_scale: float, d_pos=None) -> None:
+        self.ctx._check(self._l.wick_rocm_qk_norm_rope(self.ctx._h, _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(k_cache),
+                                                       _ptr(v_cache), pos, _ptr(d_pos), max_seq, head_dim, n_heads, n_kv_heads, eps, theta_scale))
+
+    def encode_attention(self, q, k_cache, v_cache, out, scores, seq_len: int, max_seq: int, n_heads: int, n_kv_heads: int, head_dim: int,
+                         d_pos=None) -> None:
+        self.ctx._check(self._l.wick_rocm_attention_decode(self.ctx._h, _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(scores), seq_len,
+                                                           _ptr(d_pos), max_seq, n_heads, n_kv_heads, head_dim))
+
+    def encode_conv1d_fused(self, proj, buffer, conv_weight, out, hidden: int, kernel_size: int) -> None:
+        self.ctx._check(self._l.wick_rocm_shortconv_step(self.ctx._h, _ptr(proj), _ptr(buffer), _ptr(conv_weight), _ptr(out), hidden, kernel_size))
+
+    def silu_mul_inplace(self, gate, up, n: int) -> None:
+        self.ctx._check(self._l.wick_rocm_silu_mul(self.ctx._h, _ptr(gate), _ptr(up), n))
+
+    def argmax(self, logits, n: int, out, d_token=None, d_pos=None) -> None:
+        self.ctx._check(self._l.wick_rocm_argmax(self.ctx._h, _ptr(logits), n, _ptr(out), _ptr(d_token), _ptr(d_pos)))
+
+
+class RocmLfm2Model:
+    """load_model_* counterpart (wick/src/model/mod.rs:385-403): owns weights, KV caches, conv state and scratch on the GPU."""
+
+    def __init__(self, ctx: RocmContext, gguf, context_size: int):
+        self.ctx, self._l = ctx, _lib()
+        h = _P()
+        ctx._check(self._l.wick_rocm_lfm2_load(ctx._h, gguf.handle, context_size, C.byref(h)))
+        self._h = h.value
+        cfg = Lfm2Config()
+        ctx._check(self._l.wick_rocm_lfm2_get_config(self._h, C.byref(cfg)))
+        self.config = {n: getattr(cfg, n) for n, _ in Lfm2Config._fields_}
+        kv = _U32()
+        self.kv_heads_per_layer = []
+        for i in range(cfg.n_layers):
+            ctx._check(self._l.wick_rocm_lfm2_layer_kv_heads(self._h, i, C.byref(kv)))
+            self.kv_heads_per_layer.append(kv.value)
+
+    def free(self) -> None:
+        if self._h:
+            self.ctx._check(self._l.wick_rocm_lfm2_free(self.ctx._h, self._h))
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.free()
+
+    def gpu_memory_bytes(self) -> int:
+        return self._l.wick_rocm_lfm2_gpu_memory_bytes(self._h)
+
+    def reset(self) -> None:
+        self.ctx._check(self._l.wick_rocm_lfm2_reset(self.ctx._h, self._h))
+
+    def forward(self, token: int, pos: int) -> np.ndarray:
+        logits = np.empty(self.config["vocab_size"], np.float32)
+        self.ctx._check(self._l.wick_rocm_lfm2_forward(self.ctx._h, self._h, token, pos, logits.ctypes.data))
+        return logits
+
+    def forward_greedy(self, token: int, pos: int) -> int:
+        nxt = _U32()
+        self.ctx._check(self._l.wick_rocm_lfm2_forward_greedy(self.ctx._h, self._h, token, pos, C.byref(nxt)))
+        return nxt.value
+
+    def generate_greedy(self, token: int, pos: int, n: int) -> np.ndarray:
+        out = np.empty(n, np.uint32)
+        self.ctx._check(self._l.wick_rocm_lfm2_generate_greedy(self.ctx._h, self._h, token, pos, n, out.ctypes.data))
+        return out
+
+    def hidden(self) -> np.ndarray:
+        """Final normed hidden state of the last step."""
+        out = np.empty(self.config["hidden_size"], np.float32)
+        self.ctx._check(self.ctx._lib.wick_rocm_download(self.ctx._h, out.ctypes.data, self._l.wick_rocm_lfm2_hidden_device(self._h), out.nbytes))
+        return out
