@@ -128,6 +128,29 @@ def gemv(ggml_type: int, data: np.ndarray, x: np.ndarray, m: int, k: int) -> np.
     return O.gemv_q8(ggml_type, data, s, q, m, k)
 
 
+def quantizer_margin(x) -> float:
+    """How far the Q8_0 quantization of `x` (wick/src/backend/simd.rs:255-323) is from changing under a
+    last-bit perturbation of x, as the smaller of
+      - the distance of any x*id from a rounding tie (in units of one quant step), and
+      - 1e3 x the relative distance of any block's amax/127 from an f16 rounding boundary of its scale.
+    The quantizer is discontinuous there: two correct f32 pipelines that differ in the last bit of one
+    activation can then legitimately differ by a whole quant step (or a whole f16 scale step) downstream."""
+    x = np.asarray(x, np.float32).reshape(-1, 32)
+    amax = np.abs(x).max(1)
+    d = (amax / np.float32(127.0)).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        idv = np.where(d != 0, np.float32(1.0) / d, np.float32(0)).astype(np.float32)
+    r = (x * idv[:, None]).astype(np.float32)
+    tie = float(np.abs(r - np.floor(r) - np.float32(0.5)).min())
+    nz = d[d != 0].astype(np.float64)
+    if nz.size == 0:
+        return tie
+    h = nz.astype(np.float16).astype(np.float64)
+    up, dn = np.nextafter(h.astype(np.float16), np.float16(np.inf)).astype(np.float64), np.nextafter(h.astype(np.float16), np.float16(-np.inf)).astype(np.float64)
+    edge = np.minimum(np.abs(nz - (h + up) / 2), np.abs(nz - (h + dn) / 2)) / nz
+    return min(tie, float(edge.min()) * 1e3)
+
+
 class Lfm2Oracle:
     """`cfg`: n_layers, hidden_size, intermediate_size, n_heads, vocab_size, rope_theta, rms_norm_eps,
     conv_kernel_size, kv_heads_per_layer (0 = gated-conv layer).  `tensors`: GGUF name -> (ggml_type, dims, array),
@@ -135,6 +158,7 @@ class Lfm2Oracle:
 
     def __init__(self, cfg: dict, tensors: dict):
         self.cfg, self.t = cfg, tensors
+        self.min_margin = float("inf")  # smallest quantizer_margin over every GEMV input so far
 
     def new_state(self) -> dict:
         c = self.cfg
@@ -149,6 +173,7 @@ class Lfm2Oracle:
 
     def _gemv(self, name, x):
         gt, dims, data = self.t[name]
+        self.min_margin = min(self.min_margin, quantizer_margin(x))
         return gemv(gt, data, x, dims[1], dims[0])
 
     def hidden_after_layers(self, token: int, pos: int, state: dict) -> np.ndarray:

@@ -12,9 +12,34 @@ from wick_amd.lfm2 import RocmLfm2Model
 
 pytestmark = pytest.mark.gpu
 
-# f32 tolerance of a whole step: every operation is within a few ulp of the oracle's, a 4..6-layer
-# residual stream amplifies that to ~1e-6; 1e-5 rel-L2 is the bar of the matmul path itself.
+# f32 tolerance of a whole step: every operation is within a few ulp of the oracle's and the residual
+# stream keeps that near 1e-7; 1e-5 rel-L2 is the bar of the matmul path itself.
 LOGITS_REL_L2 = 1e-5
+# The step re-quantizes f32 activations to Q8_0 before every GEMV, and that quantizer is discontinuous:
+# when some x/d sits within the f32 noise of a rounding tie, two correct pipelines that differ in the last
+# bit of one activation differ by a whole quant step afterwards (about 1e-3 of a GEMV output per flipped
+# quant), and the KV cache / conv state carry it to later positions.  The oracle reports how close every
+# GEMV input came to such a tie (quantizer_margin); positions are held to the strict bar until the first
+# near-tie, to the loose one (what one flipped quant can do) from there on.
+NEAR_TIE = 3e-5  # in quant steps; the GPU's activations differ from the oracle's by <= ~1e-5 of a step
+LOOSE_REL_L2 = 5e-2
+LOOSE_COSINE = 0.999
+
+
+def cosine(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return float(a @ b / (np.linalg.norm(a) * np.linalg.norm(b)))
+
+
+def check_step(logits, want, margin, what):
+    """Returns True when the step was held to the strict bar."""
+    assert np.isfinite(logits).all(), what
+    if margin >= NEAR_TIE:
+        assert rel_l2(logits, want) <= LOGITS_REL_L2, f"{what}: rel-L2 {rel_l2(logits, want):.2e} (margin {margin:.1e})"
+        assert int(np.argmax(logits)) == int(np.argmax(want)), what
+        return True
+    assert rel_l2(logits, want) <= LOOSE_REL_L2 and cosine(logits, want) >= LOOSE_COSINE, f"{what}: rel-L2 {rel_l2(logits, want):.2e} after a near-tie"
+    return False
 
 
 def load(ctx, oracle, tmp_path, context=64, **kw):
@@ -26,26 +51,58 @@ def load(ctx, oracle, tmp_path, context=64, **kw):
     return model, L.Lfm2Oracle(cfg, tensors), cfg
 
 
-@pytest.mark.parametrize("kw", [
-    dict(),                                                                              # Q4_0 body, Q6_K embedding (a shipped Q4_0 file)
-    dict(wtype=W.Q8_0, embd_type=W.Q8_0, seed=2),
-    dict(n_layers=6, hidden=512, inter=1024, n_heads=8, kv_heads=(0, 0, 4, 0, 8, 2), vocab=1000, embd_type=W.Q4_0, seed=3),
-    dict(kernel=4, kv_heads=(2, 0, 0, 4), seed=4, rope_theta=10000.0, eps=1e-6),
-    dict(mixed_qkv=True, seed=5),                                                        # Q/K Q4_0, V Q8_0: separate launches
-], ids=["q4_0+q6k", "q8_0", "6-layer", "kernel4", "mixed-qkv"])
-def test_forward_matches_the_oracle_step_by_step(ctx, oracle, tmp_path, kw):
+# Small models and seeds picked so that the whole token sequence stays clear of quantizer ties (the search ran
+# on the oracle alone; the test re-checks the margin, so a change of the generator cannot go unnoticed).
+CLEAR = {
+    "q4_0+q6k": dict(hidden=256, inter=256, vocab=256, seed=16),                      # Q4_0 body, Q6_K embedding: a shipped Q4_0 file
+    "q8_0": dict(hidden=256, inter=256, vocab=256, wtype=W.Q8_0, embd_type=W.Q8_0, seed=25),
+    "kernel4": dict(hidden=256, inter=256, vocab=256, kernel=4, kv_heads=(2, 0, 0, 4), rope_theta=10000.0, eps=1e-6, seed=20),
+    "mixed-qkv": dict(hidden=256, inter=256, vocab=256, mixed_qkv=True, seed=27),      # Q/K Q4_0, V Q8_0: separate launches
+    "3-layer-q4embd": dict(n_layers=3, hidden=512, inter=512, n_heads=8, kv_heads=(0, 4, 8), vocab=512, embd_type=W.Q4_0, seed=1),
+}
+
+
+@pytest.mark.parametrize("name", list(CLEAR))
+def test_forward_matches_the_oracle_step_by_step(ctx, oracle, tmp_path, name):
+    kw = CLEAR[name]
     model, ref, cfg = load(ctx, oracle, tmp_path, **kw)
     assert model.kv_heads_per_layer == cfg["kv_heads_per_layer"]
     assert model.config["max_seq_len"] == 64 and model.config["n_kv_heads"] == max(cfg["kv_heads_per_layer"])
     state = ref.new_state()
-    rng = np.random.default_rng(11)
-    tokens = rng.integers(0, cfg["vocab_size"], 9)
+    tokens = np.random.default_rng(100 + kw["seed"]).integers(0, cfg["vocab_size"], 6)
     for pos, tok in enumerate(tokens):
         logits = model.forward(int(tok), pos)
         want = ref.forward(int(tok), pos, state)
-        assert np.isfinite(logits).all()
-        assert rel_l2(logits, want) <= LOGITS_REL_L2, f"pos {pos}: rel-L2 {rel_l2(logits, want):.2e}"
-        assert int(np.argmax(logits)) == int(np.argmax(want))
+        assert ref.min_margin >= NEAR_TIE, "this seed no longer stays clear of quantizer ties: search another"
+        assert check_step(logits, want, ref.min_margin, f"{name} pos {pos}")
+    model.free()
+
+
+def test_larger_model_longer_sequence(ctx, oracle, tmp_path):
+    """Six layers, 24 positions: strict until the oracle reports the first near-tie, bounded afterwards."""
+    model, ref, cfg = load(ctx, oracle, tmp_path, n_layers=6, hidden=512, inter=1024, n_heads=8, kv_heads=(0, 0, 4, 0, 8, 2), vocab=1000,
+                           embd_type=W.Q4_0, seed=3)
+    state = ref.new_state()
+    tokens = np.random.default_rng(11).integers(0, cfg["vocab_size"], 24)
+    strict = sum(check_step(model.forward(int(t), p), ref.forward(int(t), p, state), ref.min_margin, f"pos {p}") for p, t in enumerate(tokens))
+    assert strict >= 1
+    model.free()
+
+
+def test_a_quantizer_tie_is_the_only_thing_that_loosens_the_bar(ctx, oracle, tmp_path):
+    """Token 42 of this model puts an FFN input at x/d = 61.499996: the oracle flags it, the GPU step stays
+    within what one flipped quant can do, and the very same model is strict on tokens that stay clear of ties."""
+    model, ref, cfg = load(ctx, oracle, tmp_path, wtype=W.Q8_0, embd_type=W.Q8_0, seed=2)
+    state = ref.new_state()
+    want = ref.forward(42, 0, state)
+    assert ref.min_margin < 1e-5
+    assert check_step(model.forward(42, 0), want, ref.min_margin, "token 42") is False
+    model.reset()
+    ref2 = L.Lfm2Oracle(cfg, ref.t)
+    state = ref2.new_state()
+    want = ref2.forward(3, 0, state)
+    assert ref2.min_margin >= NEAR_TIE
+    assert check_step(model.forward(3, 0), want, ref2.min_margin, "clear token 3") is True
     model.free()
 
 
@@ -62,22 +119,24 @@ def test_reset_starts_a_fresh_state(ctx, oracle, tmp_path):
 def test_greedy_generation_stays_on_the_device(ctx, oracle, tmp_path):
     """forward_greedy == argmax(forward) with the reference's tie rule; n steps without a host round trip
     give the same tokens as n single steps."""
-    model, ref, cfg = load(ctx, oracle, tmp_path, seed=7)
+    model, ref, cfg = load(ctx, oracle, tmp_path, hidden=256, inter=256, vocab=256, seed=26)
     state, tok, want = ref.new_state(), 17, []
-    for pos in range(12):
+    for pos in range(10):
         tok = L.argmax(ref.forward(tok, pos, state))
         want.append(tok)
-    got = model.generate_greedy(17, 0, 12)
+    assert ref.min_margin >= NEAR_TIE, "this seed walks into a quantizer tie: pick another"
+    got = model.generate_greedy(17, 0, 10)
     assert got.tolist() == want
     model.reset()
     tok, single = 17, []
-    for pos in range(12):
+    for pos in range(10):
         tok = model.forward_greedy(tok, pos)
         single.append(tok)
     assert single == want
     # the two kinds of step interleave on one state: logits of the next position follow the greedy prefix
-    logits = model.forward(want[-1], 12)
-    assert rel_l2(logits, ref.forward(want[-1], 12, state)) <= LOGITS_REL_L2
+    logits = model.forward(want[-1], 10)
+    expect = ref.forward(want[-1], 10, state)
+    check_step(logits, expect, ref.min_margin, "logits after the greedy prefix")
     model.free()
 
 
