@@ -217,6 +217,83 @@ def bench_single_gemv(ctx, W, O, dtype, m, k, launches=200, wb=None):
             "kernel_us": kus, "kernel_GBps": b / kus / 1e3, "kernel_frac_of_hbm_peak": b / kus / 1e3 / HBM_PEAK_GBS}
 
 
+def lfm2_350m_image(O, body=2, embd=14):
+    """A randomly initialised LFM2-350M-shaped model as a GGUF image: 16 layers (gated conv except attention at
+    2, 5, 8, 10, 12, 14), hidden 1024, FFN 4608, 16 heads / 8 KV heads, vocabulary 65536, Q4_0 body with the tied
+    embedding in Q6_K like the shipped Q4_0 files (tensor names of wick/src/model/lfm2.rs:97-300)."""
+    from wick_amd import gguf as G
+
+    attn = {2, 5, 8, 10, 12, 14}
+    n_layers, hd = N_CONV + N_ATTN, 64
+    names, jobs = ["token_embd.weight"], [(embd, VOCAB, HS, 9000)]
+    for i in range(n_layers):
+        p = f"blk.{i}."
+        mats = ([("attn_q", HS, HS), ("attn_k", KV, HS), ("attn_v", KV, HS), ("attn_output", HS, HS)] if i in attn else
+                [("shortconv.in_proj", 3 * HS, HS), ("shortconv.out_proj", HS, HS)])
+        for j, (n, m, k) in enumerate(mats + [("ffn_gate", IS, HS), ("ffn_up", IS, HS), ("ffn_down", HS, IS)]):
+            names.append(p + n + ".weight")
+            jobs.append((body, m, k, 9100 + 16 * i + j))
+    tensors = [(n, [j[2], j[1]], j[0], b) for n, j, b in zip(names, jobs, synth_many(O, jobs))]
+    rng = np.random.default_rng(5)
+    norm = lambda n: (1.0 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    tensors.append(("token_embd_norm.weight", [HS], 0, norm(HS)))
+    for i in range(n_layers):
+        p = f"blk.{i}."
+        tensors += [(p + "attn_norm.weight", [HS], 0, norm(HS)), (p + "ffn_norm.weight", [HS], 0, norm(HS))]
+        if i in attn:
+            tensors += [(p + "attn_q_norm.weight", [hd], 0, norm(hd)), (p + "attn_k_norm.weight", [hd], 0, norm(hd))]
+        else:
+            tensors.append((p + "shortconv.conv.weight", [3, HS], 0, (0.3 * rng.standard_normal(3 * HS)).astype(np.float32)))
+    meta = [("general.architecture", G.T_STRING, "lfm2"), ("lfm2.block_count", G.T_U32, n_layers), ("lfm2.embedding_length", G.T_U32, HS),
+            ("lfm2.feed_forward_length", G.T_U32, IS), ("lfm2.attention.head_count", G.T_U32, HS // hd), ("lfm2.vocab_size", G.T_U32, VOCAB),
+            ("lfm2.rope.freq_base", G.T_F32, 1000000.0), ("lfm2.attention.layer_norm_rms_epsilon", G.T_F32, 1e-5),
+            ("lfm2.shortconv.l_cache", G.T_U32, 3),
+            ("lfm2.attention.head_count_kv", G.T_ARRAY, (G.T_I32, [KV // hd if i in attn else 0 for i in range(n_layers)]))]
+    return G.build_image(meta, tensors)
+
+
+def trace_lfm2_step(ctx, W, O, tokens=32, context=4096):
+    """The same decode steps enqueued one by one (no graph replay), for a kernel tracer: 32 tokens from position 1024."""
+    from wick_amd import gguf as G
+    from wick_amd.lfm2 import RocmLfm2Model
+
+    with G.GgufFile.from_bytes(lfm2_350m_image(O)) as g:
+        model = RocmLfm2Model(ctx, g, context)
+    model.set_graph_replay(False)
+    picks = model.generate_greedy(1, 1024, tokens)
+    model.free()
+    return {"tokens": tokens, "start_pos": 1024, "last_pick": int(picks[-1])}
+
+
+def bench_lfm2_step(ctx, W, O, tokens=64, context=4096):
+    """Whole decode steps of the model handle (embedding, 16 layers with their norms / conv / attention / gates, tied
+    LM head, greedy pick), replayed as one graph per token with token and position resident on the device."""
+    from wick_amd import gguf as G
+    from wick_amd.lfm2 import RocmLfm2Model
+
+    with G.GgufFile.from_bytes(lfm2_350m_image(O)) as g:
+        model = RocmLfm2Model(ctx, g, context)
+    model.generate_greedy(1, 0, 8)  # captures the graph, warms up
+    out = {"model": "LFM2-350M-shaped, Q4_0 body + Q6_K tied embedding, random init", "context": context,
+           "gpu_memory_MB": model.gpu_memory_bytes() / 1e6, "runs": []}
+    for start in (0, 1024, context - tokens):  # attention cost grows with the position
+        model.reset()
+        t0 = time.perf_counter()
+        model.generate_greedy(1, start, tokens)
+        dt = time.perf_counter() - t0
+        out["runs"].append({"start_pos": start, "tokens": tokens, "ms_per_token": dt / tokens * 1e3, "tokens_per_s": tokens / dt})
+    # where the time goes: the same steps enqueued one by one with per-dispatch timestamps
+    model.set_graph_replay(False)
+    model.reset()
+    model.generate_greedy(1, 1024, 4)
+    ctx.kernel_timing_begin()
+    model.generate_greedy(1, 1028, 16)
+    kt = ctx.kernel_timing_end()
+    out["kernel_time_per_token_at_pos_1024"] = {fam: {"us": ms / 16 * 1e3, "launches": n // 16} for fam, (ms, n) in kt.items() if n}
+    model.free()
+    return out
+
+
 def bench_gemm(ctx, W, O, dtype, m, n, k, reps=20, wb=None, with_quantize=True):
     wb = O.synth_weight(dtype, m, k, seed=777) if wb is None else wb
     w = ctx.upload_weight(wb, dtype, m, k)
@@ -388,6 +465,8 @@ def main():
             "prefill_sites": lambda: bench_prefill_sites(ctx, W, O),
             "lm_head": lambda: bench_lm_head_sweep(ctx, W, O),
             "lm_head_q6k": lambda: bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024),
+            "lfm2_step": lambda: bench_lfm2_step(ctx, W, O),
+            "lfm2_step_trace": lambda: trace_lfm2_step(ctx, W, O),
             "copy": lambda: bench_copy(ctx),
             "probe": lambda: bench_probe(ctx),
         }
@@ -457,6 +536,7 @@ def main():
         out["lm_head_sweep"] = bench_lm_head_sweep(ctx, W, O)
         # shipped LFM2 Q4_0 files keep the tied embedding / LM head in Q6_K (wick/src/model/metal_lfm2.rs:175-180)
         out["lm_head_q6_k_65536x1024"] = bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024)
+        out["lfm2_decode_step"] = bench_lfm2_step(ctx, W, O)
         host_weights = None
     ctx.close()
     if not args.skip_cpu:

@@ -191,6 +191,20 @@ int wick_rocm_matmul_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const fl
 int wick_rocm_gemv_f32_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *ws, float *const *d_ys, uint32_t count,
                              const float *d_x, size_t x_off_bytes, int accumulate);
 
+/* encode_gemv_rmsnorm_gate_up (wick/src/model/metal_lfm2.rs:1157-1186), for any group of 1..4 weights that share
+ * the activation: y_i (+)= W_i * quantize(rmsnorm(x, norm_weight, eps)) in one launch.  cpu::rmsnorm
+ * (wick/src/backend/cpu.rs:577-594) is applied to the f32 vector inside the GEMV kernel, in front of its Q8_0
+ * quantization; results equal wick_rocm_rmsnorm followed by wick_rocm_gemv_f32_multi up to the last bit of the f64
+ * sum of squares.  Weights that cannot take the fused kernel (Q6_K, odd block counts, k > 8192) run the norm as
+ * a launch of its own into context scratch (wick_rocm_reserve_scratch before a capture). */
+int wick_rocm_gemv_rmsnorm_f32_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *ws, float *const *d_ys, uint32_t count,
+                                     const float *d_x, const float *d_norm_weight, float eps, int accumulate);
+/* The FFN's down projection with its gate folded in: y (+)= W * quantize(silu(gate) * up), cpu::silu_mul_inplace
+ * (wick/src/backend/cpu.rs:668-673) applied inside the GEMV kernel (bit-identical to the two separate launches).
+ * d_gate is left unchanged. */
+int wick_rocm_gemv_silu_mul_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const float *d_gate, const float *d_up, float *d_y,
+                                int accumulate);
+
 /* Pre-sizes the scratch used by wick_rocm_matmul_f32 for up to max_n columns of
  * up to max_k elements (call before capturing a graph). */
 int wick_rocm_reserve_scratch(wick_rocm_ctx *ctx, uint32_t max_n, uint32_t max_k);

@@ -51,10 +51,13 @@ float wick_rocm_rope_theta_scale(uint32_t head_dim, float freq_base);
 
 /* encode_attention (wick/src/model/metal_lfm2.rs:1736-1867) = attn_scores + softmax_inplace + attn_values per
  * query head (wick/src/model/lfm2.rs:984-1006) over cache rows [0, seq_len) (seq_len = *d_pos + 1 when d_pos is
- * given), grouped-query: head h reads KV head h / (n_heads / n_kv_heads).  d_scores is scratch of
- * n_heads * max_seq floats.  head_dim % 4 == 0, <= 256. */
+ * given), grouped-query: head h reads KV head h / (n_heads / n_kv_heads).  d_scratch holds
+ * wick_rocm_attention_scratch_floats(max_seq, n_heads, head_dim) floats (contents need not be kept between calls).
+ * head_dim % 4 == 0, <= 256.  Contexts longer than 256 positions with head_dim 32 / 64 / 128 / 256 are split over the
+ * sequence (many workgroups per head, streaming softmax, a second small launch merges the partials). */
+size_t wick_rocm_attention_scratch_floats(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim);
 int wick_rocm_attention_decode(wick_rocm_ctx *ctx, const float *d_q, const float *d_k_cache, const float *d_v_cache, float *d_out,
-                               float *d_scores, uint32_t seq_len, const uint32_t *d_pos, uint32_t max_seq, uint32_t n_heads,
+                               float *d_scratch, uint32_t seq_len, const uint32_t *d_pos, uint32_t max_seq, uint32_t n_heads,
                                uint32_t n_kv_heads, uint32_t head_dim);
 
 /* encode_conv1d_fused (wick/src/model/metal_lfm2.rs:1959-1991) = the middle of forward_conv_block
@@ -96,6 +99,12 @@ size_t wick_rocm_lfm2_gpu_memory_bytes(const wick_rocm_lfm2 *model);
 /* A fresh InferenceState: conv state zeroed, caches logically empty. */
 int wick_rocm_lfm2_reset(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model);
 
+/* Steps replay a captured graph (the counterpart of one command buffer per token, wick/src/model/metal_lfm2.rs:1-4).
+ * With enabled = 0 the same launches are enqueued one by one instead, which per-dispatch timing
+ * (wick_rocm_kernel_timing_begin) and kernel tracers need; results are identical.  The counterpart of the
+ * reference's profiled encode path (encode_layers_profiled, wick/src/model/metal_lfm2.rs:4559-4712). */
+int wick_rocm_lfm2_set_graph_replay(wick_rocm_lfm2 *model, int enabled);
+
 /* Model::forward (wick/src/model/lfm2.rs:2258-2289): one token at position `pos` (= tokens seen so far) ->
  * vocab_size logits copied to `logits` (host memory; may be null to leave them on the device).  Waits for the step. */
 int wick_rocm_lfm2_forward(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t token, uint32_t pos, float *logits);
@@ -105,9 +114,8 @@ int wick_rocm_lfm2_forward_greedy(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uin
  * pick after step i (which is also step i+1's input). */
 int wick_rocm_lfm2_generate_greedy(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t token, uint32_t pos, uint32_t n,
                                    uint32_t *out_tokens);
-/* Device buffers of the last step, for inspection: logits [vocab_size], final normed hidden state [hidden_size]. */
+/* The logits of the last step on the device ([vocab_size] floats). */
 const float *wick_rocm_lfm2_logits_device(const wick_rocm_lfm2 *model);
-const float *wick_rocm_lfm2_hidden_device(const wick_rocm_lfm2 *model);
 
 #ifdef __cplusplus
 }

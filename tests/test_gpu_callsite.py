@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import wick_amd as W
-from conftest import assert_f32_parity
+from conftest import assert_f32_parity, rel_l2
 
 pytestmark = pytest.mark.gpu
 
@@ -168,3 +168,60 @@ def test_rate_probes(ctx):
         ctx.probe_rate(3, 10)
     with pytest.raises(W.RocmError):
         ctx.probe_rate(0, 0)
+
+
+# ---- projections with the preceding norm / gate folded into their launch -----------------------------------
+
+NEAR_TIE = 3e-5  # see tests/test_gpu_lfm2_model.py: closer to a Q8_0 rounding tie than this, one quant may legitimately flip
+
+
+def _close_unless_tie(got, x_transformed, ref, what):
+    from oracle import lfm2_oracle as L
+    margin = L.quantizer_margin(x_transformed)
+    tol = 1e-5 if margin >= NEAR_TIE else 3e-3
+    assert rel_l2(got, ref) <= tol, f"{what}: rel-L2 {rel_l2(got, ref):.2e} (quantizer margin {margin:.1e})"
+
+
+@pytest.mark.parametrize("dtype,ms,k", [(W.Q4_0, [3072], 1024), (W.Q4_0, [1024, 512, 512], 1024), (W.Q8_0, [4608, 4608], 1024), (W.Q4_0, [100], 2048),
+                                        (W.Q8_0, [64, 32], 256), (W.Q4_0, [40], 4608), (W.Q4_0, [70], 8192), (W.Q4_0, [33], 96),
+                                        (W.Q6_K, [515], 1024), (W.Q8_0, [16], 16384)])
+def test_gemv_with_the_norm_folded_in(ctx, oracle, dtype, ms, k):
+    """wick_rocm_gemv_rmsnorm_f32_multi == rmsnorm, quantize, GEMV of the oracle (encode_gemv_rmsnorm_gate_up's fusion,
+    wick/src/model/metal_lfm2.rs:1157-1186); the last three shapes take the unfused fallback (odd block count, Q6_K, k > 8192)."""
+    from oracle import lfm2_oracle as L
+    x = oracle.fill_normal(k + 1, 2.0, k)
+    nw = (1.0 + 0.2 * oracle.fill_normal(k + 2, 1.0, k)).astype(np.float32)
+    eps = 1e-5
+    wbs = [oracle.synth_weight(dtype, m, k, seed=m + i) for i, m in enumerate(ms)]
+    ws = [ctx.upload_weight(b, dtype, m, k) for b, m in zip(wbs, ms)]
+    d_x, d_nw = ctx.to_device(x), ctx.to_device(nw)
+    ys = [ctx.to_device(np.full(m, 3.0, np.float32)) for m in ms]
+    ctx.encode_gemv_rmsnorm_fused(ws, d_x, d_nw, eps, ys)
+    normed = L.rmsnorm(x, nw, eps)
+    for b, m, y in zip(wbs, ms, ys):
+        _close_unless_tie(y.download(np.float32, m), normed, L.gemv(dtype, b, normed, m, k), f"norm+gemv {dtype} {m}x{k}")
+    ctx.encode_gemv_rmsnorm_fused(ws[:1], d_x, d_nw, eps, ys[:1], accumulate=True)  # y += W norm(x): y becomes 2 W norm(x)
+    _close_unless_tie(ys[0].download(np.float32, ms[0]), normed, 2 * L.gemv(dtype, wbs[0], normed, ms[0], k), "norm+gemv accumulate")
+    for b in ws + [d_x, d_nw] + ys:
+        b.free()
+
+
+@pytest.mark.parametrize("dtype,m,k", [(W.Q4_0, 1024, 4608), (W.Q8_0, 1024, 4608), (W.Q4_0, 256, 512), (W.Q4_0, 77, 8192), (W.Q8_0, 50, 96)])
+def test_down_projection_with_the_gate_folded_in(ctx, oracle, dtype, m, k):
+    """wick_rocm_gemv_silu_mul_f32 is bit-identical to silu_mul followed by the plain f32 GEMV, and matches the oracle."""
+    from oracle import lfm2_oracle as L
+    from wick_amd.lfm2 import Lfm2Ops
+    g, u = oracle.fill_normal(k + 5, 2.0, k), oracle.fill_normal(k + 6, 1.0, k)
+    wb = oracle.synth_weight(dtype, m, k, seed=m)
+    w = ctx.upload_weight(wb, dtype, m, k)
+    d_g, d_u, d_y, d_z = ctx.to_device(g), ctx.to_device(u), ctx.to_device(np.ones(m, np.float32)), ctx.to_device(np.ones(m, np.float32))
+    ctx.encode_gemv_silu_mul(w, d_g, d_u, d_y, accumulate=True)
+    assert np.array_equal(d_g.download(np.float32, k).view(np.uint32), g.view(np.uint32))  # the gate is left alone
+    Lfm2Ops(ctx).silu_mul_inplace(d_g, d_u, k)
+    ctx.encode_gemv(w, d_g, 0, d_z, 0, accumulate=True)
+    y, z = d_y.download(np.float32, m), d_z.download(np.float32, m)
+    assert np.array_equal(y.view(np.uint32), z.view(np.uint32))
+    sm = L.silu_mul(g, u)
+    assert rel_l2(y, 1 + L.gemv(dtype, wb, sm, m, k)) <= 1e-5  # silu_mul is bit-exact: the quantizer sees the oracle's very input
+    for b in (w, d_g, d_u, d_y, d_z):
+        b.free()

@@ -140,6 +140,19 @@ def test_greedy_generation_stays_on_the_device(ctx, oracle, tmp_path):
     model.free()
 
 
+def test_graph_replay_and_plain_launches_agree(ctx, oracle, tmp_path):
+    model, ref, cfg = load(ctx, oracle, tmp_path, seed=9)
+    replayed = [model.forward(t, p) for p, t in enumerate([4, 8, 15, 16])]
+    picks = model.generate_greedy(23, 4, 5)
+    model.reset()
+    model.set_graph_replay(False)
+    plain = [model.forward(t, p) for p, t in enumerate([4, 8, 15, 16])]
+    for a, b in zip(replayed, plain):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert model.generate_greedy(23, 4, 5).tolist() == picks.tolist()
+    model.free()
+
+
 def test_load_and_step_errors(ctx, oracle, tmp_path):
     model, ref, cfg = load(ctx, oracle, tmp_path, context=8, context_length=6)
     assert model.config["max_seq_len"] == 6  # min(context_size, lfm2.context_length), wick/src/model/lfm2.rs:121-125

@@ -21,8 +21,8 @@ int check_weight(wick_rocm_ctx* ctx, const wick_rocm_weight* w) {
     return WICK_ROCM_OK;
 }
 
-int ensure_scratch(wick_rocm_ctx* ctx, size_t q_bytes, size_t s_floats) {
-    if (q_bytes <= ctx->scratch_q_cap && s_floats <= ctx->scratch_s_cap) return WICK_ROCM_OK;
+int ensure_scratch(wick_rocm_ctx* ctx, size_t q_bytes, size_t s_floats, size_t f_floats = 0) {
+    if (q_bytes <= ctx->scratch_q_cap && s_floats <= ctx->scratch_s_cap && f_floats <= ctx->scratch_f_cap) return WICK_ROCM_OK;
     if (ctx->capturing)
         return fail(ctx, WICK_ROCM_ERR_STATE, "activation scratch too small during graph capture; call wick_rocm_reserve_scratch first");
     WR_HIP(ctx, hipStreamSynchronize(ctx->stream));  // earlier launches may still read the old scratch
@@ -37,6 +37,12 @@ int ensure_scratch(wick_rocm_ctx* ctx, size_t q_bytes, size_t s_floats) {
         ctx->scratch_s = nullptr, ctx->scratch_s_cap = 0;
         WR_HIP(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->scratch_s), s_floats * sizeof(float)));
         ctx->scratch_s_cap = s_floats;
+    }
+    if (f_floats > ctx->scratch_f_cap) {
+        if (ctx->scratch_f) WR_HIP(ctx, hipFree(ctx->scratch_f));
+        ctx->scratch_f = nullptr, ctx->scratch_f_cap = 0;
+        WR_HIP(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->scratch_f), f_floats * sizeof(float)));
+        ctx->scratch_f_cap = f_floats;
     }
     return WICK_ROCM_OK;
 }
@@ -125,6 +131,8 @@ void wick_rocm_ctx_destroy(wick_rocm_ctx* ctx) {
         }
         if (ctx->scratch_q) (void)hipFree(ctx->scratch_q);
         if (ctx->scratch_s) (void)hipFree(ctx->scratch_s);
+        if (ctx->scratch_f) (void)hipFree(ctx->scratch_f);
+        if (ctx->argmax_partial) (void)hipFree(ctx->argmax_partial);
         if (ctx->probe_sink) (void)hipFree(ctx->probe_sink);
         for (auto* v : {&ctx->timer.recs, &ctx->timer.spares})
             for (KernelTimer::Rec& r : *v) {
@@ -379,6 +387,54 @@ int wick_rocm_gemv_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* w
     return WICK_ROCM_OK;
 }
 
+namespace {
+
+// y_i (+)= W_i xform(x) for weights that share x (lock held).  The fused kernel applies the transform in its
+// prologue; shapes / types it does not take run the transform as a launch of its own into scratch first.
+int gemv_xform_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count, const float* x, int xform,
+                      const float* d_aux, float eps, int accumulate) {
+    if (!x || !d_aux) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv: null activation pointer");
+    GemvBatch b{};
+    if (int rc = make_batch(ctx, ws, d_ys, count, b)) return rc;
+    const uint32_t k = ws[0]->k;
+    const auto aligned16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16u == 0; };
+    if (ws[0]->type != kTypeQ6_K && pairs_kernel_applies(b, k) && aligned16(x) && aligned16(d_aux)) {
+        hipError_t e = launch_gemv_f32(ws[0]->type, b, k, x, accumulate, ctx->num_cus, ctx->launch(), xform, d_aux, eps);
+        return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "fused gemv launch");
+    }
+    if (int rc = ensure_scratch(ctx, k, k / 32u, k)) return rc;
+    hipError_t e;
+    if (xform == kXformRmsNorm) {
+        e = launch_rmsnorm(x, d_aux, ctx->scratch_f, 1, k, k, k, eps, ctx->launch());
+    } else {
+        e = hipMemcpyAsync(ctx->scratch_f, x, (size_t)k * sizeof(float), hipMemcpyDeviceToDevice, ctx->stream);
+        if (e == hipSuccess) e = launch_silu_mul(ctx->scratch_f, d_aux, k, ctx->launch());
+    }
+    if (e != hipSuccess) return fail_hip(ctx, e, "activation transform launch");
+    if (ws[0]->type == kTypeQ6_K) {
+        e = launch_quantize_q8_0(ctx->scratch_f, 1, k, k, ctx->scratch_q, ctx->scratch_s, ctx->launch());
+        if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
+        return q6k_gemv_locked(ctx, ws, d_ys, count, ctx->scratch_q, ctx->scratch_s, accumulate);
+    }
+    return gemv_f32_locked(ctx, b, ws[0]->type, k, ctx->scratch_f, accumulate);
+}
+
+}  // namespace
+
+int wick_rocm_gemv_rmsnorm_f32_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count,
+                                     const float* d_x, const float* d_norm_weight, float eps, int accumulate) {
+    WR_ENTER(ctx);
+    return gemv_xform_locked(ctx, ws, d_ys, count, d_x, kXformRmsNorm, d_norm_weight, eps, accumulate);
+}
+
+int wick_rocm_gemv_silu_mul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const float* d_gate, const float* d_up, float* d_y,
+                                int accumulate) {
+    WR_ENTER(ctx);
+    const wick_rocm_weight* ws[1] = {w};
+    float* ys[1] = {d_y};
+    return gemv_xform_locked(ctx, ws, ys, 1, d_gate, kXformSiluMul, d_up, 0.0f, accumulate);
+}
+
 int wick_rocm_gemv_f32_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count,
                              const float* d_x, size_t x_off_bytes, int accumulate) {
     WR_ENTER(ctx);
@@ -414,7 +470,7 @@ int wick_rocm_gemm_q8(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_
 int wick_rocm_reserve_scratch(wick_rocm_ctx* ctx, uint32_t max_n, uint32_t max_k) {
     WR_ENTER(ctx);
     if (max_k % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "reserve_scratch: max_k % 32 != 0");
-    return ensure_scratch(ctx, (size_t)max_n * max_k, (size_t)max_n * (max_k / 32u));
+    return ensure_scratch(ctx, (size_t)max_n * max_k, (size_t)max_n * (max_k / 32u), max_k);
 }
 
 int wick_rocm_matmul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const float* d_x, size_t x_off_bytes, uint32_t n,

@@ -35,6 +35,9 @@ struct GemvArgs {
     const int8_t* xq;   // [n][k]      (pre-quantized activations)
     const float* xs;    // [n][k/32]
     const float* xf;    // [n][x_stride] f32 activations, quantized in-kernel (FUSEQ variants)
+    const float* xaux;  // FUSEQ with a transform: RMSNorm weights [k] / the "up" vector [k]
+    float eps;          // RMSNorm epsilon
+    int xform;          // kXformNone / kXformRmsNorm / kXformSiluMul (host-side selector of the kernel variant)
     uint32_t x_stride;
     uint32_t k;
     uint32_t n;         // tokens (1 for decode)
@@ -68,6 +71,15 @@ constexpr int kFusedMaxK = 8192;
 //              slot and LDS operations of a wave execute in order, so no barrier is involved.
 enum { kDirect = 0, kDirectNT = 1, kSpan = 2 };
 
+// What the fused variant does to the f32 activations before quantizing them (XF):
+//   kXformRmsNorm  x * inv_rms * weight (cpu::rmsnorm, wick/src/backend/cpu.rs:577-594): the norm in front of
+//                  every projection of a decode step, folded into the projection's launch like the reference's
+//                  encode_gemv_rmsnorm_gate_up (wick/src/model/metal_lfm2.rs:1157-1186);
+//   kXformSiluMul  silu(x) * up (cpu::silu_mul_inplace, wick/src/backend/cpu.rs:668-673) in front of the FFN's
+//                  down projection.
+// Every workgroup redoes the transform on the whole vector (k <= 8192 floats, a few per thread): cheaper than a
+// launch of its own.
+
 // The leading scalar parameters repeat fields of `a` (x = a.xf for the fused variant, a.xq
 // otherwise; w0 / y0 / rows0 = weight 0 of the batch).  Passed on their own, at the front,
 // they are the kernel arguments the hardware preloads into SGPRs at wave launch (the build
@@ -75,11 +87,12 @@ enum { kDirect = 0, kDirectNT = 1, kSpan = 2 };
 // and weight loads of a single-weight launch is there at the first instruction, instead of
 // after one or two scalar-load round trips (~0.15 us each, on the critical path of a
 // 2-3 us launch).  The rest of `a` is still fetched the ordinary way, under those loads.
-template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI, int MODE>
+template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI, int MODE, int XF = kXformNone>
 __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kernel(const void* p_x, const uint8_t* p_w0, float* p_y0,
                                                                                   uint32_t p_k, uint32_t p_rows0,
                                                                                   uint32_t p_rows_per_wave, uint32_t p_total_waves,
                                                                                   int p_accumulate, GemvArgs a) {
+    static_assert(XF == kXformNone || FUSEQ, "activation transforms belong to the fused-quantizer variant");
     using PT = PairTraits<TYPE>;
     constexpr int RPW = 64 / LPR;  // rows per wave pass
     const uint32_t lane = threadIdx.x & 63u;
@@ -95,6 +108,7 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     // scalars of the argument block, and everything below overlaps with their latency.
     constexpr int kQuadRounds = kFusedMaxK / 4 / (64 * kFusedWaves);  // 8
     float4 xv[FUSEQ ? kQuadRounds : 1];
+    float4 av[XF != kXformNone ? kQuadRounds : 1];  // the transform's second operand, same quads
     if constexpr (FUSEQ) {
         const uint32_t quads = p_k >> 2;
 #pragma unroll
@@ -104,6 +118,15 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
             // within a round: clamped
             if (i > 0 && i * 64 * kFusedWaves >= quads) break;
             xv[i] = reinterpret_cast<const float4*>(p_x)[min(quad, quads - 1)];
+        }
+        if constexpr (XF != kXformNone) {
+            const float4* aux = reinterpret_cast<const float4*>(a.xaux);
+#pragma unroll
+            for (int i = 0; i < kQuadRounds; i++) {
+                const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
+                if (i > 0 && i * 64 * kFusedWaves >= quads) break;
+                av[i] = aux[min(quad, quads - 1)];
+            }
         }
         // keep the compiler from moving the weight loads in front of these
         asm volatile("" ::: "memory");
@@ -237,6 +260,41 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     // kernel), instead of every wave redoing it.  Only n = 1 uses this variant.
     if constexpr (FUSEQ) {
         const uint32_t quads = p_k >> 2;
+        if constexpr (XF == kXformSiluMul) {
+#pragma unroll
+            for (int i = 0; i < kQuadRounds; i++) {
+                if (i * 64 * kFusedWaves < quads) {
+                    xv[i].x = silu_mul(xv[i].x, av[i].x), xv[i].y = silu_mul(xv[i].y, av[i].y);
+                    xv[i].z = silu_mul(xv[i].z, av[i].z), xv[i].w = silu_mul(xv[i].w, av[i].w);
+                }
+            }
+        }
+        if constexpr (XF == kXformRmsNorm) {
+            // f64 sum of squares over the whole vector (clamped duplicates of the last quad left out), one barrier
+            __shared__ double sq[kFusedWaves];
+            double part = 0.0;
+#pragma unroll
+            for (int i = 0; i < kQuadRounds; i++) {
+                const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
+                if (i * 64 * kFusedWaves < quads && quad < quads) {
+                    const double x0 = xv[i].x, x1 = xv[i].y, x2 = xv[i].z, x3 = xv[i].w;
+                    part += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
+                }
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+            if (lane == 0) sq[threadIdx.x >> 6] = part;
+            __syncthreads();
+            const double total = (sq[0] + sq[1]) + (sq[2] + sq[3]);
+            const float inv_rms = (float)(1.0 / sqrt(total / (double)p_k + (double)a.eps));
+#pragma unroll
+            for (int i = 0; i < kQuadRounds; i++) {
+                if (i * 64 * kFusedWaves < quads) {
+                    xv[i].x = __fmul_rn(__fmul_rn(xv[i].x, inv_rms), av[i].x), xv[i].y = __fmul_rn(__fmul_rn(xv[i].y, inv_rms), av[i].y);
+                    xv[i].z = __fmul_rn(__fmul_rn(xv[i].z, inv_rms), av[i].z), xv[i].w = __fmul_rn(__fmul_rn(xv[i].w, inv_rms), av[i].w);
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < kQuadRounds; i++) {
             const uint32_t quad = threadIdx.x + i * 64 * kFusedWaves;
@@ -436,7 +494,19 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
         return launch_kernel(L, kFamGemv, kernel, grid, block, FUSEQ ? static_cast<const void*>(a.xf) : static_cast<const void*>(a.xq),
                              a.batch.w[0], a.batch.y[0], a.k, a.batch.row_end[0], a.rows_per_wave, a.total_waves, a.accumulate, a);
     };
-    if constexpr (NT == 1) {
+    if constexpr (NT == 1 && FUSEQ) {
+        // the activation transforms exist for the fused single-token variant only
+        auto with_xform = [&](auto xf) {
+            constexpr int XF = decltype(xf)::value;
+            if (mode == kSpan && multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSpan, XF>);
+            if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan, XF>);
+            if (multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSmall, XF>);
+            return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall, XF>);
+        };
+        if (a.xform == kXformRmsNorm) return with_xform(std::integral_constant<int, kXformRmsNorm>{});
+        if (a.xform == kXformSiluMul) return with_xform(std::integral_constant<int, kXformSiluMul>{});
+        return with_xform(std::integral_constant<int, kXformNone>{});
+    } else if constexpr (NT == 1) {
         if (mode == kSpan && multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSpan>);
         if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan>);
         if (multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSmall>);
@@ -510,10 +580,11 @@ bool pairs_kernel_applies(const GemvBatch& batch, uint32_t k) {
 
 // f32 activations in, quantized inside the GEMV kernel: one launch instead of two.
 hipError_t launch_gemv_f32(int type, const GemvBatch& batch, uint32_t k, const float* d_x, int accumulate, int num_cus,
-                           const Launch& L) {
+                           const Launch& L, int xform, const float* d_aux, float eps) {
     GemvArgs a{};
     a.batch = batch;
     a.xf = d_x;
+    a.xform = xform, a.xaux = d_aux, a.eps = eps;
     a.x_stride = k;
     a.k = k;
     a.n = 1;

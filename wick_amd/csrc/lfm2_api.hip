@@ -37,6 +37,10 @@ int wick_rocm_rmsnorm(wick_rocm_ctx* ctx, const float* d_x, const float* d_weigh
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "rmsnorm launch");
 }
 
+size_t wick_rocm_attention_scratch_floats(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim) {
+    return attention_scratch_floats(max_seq, n_heads, head_dim);
+}
+
 float wick_rocm_rope_theta_scale(uint32_t head_dim, float freq_base) { return powf(freq_base, -2.0f / (float)head_dim); }
 
 int wick_rocm_qk_norm_rope(wick_rocm_ctx* ctx, float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
@@ -60,7 +64,7 @@ int wick_rocm_attention_decode(wick_rocm_ctx* ctx, const float* d_q, const float
     if (!d_q || !d_k_cache || !d_v_cache || !d_out || !d_scores) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention: null device pointer");
     if (head_dim == 0 || head_dim % 4u != 0 || head_dim > 256u || n_heads == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0)
         return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "attention: head_dim must be a multiple of 4 and <= 256, n_kv_heads must divide n_heads");
-    if (misaligned(d_k_cache, 16)) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention: key cache must be 16-byte aligned");
+    if (misaligned(d_k_cache, 16) || misaligned(d_q, 16)) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention: q and the key cache must be 16-byte aligned");
     if (!d_pos && seq_len > max_seq) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention: seq_len beyond the cache");
     const float scale = 1.0f / sqrtf((float)head_dim);  // wick/src/model/lfm2.rs:862
     hipError_t e = launch_attention_decode(d_q, d_k_cache, d_v_cache, d_out, d_scores, seq_len, d_pos, max_seq, n_heads, n_kv_heads, head_dim, scale,
@@ -87,7 +91,12 @@ int wick_rocm_silu_mul(wick_rocm_ctx* ctx, float* d_gate, const float* d_up, uin
 int wick_rocm_argmax(wick_rocm_ctx* ctx, const float* d_logits, uint32_t n, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos) {
     WR_ENTER(ctx);
     if (!d_logits || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "argmax: null device pointer");
-    hipError_t e = launch_argmax(d_logits, n, d_out, d_token, d_pos, nullptr, 0, ctx->launch());
+    if (misaligned(d_logits, 16)) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "argmax: logits must be 16-byte aligned");
+    if (!ctx->argmax_partial) {
+        if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "argmax: first use inside a graph capture (call it once before capturing)");
+        WR_HIP(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->argmax_partial), kArgmaxPartials * sizeof(unsigned long long)));
+    }
+    hipError_t e = launch_argmax(d_logits, n, ctx->argmax_partial, d_out, d_token, d_pos, nullptr, 0, ctx->launch());
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
 }
 
@@ -119,10 +128,12 @@ struct wick_rocm_lfm2 {
     size_t bytes = 0;
     float theta_scale = 0.0f;
     // step scratch (device)
-    float *hidden = nullptr, *normed = nullptr, *proj = nullptr, *gated = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr,
-          *gate = nullptr, *up = nullptr, *scores = nullptr, *final_hidden = nullptr, *logits = nullptr;
+    float *hidden = nullptr, *proj = nullptr, *gated = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr,
+          *gate = nullptr, *up = nullptr, *scores = nullptr, *logits = nullptr;
     uint32_t *d_token = nullptr, *d_pos = nullptr, *d_pick = nullptr, *d_history = nullptr;
+    unsigned long long* d_argmax_partial = nullptr;
     wick_rocm_graph *g_logits = nullptr, *g_greedy = nullptr;
+    bool use_graph = true;
     std::mutex mu;
 };
 
@@ -181,16 +192,24 @@ void release(wick_rocm_ctx* ctx, wick_rocm_lfm2* m) {
     delete m;
 }
 
-// y (+)= W x for 1..3 weights that share x; one launch when their types agree.
-int gemv(wick_rocm_ctx* ctx, std::initializer_list<const wick_rocm_weight*> ws, std::initializer_list<float*> ys, const float* x, int accumulate) {
+// y_i = W_i rmsnorm(x) for 1..3 weights that share x, the norm folded into the projection's launch; one launch when
+// the weights' types agree.
+int gemv_normed(wick_rocm_ctx* ctx, std::initializer_list<const wick_rocm_weight*> ws, std::initializer_list<float*> ys, const float* x,
+                const float* norm_weight, float eps) {
     bool same = true;
     for (const wick_rocm_weight* w : ws) same = same && w->type == (*ws.begin())->type;
-    if (same) return wick_rocm_gemv_f32_multi(ctx, ws.begin(), ys.begin(), (uint32_t)ws.size(), x, 0, accumulate);
+    if (same) return wick_rocm_gemv_rmsnorm_f32_multi(ctx, ws.begin(), ys.begin(), (uint32_t)ws.size(), x, norm_weight, eps, 0);
     auto y = ys.begin();
-    for (const wick_rocm_weight* w : ws) {
-        if (int rc = wick_rocm_matmul_f32(ctx, w, x, 0, 1, w->k, *y++, 0, w->m, accumulate)) return rc;
+    for (const wick_rocm_weight* const& w : ws) {
+        float* const out = *y++;
+        if (int rc = wick_rocm_gemv_rmsnorm_f32_multi(ctx, &w, &out, 1, x, norm_weight, eps, 0)) return rc;
     }
     return WICK_ROCM_OK;
+}
+
+// y += W x (the residual form of the out / output projections).
+int gemv_residual(wick_rocm_ctx* ctx, const wick_rocm_weight* w, float* y, const float* x) {
+    return wick_rocm_matmul_f32(ctx, w, x, 0, 1, w->k, y, 0, w->m, 1);
 }
 
 // Enqueues one decode step that reads token / pos from the device: run_layers + the tied LM head
@@ -201,32 +220,28 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
     int rc = wick_rocm_embed_row(ctx, m->embd, 0, m->d_token, m->hidden);
     for (uint32_t i = 0; rc == 0 && i < c.n_layers; i++) {
         const LayerWeights& L = m->layers[i];
-        rc = wick_rocm_rmsnorm(ctx, m->hidden, L.attn_norm, m->normed, 1, hs, hs, hs, c.rms_norm_eps);
-        if (rc) break;
         if (L.n_kv == 0) {
-            if ((rc = gemv(ctx, {L.in_proj}, {m->proj}, m->normed, 0))) break;
+            if ((rc = gemv_normed(ctx, {L.in_proj}, {m->proj}, m->hidden, L.attn_norm, c.rms_norm_eps))) break;
             if ((rc = wick_rocm_shortconv_step(ctx, m->proj, L.conv_state, L.conv_w, m->gated, hs, c.conv_kernel_size))) break;
-            if ((rc = gemv(ctx, {L.out_proj}, {m->hidden}, m->gated, 1))) break;  // hidden += out_proj(gated)
+            if ((rc = gemv_residual(ctx, L.out_proj, m->hidden, m->gated))) break;
         } else {
-            if ((rc = gemv(ctx, {L.q, L.k, L.v}, {m->q, m->k, m->v}, m->normed, 0))) break;
+            if ((rc = gemv_normed(ctx, {L.q, L.k, L.v}, {m->q, m->k, m->v}, m->hidden, L.attn_norm, c.rms_norm_eps))) break;
             if ((rc = wick_rocm_qk_norm_rope(ctx, m->q, m->k, m->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, 0, m->d_pos, c.max_seq_len, hd, c.n_heads,
                                              L.n_kv, c.rms_norm_eps, m->theta_scale)))
                 break;
             if ((rc = wick_rocm_attention_decode(ctx, m->q, L.k_cache, L.v_cache, m->attn, m->scores, 0, m->d_pos, c.max_seq_len, c.n_heads, L.n_kv, hd)))
                 break;
-            if ((rc = gemv(ctx, {L.o}, {m->hidden}, m->attn, 1))) break;
+            if ((rc = gemv_residual(ctx, L.o, m->hidden, m->attn))) break;
         }
-        if ((rc = wick_rocm_rmsnorm(ctx, m->hidden, L.ffn_norm, m->normed, 1, hs, hs, hs, c.rms_norm_eps))) break;
-        if ((rc = gemv(ctx, {L.gate, L.up}, {m->gate, m->up}, m->normed, 0))) break;
-        if ((rc = wick_rocm_silu_mul(ctx, m->gate, m->up, c.intermediate_size))) break;
-        rc = gemv(ctx, {L.down}, {m->hidden}, m->gate, 1);
+        if ((rc = gemv_normed(ctx, {L.gate, L.up}, {m->gate, m->up}, m->hidden, L.ffn_norm, c.rms_norm_eps))) break;
+        rc = wick_rocm_gemv_silu_mul_f32(ctx, L.down, m->gate, m->up, m->hidden, 1);  // hidden += down(silu(gate) * up)
     }
     if (rc) return rc;
-    if ((rc = wick_rocm_rmsnorm(ctx, m->hidden, m->out_norm, m->final_hidden, 1, hs, hs, hs, c.rms_norm_eps))) return rc;
-    if ((rc = gemv(ctx, {m->embd}, {m->logits}, m->final_hidden, 0))) return rc;
+    if ((rc = gemv_normed(ctx, {m->embd}, {m->logits}, m->hidden, m->out_norm, c.rms_norm_eps))) return rc;
     if (!greedy) return WICK_ROCM_OK;
     std::lock_guard<std::mutex> lk(ctx->mu);
-    hipError_t e = launch_argmax(m->logits, c.vocab_size, m->d_pick, m->d_token, m->d_pos, m->d_history, c.max_seq_len, ctx->launch());
+    hipError_t e = launch_argmax(m->logits, c.vocab_size, m->d_argmax_partial, m->d_pick, m->d_token, m->d_pos, m->d_history, c.max_seq_len,
+                                 ctx->launch());
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
 }
 
@@ -246,6 +261,14 @@ int step_graph(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy, wick_rocm_gra
     }
     *out = g;
     return WICK_ROCM_OK;
+}
+
+// One step on the context's stream: a replay of the captured graph, or the same launches enqueued one by one.
+int run_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
+    if (!m->use_graph) return enqueue_step(ctx, m, greedy);
+    wick_rocm_graph* g = nullptr;
+    if (int rc = step_graph(ctx, m, greedy, &g)) return rc;
+    return wick_rocm_graph_launch(ctx, g);
 }
 
 int set_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t token, uint32_t pos) {
@@ -348,12 +371,12 @@ int wick_rocm_lfm2_load(wick_rocm_ctx* ctx, const wick_gguf* g, uint32_t context
     if ((rc = upload_weight(ctx, m, g, "token_embd.weight", c.vocab_size, hs, &m->embd))) return bail(rc);
 
     const uint32_t kv_max = (c.n_kv_heads ? c.n_kv_heads : 1) * hd;
-    if ((rc = alloc_t(ctx, m, hs, &m->hidden)) || (rc = alloc_t(ctx, m, hs, &m->normed)) || (rc = alloc_t(ctx, m, 3 * (size_t)hs, &m->proj)) ||
+    if ((rc = alloc_t(ctx, m, hs, &m->hidden)) || (rc = alloc_t(ctx, m, 3 * (size_t)hs, &m->proj)) ||
         (rc = alloc_t(ctx, m, hs, &m->gated)) || (rc = alloc_t(ctx, m, hs, &m->q)) || (rc = alloc_t(ctx, m, kv_max, &m->k)) ||
         (rc = alloc_t(ctx, m, kv_max, &m->v)) || (rc = alloc_t(ctx, m, hs, &m->attn)) || (rc = alloc_t(ctx, m, inter, &m->gate)) ||
-        (rc = alloc_t(ctx, m, inter, &m->up)) || (rc = alloc_t(ctx, m, (size_t)c.n_heads * c.max_seq_len, &m->scores)) ||
-        (rc = alloc_t(ctx, m, hs, &m->final_hidden)) || (rc = alloc_t(ctx, m, c.vocab_size, &m->logits)) || (rc = alloc_t(ctx, m, 1, &m->d_token)) ||
-        (rc = alloc_t(ctx, m, 1, &m->d_pos)) || (rc = alloc_t(ctx, m, 1, &m->d_pick)) || (rc = alloc_t(ctx, m, c.max_seq_len, &m->d_history)))
+        (rc = alloc_t(ctx, m, inter, &m->up)) || (rc = alloc_t(ctx, m, attention_scratch_floats(c.max_seq_len, c.n_heads, hd), &m->scores)) ||
+        (rc = alloc_t(ctx, m, c.vocab_size, &m->logits)) || (rc = alloc_t(ctx, m, 1, &m->d_token)) ||
+        (rc = alloc_t(ctx, m, 1, &m->d_pos)) || (rc = alloc_t(ctx, m, 1, &m->d_pick)) || (rc = alloc_t(ctx, m, kArgmaxPartials, &m->d_argmax_partial)) || (rc = alloc_t(ctx, m, c.max_seq_len, &m->d_history)))
         return bail(rc);
     // GEMVs that cannot take the fused-quantizer kernel quantize into the context's scratch: size it before any capture
     if ((rc = wick_rocm_reserve_scratch(ctx, 1, hs > inter ? hs : inter))) return bail(rc);
@@ -398,14 +421,19 @@ int wick_rocm_lfm2_reset(wick_rocm_ctx* ctx, wick_rocm_lfm2* model) {
     return WICK_ROCM_OK;
 }
 
+int wick_rocm_lfm2_set_graph_replay(wick_rocm_lfm2* model, int enabled) {
+    if (!model) return WICK_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lk(model->mu);
+    model->use_graph = enabled != 0;
+    return WICK_ROCM_OK;
+}
+
 int wick_rocm_lfm2_forward(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t token, uint32_t pos, float* logits) {
     if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
     std::lock_guard<std::mutex> lk(model->mu);
     if (int rc = check_step(ctx, model, token, pos, 1)) return rc;
-    wick_rocm_graph* g = nullptr;
-    if (int rc = step_graph(ctx, model, false, &g)) return rc;
     if (int rc = set_step(ctx, model, token, pos)) return rc;
-    if (int rc = wick_rocm_graph_launch(ctx, g)) return rc;
+    if (int rc = run_step(ctx, model, false)) return rc;
     if (logits) return wick_rocm_download(ctx, logits, model->logits, (size_t)model->cfg.vocab_size * sizeof(float));
     return wick_rocm_sync(ctx);
 }
@@ -420,15 +448,12 @@ int wick_rocm_lfm2_generate_greedy(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, ui
     if (n == 0) return WICK_ROCM_OK;
     std::lock_guard<std::mutex> lk(model->mu);
     if (int rc = check_step(ctx, model, token, pos, n)) return rc;
-    wick_rocm_graph* g = nullptr;
-    if (int rc = step_graph(ctx, model, true, &g)) return rc;
     if (int rc = set_step(ctx, model, token, pos)) return rc;
     for (uint32_t i = 0; i < n; i++)  // the pick of step i is written to the device-side token and position pos + i of the history
-        if (int rc = wick_rocm_graph_launch(ctx, g)) return rc;
+        if (int rc = run_step(ctx, model, true)) return rc;
     return wick_rocm_download(ctx, out_tokens, model->d_history + pos, (size_t)n * sizeof(uint32_t));
 }
 
 const float* wick_rocm_lfm2_logits_device(const wick_rocm_lfm2* model) { return model ? model->logits : nullptr; }
-const float* wick_rocm_lfm2_hidden_device(const wick_rocm_lfm2* model) { return model ? model->final_hidden : nullptr; }
 
 }  // extern "C"

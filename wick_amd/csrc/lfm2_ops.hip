@@ -10,37 +10,14 @@
 //
 // "pos" and "token" may live in device memory (d_pos / d_token non-null): a captured graph of
 // the step can then be replayed for every token without new kernel arguments.
+#include <type_traits>
+
 #include "wick_rocm_device.h"
 #include "wick_rocm_internal.h"
 
 namespace wick_rocm {
 
 namespace {
-
-__device__ __forceinline__ float bits_f(uint32_t u) { return __uint_as_float(u); }
-
-// ggml_expf (wick/src/backend/cpu.rs:604-652), operation for operation: bit-exact.
-__device__ __forceinline__ float ggml_expf(float x) {
-    const float R = bits_f(0x4B400000u), LOG2E = bits_f(0x3FB8AA3Bu);
-    const float LN2_HI = bits_f(0x3F317200u), LN2_LO = bits_f(0x35BFBE8Eu);
-    const float C1 = bits_f(0x3F7FFFF6u), C2 = bits_f(0x3EFFFEDBu), C3 = bits_f(0x3E2AAF33u);
-    const float C4 = bits_f(0x3D2B9F17u), C5 = bits_f(0x3C072010u);
-    const float z = __fadd_rn(R, __fmul_rn(x, LOG2E));
-    const float n = __fsub_rn(z, R);
-    const float b = __fsub_rn(__fsub_rn(x, __fmul_rn(n, LN2_HI)), __fmul_rn(n, LN2_LO));
-    const uint32_t e = __float_as_uint(z) << 23;
-    const float k = bits_f(e + 0x3F800000u);
-    const float u = __fmul_rn(b, b);
-    const float inner = __fadd_rn(__fadd_rn(C2, __fmul_rn(C3, b)), __fmul_rn(__fadd_rn(C4, __fmul_rn(C5, b)), u));
-    const float j = __fadd_rn(__fmul_rn(C1, b), __fmul_rn(inner, u));
-    const float abs_n = fabsf(n);
-    if (abs_n <= 126.0f) return __fadd_rn(k, __fmul_rn(j, k));
-    if (abs_n > 192.0f) return n > 0.0f ? __builtin_inff() : 0.0f;
-    const uint32_t d = n <= 0.0f ? 0x82000000u : 0u;
-    const float s1 = bits_f(d + 0x7f000000u);
-    const float s2 = bits_f(e - d);
-    return __fmul_rn(__fadd_rn(s2, __fmul_rn(s2, j)), s1);
-}
 
 __device__ __forceinline__ double wave_sum_f64(double v) {
 #pragma unroll
@@ -252,6 +229,169 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttentionArgs a) 
     }
 }
 
+// Long sequences: the same attention split over the sequence.  Workgroup (head, split) walks chunks
+// split, split + splits, ... of kAttnChunk positions with a running maximum and rescaled sums (the usual
+// streaming softmax), reading whole cache rows with consecutive lanes (a float4 per lane), and leaves
+// {max, sum, acc[head_dim]} in scratch; attention_combine_kernel merges the partials of a head.
+// Against the single-workgroup kernel above only the summation order and the point where exp() is taken
+// change: results agree to a few 1e-7.  head_dim in {32, 64, 128, 256}.
+constexpr uint32_t kAttnChunk = 64;       // positions a workgroup handles per pass
+constexpr uint32_t kAttnMaxSplits = 64;   // workgroups per head; contexts beyond 64 * 64 positions make them loop
+
+__device__ __forceinline__ float block_max_f32(float v, float* slots) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(slots[0], slots[1]), fmaxf(slots[2], slots[3]));
+}
+
+__device__ __forceinline__ float block_sum_f32(float v, float* slots) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (slots[0] + slots[1]) + (slots[2] + slots[3]);
+}
+
+template <int HD>
+__global__ __launch_bounds__(256) void attention_split_kernel(AttentionArgs a, uint32_t splits) {
+    constexpr uint32_t LR = HD / 4;                  // lanes per cache row
+    constexpr uint32_t RPP = 256 / LR;               // rows per pass of the block
+    constexpr uint32_t KROWS = kAttnChunk / RPP;     // key rows per thread and chunk
+    constexpr uint32_t KB = KROWS < 8 ? KROWS : 8;   // ... loaded in batches of
+    constexpr uint32_t VG = 256 / HD;                // position groups of the value sum
+    constexpr uint32_t VROWS = kAttnChunk / VG;
+    constexpr uint32_t VB = VROWS < 16 ? VROWS : 16;
+    static_assert(KROWS >= 1 && KROWS % KB == 0 && VROWS % VB == 0, "chunk does not tile");
+    __shared__ float sc[kAttnChunk];
+    __shared__ float red[256];
+    __shared__ float slots[4];
+    const uint32_t h = blockIdx.x / splits, split = blockIdx.x % splits;
+    const uint32_t kv_dim = a.n_kv_heads * HD;
+    uint32_t seq = a.d_pos ? *a.d_pos + 1u : a.seq_len;
+    if (seq > a.max_seq) seq = a.max_seq;
+    if (split * kAttnChunk >= seq) return;  // the combine step derives the number of partials from seq as well
+    const uint32_t kvh = h / (a.n_heads / a.n_kv_heads);
+    const float* kbase = a.k_cache + (size_t)kvh * HD;
+    const float* vbase = a.v_cache + (size_t)kvh * HD;
+    const uint32_t tid = threadIdx.x, quad = tid % LR, prow = tid / LR, d = tid % HD, g = tid / HD;
+    const float4 q4 = reinterpret_cast<const float4*>(a.q + (size_t)h * HD)[quad];
+    const uint32_t last = seq - 1u;
+
+    float m_run = -__builtin_inff(), l_run = 0.0f, acc = 0.0f;
+    for (uint32_t c = split; c * kAttnChunk < seq; c += splits) {
+        const uint32_t t0 = c * kAttnChunk;
+        const uint32_t nt = seq - t0 < kAttnChunk ? seq - t0 : kAttnChunk;
+        // Loads are unconditional (rows past the end are clamped to the last one and masked afterwards), so the
+        // compiler can put a whole batch of them in flight instead of one round trip per row.
+#pragma unroll
+        for (uint32_t i = 0; i < KROWS; i += KB) {
+            float4 kv[KB];
+#pragma unroll
+            for (uint32_t j = 0; j < KB; j++) {
+                const uint32_t row = t0 + prow + (i + j) * RPP;
+                kv[j] = reinterpret_cast<const float4*>(kbase + (size_t)(row < last ? row : last) * kv_dim)[quad];
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < KB; j++) {
+                const uint32_t r = prow + (i + j) * RPP;
+                float p = q4.x * kv[j].x + q4.y * kv[j].y + q4.z * kv[j].z + q4.w * kv[j].w;
+#pragma unroll
+                for (uint32_t off = LR / 2; off > 0; off >>= 1) p += __shfl_xor(p, off, 64);
+                if (quad == 0) sc[r] = r < nt ? p * a.scale : -__builtin_inff();
+            }
+        }
+        __syncthreads();
+        const float s = tid < kAttnChunk ? sc[tid] : -__builtin_inff();
+        const float m_new = fmaxf(m_run, block_max_f32(s, slots));
+        const float e = tid < nt ? ggml_expf(s - m_new) : 0.0f;
+        if (tid < kAttnChunk) sc[tid] = e;  // every thread read its own score above; positions past the end weigh 0
+        const float l_chunk = block_sum_f32(e, slots);  // its barriers publish sc[]
+        const float corr = ggml_expf(m_run - m_new);    // 0 on the first chunk (m_run = -inf)
+        l_run = l_run * corr + l_chunk;
+        acc *= corr;
+#pragma unroll
+        for (uint32_t i = 0; i < VROWS; i += VB) {
+            float vv[VB];
+#pragma unroll
+            for (uint32_t j = 0; j < VB; j++) {
+                const uint32_t row = t0 + g + (i + j) * VG;
+                vv[j] = vbase[(size_t)(row < last ? row : last) * kv_dim + d];
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < VB; j++) acc += sc[g + (i + j) * VG] * vv[j];
+        }
+        m_run = m_new;
+        __syncthreads();  // sc[] is rewritten by the next chunk
+    }
+    red[tid] = acc;
+    __syncthreads();
+    float* part = a.scores + ((size_t)h * splits + split) * (HD + 2);
+    if (tid < HD) {
+        float r = red[tid];
+#pragma unroll
+        for (uint32_t p = 1; p < VG; p++) r += red[p * HD + tid];
+        part[2 + tid] = r;
+    }
+    if (tid == 0) part[0] = m_run, part[1] = l_run;
+}
+
+// Merges the partials of one head: the first wave turns the (max, sum) pairs into weights, then every thread sums
+// its share of the weighted accumulators (again with its loads batched).
+template <int HD>
+__global__ __launch_bounds__(256) void attention_combine_kernel(AttentionArgs a, uint32_t splits) {
+    constexpr uint32_t G = 256 / HD;  // partial groups
+    __shared__ float wts[kAttnMaxSplits];
+    __shared__ float red[256];
+    __shared__ float total;
+    const uint32_t h = blockIdx.x, tid = threadIdx.x, d = tid % HD, grp = tid / HD;
+    uint32_t seq = a.d_pos ? *a.d_pos + 1u : a.seq_len;
+    if (seq > a.max_seq) seq = a.max_seq;
+    uint32_t active = (seq + kAttnChunk - 1) / kAttnChunk;
+    active = active < splits ? active : splits;
+    const float* parts = a.scores + (size_t)h * splits * (HD + 2);
+    if (tid < 64) {  // splits <= 64: one lane per partial
+        const bool on = tid < active;
+        const float m_i = on ? parts[(size_t)tid * (HD + 2)] : -__builtin_inff();
+        const float l_i = on ? parts[(size_t)tid * (HD + 2) + 1] : 0.0f;
+        float m = m_i;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+        const float w = on ? ggml_expf(m_i - m) : 0.0f;
+        float l = l_i * w;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off, 64);
+        wts[tid] = w;
+        if (tid == 0) total = l;
+    }
+    __syncthreads();
+    float o = 0.0f;
+    for (uint32_t i0 = grp; i0 < active; i0 += 4 * G) {
+        float v[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; j++) {
+            const uint32_t i = i0 + j * G;
+            v[j] = parts[(size_t)(i < active ? i : i0) * (HD + 2) + 2 + d];
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 4; j++) {
+            const uint32_t i = i0 + j * G;
+            o += i < active ? v[j] * wts[i] : 0.0f;
+        }
+    }
+    red[tid] = o;
+    __syncthreads();
+    if (tid < HD) {
+        float r = red[tid];
+#pragma unroll
+        for (uint32_t p = 1; p < G; p++) r += red[p * HD + tid];
+        a.out[(size_t)h * HD + tid] = active ? __fdiv_rn(r, total) : 0.0f;
+    }
+}
+
 // ---- gated short convolution, one step ---------------------------------------------------
 // forward_conv_block's middle (wick/src/model/lfm2.rs:694-726): proj = [b | c | x]; bx = b*x;
 // out = c * (sum_k buffer[k][ch]*w[ch][k] + bx*w[ch][K-1]); the rolling buffer shifts by one slot and takes bx.
@@ -286,7 +426,8 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(float* __restrict__ gate,
 
 // ---- greedy pick ----------------------------------------------------------------------
 // cpu_argmax (wick/src/sampler.rs:7-19): NaN counts as -inf, values order by f32::total_cmp, the LAST of
-// equal maxima wins; bit-exact.  One 1024-thread block.  Optionally publishes the pick as the next step's
+// equal maxima wins; bit-exact.  Two small launches (64 blocks, then one wave over their partial keys): a single
+// block would spend 20 us walking a 65536-entry vocabulary.  Optionally publishes the pick as the next step's
 // token and advances the device-side position.
 __device__ __forceinline__ unsigned long long argmax_key(float f, uint32_t index) {
     if (f != f) f = -__builtin_inff();
@@ -296,23 +437,60 @@ __device__ __forceinline__ unsigned long long argmax_key(float f, uint32_t index
     return ((unsigned long long)ordered << 32) | index;          // equal values: the larger index wins
 }
 
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ x, uint32_t n, uint32_t* __restrict__ out,
-                                                      uint32_t* __restrict__ d_token, uint32_t* __restrict__ d_pos,
-                                                      uint32_t* __restrict__ d_history, uint32_t history_len) {
-    __shared__ unsigned long long red[1024];
+constexpr uint32_t kArgmaxBlocks = 64;
+
+// Stage 1: every block leaves the best key of its slice (float4 loads, all of a thread's loads in flight at once).
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ x, uint32_t n, unsigned long long* __restrict__ partial) {
+    __shared__ unsigned long long red[4];
     unsigned long long best = 0ull;  // below every real key
-    for (uint32_t i = threadIdx.x; i < n; i += 1024) {
-        const unsigned long long key = argmax_key(x[i], i);
-        best = key > best ? key : best;
+    const uint32_t quads = n >> 2, stride = gridDim.x * 256u;
+    for (uint32_t q0 = blockIdx.x * 256u + threadIdx.x; q0 < quads; q0 += 4u * stride) {
+        float4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t q = q0 + j * stride;
+            v[j] = reinterpret_cast<const float4*>(x)[q < quads ? q : q0];  // clamped: a repeated quad cannot change the maximum
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t q = q0 + j * stride;
+            const uint32_t i = 4u * (q < quads ? q : q0);
+            const unsigned long long k0 = argmax_key(v[j].x, i), k1 = argmax_key(v[j].y, i + 1), k2 = argmax_key(v[j].z, i + 2),
+                                     k3 = argmax_key(v[j].w, i + 3);
+            const unsigned long long a = k0 > k1 ? k0 : k1, b = k2 > k3 ? k2 : k3, c = a > b ? a : b;
+            best = c > best ? c : best;
+        }
     }
-    red[threadIdx.x] = best;
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {  // the last n % 4 elements
+        const uint32_t i = (n & ~3u) + threadIdx.x;
+        const unsigned long long k = argmax_key(x[i], i);
+        best = k > best ? k : best;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long o = __shfl_xor(best, off, 64);
+        best = o > best ? o : best;
+    }
+    if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = best;
     __syncthreads();
-    for (uint32_t off = 512; off > 0; off >>= 1) {
-        if (threadIdx.x < off) red[threadIdx.x] = red[threadIdx.x] > red[threadIdx.x + off] ? red[threadIdx.x] : red[threadIdx.x + off];
-        __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned long long a = red[0] > red[1] ? red[0] : red[1], b = red[2] > red[3] ? red[2] : red[3];
+        partial[blockIdx.x] = a > b ? a : b;
+    }
+}
+
+// Stage 2: one wave merges the partial keys and publishes the pick.
+__global__ __launch_bounds__(64) void argmax_final_kernel(const unsigned long long* __restrict__ partial, uint32_t blocks, uint32_t n,
+                                                          uint32_t* __restrict__ out, uint32_t* __restrict__ d_token, uint32_t* __restrict__ d_pos,
+                                                          uint32_t* __restrict__ d_history, uint32_t history_len) {
+    unsigned long long best = threadIdx.x < blocks ? partial[threadIdx.x] : 0ull;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long o = __shfl_xor(best, off, 64);
+        best = o > best ? o : best;
     }
     if (threadIdx.x == 0) {
-        const uint32_t pick = n ? (uint32_t)(red[0] & 0xffffffffull) : 0u;
+        const uint32_t pick = n ? (uint32_t)(best & 0xffffffffull) : 0u;
         out[0] = pick;
         if (d_token) *d_token = pick;
         if (d_pos) {
@@ -360,7 +538,35 @@ hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, con
                                    uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
                                    uint32_t head_dim, float scale, const Launch& L) {
     AttentionArgs a{d_q, d_k_cache, d_v_cache, d_out, d_scores, d_pos, seq_len, max_seq, n_heads, n_kv_heads, head_dim, scale};
+    const uint32_t splits = attention_splits(max_seq);
+    auto split_path = [&](auto hd) -> hipError_t {
+        constexpr int HD = decltype(hd)::value;
+        hipError_t e = launch_kernel(L, kFamOther, attention_split_kernel<HD>, dim3(n_heads * splits), dim3(256), a, splits);
+        if (e != hipSuccess) return e;
+        return launch_kernel(L, kFamOther, attention_combine_kernel<HD>, dim3(n_heads), dim3(256), a, splits);
+    };
+    // a short context gains nothing from the second launch
+    if (max_seq > 256u) {
+        switch (head_dim) {
+            case 32: return split_path(std::integral_constant<int, 32>{});
+            case 64: return split_path(std::integral_constant<int, 64>{});
+            case 128: return split_path(std::integral_constant<int, 128>{});
+            case 256: return split_path(std::integral_constant<int, 256>{});
+            default: break;
+        }
+    }
     return launch_kernel(L, kFamOther, attention_decode_kernel, dim3(n_heads), dim3(256), a);
+}
+
+uint32_t attention_splits(uint32_t max_seq) {
+    const uint32_t chunks = (max_seq + kAttnChunk - 1) / kAttnChunk;
+    return chunks < 1u ? 1u : (chunks < kAttnMaxSplits ? chunks : kAttnMaxSplits);
+}
+
+size_t attention_scratch_floats(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim) {
+    const size_t single = (size_t)n_heads * max_seq;                                        // scores of the one-workgroup kernel
+    const size_t split = (size_t)n_heads * attention_splits(max_seq) * (head_dim + 2);      // {max, sum, acc[head_dim]} per partial
+    return single > split ? single : split;
 }
 
 hipError_t launch_shortconv_step(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
@@ -374,9 +580,12 @@ hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const L
     return launch_kernel(L, kFamOther, silu_mul_kernel, dim3((n + 255u) / 256u), dim3(256), d_gate, d_up, n);
 }
 
-hipError_t launch_argmax(const float* d_x, uint32_t n, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos, uint32_t* d_history,
-                         uint32_t history_len, const Launch& L) {
-    return launch_kernel(L, kFamOther, argmax_kernel, dim3(1), dim3(1024), d_x, n, d_out, d_token, d_pos, d_history, history_len);
+hipError_t launch_argmax(const float* d_x, uint32_t n, unsigned long long* d_partial, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos,
+                         uint32_t* d_history, uint32_t history_len, const Launch& L) {
+    const uint32_t blocks = n >= 4096u ? kArgmaxBlocks : 1u;
+    hipError_t e = launch_kernel(L, kFamOther, argmax_partial_kernel, dim3(blocks), dim3(256), d_x, n, d_partial);
+    if (e != hipSuccess) return e;
+    return launch_kernel(L, kFamOther, argmax_final_kernel, dim3(1), dim3(64), d_partial, blocks, n, d_out, d_token, d_pos, d_history, history_len);
 }
 
 hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L) {

@@ -24,9 +24,12 @@ struct wick_rocm_ctx {
     float* scratch_s = nullptr;
     size_t scratch_q_cap = 0;  // bytes
     size_t scratch_s_cap = 0;  // floats
+    float* scratch_f = nullptr;  // one transformed f32 activation vector (norm / gate folded into a GEMV that cannot take the fused kernel)
+    size_t scratch_f_cap = 0;  // floats
     uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
     KernelTimer timer;
     int64_t gemv_direct_max_bytes = -1;
+    unsigned long long* argmax_partial = nullptr;  // kArgmaxPartials keys for wick_rocm_argmax
     void* probe_sink = nullptr;  // 64 bytes the rate probes may (never do) write to
     Launch launch() { return Launch{stream, &timer, gemv_direct_max_bytes}; }
 };

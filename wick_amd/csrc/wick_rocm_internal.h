@@ -86,8 +86,10 @@ hipError_t launch_gemv(int type, const GemvBatch& batch, uint32_t k, const int8_
 // Decode GEMV straight from f32 activations (Q8_0 quantization fused into the
 // kernel).  Only when pairs_kernel_applies() and d_x is 16-byte aligned.
 bool pairs_kernel_applies(const GemvBatch& batch, uint32_t k);
+// xform: what is done to x before it is quantized (d_aux: the RMSNorm weights / the "up" vector, k floats, 16-byte aligned).
+enum { kXformNone = 0, kXformRmsNorm = 1, kXformSiluMul = 2 };
 hipError_t launch_gemv_f32(int type, const GemvBatch& batch, uint32_t k, const float* d_x, int accumulate, int num_cus,
-                           const Launch& L);
+                           const Launch& L, int xform = kXformNone, const float* d_aux = nullptr, float eps = 0.0f);
 
 // Q6_K decode GEMV, one token (gemv_q6k.hip).  k % 256 == 0, k <= 8192; the weight allocation is padded by
 // 16 bytes; y[row * y_row_stride].  launch_group_dots_q6k is its parity hook: out[i * (k/16) + g] = exact i32 dot of 16-weight group g.
@@ -128,15 +130,20 @@ hipError_t launch_rmsnorm(const float* d_x, const float* d_weight, float* d_y, u
 hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm, float* d_k_cache,
                                float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
                                uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L);
+// d_scores is scratch of attention_scratch_floats(max_seq, n_heads, head_dim) floats.
+uint32_t attention_splits(uint32_t max_seq);
+size_t attention_scratch_floats(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim);
 hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scores,
                                    uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
                                    uint32_t head_dim, float scale, const Launch& L);
 hipError_t launch_shortconv_step(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
                                  uint32_t kernel_size, const Launch& L);
 hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const Launch& L);
-// d_history[pos] = pick (pos = *d_pos before it is advanced), when given.
-hipError_t launch_argmax(const float* d_x, uint32_t n, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos, uint32_t* d_history,
-                         uint32_t history_len, const Launch& L);
+// d_history[pos] = pick (pos = *d_pos before it is advanced), when given.  d_partial: scratch of kArgmaxPartials keys, 8-byte aligned;
+// d_x 16-byte aligned.
+constexpr uint32_t kArgmaxPartials = 64;
+hipError_t launch_argmax(const float* d_x, uint32_t n, unsigned long long* d_partial, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos,
+                         uint32_t* d_history, uint32_t history_len, const Launch& L);
 hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L);
 hipError_t launch_advance_pos(uint32_t* d_pos, const Launch& L);
 

@@ -234,3 +234,43 @@ class GgufFile:
         off, rows, cols, t = C.c_uint64(), C.c_uint64(), C.c_uint64(), C.c_int()
         _check(_lib().wick_gguf_tensor_meta(self._h, name.encode(), C.byref(off), C.byref(rows), C.byref(cols), C.byref(t)))
         return off.value, rows.value, cols.value, t.value
+
+
+# ---- writing (synthetic models for benchmarks; the reference only reads GGUF) ----------------------------
+
+def _gstr(s) -> bytes:
+    b = s if isinstance(s, bytes) else str(s).encode()
+    return len(b).to_bytes(8, "little") + b
+
+
+def _gvalue(type_id: int, v) -> bytes:
+    if type_id in _NP:
+        return np.array(v, dtype=_NP[type_id]).tobytes()
+    if type_id == T_STRING:
+        return _gstr(v)
+    if type_id == T_ARRAY:
+        elem_type, items = v
+        return int(elem_type).to_bytes(4, "little") + len(items).to_bytes(8, "little") + b"".join(_gvalue(elem_type, x) for x in items)
+    raise ValueError(f"unknown GGUF value type {type_id}")
+
+
+def build_image(metadata, tensors, alignment: int = 32) -> bytes:
+    """A GGUF v3 image from ``[(key, value_type, value)]`` and ``[(name, dims, ggml_type, bytes-like)]``
+    (dims in GGUF order: ne0 first).  Tensor data is laid out in the given order, each padded to `alignment`."""
+    head = bytearray(b"GGUF" + (3).to_bytes(4, "little") + len(tensors).to_bytes(8, "little") + len(metadata).to_bytes(8, "little"))
+    for key, t, v in metadata:
+        head += _gstr(key) + int(t).to_bytes(4, "little") + _gvalue(t, v)
+    blobs = [np.ascontiguousarray(d).view(np.uint8).ravel() if isinstance(d, np.ndarray) else np.frombuffer(bytes(d), np.uint8) for *_, d in tensors]
+    rel = 0
+    for (name, dims, gt, _), blob in zip(tensors, blobs):
+        head += _gstr(name) + len(dims).to_bytes(4, "little") + b"".join(int(d).to_bytes(8, "little") for d in dims)
+        head += int(gt).to_bytes(4, "little") + rel.to_bytes(8, "little")
+        rel += -(-blob.size // alignment) * alignment
+    data_offset = -(-len(head) // alignment) * alignment
+    out = np.zeros(data_offset + rel, np.uint8)
+    out[: len(head)] = np.frombuffer(bytes(head), np.uint8)
+    at = data_offset
+    for blob in blobs:
+        out[at: at + blob.size] = blob
+        at += -(-blob.size // alignment) * alignment
+    return out.tobytes()

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "wick_rocm_qk_norm_rope": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32, _F, _F]),
     "wick_rocm_rope_theta_scale": (_F, [_U32, _F]),
     "wick_rocm_attention_decode": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32]),
+    "wick_rocm_attention_scratch_floats": (C.c_size_t, [_U32, _U32, _U32]),
     "wick_rocm_shortconv_step": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32]),
     "wick_rocm_silu_mul": (C.c_int, [_P, _P, _P, _U32]),
     "wick_rocm_argmax": (C.c_int, [_P, _P, _U32, _P, _P, _P]),
@@ -38,11 +39,11 @@ _SIGNATURES = {
     "wick_rocm_lfm2_layer_kv_heads": (C.c_int, [_P, _U32, C.POINTER(_U32)]),
     "wick_rocm_lfm2_gpu_memory_bytes": (C.c_size_t, [_P]),
     "wick_rocm_lfm2_reset": (C.c_int, [_P, _P]),
+    "wick_rocm_lfm2_set_graph_replay": (C.c_int, [_P, C.c_int]),
     "wick_rocm_lfm2_forward": (C.c_int, [_P, _P, _U32, _U32, _P]),
     "wick_rocm_lfm2_forward_greedy": (C.c_int, [_P, _P, _U32, _U32, C.POINTER(_U32)]),
     "wick_rocm_lfm2_generate_greedy": (C.c_int, [_P, _P, _U32, _U32, _U32, _P]),
     "wick_rocm_lfm2_logits_device": (_P, [_P]),
-    "wick_rocm_lfm2_hidden_device": (_P, [_P]),
 }
 
 _bound = False
@@ -58,6 +59,10 @@ def _lib() -> C.CDLL:
             fn.argtypes = args
         _bound = True
     return lib
+
+
+def attention_scratch_floats(max_seq: int, n_heads: int, head_dim: int) -> int:
+    return int(_lib().wick_rocm_attention_scratch_floats(max_seq, n_heads, head_dim))
 
 
 def rope_theta_scale(head_dim: int, freq_base: float) -> float:
@@ -131,6 +136,9 @@ class RocmLfm2Model:
     def reset(self) -> None:
         self.ctx._check(self._l.wick_rocm_lfm2_reset(self.ctx._h, self._h))
 
+    def set_graph_replay(self, enabled: bool) -> None:
+        self.ctx._check(self._l.wick_rocm_lfm2_set_graph_replay(self._h, int(enabled)))
+
     def forward(self, token: int, pos: int) -> np.ndarray:
         logits = np.empty(self.config["vocab_size"], np.float32)
         self.ctx._check(self._l.wick_rocm_lfm2_forward(self.ctx._h, self._h, token, pos, logits.ctypes.data))
@@ -144,10 +152,4 @@ class RocmLfm2Model:
     def generate_greedy(self, token: int, pos: int, n: int) -> np.ndarray:
         out = np.empty(n, np.uint32)
         self.ctx._check(self._l.wick_rocm_lfm2_generate_greedy(self.ctx._h, self._h, token, pos, n, out.ctypes.data))
-        return out
-
-    def hidden(self) -> np.ndarray:
-        """Final normed hidden state of the last step."""
-        out = np.empty(self.config["hidden_size"], np.float32)
-        self.ctx._check(self.ctx._lib.wick_rocm_download(self.ctx._h, out.ctypes.data, self._l.wick_rocm_lfm2_hidden_device(self._h), out.nbytes))
         return out

@@ -86,6 +86,8 @@ _SIGNATURES = {
     "wick_rocm_gemm_q8": (C.c_int, [_P, _P, _P, _P, C.c_uint32, _P, C.c_uint32, C.c_int, C.c_int]),
     "wick_rocm_matmul_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_uint32, C.c_uint32, _P, C.c_size_t, C.c_uint32, C.c_int]),
     "wick_rocm_gemv_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, C.c_size_t, C.c_int]),
+    "wick_rocm_gemv_rmsnorm_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, _P, C.c_float, C.c_int]),
+    "wick_rocm_gemv_silu_mul_f32": (C.c_int, [_P, _P, _P, _P, _P, C.c_int]),
     "wick_rocm_reserve_scratch": (C.c_int, [_P, C.c_uint32, C.c_uint32]),
     "wick_rocm_block_dots_i32": (C.c_int, [_P, _P, _P, C.c_uint32, _P]),
     "wick_rocm_graph_begin": (C.c_int, [_P]),
@@ -293,6 +295,17 @@ class RocmContext:
         wa = (_P * n)(*[w.handle for w in ws])
         ya = (_P * n)(*[_ptr(y) for y in ys])
         self._check(self._lib.wick_rocm_gemv_f32_multi(self._h, wa, ya, n, _ptr(x), x_off_bytes, int(accumulate)))
+
+    def encode_gemv_rmsnorm_fused(self, ws: Sequence[RocmWeight], x, norm_weight, eps: float, ys, accumulate: bool = False) -> None:
+        """encode_gemv_rmsnorm_gate_up (wick/src/model/metal_lfm2.rs:1157-1186) for any 1..4 weights."""
+        n = len(ws)
+        wa = (_P * n)(*[w.handle for w in ws])
+        ya = (_P * n)(*[_ptr(y) for y in ys])
+        self._check(self._lib.wick_rocm_gemv_rmsnorm_f32_multi(self._h, wa, ya, n, _ptr(x), _ptr(norm_weight), eps, int(accumulate)))
+
+    def encode_gemv_silu_mul(self, w: RocmWeight, gate, up, y, accumulate: bool = False) -> None:
+        """Down projection of silu(gate) * up in one launch."""
+        self._check(self._lib.wick_rocm_gemv_silu_mul_f32(self._h, w.handle, _ptr(gate), _ptr(up), _ptr(y), int(accumulate)))
 
     def reserve_scratch(self, max_n: int, max_k: int) -> None:
         self._check(self._lib.wick_rocm_reserve_scratch(self._h, max_n, max_k))
