@@ -205,8 +205,19 @@ int wick_rocm_gemv_rmsnorm_f32_multi(wick_rocm_ctx *ctx, const wick_rocm_weight 
 int wick_rocm_gemv_silu_mul_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const float *d_gate, const float *d_up, float *d_y,
                                 int accumulate);
 
-/* Pre-sizes the scratch used by wick_rocm_matmul_f32 for up to max_n columns of
- * up to max_k elements (call before capturing a graph). */
+/* The FFN's gate and up projections with the gate applied in the same launch:
+ *   d_act[r] = silu(W_gate[r] . x') * (W_up[r] . x'),  x' = rmsnorm(x, norm_weight, eps) (or x when d_norm_weight is
+ * null), quantized to Q8_0 inside the kernel.  One lane ends up with both row sums and applies cpu::silu_mul_inplace
+ * (wick/src/backend/cpu.rs:668-673) to them: bit-identical to encode_gemv_rmsnorm_gate_up followed by the silu_mul
+ * dispatch (wick/src/model/metal_lfm2.rs:1157-1186, 4225-4238), one launch and one round trip through memory less.
+ * Both weights m x k of one type; shapes the kernel does not take (k > 4096, odd block counts, Q6_K) run the three
+ * steps separately through context scratch. */
+int wick_rocm_ffn_gate_up_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w_gate, const wick_rocm_weight *w_up, const float *d_x,
+                              const float *d_norm_weight, float eps, float *d_act);
+
+/* Pre-sizes the context's scratch for up to max_n columns of up to max_k elements (max_k: the largest row length
+ * or row count of any weight used; call before capturing a graph).  Used by wick_rocm_matmul_f32 (n > 1 or a shape
+ * the fused kernels do not take) and by the unfused fallbacks of the calls above. */
 int wick_rocm_reserve_scratch(wick_rocm_ctx *ctx, uint32_t max_n, uint32_t max_k);
 
 /* ---- parity hook ----------------------------------------------------------

@@ -225,3 +225,30 @@ def test_down_projection_with_the_gate_folded_in(ctx, oracle, dtype, m, k):
     assert rel_l2(y, 1 + L.gemv(dtype, wb, sm, m, k)) <= 1e-5  # silu_mul is bit-exact: the quantizer sees the oracle's very input
     for b in (w, d_g, d_u, d_y, d_z):
         b.free()
+
+
+@pytest.mark.parametrize("dtype,m,k,norm", [(W.Q4_0, 4608, 1024, True), (W.Q8_0, 4608, 1024, True), (W.Q4_0, 512, 256, False), (W.Q4_0, 1030, 2048, True),
+                                            (W.Q8_0, 77, 4096, True), (W.Q4_0, 64, 8192, True), (W.Q8_0, 50, 96, False), (W.Q4_0, 3, 64, True)])
+def test_gate_and_up_with_the_gate_applied(ctx, oracle, dtype, m, k, norm):
+    """wick_rocm_ffn_gate_up_f32 is bit-identical to the two projections followed by silu_mul (the last three shapes
+    take its unfused fallback or the smallest kernel tier), and matches the oracle."""
+    from oracle import lfm2_oracle as L
+    from wick_amd.lfm2 import Lfm2Ops
+    x = oracle.fill_normal(k + 9, 1.5, k)
+    nw = (1.0 + 0.2 * oracle.fill_normal(k + 3, 1.0, k)).astype(np.float32)
+    wg, wu = oracle.synth_weight(dtype, m, k, seed=m + 1), oracle.synth_weight(dtype, m, k, seed=m + 2)
+    hg, hu = ctx.upload_weight(wg, dtype, m, k), ctx.upload_weight(wu, dtype, m, k)
+    d_x, d_nw = ctx.to_device(x), ctx.to_device(nw)
+    d_act, d_g, d_u = ctx.to_device(np.full(m, 9.0, np.float32)), ctx.alloc(m * 4), ctx.alloc(m * 4)
+    ctx.encode_ffn_gate_up(hg, hu, d_x, d_nw if norm else None, 1e-5, d_act)
+    if norm:
+        ctx.encode_gemv_rmsnorm_fused([hg, hu], d_x, d_nw, 1e-5, [d_g, d_u])
+    else:
+        ctx.encode_gemv_fused([hg, hu], d_x, 0, [d_g, d_u])
+    Lfm2Ops(ctx).silu_mul_inplace(d_g, d_u, m)
+    act, sep = d_act.download(np.float32, m), d_g.download(np.float32, m)
+    assert np.array_equal(act.view(np.uint32), sep.view(np.uint32))
+    xn = L.rmsnorm(x, nw, 1e-5) if norm else x
+    _close_unless_tie(act, xn, L.silu_mul(L.gemv(dtype, wg, xn, m, k), L.gemv(dtype, wu, xn, m, k)), f"gate_up {dtype} {m}x{k}")
+    for b in (hg, hu, d_x, d_nw, d_act, d_g, d_u):
+        b.free()

@@ -389,6 +389,20 @@ int wick_rocm_gemv_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* w
 
 namespace {
 
+// y_i (+)= W_i x for weights that share the f32 activation x (lock held).
+int gemv_plain_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count, const float* x, int accumulate) {
+    GemvBatch b{};
+    if (int rc = make_batch(ctx, ws, d_ys, count, b)) return rc;
+    if (ws[0]->type == kTypeQ6_K) {  // quantize into scratch, then one launch per weight
+        const uint32_t k = ws[0]->k;
+        if (int rc = ensure_scratch(ctx, k, k / 32u)) return rc;
+        hipError_t e = launch_quantize_q8_0(x, 1, k, k, ctx->scratch_q, ctx->scratch_s, ctx->launch());
+        if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
+        return q6k_gemv_locked(ctx, ws, d_ys, count, ctx->scratch_q, ctx->scratch_s, accumulate);
+    }
+    return gemv_f32_locked(ctx, b, ws[0]->type, ws[0]->k, x, accumulate);
+}
+
 // y_i (+)= W_i xform(x) for weights that share x (lock held).  The fused kernel applies the transform in its
 // prologue; shapes / types it does not take run the transform as a launch of its own into scratch first.
 int gemv_xform_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count, const float* x, int xform,
@@ -435,22 +449,43 @@ int wick_rocm_gemv_silu_mul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, c
     return gemv_xform_locked(ctx, ws, ys, 1, d_gate, kXformSiluMul, d_up, 0.0f, accumulate);
 }
 
+int wick_rocm_ffn_gate_up_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w_gate, const wick_rocm_weight* w_up, const float* d_x,
+                              const float* d_norm_weight, float eps, float* d_act) {
+    WR_ENTER(ctx);
+    if (int rc = check_weight(ctx, w_gate)) return rc;
+    if (int rc = check_weight(ctx, w_up)) return rc;
+    if (!d_x || !d_act) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "ffn_gate_up: null device pointer");
+    if (w_gate->m != w_up->m || w_gate->k != w_up->k) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "ffn_gate_up: gate and up must have one shape");
+    const uint32_t m = w_gate->m, k = w_gate->k;
+    const auto aligned16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16u == 0; };
+    const auto *g = static_cast<const uint8_t*>(w_gate->d), *u = static_cast<const uint8_t*>(w_up->d);
+    if (w_gate->type == w_up->type && w_gate->type != kTypeQ6_K && gated_kernel_applies(g, u, k) && aligned16(d_x) &&
+        (!d_norm_weight || aligned16(d_norm_weight))) {
+        hipError_t e = launch_gemv_gated_f32(w_gate->type, g, u, m, k, d_x, d_act, ctx->num_cus, ctx->launch(),
+                                             d_norm_weight ? kXformRmsNorm : kXformNone, d_norm_weight, eps);
+        return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "gated gemv launch");
+    }
+    // Shapes / types the gated kernel does not take: gate into d_act, up into scratch (after the quantization /
+    // transform scratch of k floats), then the gate as a launch of its own.
+    if (int rc = ensure_scratch(ctx, k, k / 32u, (size_t)k + m)) return rc;
+    float* up_out = ctx->scratch_f + k;
+    const wick_rocm_weight* ws[2] = {w_gate, w_up};
+    float* ys[2] = {d_act, up_out};
+    for (int i = 0; i < 2; i++) {
+        const int rc = d_norm_weight ? gemv_xform_locked(ctx, ws + i, ys + i, 1, d_x, kXformRmsNorm, d_norm_weight, eps, 0)
+                                     : gemv_plain_locked(ctx, ws + i, ys + i, 1, d_x, 0);
+        if (rc) return rc;
+    }
+    hipError_t e = launch_silu_mul(d_act, up_out, m, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "silu_mul launch");
+}
+
 int wick_rocm_gemv_f32_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count,
                              const float* d_x, size_t x_off_bytes, int accumulate) {
     WR_ENTER(ctx);
     if (!d_x) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv_f32_multi: null activation pointer");
     if (x_off_bytes % 4u) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemv_f32_multi: offset must be a multiple of 4");
-    GemvBatch b{};
-    if (int rc = make_batch(ctx, ws, d_ys, count, b)) return rc;
-    const float* x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes);
-    if (ws[0]->type == kTypeQ6_K) {  // quantize into scratch, then one launch per weight
-        const uint32_t k = ws[0]->k;
-        if (int rc = ensure_scratch(ctx, k, k / 32u)) return rc;
-        hipError_t e = launch_quantize_q8_0(x, 1, k, k, ctx->scratch_q, ctx->scratch_s, ctx->launch());
-        if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
-        return q6k_gemv_locked(ctx, ws, d_ys, count, ctx->scratch_q, ctx->scratch_s, accumulate);
-    }
-    return gemv_f32_locked(ctx, b, ws[0]->type, ws[0]->k, x, accumulate);
+    return gemv_plain_locked(ctx, ws, d_ys, count, reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes), accumulate);
 }
 
 int wick_rocm_gemv_q8(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_quants, const float* d_scales,
@@ -470,7 +505,8 @@ int wick_rocm_gemm_q8(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_
 int wick_rocm_reserve_scratch(wick_rocm_ctx* ctx, uint32_t max_n, uint32_t max_k) {
     WR_ENTER(ctx);
     if (max_k % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "reserve_scratch: max_k % 32 != 0");
-    return ensure_scratch(ctx, (size_t)max_n * max_k, (size_t)max_n * (max_k / 32u), max_k);
+    // f32 scratch: one transformed activation vector + one projection output of the unfused fallbacks
+    return ensure_scratch(ctx, (size_t)max_n * max_k, (size_t)max_n * (max_k / 32u), 2 * (size_t)max_k);
 }
 
 int wick_rocm_matmul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const float* d_x, size_t x_off_bytes, uint32_t n,

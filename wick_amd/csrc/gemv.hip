@@ -38,6 +38,7 @@ struct GemvArgs {
     const float* xaux;  // FUSEQ with a transform: RMSNorm weights [k] / the "up" vector [k]
     float eps;          // RMSNorm epsilon
     int xform;          // kXformNone / kXformRmsNorm / kXformSiluMul (host-side selector of the kernel variant)
+    int gated;          // host-side selector of the GATED variant: batch.w[0] = gate, batch.w[1] = up, y[0][r] = silu(gate_r) * up_r
     uint32_t x_stride;
     uint32_t k;
     uint32_t n;         // tokens (1 for decode)
@@ -87,12 +88,19 @@ enum { kDirect = 0, kDirectNT = 1, kSpan = 2 };
 // and weight loads of a single-weight launch is there at the first instruction, instead of
 // after one or two scalar-load round trips (~0.15 us each, on the critical path of a
 // 2-3 us launch).  The rest of `a` is still fetched the ordinary way, under those loads.
-template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI, int MODE, int XF = kXformNone>
+// GATED: the FFN's gate and up projections in one pass with the gate applied to the results.  Lane slots u = 0, 2, ..
+// hold rows of weight 0 (gate), u = 1, 3, .. the same rows of weight 1 (up); the lane that ends up with both row sums
+// stores silu(gate) * up (cpu::silu_mul_inplace, wick/src/backend/cpu.rs:668-673): the same f32 values the two plain
+// projections would have written, so the result is bit-identical to projection + projection + silu_mul, without the
+// launch and the round trip through memory in between.
+template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI, int MODE, int XF = kXformNone, bool GATED = false>
 __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kernel(const void* p_x, const uint8_t* p_w0, float* p_y0,
                                                                                   uint32_t p_k, uint32_t p_rows0,
                                                                                   uint32_t p_rows_per_wave, uint32_t p_total_waves,
                                                                                   int p_accumulate, GemvArgs a) {
     static_assert(XF == kXformNone || FUSEQ, "activation transforms belong to the fused-quantizer variant");
+    static_assert(!GATED || (FUSEQ && !MULTI && NT == 1 && U % 2 == 0), "the gated variant pairs lane slots");
+    constexpr int UR = GATED ? U / 2 : U;  // distinct rows per lane and pass
     using PT = PairTraits<TYPE>;
     constexpr int RPW = 64 / LPR;  // rows per wave pass
     const uint32_t lane = threadIdx.x & 63u;
@@ -188,14 +196,18 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     // Loads are unconditional (row and pair indices clamped into range) so that the number
     // of outstanding loads is known at every wait; a clamped load's data is neutralised by
     // zero activation scales (pair out of range) or simply not stored (row out of range).
+    const uint8_t* const wbase_of_wave = wbase;
+    const uint8_t* wbase1 = GATED ? a.batch.w[1] : wbase;
     auto issue_pass = [&](uint32_t base) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            lrow[u] = base + u * RPW + rsel;
+            const int ur = GATED ? u >> 1 : u;
+            const uint8_t* wbase = (GATED && (u & 1)) ? wbase1 : wbase_of_wave;
+            lrow[u] = base + ur * RPW + rsel;
             rvalid[u] = lrow[u] < wave_row1;
             if constexpr (MODE == kSpan) {
                 // First row of this pass (wave-uniform) and the rows of it that exist.
-                const uint32_t row0 = base + u * RPW;
+                const uint32_t row0 = base + ur * RPW;
                 const uint32_t nrows = row0 < rows ? min((uint32_t)RPW, rows - row0) : 0u;
 #pragma unroll
                 for (int c = 0; c < NCHUNK; c++) {
@@ -352,9 +364,10 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
         }
     }
 
-    for (uint32_t base = wave_row0; base < wave_row1; base += RPW * U) {
+    for (uint32_t base = wave_row0; base < wave_row1; base += RPW * UR) {
         if (base != wave_row0) issue_pass(base);
         // Consume.
+        float gate_sum = 0.0f;  // GATED: the row sum of the even slot, waiting for its odd partner
 #pragma unroll
         for (int u = 0; u < U; u++) {
             float acc[NT];
@@ -377,7 +390,10 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const float tot = group_sum<LPR>(acc[t]);
-                if (sub == 0 && rvalid[u] && tok0 + t < a.n) {
+                if constexpr (GATED) {
+                    if ((u & 1) == 0) gate_sum = tot;
+                    else if (sub == 0 && rvalid[u]) ybase[lrow[u]] = silu_mul(gate_sum, tot);
+                } else if (sub == 0 && rvalid[u] && tok0 + t < a.n) {
                     float* dst = a.y_row_major ? ybase + (size_t)lrow[u] * a.y_stride + (tok0 + t)
                                                : ybase + (size_t)(tok0 + t) * a.y_stride + lrow[u];
                     *dst = p_accumulate ? *dst + tot : tot;
@@ -473,7 +489,7 @@ constexpr uint64_t kDirectMaxBytesQ4 = 3ull << 20;
 constexpr uint64_t kDirectMaxBytesQ8 = 512ull << 10;
 template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ, int U>
 hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
-    constexpr uint32_t pass_rows = (64 / LPR) * U;
+    const uint32_t pass_rows = (64 / LPR) * (a.gated ? U / 2 : U);
     // Enough waves to give every CU ~16, and every wave at least one full pass.
     const uint32_t max_waves = (uint32_t)num_cus * 16u;
     uint32_t passes = (total_rows + pass_rows - 1) / pass_rows;
@@ -484,7 +500,7 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
     const dim3 grid = FUSEQ ? dim3((waves + kFusedWaves - 1) / kFusedWaves, 1) : dim3(waves, (a.n + NT - 1) / NT);
     const dim3 block(FUSEQ ? 64 * kFusedWaves : 64);
     // Several tokens re-read the weights: only single-token launches stream them.
-    const uint64_t bytes = (uint64_t)total_rows * (a.k >> 5) * (TYPE == 2 ? 18u : 34u);
+    const uint64_t bytes = (uint64_t)total_rows * (a.k >> 5) * (TYPE == 2 ? 18u : 34u) * (a.gated ? 2u : 1u);
     constexpr int kSmall = TYPE == 2 ? kDirectNT : kDirect;
     const uint64_t direct_max = L.gemv_direct_max_bytes >= 0 ? (uint64_t)L.gemv_direct_max_bytes : (TYPE == 2 ? kDirectMaxBytesQ4 : kDirectMaxBytesQ8);
     const int mode = NT > 1 ? kDirect : (bytes < direct_max ? kSmall : kSpan);
@@ -496,6 +512,18 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
     };
     if constexpr (NT == 1 && FUSEQ) {
         // the activation transforms exist for the fused single-token variant only
+        if (a.gated) {  // gate | up pairs: two lane slots per row, no transform other than the norm
+            if constexpr (U == 2 && NCHUNK == 1) {
+                if (a.xform == kXformRmsNorm) {
+                    if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan, kXformRmsNorm, true>);
+                    return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall, kXformRmsNorm, true>);
+                }
+                if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan, kXformNone, true>);
+                return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall, kXformNone, true>);
+            } else {
+                return hipErrorInvalidValue;  // launch_pairs picks U = 2 for gated launches; gated_kernel_applies() keeps NCHUNK at 1
+            }
+        }
         auto with_xform = [&](auto xf) {
             constexpr int XF = decltype(xf)::value;
             if (mode == kSpan && multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSpan, XF>);
@@ -533,6 +561,10 @@ inline int gemv_u_override() {
 template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ>
 hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
     constexpr int UMAX = (NT > 1 || NCHUNK > 1) ? (TYPE == 2 && NT == 1 ? 2 : 1) : (TYPE == 2 ? 4 : 2);
+    if (a.gated) {  // one gate row and one up row per lane and pass
+        if constexpr (FUSEQ && NT == 1 && NCHUNK == 1) return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 2>(a, total_rows, num_cus, L);
+        else return hipErrorInvalidValue;
+    }
     int u = UMAX;
     const uint32_t want_waves = (uint32_t)num_cus * 8u;
     while (u > 1 && total_rows / ((64 / LPR) * u) < want_waves) u >>= 1;
@@ -589,6 +621,27 @@ hipError_t launch_gemv_f32(int type, const GemvBatch& batch, uint32_t k, const f
     a.k = k;
     a.n = 1;
     a.accumulate = accumulate;
+    return type == kTypeQ4_0 ? dispatch<2, 1, true>(a, num_cus, L) : dispatch<8, 1, true>(a, num_cus, L);
+}
+
+bool gated_kernel_applies(const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t k) {
+    const uint32_t nb = k >> 5;
+    return nb % 2u == 0 && (nb >> 1) <= 64 && reinterpret_cast<uintptr_t>(d_w_gate) % 4u == 0 && reinterpret_cast<uintptr_t>(d_w_up) % 4u == 0;
+}
+
+// out[r] = silu(W_gate[r] . x') * (W_up[r] . x'), x' = xform(x) quantized to Q8_0, in one launch.
+hipError_t launch_gemv_gated_f32(int type, const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t m, uint32_t k, const float* d_x,
+                                 float* d_out, int num_cus, const Launch& L, int xform, const float* d_aux, float eps) {
+    GemvArgs a{};
+    a.batch.w[0] = d_w_gate, a.batch.w[1] = d_w_up;
+    a.batch.y[0] = d_out;
+    a.batch.row_end[0] = m;
+    a.batch.count = 1;  // the waves are laid out over the rows of one weight; each handles both
+    a.xf = d_x;
+    a.xform = xform, a.xaux = d_aux, a.eps = eps, a.gated = 1;
+    a.x_stride = k;
+    a.k = k;
+    a.n = 1;
     return type == kTypeQ4_0 ? dispatch<2, 1, true>(a, num_cus, L) : dispatch<8, 1, true>(a, num_cus, L);
 }
 

@@ -129,7 +129,7 @@ struct wick_rocm_lfm2 {
     float theta_scale = 0.0f;
     // step scratch (device)
     float *hidden = nullptr, *proj = nullptr, *gated = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr,
-          *gate = nullptr, *up = nullptr, *scores = nullptr, *logits = nullptr;
+          *gate = nullptr, *scores = nullptr, *logits = nullptr;
     uint32_t *d_token = nullptr, *d_pos = nullptr, *d_pick = nullptr, *d_history = nullptr;
     unsigned long long* d_argmax_partial = nullptr;
     wick_rocm_graph *g_logits = nullptr, *g_greedy = nullptr;
@@ -233,8 +233,9 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
                 break;
             if ((rc = gemv_residual(ctx, L.o, m->hidden, m->attn))) break;
         }
-        if ((rc = gemv_normed(ctx, {L.gate, L.up}, {m->gate, m->up}, m->hidden, L.ffn_norm, c.rms_norm_eps))) break;
-        rc = wick_rocm_gemv_silu_mul_f32(ctx, L.down, m->gate, m->up, m->hidden, 1);  // hidden += down(silu(gate) * up)
+        // gate = silu(W_gate n(hidden)) * (W_up n(hidden)); hidden += W_down gate
+        if ((rc = wick_rocm_ffn_gate_up_f32(ctx, L.gate, L.up, m->hidden, L.ffn_norm, c.rms_norm_eps, m->gate))) break;
+        rc = gemv_residual(ctx, L.down, m->hidden, m->gate);
     }
     if (rc) return rc;
     if ((rc = gemv_normed(ctx, {m->embd}, {m->logits}, m->hidden, m->out_norm, c.rms_norm_eps))) return rc;
@@ -374,7 +375,7 @@ int wick_rocm_lfm2_load(wick_rocm_ctx* ctx, const wick_gguf* g, uint32_t context
     if ((rc = alloc_t(ctx, m, hs, &m->hidden)) || (rc = alloc_t(ctx, m, 3 * (size_t)hs, &m->proj)) ||
         (rc = alloc_t(ctx, m, hs, &m->gated)) || (rc = alloc_t(ctx, m, hs, &m->q)) || (rc = alloc_t(ctx, m, kv_max, &m->k)) ||
         (rc = alloc_t(ctx, m, kv_max, &m->v)) || (rc = alloc_t(ctx, m, hs, &m->attn)) || (rc = alloc_t(ctx, m, inter, &m->gate)) ||
-        (rc = alloc_t(ctx, m, inter, &m->up)) || (rc = alloc_t(ctx, m, attention_scratch_floats(c.max_seq_len, c.n_heads, hd), &m->scores)) ||
+        (rc = alloc_t(ctx, m, attention_scratch_floats(c.max_seq_len, c.n_heads, hd), &m->scores)) ||
         (rc = alloc_t(ctx, m, c.vocab_size, &m->logits)) || (rc = alloc_t(ctx, m, 1, &m->d_token)) ||
         (rc = alloc_t(ctx, m, 1, &m->d_pos)) || (rc = alloc_t(ctx, m, 1, &m->d_pick)) || (rc = alloc_t(ctx, m, kArgmaxPartials, &m->d_argmax_partial)) || (rc = alloc_t(ctx, m, c.max_seq_len, &m->d_history)))
         return bail(rc);

@@ -91,6 +91,14 @@ enum { kXformNone = 0, kXformRmsNorm = 1, kXformSiluMul = 2 };
 hipError_t launch_gemv_f32(int type, const GemvBatch& batch, uint32_t k, const float* d_x, int accumulate, int num_cus,
                            const Launch& L, int xform = kXformNone, const float* d_aux = nullptr, float eps = 0.0f);
 
+// The FFN's gate and up projections with the gate applied to the row sums: out[r] = silu(W_gate[r] . x') * (W_up[r] . x'),
+// x' = xform(x) quantized to Q8_0 (xform: none or RMSNorm).  Only when gated_kernel_applies() (even block count,
+// k <= 4096, 4-byte aligned weights) and d_x / d_aux are 16-byte aligned.
+bool gated_kernel_applies(const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t k);
+hipError_t launch_gemv_gated_f32(int type, const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t m, uint32_t k, const float* d_x,
+                                 float* d_out, int num_cus, const Launch& L, int xform = kXformNone, const float* d_aux = nullptr,
+                                 float eps = 0.0f);
+
 // Q6_K decode GEMV, one token (gemv_q6k.hip).  k % 256 == 0, k <= 8192; the weight allocation is padded by
 // 16 bytes; y[row * y_row_stride].  launch_group_dots_q6k is its parity hook: out[i * (k/16) + g] = exact i32 dot of 16-weight group g.
 constexpr int kTypeQ6_K = 14;  // ggml id, wick/src/gguf.rs:36-51

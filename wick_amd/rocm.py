@@ -88,6 +88,7 @@ _SIGNATURES = {
     "wick_rocm_gemv_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, C.c_size_t, C.c_int]),
     "wick_rocm_gemv_rmsnorm_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, _P, C.c_float, C.c_int]),
     "wick_rocm_gemv_silu_mul_f32": (C.c_int, [_P, _P, _P, _P, _P, C.c_int]),
+    "wick_rocm_ffn_gate_up_f32": (C.c_int, [_P, _P, _P, _P, _P, C.c_float, _P]),
     "wick_rocm_reserve_scratch": (C.c_int, [_P, C.c_uint32, C.c_uint32]),
     "wick_rocm_block_dots_i32": (C.c_int, [_P, _P, _P, C.c_uint32, _P]),
     "wick_rocm_graph_begin": (C.c_int, [_P]),
@@ -306,6 +307,10 @@ class RocmContext:
     def encode_gemv_silu_mul(self, w: RocmWeight, gate, up, y, accumulate: bool = False) -> None:
         """Down projection of silu(gate) * up in one launch."""
         self._check(self._lib.wick_rocm_gemv_silu_mul_f32(self._h, w.handle, _ptr(gate), _ptr(up), _ptr(y), int(accumulate)))
+
+    def encode_ffn_gate_up(self, w_gate: RocmWeight, w_up: RocmWeight, x, norm_weight, eps: float, act) -> None:
+        """act = silu(W_gate n(x)) * (W_up n(x)) in one launch (norm_weight may be None: no norm)."""
+        self._check(self._lib.wick_rocm_ffn_gate_up_f32(self._h, w_gate.handle, w_up.handle, _ptr(x), _ptr(norm_weight), eps, _ptr(act)))
 
     def reserve_scratch(self, max_n: int, max_k: int) -> None:
         self._check(self._lib.wick_rocm_reserve_scratch(self._h, max_n, max_k))
