@@ -60,6 +60,17 @@ int wick_rocm_attention_decode(wick_rocm_ctx *ctx, const float *d_q, const float
                                float *d_scratch, uint32_t seq_len, const uint32_t *d_pos, uint32_t max_seq, uint32_t n_heads,
                                uint32_t n_kv_heads, uint32_t head_dim);
 
+/* The attention block between the Q/K/V projections and the output projection: what wick_rocm_qk_norm_rope followed
+ * by wick_rocm_attention_decode compute (wick/src/model/lfm2.rs:783-1006), bit for bit, with the norm, the rotation and
+ * the KV append folded into the attention kernel (workgroups norm and rotate their own query head; those that own the
+ * new position norm, rotate and append K and V themselves), one launch less.  d_scratch:
+ * wick_rocm_attention_block_scratch_bytes(...) bytes, contents need not be kept.  d_q / d_k may be overwritten (head
+ * dims without a fused kernel run the separate launches, which work in place). */
+size_t wick_rocm_attention_block_scratch_bytes(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim);
+int wick_rocm_attention_block(wick_rocm_ctx *ctx, float *d_q, float *d_k, const float *d_v, const float *d_q_norm, const float *d_k_norm,
+                              float *d_k_cache, float *d_v_cache, float *d_out, void *d_scratch, uint32_t pos, const uint32_t *d_pos,
+                              uint32_t max_seq, uint32_t head_dim, uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale);
+
 /* encode_conv1d_fused (wick/src/model/metal_lfm2.rs:1959-1991) = the middle of forward_conv_block
  * (wick/src/model/lfm2.rs:694-726): d_proj = [b | c | x] (hidden floats each), d_buffer the rolling state
  * ((kernel_size-1) * hidden floats, updated in place), d_conv_weight [hidden][kernel_size]; d_out = c * conv(b*x). */

@@ -7,7 +7,7 @@ import pytest
 
 import wick_amd as W
 from oracle import lfm2_oracle as L
-from wick_amd.lfm2 import Lfm2Ops, attention_scratch_floats, rope_theta_scale
+from wick_amd.lfm2 import Lfm2Ops, attention_block_scratch_bytes, attention_scratch_floats, rope_theta_scale
 
 pytestmark = pytest.mark.gpu
 
@@ -159,6 +159,41 @@ def test_attention_decode(ctx, ops, oracle, n_heads, n_kv, hd, seq):
         ref = L.attention(q, kc[: 290 * kv_dim], vc[: 290 * kv_dim], n_heads, n_kv, hd, 290)
         assert np.allclose(d_out.download(np.float32, n_heads * hd), ref, rtol=0, atol=4e-6 * np.abs(ref).max())
     for b in (d_q, d_kc, d_vc, d_out, d_sc, d_pos):
+        b.free()
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,max_seq,steps", [(4, 2, 64, 300, [0, 1, 2, 63, 64, 65, 130, 299]), (16, 8, 64, 4096, [0, 700, 4095]),
+                                                           (4, 4, 32, 64, [0, 5, 63]), (2, 1, 128, 5000, [4100, 4999]), (2, 1, 256, 100, [99]),
+                                                           (3, 1, 96, 80, [0, 7, 79])])
+def test_attention_block_equals_the_separate_launches(ctx, ops, oracle, n_heads, n_kv, hd, max_seq, steps):
+    """The block (norm + RoPE + append folded into the attention kernel) against qk_norm_rope followed by attention,
+    bit for bit, over several positions of one cache; head_dim 96 takes the block's unfused path."""
+    kv_dim, eps, ts = n_kv * hd, 1e-5, rope_theta_scale(hd, 1_000_000.0)
+    cache = oracle.fill_normal(max_seq, 1.0, 2 * max_seq * kv_dim)
+    kc_a, vc_a = ctx.to_device(cache[: max_seq * kv_dim]), ctx.to_device(cache[max_seq * kv_dim:])
+    kc_b, vc_b = ctx.to_device(cache[: max_seq * kv_dim]), ctx.to_device(cache[max_seq * kv_dim:])
+    d_qn, d_kn = ctx.to_device(1 + 0.2 * oracle.fill_normal(4, 1.0, hd)), ctx.to_device(1 + 0.2 * oracle.fill_normal(5, 1.0, hd))
+    nbytes = attention_block_scratch_bytes(max_seq, n_heads, hd)
+    d_scr = ctx.alloc(nbytes)
+    d_sc2 = ctx.alloc(attention_scratch_floats(max_seq, n_heads, hd) * 4)
+    d_oa, d_ob = ctx.alloc(n_heads * hd * 4), ctx.alloc(n_heads * hd * 4)
+    for pos in steps:
+        q, k, v = (oracle.fill_normal(10 * pos + i, 1.0, n) for i, n in enumerate((n_heads * hd, kv_dim, kv_dim)))
+        qa, ka, va = ctx.to_device(q), ctx.to_device(k), ctx.to_device(v)
+        qb, kb = ctx.to_device(q), ctx.to_device(k)
+        ops.encode_attention_block(qa, ka, va, d_qn, d_kn, kc_a, vc_a, d_oa, d_scr, pos, max_seq, hd, n_heads, n_kv, eps, ts)
+        ops.encode_qk_norm_rope(qb, kb, va, d_qn, d_kn, kc_b, vc_b, pos, max_seq, hd, n_heads, n_kv, eps, ts)
+        ops.encode_attention(qb, kc_b, vc_b, d_ob, d_sc2, pos + 1, max_seq, n_heads, n_kv, hd)
+        got, sep = d_oa.download(np.float32, n_heads * hd), d_ob.download(np.float32, n_heads * hd)
+        if max_seq > 256 or hd == 96:  # the separate launches take the same sequence-split arithmetic (or the block its unfused path)
+            assert np.array_equal(bits(got), bits(sep)), f"pos {pos}"
+        else:  # short contexts: the separate attention call is the one-workgroup kernel, which sums in another order
+            assert np.allclose(got, sep, rtol=0, atol=4e-6 * np.abs(sep).max()), f"pos {pos}"
+        for b in (qa, ka, va, qb, kb):
+            b.free()
+    assert np.array_equal(bits(kc_a.download(np.float32, max_seq * kv_dim)), bits(kc_b.download(np.float32, max_seq * kv_dim)))
+    assert np.array_equal(bits(vc_a.download(np.float32, max_seq * kv_dim)), bits(vc_b.download(np.float32, max_seq * kv_dim)))
+    for b in (kc_a, vc_a, kc_b, vc_b, d_qn, d_kn, d_scr, d_sc2, d_oa, d_ob):
         b.free()
 
 

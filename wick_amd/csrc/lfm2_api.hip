@@ -72,6 +72,37 @@ int wick_rocm_attention_decode(wick_rocm_ctx* ctx, const float* d_q, const float
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "attention launch");
 }
 
+size_t wick_rocm_attention_block_scratch_bytes(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim) {
+    return attention_scratch_floats(max_seq, n_heads, head_dim) * sizeof(float);
+}
+
+int wick_rocm_attention_block(wick_rocm_ctx* ctx, float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
+                              float* d_k_cache, float* d_v_cache, float* d_out, void* d_scratch, uint32_t pos, const uint32_t* d_pos,
+                              uint32_t max_seq, uint32_t head_dim, uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale) {
+    WR_ENTER(ctx);
+    if (!d_q || !d_k || !d_v || !d_q_norm || !d_k_norm || !d_k_cache || !d_v_cache || !d_out || !d_scratch)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention_block: null device pointer");
+    if (head_dim == 0 || head_dim % 4u != 0 || head_dim > 256u || n_heads == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "attention_block: head_dim must be a multiple of 4 and <= 256, n_kv_heads must divide n_heads");
+    if (misaligned(d_k_cache, 16) || misaligned(d_q, 16) || misaligned(d_scratch, 16))
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention_block: q, the key cache and the scratch must be 16-byte aligned");
+    if (!d_pos && pos >= max_seq) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention_block: pos beyond the cache");
+    const float scale = 1.0f / sqrtf((float)head_dim);  // wick/src/model/lfm2.rs:862
+    float* partials = static_cast<float*>(d_scratch);
+    hipError_t e;
+    if (attention_layer_applies(head_dim)) {
+        e = launch_attention_layer(d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, d_out, partials, pos, d_pos, max_seq, n_heads,
+                                   n_kv_heads, head_dim, eps, theta_scale, scale, ctx->launch());
+    } else {
+        e = launch_qk_norm_rope(d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, pos, d_pos, max_seq, head_dim, n_heads, n_kv_heads, eps,
+                                theta_scale, ctx->launch());
+        if (e == hipSuccess)
+            e = launch_attention_decode(d_q, d_k_cache, d_v_cache, d_out, partials, pos + 1u, d_pos, max_seq, n_heads, n_kv_heads, head_dim, scale,
+                                        ctx->launch());
+    }
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "attention_block launch");
+}
+
 int wick_rocm_shortconv_step(wick_rocm_ctx* ctx, const float* d_proj, float* d_buffer, const float* d_conv_weight, float* d_out, uint32_t hidden,
                              uint32_t kernel_size) {
     WR_ENTER(ctx);
@@ -226,10 +257,8 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
             if ((rc = gemv_residual(ctx, L.out_proj, m->hidden, m->gated))) break;
         } else {
             if ((rc = gemv_normed(ctx, {L.q, L.k, L.v}, {m->q, m->k, m->v}, m->hidden, L.attn_norm, c.rms_norm_eps))) break;
-            if ((rc = wick_rocm_qk_norm_rope(ctx, m->q, m->k, m->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, 0, m->d_pos, c.max_seq_len, hd, c.n_heads,
-                                             L.n_kv, c.rms_norm_eps, m->theta_scale)))
-                break;
-            if ((rc = wick_rocm_attention_decode(ctx, m->q, L.k_cache, L.v_cache, m->attn, m->scores, 0, m->d_pos, c.max_seq_len, c.n_heads, L.n_kv, hd)))
+            if ((rc = wick_rocm_attention_block(ctx, m->q, m->k, m->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, m->attn, m->scores, 0, m->d_pos,
+                                                c.max_seq_len, hd, c.n_heads, L.n_kv, c.rms_norm_eps, m->theta_scale)))
                 break;
             if ((rc = gemv_residual(ctx, L.o, m->hidden, m->attn))) break;
         }

@@ -107,40 +107,43 @@ struct QkNormRopeArgs {
     float eps, theta_scale;
 };
 
+// RMSNorm + RoPE of one head by the calling wave: dst[] (and dst2[], when given) receive the result; src may equal dst.
+__device__ __forceinline__ void norm_rope_head(const float* src, const float* w, uint32_t hd, uint32_t pos, float eps, float theta_scale,
+                                               float* dst, float* dst2) {
+    const uint32_t lane = threadIdx.x & 63u, half = hd >> 1;
+    double s = 0.0;
+    for (uint32_t i = lane; i < hd; i += 64) {
+        const double v = (double)src[i];
+        s += v * v;
+    }
+    const float inv_rms = (float)(1.0 / sqrt(wave_sum_f64(s) / (double)hd + (double)eps));
+    for (uint32_t i = lane; i < half; i += 64) {
+        float theta = (float)pos;
+        for (uint32_t j = 0; j < i; j++) theta = __fmul_rn(theta, theta_scale);
+        float sn, cs;
+        sincosf(theta, &sn, &cs);
+        const float x0 = __fmul_rn(__fmul_rn(src[i], inv_rms), w[i]);
+        const float x1 = __fmul_rn(__fmul_rn(src[i + half], inv_rms), w[i + half]);
+        const float r0 = __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn));
+        const float r1 = __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, cs));
+        dst[i] = r0, dst[i + half] = r1;
+        if (dst2) dst2[i] = r0, dst2[i + half] = r1;
+    }
+}
+
 __global__ __launch_bounds__(64) void qk_norm_rope_kernel(QkNormRopeArgs a) {
     const uint32_t pos = a.d_pos ? *a.d_pos : a.pos;
     const bool is_q = blockIdx.x < a.n_heads;
     const uint32_t h = is_q ? blockIdx.x : blockIdx.x - a.n_heads;
-    const uint32_t hd = a.head_dim, half = hd >> 1, kv_dim = a.n_kv_heads * hd;
+    const uint32_t hd = a.head_dim, kv_dim = a.n_kv_heads * hd;
     float* head = (is_q ? a.q : a.k) + (size_t)h * hd;
-    const float* w = is_q ? a.q_norm : a.k_norm;
-    const uint32_t lane = threadIdx.x;
-
-    double s = 0.0;
-    for (uint32_t i = lane; i < hd; i += 64) {
-        const double v = (double)head[i];
-        s += v * v;
-    }
-    const float inv_rms = (float)(1.0 / sqrt(wave_sum_f64(s) / (double)hd + (double)a.eps));
-
     const bool store = !is_q && pos < a.max_seq;  // the host checks a by-value pos; a device-side pos past the cache is dropped
-    float* kc = a.k_cache + (size_t)pos * kv_dim + (size_t)h * hd;
-    for (uint32_t i = lane; i < half; i += 64) {
-        float theta = (float)pos;
-        for (uint32_t j = 0; j < i; j++) theta = __fmul_rn(theta, a.theta_scale);
-        float sn, cs;
-        sincosf(theta, &sn, &cs);
-        const float x0 = __fmul_rn(__fmul_rn(head[i], inv_rms), w[i]);
-        const float x1 = __fmul_rn(__fmul_rn(head[i + half], inv_rms), w[i + half]);
-        const float r0 = __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn));
-        const float r1 = __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, cs));
-        head[i] = r0, head[i + half] = r1;
-        if (store) kc[i] = r0, kc[i + half] = r1;
-    }
+    norm_rope_head(head, is_q ? a.q_norm : a.k_norm, hd, pos, a.eps, a.theta_scale, head,
+                   store ? a.k_cache + (size_t)pos * kv_dim + (size_t)h * hd : nullptr);
     if (store) {
         const float* vh = a.v + (size_t)h * hd;
         float* vc = a.v_cache + (size_t)pos * kv_dim + (size_t)h * hd;
-        for (uint32_t i = lane; i < hd; i += 64) vc[i] = vh[i];
+        for (uint32_t i = threadIdx.x; i < hd; i += 64) vc[i] = vh[i];
     }
 }
 
@@ -256,8 +259,10 @@ __device__ __forceinline__ float block_sum_f32(float v, float* slots) {
     return (slots[0] + slots[1]) + (slots[2] + slots[3]);
 }
 
+// The chunks of workgroup (h, split): scores against q (HD floats, 16-byte aligned, global or LDS), streaming softmax,
+// weighted values; leaves {max, sum, acc[HD]} in the partial record of (h, split).  All 256 threads call it.
 template <int HD>
-__global__ __launch_bounds__(256) void attention_split_kernel(AttentionArgs a, uint32_t splits) {
+__device__ __forceinline__ void attention_chunks(const AttentionArgs& a, uint32_t splits, uint32_t h, uint32_t split, uint32_t seq, const float* q) {
     constexpr uint32_t LR = HD / 4;                  // lanes per cache row
     constexpr uint32_t RPP = 256 / LR;               // rows per pass of the block
     constexpr uint32_t KROWS = kAttnChunk / RPP;     // key rows per thread and chunk
@@ -269,16 +274,12 @@ __global__ __launch_bounds__(256) void attention_split_kernel(AttentionArgs a, u
     __shared__ float sc[kAttnChunk];
     __shared__ float red[256];
     __shared__ float slots[4];
-    const uint32_t h = blockIdx.x / splits, split = blockIdx.x % splits;
     const uint32_t kv_dim = a.n_kv_heads * HD;
-    uint32_t seq = a.d_pos ? *a.d_pos + 1u : a.seq_len;
-    if (seq > a.max_seq) seq = a.max_seq;
-    if (split * kAttnChunk >= seq) return;  // the combine step derives the number of partials from seq as well
     const uint32_t kvh = h / (a.n_heads / a.n_kv_heads);
     const float* kbase = a.k_cache + (size_t)kvh * HD;
     const float* vbase = a.v_cache + (size_t)kvh * HD;
     const uint32_t tid = threadIdx.x, quad = tid % LR, prow = tid / LR, d = tid % HD, g = tid / HD;
-    const float4 q4 = reinterpret_cast<const float4*>(a.q + (size_t)h * HD)[quad];
+    const float4 q4 = reinterpret_cast<const float4*>(q)[quad];
     const uint32_t last = seq - 1u;
 
     float m_run = -__builtin_inff(), l_run = 0.0f, acc = 0.0f;
@@ -339,17 +340,15 @@ __global__ __launch_bounds__(256) void attention_split_kernel(AttentionArgs a, u
     if (tid == 0) part[0] = m_run, part[1] = l_run;
 }
 
-// Merges the partials of one head: the first wave turns the (max, sum) pairs into weights, then every thread sums
-// its share of the weighted accumulators (again with its loads batched).
+// Merges the partials of head h: the first wave turns the (max, sum) pairs into weights, then every thread sums its
+// share of the weighted accumulators (again with its loads batched).  All 256 threads call it.
 template <int HD>
-__global__ __launch_bounds__(256) void attention_combine_kernel(AttentionArgs a, uint32_t splits) {
+__device__ __forceinline__ void attention_merge(const AttentionArgs& a, uint32_t splits, uint32_t h, uint32_t seq) {
     constexpr uint32_t G = 256 / HD;  // partial groups
     __shared__ float wts[kAttnMaxSplits];
-    __shared__ float red[256];
+    __shared__ float mred[256];
     __shared__ float total;
-    const uint32_t h = blockIdx.x, tid = threadIdx.x, d = tid % HD, grp = tid / HD;
-    uint32_t seq = a.d_pos ? *a.d_pos + 1u : a.seq_len;
-    if (seq > a.max_seq) seq = a.max_seq;
+    const uint32_t tid = threadIdx.x, d = tid % HD, grp = tid / HD;
     uint32_t active = (seq + kAttnChunk - 1) / kAttnChunk;
     active = active < splits ? active : splits;
     const float* parts = a.scores + (size_t)h * splits * (HD + 2);
@@ -382,14 +381,76 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(AttentionArgs a,
             o += i < active ? v[j] * wts[i] : 0.0f;
         }
     }
-    red[tid] = o;
+    mred[tid] = o;
     __syncthreads();
     if (tid < HD) {
-        float r = red[tid];
+        float r = mred[tid];
 #pragma unroll
-        for (uint32_t p = 1; p < G; p++) r += red[p * HD + tid];
+        for (uint32_t p = 1; p < G; p++) r += mred[p * HD + tid];
         a.out[(size_t)h * HD + tid] = active ? __fdiv_rn(r, total) : 0.0f;
     }
+}
+
+__device__ __forceinline__ uint32_t attention_seq(const AttentionArgs& a) {
+    const uint32_t seq = a.d_pos ? *a.d_pos + 1u : a.seq_len;
+    return seq > a.max_seq ? a.max_seq : seq;
+}
+
+template <int HD>
+__global__ __launch_bounds__(256) void attention_split_kernel(AttentionArgs a, uint32_t splits) {
+    const uint32_t h = blockIdx.x / splits, split = blockIdx.x % splits;
+    const uint32_t seq = attention_seq(a);
+    if (split * kAttnChunk >= seq) return;  // the combine step derives the number of partials from seq as well
+    attention_chunks<HD>(a, splits, h, split, seq, a.q + (size_t)h * HD);
+}
+
+template <int HD>
+__global__ __launch_bounds__(256) void attention_combine_kernel(AttentionArgs a, uint32_t splits) {
+    attention_merge<HD>(a, splits, blockIdx.x, attention_seq(a));
+}
+
+// The attention block between the Q/K/V projections and the output projection with QK-norm, RoPE and the KV append
+// folded into the sequence-split kernel (wick/src/model/lfm2.rs:783-1006): every workgroup (head, split) norms and
+// rotates its own query head into LDS (same arithmetic as qk_norm_rope_kernel); the workgroups whose chunk holds the
+// new position norm and rotate the key head, append it and the value row to the caches (query heads that share a KV
+// head write identical bytes) and read them back after a barrier.  No workgroup depends on another; the partials are
+// merged by attention_combine_kernel as before.  Results are bit-identical to qk_norm_rope + attention_split +
+// attention_combine, one launch less.  (Merging in the last workgroup to finish, behind a ticket counter, was built
+// and measured: the device-scope fences it needs write back and invalidate the L2 per workgroup and cost far more
+// than the launch they save.)
+struct AttentionLayerArgs {
+    AttentionArgs at;     // q unused; caches as read
+    const float* q_raw;   // [n_heads * HD] projection output, left unchanged
+    const float* k_raw;   // [n_kv_heads * HD]
+    const float* v;       // [n_kv_heads * HD]
+    const float* q_norm;
+    const float* k_norm;
+    float* k_cache;       // the same caches, writable
+    float* v_cache;
+    float eps, theta_scale;
+};
+
+template <int HD>
+__global__ __launch_bounds__(256) void attention_layer_kernel(AttentionLayerArgs f, uint32_t splits) {
+    __shared__ __align__(16) float qh[HD];
+    const AttentionArgs& a = f.at;
+    const uint32_t h = blockIdx.x / splits, split = blockIdx.x % splits, tid = threadIdx.x;
+    const uint32_t seq = attention_seq(a);
+    if (seq == 0 || split * kAttnChunk >= seq) return;
+    const uint32_t pos = seq - 1u, kv_dim = a.n_kv_heads * HD, kvh = h / (a.n_heads / a.n_kv_heads);
+    if (tid < 64) norm_rope_head(f.q_raw + (size_t)h * HD, f.q_norm, HD, pos, f.eps, f.theta_scale, qh, nullptr);
+    if ((pos / kAttnChunk) % splits == split) {  // this workgroup's chunks include the new position
+        if (tid >= 64 && tid < 128)
+            norm_rope_head(f.k_raw + (size_t)kvh * HD, f.k_norm, HD, pos, f.eps, f.theta_scale, f.k_cache + (size_t)pos * kv_dim + (size_t)kvh * HD,
+                           nullptr);
+        if (tid >= 128) {
+            const float* vh = f.v + (size_t)kvh * HD;
+            float* vc = f.v_cache + (size_t)pos * kv_dim + (size_t)kvh * HD;
+            for (uint32_t i = tid - 128; i < HD; i += 128) vc[i] = vh[i];
+        }
+    }
+    __syncthreads();  // qh[] and this workgroup's cache rows are complete
+    attention_chunks<HD>(a, splits, h, split, seq, qh);
 }
 
 // ---- gated short convolution, one step ---------------------------------------------------
@@ -556,6 +617,34 @@ hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, con
         }
     }
     return launch_kernel(L, kFamOther, attention_decode_kernel, dim3(n_heads), dim3(256), a);
+}
+
+// The fused attention block; false when head_dim has no fused variant (the caller then runs the three launches).
+bool attention_layer_applies(uint32_t head_dim) { return head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256; }
+
+hipError_t launch_attention_layer(const float* d_q, const float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
+                                  float* d_k_cache, float* d_v_cache, float* d_out, float* d_scratch, uint32_t pos,
+                                  const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float eps,
+                                  float theta_scale, float scale, const Launch& L) {
+    AttentionLayerArgs f{};
+    f.at = AttentionArgs{nullptr, d_k_cache, d_v_cache, d_out, d_scratch, d_pos, pos + 1u, max_seq, n_heads, n_kv_heads, head_dim, scale};
+    f.q_raw = d_q, f.k_raw = d_k, f.v = d_v, f.q_norm = d_q_norm, f.k_norm = d_k_norm;
+    f.k_cache = d_k_cache, f.v_cache = d_v_cache, f.eps = eps, f.theta_scale = theta_scale;
+    const uint32_t splits = attention_splits(max_seq);
+    const dim3 grid(n_heads * splits), block(256);
+    auto run = [&](auto hd) -> hipError_t {
+        constexpr int HD = decltype(hd)::value;
+        hipError_t e = launch_kernel(L, kFamOther, attention_layer_kernel<HD>, grid, block, f, splits);
+        if (e != hipSuccess) return e;
+        return launch_kernel(L, kFamOther, attention_combine_kernel<HD>, dim3(n_heads), block, f.at, splits);
+    };
+    switch (head_dim) {
+        case 32: return run(std::integral_constant<int, 32>{});
+        case 64: return run(std::integral_constant<int, 64>{});
+        case 128: return run(std::integral_constant<int, 128>{});
+        case 256: return run(std::integral_constant<int, 256>{});
+        default: return hipErrorInvalidValue;
+    }
 }
 
 uint32_t attention_splits(uint32_t max_seq) {

@@ -144,6 +144,13 @@ size_t attention_scratch_floats(uint32_t max_seq, uint32_t n_heads, uint32_t hea
 hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scores,
                                    uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
                                    uint32_t head_dim, float scale, const Launch& L);
+// QK-norm + RoPE + KV append folded into the sequence-split attention kernel, then the merge (head_dim 32 / 64 / 128 / 256).
+// d_scratch as for launch_attention_decode.
+bool attention_layer_applies(uint32_t head_dim);
+hipError_t launch_attention_layer(const float* d_q, const float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
+                                  float* d_k_cache, float* d_v_cache, float* d_out, float* d_scratch, uint32_t pos,
+                                  const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float eps,
+                                  float theta_scale, float scale, const Launch& L);
 hipError_t launch_shortconv_step(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
                                  uint32_t kernel_size, const Launch& L);
 hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const Launch& L);

@@ -30,6 +30,8 @@ _SIGNATURES = {
     "wick_rocm_rope_theta_scale": (_F, [_U32, _F]),
     "wick_rocm_attention_decode": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32]),
     "wick_rocm_attention_scratch_floats": (C.c_size_t, [_U32, _U32, _U32]),
+    "wick_rocm_attention_block_scratch_bytes": (C.c_size_t, [_U32, _U32, _U32]),
+    "wick_rocm_attention_block": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32, _F, _F]),
     "wick_rocm_shortconv_step": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32]),
     "wick_rocm_silu_mul": (C.c_int, [_P, _P, _P, _U32]),
     "wick_rocm_argmax": (C.c_int, [_P, _P, _U32, _P, _P, _P]),
@@ -65,6 +67,10 @@ def attention_scratch_floats(max_seq: int, n_heads: int, head_dim: int) -> int:
     return int(_lib().wick_rocm_attention_scratch_floats(max_seq, n_heads, head_dim))
 
 
+def attention_block_scratch_bytes(max_seq: int, n_heads: int, head_dim: int) -> int:
+    return int(_lib().wick_rocm_attention_block_scratch_bytes(max_seq, n_heads, head_dim))
+
+
 def rope_theta_scale(head_dim: int, freq_base: float) -> float:
     return float(_lib().wick_rocm_rope_theta_scale(head_dim, freq_base))
 
@@ -91,6 +97,13 @@ class Lfm2Ops:
                          d_pos=None) -> None:
         self.ctx._check(self._l.wick_rocm_attention_decode(self.ctx._h, _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(scores), seq_len,
                                                            _ptr(d_pos), max_seq, n_heads, n_kv_heads, head_dim))
+
+    def encode_attention_block(self, q, k, v, q_norm, k_norm, k_cache, v_cache, out, scratch, pos: int, max_seq: int, head_dim: int,
+                               n_heads: int, n_kv_heads: int, eps: float, theta_scale: float, d_pos=None) -> None:
+        """QK-norm + RoPE + KV append folded into the attention kernel (then the merge)."""
+        self.ctx._check(self._l.wick_rocm_attention_block(self.ctx._h, _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(k_cache),
+                                                          _ptr(v_cache), _ptr(out), _ptr(scratch), pos, _ptr(d_pos), max_seq, head_dim, n_heads,
+                                                          n_kv_heads, eps, theta_scale))
 
     def encode_conv1d_fused(self, proj, buffer, conv_weight, out, hidden: int, kernel_size: int) -> None:
         self.ctx._check(self._l.wick_rocm_shortconv_step(self.ctx._h, _ptr(proj), _ptr(buffer), _ptr(conv_weight), _ptr(out), hidden, kernel_size))
