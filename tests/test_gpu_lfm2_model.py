@@ -173,3 +173,68 @@ def test_load_and_step_errors(ctx, oracle, tmp_path):
     with G.GgufFile.from_bytes(GW.build([("general.architecture", GW.T_STRING, "llama")])[0]) as g:
         with pytest.raises(W.RocmError, match="missing lfm2.block_count"):
             RocmLfm2Model(ctx, g, 16)
+
+
+# ---- prompts (batched prefill) -------------------------------------------------------------------------------
+# The reference's prefill computes what n single steps compute, with the projections batched into GEMMs
+# (prefill_layers_and_logits, wick/src/model/lfm2.rs:1139-2109; its own tests compare prefill against sequential
+# decode by cosine / top-1, wick/tests/blas_parity.rs:71-152).  The oracle for a prompt is therefore the oracle's
+# sequential decode; the same quantizer-tie rule applies.
+
+def oracle_prompt(ref, tokens, state, start=0):
+    logits = None
+    for j, t in enumerate(tokens):
+        logits = ref.forward(int(t), start + j, state)
+    return logits
+
+
+@pytest.mark.parametrize("name,n", [("q4_0+q6k", 5), ("q4_0+q6k", 24), ("q8_0", 17), ("kernel4", 33), ("mixed-qkv", 16), ("3-layer-q4embd", 40)])
+def test_prefill_matches_the_oracle(ctx, oracle, tmp_path, name, n):
+    """n < 16 runs the projections as multi-token GEMVs, n >= 16 on the int8-MFMA GEMM."""
+    kw = CLEAR[name]
+    model, ref, cfg = load(ctx, oracle, tmp_path, **kw)
+    tokens = np.random.default_rng(7 + n).integers(0, cfg["vocab_size"], n)
+    state = ref.new_state()
+    want = oracle_prompt(ref, tokens, state)
+    got = model.forward_prefill(tokens, 0)
+    check_step(got, want, ref.min_margin, f"{name}: prompt of {n}")
+    assert cosine(got, want) >= 0.9999
+    # the state the prompt left behind (KV rows, conv state) carries the next single steps
+    for pos, tok in enumerate([3, 11], start=n):
+        check_step(model.forward(tok, pos), ref.forward(tok, pos, state), ref.min_margin, f"{name}: step after the prompt")
+    model.free()
+
+
+def test_prefill_in_pieces_and_against_single_steps(ctx, oracle, tmp_path):
+    model, ref, cfg = load(ctx, oracle, tmp_path, **CLEAR["q4_0+q6k"])
+    tokens = np.random.default_rng(3).integers(0, cfg["vocab_size"], 30)
+    whole = model.forward_prefill(tokens, 0)
+    model.reset()
+    model.forward_prefill(tokens[:18], 0)
+    pieces = model.forward_prefill(tokens[18:], 18)
+    model.reset()
+    single = None
+    for pos, t in enumerate(tokens):
+        single = model.forward(int(t), pos)
+    # same arithmetic up to GEMM-vs-GEMV summation order (and what a quantizer tie may do to it)
+    assert cosine(whole, pieces) >= 0.9999 and cosine(whole, single) >= 0.9999
+    assert int(np.argmax(whole)) == int(np.argmax(single))
+    with pytest.raises(W.RocmError, match="beyond the context"):
+        model.forward_prefill(tokens, 40)
+    with pytest.raises(W.RocmError, match="token_id out of range"):
+        model.forward_prefill([1, cfg["vocab_size"]], 0)
+    with pytest.raises(W.RocmError, match="empty prompt"):
+        model.forward_prefill([], 0)
+    model.free()
+
+
+def test_long_prompt_runs_in_passes(ctx, oracle, tmp_path):
+    """530 tokens = one pass of 512 + one of 18, attention over up to 530 cached positions."""
+    model, ref, cfg = load(ctx, oracle, tmp_path, context=600, **CLEAR["q4_0+q6k"])
+    tokens = np.random.default_rng(5).integers(0, cfg["vocab_size"], 530)
+    state = ref.new_state()
+    want = oracle_prompt(ref, tokens, state)
+    got = model.forward_prefill(tokens, 0)
+    check_step(got, want, ref.min_margin, "long prompt")
+    check_step(model.forward(9, 530), ref.forward(9, 530, state), ref.min_margin, "step after the long prompt")
+    model.free()

@@ -163,6 +163,11 @@ struct wick_rocm_lfm2 {
           *gate = nullptr, *scores = nullptr, *logits = nullptr;
     uint32_t *d_token = nullptr, *d_pos = nullptr, *d_pick = nullptr, *d_history = nullptr;
     unsigned long long* d_argmax_partial = nullptr;
+    // prompt (prefill) buffers for up to `prefill_cap` tokens, allocated by the first prefill
+    uint32_t prefill_cap = 0;
+    float *pX = nullptr, *pN = nullptr, *pA = nullptr, *pG = nullptr, *pGate = nullptr, *pUp = nullptr, *pS = nullptr, *pAttn = nullptr;
+    int8_t* pQ = nullptr;
+    uint32_t* pTokens = nullptr;
     wick_rocm_graph *g_logits = nullptr, *g_greedy = nullptr;
     bool use_graph = true;
     std::mutex mu;
@@ -299,6 +304,85 @@ int run_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
     wick_rocm_graph* g = nullptr;
     if (int rc = step_graph(ctx, m, greedy, &g)) return rc;
     return wick_rocm_graph_launch(ctx, g);
+}
+
+constexpr uint32_t kPrefillChunk = 512;  // tokens per pass of a prompt (MAX_PREFILL_TOKENS, wick/src/model/metal_lfm2.rs:25)
+
+int ensure_prefill_buffers(wick_rocm_ctx* ctx, wick_rocm_lfm2* m) {
+    if (m->prefill_cap) return WICK_ROCM_OK;
+    const wick_rocm_lfm2_config& c = m->cfg;
+    const size_t P = c.max_seq_len < kPrefillChunk ? c.max_seq_len : kPrefillChunk;
+    const size_t hs = c.hidden_size, inter = c.intermediate_size, hd = hs / c.n_heads, wide = hs > inter ? hs : inter;
+    int rc;
+    if ((rc = alloc_t(ctx, m, P * hs, &m->pX)) || (rc = alloc_t(ctx, m, P * hs, &m->pN)) || (rc = alloc_t(ctx, m, P * 3 * hs, &m->pA)) ||
+        (rc = alloc_t(ctx, m, P * hs, &m->pG)) || (rc = alloc_t(ctx, m, P * inter, &m->pGate)) || (rc = alloc_t(ctx, m, P * inter, &m->pUp)) ||
+        (rc = alloc_t(ctx, m, P * wide, &m->pQ)) || (rc = alloc_t(ctx, m, P * (wide / 32), &m->pS)) ||
+        (rc = alloc_t(ctx, m, attention_prefill_scratch_floats((uint32_t)P, c.n_heads, (uint32_t)hd), &m->pAttn)) ||
+        (rc = alloc_t(ctx, m, P, &m->pTokens)))
+        return rc;
+    m->prefill_cap = (uint32_t)P;
+    return WICK_ROCM_OK;
+}
+
+// y[n][y_stride] (+)= W x for n tokens: quantized activations (q, s) against one weight, token-major output.
+int gemm(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const wick_rocm_lfm2* m, uint32_t n, float* y, uint32_t y_stride, int accumulate) {
+    return wick_rocm_gemm_q8(ctx, w, m->pQ, m->pS, n, y, y_stride, WICK_ROCM_LAYOUT_TOKEN_MAJOR, accumulate);
+}
+
+// One pass of a prompt: n <= prefill_cap tokens (already in pTokens) at positions pos0 .. pos0 + n - 1.  The batched form
+// of enqueue_step (prefill_layers_and_logits, wick/src/model/lfm2.rs:1139-2109): projections as GEMMs over the tokens,
+// the conv state and the KV append walked in token order, causal attention per (head, token).
+int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint32_t pos0) {
+    const wick_rocm_lfm2_config& c = m->cfg;
+    const uint32_t hs = c.hidden_size, hd = hs / c.n_heads, inter = c.intermediate_size;
+    const float scale = 1.0f / sqrtf((float)hd);
+    auto locked = [&](auto&& launch, const char* what) {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        const hipError_t e = launch();
+        return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, what);
+    };
+    int rc = locked([&] { return launch_embed_rows(static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m, hs, m->pTokens, n, m->pX, ctx->launch()); },
+                    "embed_rows launch");
+    for (uint32_t i = 0; rc == 0 && i < c.n_layers; i++) {
+        const LayerWeights& L = m->layers[i];
+        if ((rc = wick_rocm_rmsnorm(ctx, m->pX, L.attn_norm, m->pN, n, hs, hs, hs, c.rms_norm_eps))) break;
+        if ((rc = wick_rocm_quantize_q8_0(ctx, m->pN, n, hs, hs, m->pQ, m->pS))) break;
+        if (L.n_kv == 0) {
+            if ((rc = gemm(ctx, L.in_proj, m, n, m->pA, 3 * hs, 0))) break;
+            if ((rc = locked([&] { return launch_shortconv_seq(m->pA, L.conv_state, L.conv_w, m->pG, hs, c.conv_kernel_size, n, ctx->launch()); },
+                             "shortconv_seq launch")))
+                break;
+        } else {
+            const uint32_t kvd = L.n_kv * hd, S = hs + 2 * kvd;  // a token's [q | k | v]
+            float *q = m->pA, *k = m->pA + hs, *v = m->pA + hs + kvd;
+            if ((rc = gemm(ctx, L.q, m, n, q, S, 0)) || (rc = gemm(ctx, L.k, m, n, k, S, 0)) || (rc = gemm(ctx, L.v, m, n, v, S, 0))) break;
+            if ((rc = locked([&] {
+                     return launch_qk_norm_rope(q, k, v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, pos0, nullptr, c.max_seq_len, hd, c.n_heads, L.n_kv,
+                                                c.rms_norm_eps, m->theta_scale, ctx->launch(), n, S, S);
+                 }, "qk_norm_rope launch")))
+                break;
+            if (attention_layer_applies(hd)) {
+                rc = locked([&] {
+                    return launch_attention_prefill(q, L.k_cache, L.v_cache, m->pG, m->pAttn, pos0, nullptr, n, S, hs, c.max_seq_len, c.n_heads, L.n_kv, hd,
+                                                    scale, ctx->launch());
+                }, "attention_prefill launch");
+            } else {  // head dims without a batched kernel: the decode kernel, token by token
+                for (uint32_t j = 0; rc == 0 && j < n; j++)
+                    rc = wick_rocm_attention_decode(ctx, q + (size_t)j * S, L.k_cache, L.v_cache, m->pG + (size_t)j * hs, m->scores, pos0 + j + 1, nullptr,
+                                                    c.max_seq_len, c.n_heads, L.n_kv, hd);
+            }
+            if (rc) break;
+        }
+        if ((rc = wick_rocm_quantize_q8_0(ctx, m->pG, n, hs, hs, m->pQ, m->pS))) break;
+        if ((rc = gemm(ctx, L.n_kv == 0 ? L.out_proj : L.o, m, n, m->pX, hs, 1))) break;  // hidden += out projection
+        if ((rc = wick_rocm_rmsnorm(ctx, m->pX, L.ffn_norm, m->pN, n, hs, hs, hs, c.rms_norm_eps))) break;
+        if ((rc = wick_rocm_quantize_q8_0(ctx, m->pN, n, hs, hs, m->pQ, m->pS))) break;
+        if ((rc = gemm(ctx, L.gate, m, n, m->pGate, inter, 0)) || (rc = gemm(ctx, L.up, m, n, m->pUp, inter, 0))) break;
+        if ((rc = wick_rocm_silu_mul(ctx, m->pGate, m->pUp, n * inter))) break;
+        if ((rc = wick_rocm_quantize_q8_0(ctx, m->pGate, n, inter, inter, m->pQ, m->pS))) break;
+        rc = gemm(ctx, L.down, m, n, m->pX, hs, 1);
+    }
+    return rc;
 }
 
 int set_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t token, uint32_t pos) {
@@ -465,6 +549,29 @@ int wick_rocm_lfm2_forward(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t t
     if (int rc = set_step(ctx, model, token, pos)) return rc;
     if (int rc = run_step(ctx, model, false)) return rc;
     if (logits) return wick_rocm_download(ctx, logits, model->logits, (size_t)model->cfg.vocab_size * sizeof(float));
+    return wick_rocm_sync(ctx);
+}
+
+int wick_rocm_lfm2_forward_prefill(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, const uint32_t* tokens, uint32_t n, uint32_t start_pos, float* logits) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    if (!tokens || n == 0) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 prefill: empty prompt");
+    std::lock_guard<std::mutex> lk(model->mu);
+    const wick_rocm_lfm2_config& c = model->cfg;
+    for (uint32_t j = 0; j < n; j++)
+        if (tokens[j] >= c.vocab_size) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: token_id out of range");
+    if ((uint64_t)start_pos + n > c.max_seq_len) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: position beyond the context size");
+    if (c.conv_kernel_size > 8) return ctx_fail(ctx, WICK_ROCM_ERR_UNSUPPORTED_DTYPE, "lfm2 prefill: conv kernel size above 8");
+    if (int rc = ensure_prefill_buffers(ctx, model)) return rc;
+    uint32_t last = 0;
+    for (uint32_t done = 0; done < n; done += model->prefill_cap) {
+        last = n - done < model->prefill_cap ? n - done : model->prefill_cap;
+        if (int rc = wick_rocm_upload(ctx, model->pTokens, tokens + done, (size_t)last * sizeof(uint32_t))) return rc;
+        if (int rc = enqueue_prompt_pass(ctx, model, last, start_pos + done)) return rc;
+    }
+    // output norm + tied LM head on the last token only (wick/src/model/lfm2.rs:2080-2109)
+    const float* h_last = model->pX + (size_t)(last - 1) * c.hidden_size;
+    if (int rc = gemv_normed(ctx, {model->embd}, {model->logits}, h_last, model->out_norm, c.rms_norm_eps)) return rc;
+    if (logits) return wick_rocm_download(ctx, logits, model->logits, (size_t)c.vocab_size * sizeof(float));
     return wick_rocm_sync(ctx);
 }
 

@@ -40,33 +40,42 @@ __device__ __forceinline__ double block_sum_f64(double v, double* slots) {
 // ---- embedding row -------------------------------------------------------------------
 // dequantize_row_into (wick/src/model/lfm2.rs:621-643) for Q4_0 / Q8_0 (quant.rs:78-90, 154-161) and
 // Q6_K (quant.rs:380-412: d * sc * q left to right): bit-exact.
+__device__ __forceinline__ float dequant_element(const uint8_t* __restrict__ w, int type, uint32_t row, uint32_t k, uint32_t e) {
+    if (type == kTypeQ6_K) {
+        const uint8_t* blk = w + ((size_t)row * (k >> 8) + (e >> 8)) * kQ6KBlockBytes;
+        const uint32_t i = e & 255u, n = i >> 7, j = (i >> 5) & 3u, l = i & 31u;
+        const uint32_t lo = (blk[64 * n + 32 * (j & 1u) + l] >> (4 * (j >> 1))) & 15u;
+        const uint32_t hi = (blk[128 + 32 * n + l] >> (2 * j)) & 3u;
+        const int q = (int)(lo | (hi << 4)) - 32;
+        const float d = f16_bits_to_f32((uint32_t)blk[208] | ((uint32_t)blk[209] << 8));
+        const float sc = (float)(int)(int8_t)blk[192 + (i >> 4)];
+        return __fmul_rn(__fmul_rn(d, sc), (float)q);
+    }
+    if (type == kTypeQ4_0) {
+        const uint8_t* blk = w + ((size_t)row * (k >> 5) + (e >> 5)) * kQ4BlockBytes;
+        const uint32_t i = e & 31u;
+        const uint32_t byte = blk[2 + (i & 15u)];
+        const int q = (int)((i < 16u) ? (byte & 15u) : (byte >> 4)) - 8;
+        return __fmul_rn((float)q, f16_bits_to_f32((uint32_t)blk[0] | ((uint32_t)blk[1] << 8)));
+    }
+    const uint8_t* blk = w + ((size_t)row * (k >> 5) + (e >> 5)) * kQ8BlockBytes;
+    return __fmul_rn((float)(int)(int8_t)blk[2 + (e & 31u)], f16_bits_to_f32((uint32_t)blk[0] | ((uint32_t)blk[1] << 8)));
+}
+
 __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restrict__ w, int type, uint32_t m, uint32_t k, uint32_t token,
                                                         const uint32_t* __restrict__ d_token, float* __restrict__ out) {
     const uint32_t row = d_token ? *d_token : token;
     if (row >= m) return;  // the host checks a by-value token; a device-side token out of range leaves `out` untouched
-    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < k; e += gridDim.x * blockDim.x) {
-        float v;
-        if (type == kTypeQ6_K) {
-            const uint8_t* blk = w + ((size_t)row * (k >> 8) + (e >> 8)) * kQ6KBlockBytes;
-            const uint32_t i = e & 255u, n = i >> 7, j = (i >> 5) & 3u, l = i & 31u;
-            const uint32_t lo = (blk[64 * n + 32 * (j & 1u) + l] >> (4 * (j >> 1))) & 15u;
-            const uint32_t hi = (blk[128 + 32 * n + l] >> (2 * j)) & 3u;
-            const int q = (int)(lo | (hi << 4)) - 32;
-            const float d = f16_bits_to_f32((uint32_t)blk[208] | ((uint32_t)blk[209] << 8));
-            const float sc = (float)(int)(int8_t)blk[192 + (i >> 4)];
-            v = __fmul_rn(__fmul_rn(d, sc), (float)q);
-        } else if (type == kTypeQ4_0) {
-            const uint8_t* blk = w + ((size_t)row * (k >> 5) + (e >> 5)) * kQ4BlockBytes;
-            const uint32_t i = e & 31u;
-            const uint32_t byte = blk[2 + (i & 15u)];
-            const int q = (int)((i < 16u) ? (byte & 15u) : (byte >> 4)) - 8;
-            v = __fmul_rn((float)q, f16_bits_to_f32((uint32_t)blk[0] | ((uint32_t)blk[1] << 8)));
-        } else {
-            const uint8_t* blk = w + ((size_t)row * (k >> 5) + (e >> 5)) * kQ8BlockBytes;
-            v = __fmul_rn((float)(int)(int8_t)blk[2 + (e & 31u)], f16_bits_to_f32((uint32_t)blk[0] | ((uint32_t)blk[1] << 8)));
-        }
-        out[e] = v;
-    }
+    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < k; e += gridDim.x * blockDim.x) out[e] = dequant_element(w, type, row, k, e);
+}
+
+// The rows of a whole prompt: out[j][k] = row d_tokens[j] (blockIdx.y = j).
+__global__ __launch_bounds__(256) void embed_rows_kernel(const uint8_t* __restrict__ w, int type, uint32_t m, uint32_t k,
+                                                         const uint32_t* __restrict__ d_tokens, float* __restrict__ out) {
+    const uint32_t row = d_tokens[blockIdx.y];
+    if (row >= m) return;
+    float* o = out + (size_t)blockIdx.y * k;
+    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < k; e += gridDim.x * blockDim.x) o[e] = dequant_element(w, type, row, k, e);
 }
 
 // ---- RMSNorm ---------------------------------------------------------------------------
@@ -105,6 +114,7 @@ struct QkNormRopeArgs {
     const uint32_t* d_pos;  // may be null
     uint32_t pos, max_seq, head_dim, n_heads, n_kv_heads;
     float eps, theta_scale;
+    uint32_t q_stride, kv_stride;  // floats between consecutive tokens of q / of k and v (a prompt: blockIdx.y = token, position pos + token)
 };
 
 // RMSNorm + RoPE of one head by the calling wave: dst[] (and dst2[], when given) receive the result; src may equal dst.
@@ -132,16 +142,17 @@ __device__ __forceinline__ void norm_rope_head(const float* src, const float* w,
 }
 
 __global__ __launch_bounds__(64) void qk_norm_rope_kernel(QkNormRopeArgs a) {
-    const uint32_t pos = a.d_pos ? *a.d_pos : a.pos;
+    const uint32_t tok = blockIdx.y;
+    const uint32_t pos = (a.d_pos ? *a.d_pos : a.pos) + tok;
     const bool is_q = blockIdx.x < a.n_heads;
     const uint32_t h = is_q ? blockIdx.x : blockIdx.x - a.n_heads;
     const uint32_t hd = a.head_dim, kv_dim = a.n_kv_heads * hd;
-    float* head = (is_q ? a.q : a.k) + (size_t)h * hd;
+    float* head = (is_q ? a.q + (size_t)tok * a.q_stride : a.k + (size_t)tok * a.kv_stride) + (size_t)h * hd;
     const bool store = !is_q && pos < a.max_seq;  // the host checks a by-value pos; a device-side pos past the cache is dropped
     norm_rope_head(head, is_q ? a.q_norm : a.k_norm, hd, pos, a.eps, a.theta_scale, head,
                    store ? a.k_cache + (size_t)pos * kv_dim + (size_t)h * hd : nullptr);
     if (store) {
-        const float* vh = a.v + (size_t)h * hd;
+        const float* vh = a.v + (size_t)tok * a.kv_stride + (size_t)h * hd;
         float* vc = a.v_cache + (size_t)pos * kv_dim + (size_t)h * hd;
         for (uint32_t i = threadIdx.x; i < hd; i += 64) vc[i] = vh[i];
     }
@@ -453,6 +464,23 @@ __global__ __launch_bounds__(256) void attention_layer_kernel(AttentionLayerArgs
     attention_chunks<HD>(a, splits, h, split, seq, qh);
 }
 
+// Causal attention for the n tokens of a prompt whose K / V rows are already in the caches (pass B of the reference's
+// batched prefill, wick/src/model/lfm2.rs:1640-1700): workgroup (head, token j) attends query j over positions
+// [0, pos0 + j] with the streaming-softmax chunks above (it walks all its chunks itself: splits = 1) and normalises.
+// q: [n][q_stride] floats, out: [n][out_stride]; scratch: n * n_heads partial records.
+template <int HD>
+__global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a, uint32_t pos0, uint32_t q_stride, uint32_t out_stride) {
+    const uint32_t h = blockIdx.x, j = blockIdx.y;
+    uint32_t seq = (a.d_pos ? *a.d_pos : pos0) + j + 1u;
+    if (seq > a.max_seq) seq = a.max_seq;
+    AttentionArgs mine = a;
+    mine.scores = a.scores + (size_t)j * a.n_heads * (HD + 2);
+    attention_chunks<HD>(mine, 1u, h, 0u, seq, a.q + (size_t)j * q_stride + (size_t)h * HD);
+    __syncthreads();  // the partial record written by this workgroup
+    const float* part = mine.scores + (size_t)h * (HD + 2);
+    if (threadIdx.x < HD) a.out[(size_t)j * out_stride + (size_t)h * HD + threadIdx.x] = __fdiv_rn(part[2 + threadIdx.x], part[1]);
+}
+
 // ---- gated short convolution, one step ---------------------------------------------------
 // forward_conv_block's middle (wick/src/model/lfm2.rs:694-726): proj = [b | c | x]; bx = b*x;
 // out = c * (sum_k buffer[k][ch]*w[ch][k] + bx*w[ch][K-1]); the rolling buffer shifts by one slot and takes bx.
@@ -474,6 +502,42 @@ __global__ __launch_bounds__(256) void shortconv_step_kernel(const float* __rest
     sum = __fadd_rn(sum, __fmul_rn(bx, w[d_conv]));
     if (d_conv > 0) buffer[(size_t)(d_conv - 1) * hidden + ch] = bx;
     out[ch] = __fmul_rn(proj[hidden + ch], sum);
+}
+
+// The same step for the n tokens of a prompt in order (the sequential core of the reference's batched prefill,
+// wick/src/model/lfm2.rs:1306-1350): proj [n][3 * hidden], out [n][hidden]; one thread per channel walks the tokens,
+// the rolling state in registers.  Per token the arithmetic is shortconv_step_kernel's: bit-exact.
+template <int KMAX>
+__global__ __launch_bounds__(256) void shortconv_seq_kernel(const float* __restrict__ proj, float* __restrict__ buffer,
+                                                            const float* __restrict__ conv_w, float* __restrict__ out, uint32_t hidden,
+                                                            uint32_t kernel_size, uint32_t n) {
+    const uint32_t ch = blockIdx.x * blockDim.x + threadIdx.x;
+    if (ch >= hidden) return;
+    const uint32_t d_conv = kernel_size - 1;  // <= KMAX - 1
+    float w[KMAX], st[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; k++) {
+        w[k] = (uint32_t)k < kernel_size ? conv_w[(size_t)ch * kernel_size + k] : 0.0f;
+        st[k] = (uint32_t)k < d_conv ? buffer[(size_t)k * hidden + ch] : 0.0f;
+    }
+    for (uint32_t j = 0; j < n; j++) {
+        const float* p = proj + (size_t)j * 3 * hidden;
+        const float bx = __fmul_rn(p[ch], p[2 * hidden + ch]);
+        float sum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KMAX - 1; k++)
+            if ((uint32_t)k < d_conv) sum = __fadd_rn(sum, __fmul_rn(st[k], w[k]));
+        float wl = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KMAX; k++) wl = (uint32_t)k == d_conv ? w[k] : wl;
+        sum = __fadd_rn(sum, __fmul_rn(bx, wl));
+#pragma unroll
+        for (int k = 0; k < KMAX - 1; k++) st[k] = (uint32_t)(k + 1) < d_conv ? st[k + 1] : ((uint32_t)(k + 1) == d_conv ? bx : st[k]);
+        out[(size_t)j * hidden + ch] = __fmul_rn(p[hidden + ch], sum);
+    }
+#pragma unroll
+    for (int k = 0; k < KMAX - 1; k++)
+        if ((uint32_t)k < d_conv) buffer[(size_t)k * hidden + ch] = st[k];
 }
 
 // ---- SiLU gate ------------------------------------------------------------------------
@@ -590,9 +654,12 @@ hipError_t launch_rmsnorm(const float* d_x, const float* d_weight, float* d_y, u
 
 hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm, float* d_k_cache,
                                float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
-                               uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L) {
-    QkNormRopeArgs a{d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, d_pos, pos, max_seq, head_dim, n_heads, n_kv_heads, eps, theta_scale};
-    return launch_kernel(L, kFamOther, qk_norm_rope_kernel, dim3(n_heads + n_kv_heads), dim3(64), a);
+                               uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L, uint32_t n_tokens, uint32_t q_stride,
+                               uint32_t kv_stride) {
+    if (n_tokens == 0) return hipSuccess;
+    QkNormRopeArgs a{d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, d_pos, pos, max_seq, head_dim, n_heads, n_kv_heads, eps, theta_scale,
+                     q_stride, kv_stride};
+    return launch_kernel(L, kFamOther, qk_norm_rope_kernel, dim3(n_heads + n_kv_heads, n_tokens), dim3(64), a);
 }
 
 hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scores,
@@ -662,6 +729,39 @@ hipError_t launch_shortconv_step(const float* d_proj, float* d_buffer, const flo
                                  uint32_t kernel_size, const Launch& L) {
     return launch_kernel(L, kFamOther, shortconv_step_kernel, dim3((hidden + 255u) / 256u), dim3(256), d_proj, d_buffer, d_conv_w, d_out, hidden,
                          kernel_size);
+}
+
+hipError_t launch_embed_rows(const uint8_t* d_w, int type, uint32_t m, uint32_t k, const uint32_t* d_tokens, uint32_t n, float* d_out,
+                             const Launch& L) {
+    if (n == 0) return hipSuccess;
+    const uint32_t blocks = (k + 255u) / 256u;
+    return launch_kernel(L, kFamOther, embed_rows_kernel, dim3(blocks < 16u ? blocks : 16u, n), dim3(256), d_w, type, m, k, d_tokens, d_out);
+}
+
+hipError_t launch_shortconv_seq(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
+                                uint32_t kernel_size, uint32_t n, const Launch& L) {
+    if (n == 0) return hipSuccess;
+    const dim3 grid((hidden + 255u) / 256u), block(256);
+    if (kernel_size <= 4) return launch_kernel(L, kFamOther, shortconv_seq_kernel<4>, grid, block, d_proj, d_buffer, d_conv_w, d_out, hidden, kernel_size, n);
+    if (kernel_size <= 8) return launch_kernel(L, kFamOther, shortconv_seq_kernel<8>, grid, block, d_proj, d_buffer, d_conv_w, d_out, hidden, kernel_size, n);
+    return hipErrorInvalidValue;
+}
+
+size_t attention_prefill_scratch_floats(uint32_t n, uint32_t n_heads, uint32_t head_dim) { return (size_t)n * n_heads * (head_dim + 2); }
+
+hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scratch,
+                                    uint32_t pos0, const uint32_t* d_pos, uint32_t n, uint32_t q_stride, uint32_t out_stride, uint32_t max_seq,
+                                    uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L) {
+    if (n == 0) return hipSuccess;
+    AttentionArgs a{d_q, d_k_cache, d_v_cache, d_out, d_scratch, d_pos, 0u, max_seq, n_heads, n_kv_heads, head_dim, scale};
+    const dim3 grid(n_heads, n), block(256);
+    switch (head_dim) {
+        case 32: return launch_kernel(L, kFamOther, attention_prefill_kernel<32>, grid, block, a, pos0, q_stride, out_stride);
+        case 64: return launch_kernel(L, kFamOther, attention_prefill_kernel<64>, grid, block, a, pos0, q_stride, out_stride);
+        case 128: return launch_kernel(L, kFamOther, attention_prefill_kernel<128>, grid, block, a, pos0, q_stride, out_stride);
+        case 256: return launch_kernel(L, kFamOther, attention_prefill_kernel<256>, grid, block, a, pos0, q_stride, out_stride);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const Launch& L) {

@@ -137,7 +137,19 @@ hipError_t launch_rmsnorm(const float* d_x, const float* d_weight, float* d_y, u
                           uint32_t y_stride, float eps, const Launch& L);
 hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm, float* d_k_cache,
                                float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
-                               uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L);
+                               uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L, uint32_t n_tokens = 1, uint32_t q_stride = 0,
+                               uint32_t kv_stride = 0);
+// A prompt of n tokens at once (token j at position pos + j): embedding rows [n][k], the short conv walked over the tokens
+// (kernel_size <= 8), causal attention over caches that already hold the prompt's K / V rows (head_dim 32 / 64 / 128 / 256;
+// scratch: attention_prefill_scratch_floats).
+hipError_t launch_embed_rows(const uint8_t* d_w, int type, uint32_t m, uint32_t k, const uint32_t* d_tokens, uint32_t n, float* d_out,
+                             const Launch& L);
+hipError_t launch_shortconv_seq(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
+                                uint32_t kernel_size, uint32_t n, const Launch& L);
+size_t attention_prefill_scratch_floats(uint32_t n, uint32_t n_heads, uint32_t head_dim);
+hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scratch,
+                                    uint32_t pos0, const uint32_t* d_pos, uint32_t n, uint32_t q_stride, uint32_t out_stride, uint32_t max_seq,
+                                    uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L);
 // d_scores is scratch of attention_scratch_floats(max_seq, n_heads, head_dim) floats.
 uint32_t attention_splits(uint32_t max_seq);
 size_t attention_scratch_floats(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim);

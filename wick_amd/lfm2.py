@@ -43,6 +43,7 @@ _SIGNATURES = {
     "wick_rocm_lfm2_reset": (C.c_int, [_P, _P]),
     "wick_rocm_lfm2_set_graph_replay": (C.c_int, [_P, C.c_int]),
     "wick_rocm_lfm2_forward": (C.c_int, [_P, _P, _U32, _U32, _P]),
+    "wick_rocm_lfm2_forward_prefill": (C.c_int, [_P, _P, _P, _U32, _U32, _P]),
     "wick_rocm_lfm2_forward_greedy": (C.c_int, [_P, _P, _U32, _U32, C.POINTER(_U32)]),
     "wick_rocm_lfm2_generate_greedy": (C.c_int, [_P, _P, _U32, _U32, _U32, _P]),
     "wick_rocm_lfm2_logits_device": (_P, [_P]),
@@ -155,6 +156,13 @@ class RocmLfm2Model:
     def forward(self, token: int, pos: int) -> np.ndarray:
         logits = np.empty(self.config["vocab_size"], np.float32)
         self.ctx._check(self._l.wick_rocm_lfm2_forward(self.ctx._h, self._h, token, pos, logits.ctypes.data))
+        return logits
+
+    def forward_prefill(self, tokens, start_pos: int) -> np.ndarray:
+        """Model::forward_prefill: the logits of the last prompt token."""
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        logits = np.empty(self.config["vocab_size"], np.float32)
+        self.ctx._check(self._l.wick_rocm_lfm2_forward_prefill(self.ctx._h, self._h, t.ctypes.data, t.size, start_pos, logits.ctypes.data))
         return logits
 
     def forward_greedy(self, token: int, pos: int) -> int:
