@@ -282,6 +282,17 @@ def bench_lfm2_step(ctx, W, O, tokens=64, context=4096):
         model.generate_greedy(1, start, tokens)
         dt = time.perf_counter() - t0
         out["runs"].append({"start_pos": start, "tokens": tokens, "ms_per_token": dt / tokens * 1e3, "tokens_per_s": tokens / dt})
+    # prompts: the batched pass (projections on the int8-MFMA GEMM)
+    out["prefill"] = []
+    for n in (512, 2002):
+        toks = np.random.default_rng(n).integers(0, VOCAB, n)
+        model.reset()
+        model.forward_prefill(toks[:64], 0)  # buffers allocated, kernels warm
+        model.reset()
+        t0 = time.perf_counter()
+        model.forward_prefill(toks, 0)
+        dt = time.perf_counter() - t0
+        out["prefill"].append({"prompt_tokens": n, "ms": dt * 1e3, "tokens_per_s": n / dt})
     # where the time goes: the same steps enqueued one by one with per-dispatch timestamps
     model.set_graph_replay(False)
     model.reset()

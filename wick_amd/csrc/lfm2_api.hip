@@ -331,7 +331,8 @@ int gemm(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const wick_rocm_lfm2* m,
 
 // One pass of a prompt: n <= prefill_cap tokens (already in pTokens) at positions pos0 .. pos0 + n - 1.  The batched form
 // of enqueue_step (prefill_layers_and_logits, wick/src/model/lfm2.rs:1139-2109): projections as GEMMs over the tokens,
-// the conv state and the KV append walked in token order, causal attention per (head, token).
+// the short conv per (token, channel) with the rolling state behind it, the KV append per token, causal attention per
+// (head, token).
 int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint32_t pos0) {
     const wick_rocm_lfm2_config& c = m->cfg;
     const uint32_t hs = c.hidden_size, hd = hs / c.n_heads, inter = c.intermediate_size;
@@ -560,7 +561,6 @@ int wick_rocm_lfm2_forward_prefill(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, co
     for (uint32_t j = 0; j < n; j++)
         if (tokens[j] >= c.vocab_size) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: token_id out of range");
     if ((uint64_t)start_pos + n > c.max_seq_len) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: position beyond the context size");
-    if (c.conv_kernel_size > 8) return ctx_fail(ctx, WICK_ROCM_ERR_UNSUPPORTED_DTYPE, "lfm2 prefill: conv kernel size above 8");
     if (int rc = ensure_prefill_buffers(ctx, model)) return rc;
     uint32_t last = 0;
     for (uint32_t done = 0; done < n; done += model->prefill_cap) {

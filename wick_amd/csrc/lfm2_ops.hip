@@ -504,40 +504,53 @@ __global__ __launch_bounds__(256) void shortconv_step_kernel(const float* __rest
     out[ch] = __fmul_rn(proj[hidden + ch], sum);
 }
 
-// The same step for the n tokens of a prompt in order (the sequential core of the reference's batched prefill,
-// wick/src/model/lfm2.rs:1306-1350): proj [n][3 * hidden], out [n][hidden]; one thread per channel walks the tokens,
-// the rolling state in registers.  Per token the arithmetic is shortconv_step_kernel's: bit-exact.
-template <int KMAX>
-__global__ __launch_bounds__(256) void shortconv_seq_kernel(const float* __restrict__ proj, float* __restrict__ buffer,
+// The same step for the n tokens of a prompt (the sequential core of the reference's batched prefill,
+// wick/src/model/lfm2.rs:1306-1350).  The convolution has no recurrence -- token j sees the gated inputs b*x of
+// tokens j - (K-1) .. j, the ones before the prompt coming from the rolling state -- so every (token, channel) is
+// computed on its own, taps summed oldest first exactly like shortconv_step_kernel: bit-exact.  The state is brought
+// up to date by a second small kernel once every token has read the old one.
+// proj [n][3 * hidden], out [n][hidden]; blockIdx.y = token.
+__global__ __launch_bounds__(256) void shortconv_seq_kernel(const float* __restrict__ proj, const float* __restrict__ buffer,
                                                             const float* __restrict__ conv_w, float* __restrict__ out, uint32_t hidden,
-                                                            uint32_t kernel_size, uint32_t n) {
+                                                            uint32_t kernel_size) {
+    const uint32_t ch = blockIdx.x * blockDim.x + threadIdx.x, j = blockIdx.y;
+    if (ch >= hidden) return;
+    const uint32_t d_conv = kernel_size - 1;
+    const float* w = conv_w + (size_t)ch * kernel_size;
+    float sum = 0.0f;
+    for (uint32_t k = 0; k < d_conv; k++) {
+        const int t = (int)j - (int)d_conv + (int)k;  // token of this tap, < 0: before the prompt
+        float tap;
+        if (t < 0) {
+            tap = buffer[(size_t)(t + (int)d_conv) * hidden + ch];
+        } else {
+            const float* p = proj + (size_t)t * 3 * hidden;
+            tap = __fmul_rn(p[ch], p[2 * hidden + ch]);
+        }
+        sum = __fadd_rn(sum, __fmul_rn(tap, w[k]));
+    }
+    const float* p = proj + (size_t)j * 3 * hidden;
+    sum = __fadd_rn(sum, __fmul_rn(__fmul_rn(p[ch], p[2 * hidden + ch]), w[d_conv]));
+    out[(size_t)j * hidden + ch] = __fmul_rn(p[hidden + ch], sum);
+}
+
+// New rolling state after n prompt tokens: slot s holds b*x of token n - (K-1) + s (an old slot when that is negative).
+__global__ __launch_bounds__(256) void shortconv_state_kernel(const float* __restrict__ proj, float* __restrict__ buffer, uint32_t hidden,
+                                                              uint32_t kernel_size, uint32_t n) {
     const uint32_t ch = blockIdx.x * blockDim.x + threadIdx.x;
     if (ch >= hidden) return;
-    const uint32_t d_conv = kernel_size - 1;  // <= KMAX - 1
-    float w[KMAX], st[KMAX];
-#pragma unroll
-    for (int k = 0; k < KMAX; k++) {
-        w[k] = (uint32_t)k < kernel_size ? conv_w[(size_t)ch * kernel_size + k] : 0.0f;
-        st[k] = (uint32_t)k < d_conv ? buffer[(size_t)k * hidden + ch] : 0.0f;
+    const int d_conv = (int)kernel_size - 1;
+    for (int s = 0; s < d_conv; s++) {  // ascending: slot s only ever takes a value from a slot above it
+        const int t = (int)n - d_conv + s;
+        float v;
+        if (t < 0) {
+            v = buffer[(size_t)(t + d_conv) * hidden + ch];
+        } else {
+            const float* p = proj + (size_t)t * 3 * hidden;
+            v = __fmul_rn(p[ch], p[2 * hidden + ch]);
+        }
+        buffer[(size_t)s * hidden + ch] = v;
     }
-    for (uint32_t j = 0; j < n; j++) {
-        const float* p = proj + (size_t)j * 3 * hidden;
-        const float bx = __fmul_rn(p[ch], p[2 * hidden + ch]);
-        float sum = 0.0f;
-#pragma unroll
-        for (int k = 0; k < KMAX - 1; k++)
-            if ((uint32_t)k < d_conv) sum = __fadd_rn(sum, __fmul_rn(st[k], w[k]));
-        float wl = 0.0f;
-#pragma unroll
-        for (int k = 0; k < KMAX; k++) wl = (uint32_t)k == d_conv ? w[k] : wl;
-        sum = __fadd_rn(sum, __fmul_rn(bx, wl));
-#pragma unroll
-        for (int k = 0; k < KMAX - 1; k++) st[k] = (uint32_t)(k + 1) < d_conv ? st[k + 1] : ((uint32_t)(k + 1) == d_conv ? bx : st[k]);
-        out[(size_t)j * hidden + ch] = __fmul_rn(p[hidden + ch], sum);
-    }
-#pragma unroll
-    for (int k = 0; k < KMAX - 1; k++)
-        if ((uint32_t)k < d_conv) buffer[(size_t)k * hidden + ch] = st[k];
 }
 
 // ---- SiLU gate ------------------------------------------------------------------------
@@ -741,10 +754,11 @@ hipError_t launch_embed_rows(const uint8_t* d_w, int type, uint32_t m, uint32_t 
 hipError_t launch_shortconv_seq(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
                                 uint32_t kernel_size, uint32_t n, const Launch& L) {
     if (n == 0) return hipSuccess;
-    const dim3 grid((hidden + 255u) / 256u), block(256);
-    if (kernel_size <= 4) return launch_kernel(L, kFamOther, shortconv_seq_kernel<4>, grid, block, d_proj, d_buffer, d_conv_w, d_out, hidden, kernel_size, n);
-    if (kernel_size <= 8) return launch_kernel(L, kFamOther, shortconv_seq_kernel<8>, grid, block, d_proj, d_buffer, d_conv_w, d_out, hidden, kernel_size, n);
-    return hipErrorInvalidValue;
+    const uint32_t blocks = (hidden + 255u) / 256u;
+    hipError_t e = launch_kernel(L, kFamOther, shortconv_seq_kernel, dim3(blocks, n), dim3(256), d_proj, static_cast<const float*>(d_buffer), d_conv_w,
+                                 d_out, hidden, kernel_size);
+    if (e != hipSuccess || kernel_size < 2) return e;
+    return launch_kernel(L, kFamOther, shortconv_state_kernel, dim3(blocks), dim3(256), d_proj, d_buffer, hidden, kernel_size, n);
 }
 
 size_t attention_prefill_scratch_floats(uint32_t n, uint32_t n_heads, uint32_t head_dim) { return (size_t)n * n_heads * (head_dim + 2); }

@@ -139,8 +139,7 @@ hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const f
                                float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
                                uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L, uint32_t n_tokens = 1, uint32_t q_stride = 0,
                                uint32_t kv_stride = 0);
-// A prompt of n tokens at once (token j at position pos + j): embedding rows [n][k], the short conv walked over the tokens
-// (kernel_size <= 8), causal attention over caches that already hold the prompt's K / V rows (head_dim 32 / 64 / 128 / 256;
+// A prompt of n tokens at once (token j at position pos + j): embedding rows [n][k], the short conv of every (token, channel), causal attention over caches that already hold the prompt's K / V rows (head_dim 32 / 64 / 128 / 256;
 // scratch: attention_prefill_scratch_floats).
 hipError_t launch_embed_rows(const uint8_t* d_w, int type, uint32_t m, uint32_t k, const uint32_t* d_tokens, uint32_t n, float* d_out,
                              const Launch& L);
