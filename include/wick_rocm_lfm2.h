@@ -120,7 +120,7 @@ int wick_rocm_lfm2_set_graph_replay(wick_rocm_lfm2 *model, int enabled);
  * vocab_size logits copied to `logits` (host memory; may be null to leave them on the device).  Waits for the step. */
 int wick_rocm_lfm2_forward(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t token, uint32_t pos, float *logits);
 /* Model::forward_prefill (wick/src/model/lfm2.rs:2351-2443, prefill_layers_and_logits :1139-2109): n prompt tokens at
- * positions start_pos .. start_pos + n - 1 in passes of up to 512; projections run as GEMMs over the tokens, the conv
+ * positions start_pos .. start_pos + n - 1 in passes of up to 2048; projections run as GEMMs over the tokens, the conv
  * state and the KV append are walked in token order, attention is causal per (head, token).  Leaves the state as n
  * single steps would (up to the rounding of GEMM against GEMV sums) and returns the logits of the LAST token. */
 int wick_rocm_lfm2_forward_prefill(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, const uint32_t *tokens, uint32_t n, uint32_t start_pos,

@@ -229,12 +229,12 @@ def test_prefill_in_pieces_and_against_single_steps(ctx, oracle, tmp_path):
 
 
 def test_long_prompt_runs_in_passes(ctx, oracle, tmp_path):
-    """530 tokens = one pass of 512 + one of 18, attention over up to 530 cached positions."""
-    model, ref, cfg = load(ctx, oracle, tmp_path, context=600, **CLEAR["q4_0+q6k"])
-    tokens = np.random.default_rng(5).integers(0, cfg["vocab_size"], 530)
+    """2100 tokens = one pass of 2048 + one of 52, attention over up to 2100 cached positions."""
+    model, ref, cfg = load(ctx, oracle, tmp_path, context=2200, **CLEAR["q4_0+q6k"])
+    tokens = np.random.default_rng(5).integers(0, cfg["vocab_size"], 2100)
     state = ref.new_state()
     want = oracle_prompt(ref, tokens, state)
     got = model.forward_prefill(tokens, 0)
     check_step(got, want, ref.min_margin, "long prompt")
-    check_step(model.forward(9, 530), ref.forward(9, 530, state), ref.min_margin, "step after the long prompt")
+    check_step(model.forward(9, 2100), ref.forward(9, 2100, state), ref.min_margin, "step after the long prompt")
     model.free()

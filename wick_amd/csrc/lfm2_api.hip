@@ -306,7 +306,8 @@ int run_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
     return wick_rocm_graph_launch(ctx, g);
 }
 
-constexpr uint32_t kPrefillChunk = 512;  // tokens per pass of a prompt (MAX_PREFILL_TOKENS, wick/src/model/metal_lfm2.rs:25)
+constexpr uint32_t kPrefillChunk = 2048;  // tokens per pass of a prompt (the reference's Metal path uses 512, MAX_PREFILL_TOKENS, wick/src/model/metal_lfm2.rs:25;
+                                          // 288 GB of HBM afford four times that, and the GEMMs run better the wider they are)
 
 int ensure_prefill_buffers(wick_rocm_ctx* ctx, wick_rocm_lfm2* m) {
     if (m->prefill_cap) return WICK_ROCM_OK;
