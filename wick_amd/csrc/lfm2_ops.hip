@@ -465,20 +465,116 @@ __global__ __launch_bounds__(256) void attention_layer_kernel(AttentionLayerArgs
 }
 
 // Causal attention for the n tokens of a prompt whose K / V rows are already in the caches (pass B of the reference's
-// batched prefill, wick/src/model/lfm2.rs:1640-1700): workgroup (head, token j) attends query j over positions
-// [0, pos0 + j] with the streaming-softmax chunks above (it walks all its chunks itself: splits = 1) and normalises.
-// q: [n][q_stride] floats, out: [n][out_stride]; scratch: n * n_heads partial records.
+// batched prefill, wick/src/model/lfm2.rs:1640-1700).  A workgroup takes QB = 8 consecutive query tokens of one head and
+// walks the 64-position chunks of the cache once for all of them: every key / value row it loads serves eight queries
+// (one workgroup per query re-read the caches 2002 times for a 2002-token prompt and was L2-bound at 1 ms per layer).
+// Per chunk: scores of the 8 queries (rows past a query's own position masked), streaming softmax with each wave
+// owning two queries (64 positions = one wave: shuffles only), then the weighted value sums for all eight from one set
+// of value loads.  q: [n][q_stride] floats, out: [n][out_stride].
 template <int HD>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a, uint32_t pos0, uint32_t q_stride, uint32_t out_stride) {
-    const uint32_t h = blockIdx.x, j = blockIdx.y;
-    uint32_t seq = (a.d_pos ? *a.d_pos : pos0) + j + 1u;
-    if (seq > a.max_seq) seq = a.max_seq;
-    AttentionArgs mine = a;
-    mine.scores = a.scores + (size_t)j * a.n_heads * (HD + 2);
-    attention_chunks<HD>(mine, 1u, h, 0u, seq, a.q + (size_t)j * q_stride + (size_t)h * HD);
-    __syncthreads();  // the partial record written by this workgroup
-    const float* part = mine.scores + (size_t)h * (HD + 2);
-    if (threadIdx.x < HD) a.out[(size_t)j * out_stride + (size_t)h * HD + threadIdx.x] = __fdiv_rn(part[2 + threadIdx.x], part[1]);
+__global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride) {
+    constexpr uint32_t QB = 8;
+    constexpr uint32_t LR = HD / 4, RPP = 256 / LR, KROWS = kAttnChunk / RPP, KB = KROWS < 4 ? KROWS : 4;
+    constexpr uint32_t VG = 256 / HD, VROWS = kAttnChunk / VG, VB = VROWS < 8 ? VROWS : 8;
+    static_assert(kAttnChunk == 64 && KROWS % KB == 0 && VROWS % VB == 0, "one wave per query's softmax needs 64-position chunks");
+    __shared__ float sc[QB][kAttnChunk];
+    __shared__ float corr[QB], lsum[QB];
+    __shared__ float red[256];
+    const uint32_t h = blockIdx.x, j0 = blockIdx.y * QB;
+    const uint32_t nq = n - j0 < QB ? n - j0 : QB;  // queries of this workgroup
+    const uint32_t base = a.d_pos ? *a.d_pos : pos0;
+    const uint32_t kv_dim = a.n_kv_heads * HD, kvh = h / (a.n_heads / a.n_kv_heads);
+    const float* kbase = a.k_cache + (size_t)kvh * HD;
+    const float* vbase = a.v_cache + (size_t)kvh * HD;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, quad = tid % LR, prow = tid / LR, d = tid % HD, g = tid / HD;
+    uint32_t seq_max = base + j0 + nq;  // positions the last query sees
+    if (seq_max > a.max_seq) seq_max = a.max_seq;
+    const uint32_t last = seq_max - 1u;
+
+    float4 q4[QB];
+#pragma unroll
+    for (uint32_t q = 0; q < QB; q++)
+        q4[q] = reinterpret_cast<const float4*>(a.q + (size_t)(j0 + (q < nq ? q : 0u)) * q_stride + (size_t)h * HD)[quad];
+    float acc[QB];
+#pragma unroll
+    for (uint32_t q = 0; q < QB; q++) acc[q] = 0.0f;
+    float m_run[2] = {-__builtin_inff(), -__builtin_inff()}, l_run[2] = {0.0f, 0.0f};  // of queries 2 * wave, 2 * wave + 1
+
+    for (uint32_t t0 = 0; t0 < seq_max; t0 += kAttnChunk) {
+#pragma unroll
+        for (uint32_t i = 0; i < KROWS; i += KB) {
+            float4 kv[KB];
+#pragma unroll
+            for (uint32_t jj = 0; jj < KB; jj++) {
+                const uint32_t row = t0 + prow + (i + jj) * RPP;
+                kv[jj] = reinterpret_cast<const float4*>(kbase + (size_t)(row < last ? row : last) * kv_dim)[quad];
+            }
+#pragma unroll
+            for (uint32_t jj = 0; jj < KB; jj++) {
+                const uint32_t r = prow + (i + jj) * RPP;
+#pragma unroll
+                for (uint32_t q = 0; q < QB; q++) {
+                    float p = q4[q].x * kv[jj].x + q4[q].y * kv[jj].y + q4[q].z * kv[jj].z + q4[q].w * kv[jj].w;
+#pragma unroll
+                    for (uint32_t off = LR / 2; off > 0; off >>= 1) p += __shfl_xor(p, off, 64);
+                    // causal: query q (token j0 + q) sees positions <= base + j0 + q
+                    if (quad == 0) sc[q][r] = (q < nq && t0 + r <= base + j0 + q && t0 + r < a.max_seq) ? p * a.scale : -__builtin_inff();
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (uint32_t w2 = 0; w2 < 2; w2++) {  // this wave's two queries: one lane per position of the chunk
+            const uint32_t q = 2 * wave + w2;
+            const float s = sc[q][lane];
+            float mx = s;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+            const float m_new = fmaxf(m_run[w2], mx);
+            // a chunk (or a query slot) with nothing to see keeps -inf: weights 0, nothing rescaled
+            const float e = m_new == -__builtin_inff() ? 0.0f : ggml_expf(s - m_new);
+            float l = e;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off, 64);
+            const float c = m_new == -__builtin_inff() ? 1.0f : ggml_expf(m_run[w2] - m_new);
+            sc[q][lane] = e;
+            l_run[w2] = l_run[w2] * c + l;
+            m_run[w2] = m_new;
+            if (lane == 0) corr[q] = c;
+        }
+        __syncthreads();
+#pragma unroll
+        for (uint32_t q = 0; q < QB; q++) acc[q] *= corr[q];
+#pragma unroll
+        for (uint32_t i = 0; i < VROWS; i += VB) {
+            float vv[VB];
+#pragma unroll
+            for (uint32_t jj = 0; jj < VB; jj++) {
+                const uint32_t row = t0 + g + (i + jj) * VG;
+                vv[jj] = vbase[(size_t)(row < last ? row : last) * kv_dim + d];
+            }
+#pragma unroll
+            for (uint32_t jj = 0; jj < VB; jj++) {
+                const uint32_t t = g + (i + jj) * VG;
+#pragma unroll
+                for (uint32_t q = 0; q < QB; q++) acc[q] += sc[q][t] * vv[jj];
+            }
+        }
+        __syncthreads();  // sc[] and corr[] are rewritten by the next chunk
+    }
+    if (lane == 0) lsum[2 * wave] = l_run[0], lsum[2 * wave + 1] = l_run[1];
+#pragma unroll
+    for (uint32_t q = 0; q < QB; q++) {
+        __syncthreads();  // red[] of the previous query has been read; lsum[] is published before the first read
+        red[tid] = acc[q];
+        __syncthreads();
+        if (tid < HD && q < nq) {
+            float r = red[tid];
+#pragma unroll
+            for (uint32_t p = 1; p < VG; p++) r += red[p * HD + tid];
+            a.out[(size_t)(j0 + q) * out_stride + (size_t)h * HD + tid] = __fdiv_rn(r, lsum[q]);
+        }
+    }
 }
 
 // ---- gated short convolution, one step ---------------------------------------------------
@@ -761,19 +857,19 @@ hipError_t launch_shortconv_seq(const float* d_proj, float* d_buffer, const floa
     return launch_kernel(L, kFamOther, shortconv_state_kernel, dim3(blocks), dim3(256), d_proj, d_buffer, hidden, kernel_size, n);
 }
 
-size_t attention_prefill_scratch_floats(uint32_t n, uint32_t n_heads, uint32_t head_dim) { return (size_t)n * n_heads * (head_dim + 2); }
+size_t attention_prefill_scratch_floats(uint32_t, uint32_t, uint32_t) { return 4; }  // the kernel keeps everything on chip
 
 hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scratch,
                                     uint32_t pos0, const uint32_t* d_pos, uint32_t n, uint32_t q_stride, uint32_t out_stride, uint32_t max_seq,
                                     uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L) {
     if (n == 0) return hipSuccess;
     AttentionArgs a{d_q, d_k_cache, d_v_cache, d_out, d_scratch, d_pos, 0u, max_seq, n_heads, n_kv_heads, head_dim, scale};
-    const dim3 grid(n_heads, n), block(256);
+    const dim3 grid(n_heads, (n + 7u) / 8u), block(256);
     switch (head_dim) {
-        case 32: return launch_kernel(L, kFamOther, attention_prefill_kernel<32>, grid, block, a, pos0, q_stride, out_stride);
-        case 64: return launch_kernel(L, kFamOther, attention_prefill_kernel<64>, grid, block, a, pos0, q_stride, out_stride);
-        case 128: return launch_kernel(L, kFamOther, attention_prefill_kernel<128>, grid, block, a, pos0, q_stride, out_stride);
-        case 256: return launch_kernel(L, kFamOther, attention_prefill_kernel<256>, grid, block, a, pos0, q_stride, out_stride);
+        case 32: return launch_kernel(L, kFamOther, attention_prefill_kernel<32>, grid, block, a, pos0, n, q_stride, out_stride);
+        case 64: return launch_kernel(L, kFamOther, attention_prefill_kernel<64>, grid, block, a, pos0, n, q_stride, out_stride);
+        case 128: return launch_kernel(L, kFamOther, attention_prefill_kernel<128>, grid, block, a, pos0, n, q_stride, out_stride);
+        case 256: return launch_kernel(L, kFamOther, attention_prefill_kernel<256>, grid, block, a, pos0, n, q_stride, out_stride);
         default: return hipErrorInvalidValue;
     }
 }
