@@ -311,8 +311,7 @@ __device__ __forceinline__ void attention_chunks(const AttentionArgs& a, uint32_
             for (uint32_t j = 0; j < KB; j++) {
                 const uint32_t r = prow + (i + j) * RPP;
                 float p = q4.x * kv[j].x + q4.y * kv[j].y + q4.z * kv[j].z + q4.w * kv[j].w;
-#pragma unroll
-                for (uint32_t off = LR / 2; off > 0; off >>= 1) p += __shfl_xor(p, off, 64);
+                p = group_sum<LR>(p);  // DPP adds inside 16 lanes: no trip through the LDS crossbar
                 if (quad == 0) sc[r] = r < nt ? p * a.scale : -__builtin_inff();
             }
         }
@@ -476,8 +475,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
     constexpr uint32_t QB = 8;
     constexpr uint32_t LR = HD / 4, RPP = 256 / LR, KROWS = kAttnChunk / RPP, KB = KROWS < 4 ? KROWS : 4;
     constexpr uint32_t VG = 256 / HD, VROWS = kAttnChunk / VG, VB = VROWS < 8 ? VROWS : 8;
+    static_assert(VB % 4 == 0, "weights are read four at a time");
     static_assert(kAttnChunk == 64 && KROWS % KB == 0 && VROWS % VB == 0, "one wave per query's softmax needs 64-position chunks");
-    __shared__ float sc[QB][kAttnChunk];
+    __shared__ __align__(16) float sc[QB][kAttnChunk];
     __shared__ float corr[QB], lsum[QB];
     __shared__ float red[256];
     const uint32_t h = blockIdx.x, j0 = blockIdx.y * QB;
@@ -515,8 +515,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
 #pragma unroll
                 for (uint32_t q = 0; q < QB; q++) {
                     float p = q4[q].x * kv[jj].x + q4[q].y * kv[jj].y + q4[q].z * kv[jj].z + q4[q].w * kv[jj].w;
-#pragma unroll
-                    for (uint32_t off = LR / 2; off > 0; off >>= 1) p += __shfl_xor(p, off, 64);
+                    p = group_sum<LR>(p);  // DPP adds inside 16 lanes: no trip through the LDS crossbar
                     // causal: query q (token j0 + q) sees positions <= base + j0 + q
                     if (quad == 0) sc[q][r] = (q < nq && t0 + r <= base + j0 + q && t0 + r < a.max_seq) ? p * a.scale : -__builtin_inff();
                 }
@@ -545,19 +544,22 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
         __syncthreads();
 #pragma unroll
         for (uint32_t q = 0; q < QB; q++) acc[q] *= corr[q];
+        // group g takes the contiguous positions g * VROWS .. of the chunk: its weights come as 16-byte LDS reads
 #pragma unroll
         for (uint32_t i = 0; i < VROWS; i += VB) {
             float vv[VB];
 #pragma unroll
             for (uint32_t jj = 0; jj < VB; jj++) {
-                const uint32_t row = t0 + g + (i + jj) * VG;
+                const uint32_t row = t0 + g * VROWS + i + jj;
                 vv[jj] = vbase[(size_t)(row < last ? row : last) * kv_dim + d];
             }
 #pragma unroll
-            for (uint32_t jj = 0; jj < VB; jj++) {
-                const uint32_t t = g + (i + jj) * VG;
+            for (uint32_t q = 0; q < QB; q++) {
 #pragma unroll
-                for (uint32_t q = 0; q < QB; q++) acc[q] += sc[q][t] * vv[jj];
+                for (uint32_t jj = 0; jj < VB; jj += 4) {
+                    const float4 w4 = *reinterpret_cast<const float4*>(&sc[q][g * VROWS + i + jj]);
+                    acc[q] += w4.x * vv[jj] + w4.y * vv[jj + 1] + w4.z * vv[jj + 2] + w4.w * vv[jj + 3];
+                }
             }
         }
         __syncthreads();  // sc[] and corr[] are rewritten by the next chunk
