@@ -112,7 +112,8 @@ int wick_rocm_lfm2_reset(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model);
 
 /* Steps replay a captured graph (the counterpart of one command buffer per token, wick/src/model/metal_lfm2.rs:1-4).
  * With enabled = 0 the same launches are enqueued one by one instead, which per-dispatch timing
- * (wick_rocm_kernel_timing_begin) and kernel tracers need; results are identical.  The counterpart of the
+ * (wick_rocm_kernel_timing_begin) and kernel tracers need; results are identical.  While per-dispatch timing is on,
+ * steps are enqueued one by one whatever this switch says.  The counterpart of the
  * reference's profiled encode path (encode_layers_profiled, wick/src/model/metal_lfm2.rs:4559-4712). */
 int wick_rocm_lfm2_set_graph_replay(wick_rocm_lfm2 *model, int enabled);
 

@@ -153,6 +153,22 @@ def test_graph_replay_and_plain_launches_agree(ctx, oracle, tmp_path):
     model.free()
 
 
+def test_per_dispatch_timing_sees_the_step(ctx, oracle, tmp_path):
+    """While per-dispatch timing is on, a step is enqueued launch by launch (a graph hides its kernels from
+    the timer) and still gives the replayed step's logits."""
+    model, ref, cfg = load(ctx, oracle, tmp_path, seed=9)
+    replayed = [model.forward(4, 0), model.forward(8, 1)]
+    model.reset()
+    ctx.kernel_timing_begin()
+    timed = model.forward(4, 0)
+    fams = ctx.kernel_timing_end()
+    assert np.array_equal(replayed[0].view(np.uint32), timed.view(np.uint32))
+    assert sum(n for _, n in fams.values()) >= 4 * cfg["n_layers"], fams
+    # the state the timed step left carries the next replayed one
+    assert np.array_equal(replayed[1].view(np.uint32), model.forward(8, 1).view(np.uint32))
+    model.free()
+
+
 def test_load_and_step_errors(ctx, oracle, tmp_path):
     model, ref, cfg = load(ctx, oracle, tmp_path, context=8, context_length=6)
     assert model.config["max_seq_len"] == 6  # min(context_size, lfm2.context_length), wick/src/model/lfm2.rs:121-125
