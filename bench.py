@@ -392,7 +392,8 @@ def bench_lm_head_sweep(ctx, W, O, dtype=8, m=65536, k=2048, ns=(1, 4, 16, 64)):
 def bench_probe(ctx, iters=20000):
     """Register-only ceilings of this GPU for the GEMM's two bounds (no memory traffic)."""
     out = {}
-    for shape, name, unit in [(0, "mfma_i32_32x32x32_i8", "TOP/s"), (1, "mfma_i32_16x16x32_i8", "TOP/s"), (2, "v_fma_f32", "TFLOP/s")]:
+    for shape, name, unit in [(0, "mfma_i32_32x32x32_i8", "TOP/s"), (1, "mfma_i32_16x16x32_i8", "TOP/s"), (2, "v_fma_f32", "TFLOP/s"),
+                              (3, "block_loop_8xmfma16_plus_64_scaling_fma", "TOP/s"), (4, "block_loop_2xmfma32_plus_64_scaling_fma", "TOP/s")]:
         ctx.probe_rate(shape, iters)
         ctx.sync()
         e0, e1 = ctx.event(), ctx.event()

@@ -96,8 +96,11 @@ int wick_rocm_sync(wick_rocm_ctx *ctx);
 /* Measurement aid with no counterpart in the reference: enqueues a register-only kernel that
  * does nothing but issue one instruction (shape 0 = v_mfma_i32_32x32x32_i8, 1 =
  * v_mfma_i32_16x16x32_i8, 2 = v_fma_f32) `iters` x 4 times per wave on every SIMD, and returns
- * the number of operations it performs (int8 ops / flops).  Timed by the caller (events or
- * kernel timing, family 3), it gives this GPU's own ceiling for the prefill GEMM's two bounds. */
+ * the number of operations it performs (int8 ops / flops).  Shapes 3 and 4 run the GEMM's whole block
+ * loop from registers instead: per iteration and wave one 32-element block of a 64 x 32 tile = 8
+ * v_mfma_i32_16x16x32_i8 (3) or 2 v_mfma_i32_32x32x32_i8 (4) plus the two scaling FMAs of each of the
+ * 32 results per lane, at the GEMM's occupancy (131072 int8 ops per wave and iteration).  Timed by the
+ * caller (events or kernel timing, family 3), they give this GPU's own ceilings for the prefill GEMM. */
 int wick_rocm_probe_rate(wick_rocm_ctx *ctx, int shape, uint32_t iters, double *ops);
 
 /* Device-to-device copy enqueued on the context's stream (the counterpart of a Metal

@@ -160,12 +160,12 @@ def test_cpp_host_mirror_selftest():
 def test_rate_probes(ctx):
     """The register-only instruction-rate probes launch, report their operation counts and
     reject bad arguments (they are measurement aids; nothing is checked about their speed)."""
-    for shape, per_iter in [(0, 4 * 65536.0), (1, 4 * 16384.0), (2, 4 * 4 * 64 * 2.0)]:
+    for shape, per_iter in [(0, 4 * 65536.0), (1, 4 * 16384.0), (2, 4 * 4 * 64 * 2.0), (3, 131072.0), (4, 131072.0)]:
         ops = ctx.probe_rate(shape, 10)
         assert ops > 0 and ops % (per_iter * 10) == 0
     ctx.sync()
     with pytest.raises(W.RocmError):
-        ctx.probe_rate(3, 10)
+        ctx.probe_rate(5, 10)
     with pytest.raises(W.RocmError):
         ctx.probe_rate(0, 0)
 

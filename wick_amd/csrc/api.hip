@@ -209,7 +209,7 @@ int wick_rocm_copy(wick_rocm_ctx* ctx, void* d_dst, const void* d_src, size_t nb
 
 int wick_rocm_probe_rate(wick_rocm_ctx* ctx, int shape, uint32_t iters, double* ops) {
     WR_ENTER(ctx);
-    if (!ops || shape < 0 || shape > 2 || iters == 0) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "probe_rate: shape must be 0..2, iters > 0");
+    if (!ops || shape < 0 || shape > 4 || iters == 0) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "probe_rate: shape must be 0..4, iters > 0");
     if (!ctx->probe_sink) {
         if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "probe_rate: first call must be outside graph capture");
         WR_HIP(ctx, hipMalloc(&ctx->probe_sink, 64));

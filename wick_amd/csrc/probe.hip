@@ -15,7 +15,7 @@ constexpr int kProbeThreads = 256;
 constexpr int kProbeChains = 4;  // independent accumulators per wave, enough to cover the MFMA latency
 
 // SHAPE 0: v_mfma_i32_32x32x32_i8 (65536 ops), 1: v_mfma_i32_16x16x32_i8 (16384 ops),
-// 2: v_fma_f32 on 16 independent registers (64 lanes x 2 flops each).
+// 2: v_fma_f32 on 16 independent registers (64 lanes x 2 flops each); 3, 4: probe_mix_kernel below.
 template <int SHAPE>
 __global__ __launch_bounds__(kProbeThreads) void probe_kernel(int* sink, uint32_t iters) {
     v4i a4 = {(int)threadIdx.x, 2, 3, 4}, b4 = {5, 6, (int)threadIdx.x, 8};
@@ -56,11 +56,71 @@ __global__ __launch_bounds__(kProbeThreads) void probe_kernel(int* sink, uint32_
     if (s == 0x7fffffff) sink[0] = s;  // keeps the loop alive, practically never stores
 }
 
+// The GEMM's block loop without its memory side: per iteration one 32-element block of a wave's 64 x 32 tile, i.e.
+// 8 v_mfma_i32_16x16x32_i8 (SHAPE 3) or 2 v_mfma_i32_32x32x32_i8 (SHAPE 4) onto the float-bias constant, and the two
+// scaling FMAs of each of the 32 results per lane (per-lane scale registers, the second FMA four instructions behind
+// the first).  512-thread workgroups, two per CU: four waves per SIMD, the GEMM's occupancy.
+constexpr int kMixThreads = 512;
+template <int SHAPE>
+__global__ __launch_bounds__(kMixThreads) void probe_mix_kernel(int* sink, uint32_t iters) {
+    float acc[32];
+#pragma unroll
+    for (int i = 0; i < 32; i++) acc[i] = (float)(threadIdx.x + i);
+    const float dw = 1e-3f + 1e-9f * (float)threadIdx.x, nb = -12582912.0f * dw, dx = 2e-3f + 1e-9f * (float)threadIdx.x;
+    long a8 = (long)threadIdx.x * 0x0101010101010101L;
+    const long b8 = 0x0203040506070809L + (long)threadIdx.x;
+    v4i c4 = {0x4B400000, 0x4B400000, 0x4B400000, 0x4B400000};
+    v16i c16;
+#pragma unroll
+    for (int r = 0; r < 16; r++) c16[r] = 0x4B400000;
+    asm volatile("" : "+v"(c4), "+v"(c16));
+    for (uint32_t it = 0; it < iters; it++) {
+        int d[32];
+        if constexpr (SHAPE == 3) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const v4i r4 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a8 + j, b8, c4, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; r++) d[4 * j + r] = r4[r];
+            }
+        } else {
+            const v4i a4 = {(int)a8, (int)(a8 >> 32), 3, 4}, b4 = {(int)b8, 6, 7, 8};
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const v16i r16 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, b4 + j, c16, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; r++) d[16 * j + r] = r16[r];
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            float t[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) t[r] = __builtin_fmaf(__int_as_float(d[4 * g + r]), dw, nb);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[4 * g + r] = __builtin_fmaf(t[r], dx, acc[4 * g + r]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        a8 += 0x0101;
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) s += acc[i];
+    if (s == 123.456f) sink[0] = 1;  // keeps the loop alive, practically never stores
+}
+
 }  // namespace
 
 // Enqueues one probe launch that fills the chip (8 workgroups of 4 waves per CU) and returns
 // the number of operations it performs (int8 ops for the MFMA shapes, flops for the FMA one).
 hipError_t launch_probe(int shape, uint32_t iters, int num_cus, int* d_sink, double* ops, const Launch& L) {
+    if (shape >= 3) {  // the block loop: 2 * 64 * 32 * 32 int8 ops per wave and iteration
+        const dim3 grid((uint32_t)num_cus * 2u), block(kMixThreads);
+        *ops = (double)grid.x * (kMixThreads / 64) * 131072.0 * iters;
+        if (shape == 3) return launch_kernel(L, kFamOther, probe_mix_kernel<3>, grid, block, d_sink, iters);
+        return launch_kernel(L, kFamOther, probe_mix_kernel<4>, grid, block, d_sink, iters);
+    }
     const dim3 grid((uint32_t)num_cus * 8u), block(kProbeThreads);
     const double waves = (double)grid.x * (kProbeThreads / 64);
     const double per_iter = kProbeChains * (shape == 0 ? 65536.0 : shape == 1 ? 16384.0 : 4 * 64 * 2.0);
