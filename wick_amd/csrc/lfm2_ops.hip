@@ -579,6 +579,158 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
     }
 }
 
+// The same causal attention on the f32 matrix cores (v_mfma_f32_16x16x4_f32: exact f32 products, f32 sums; only the
+// order of the sums differs from the scalar kernel above).  A workgroup = 4 waves = 64 consecutive queries of one head,
+// 16 per wave; it walks the cache in tiles of 64 positions that all four waves share through LDS.
+//   scores, transposed:  S^T[key][q] = sum_d K[key][d] Q[q][d]   A = K (keys are the M rows), B = Q^T
+//     lane l feeds key l % 16 and query l % 16 at head dims (l / 16) * HD/4 + s, s = 0 .. HD/4 - 1 (the order of the
+//     K steps is free as long as both operands agree, so a lane's dims are contiguous: 16-byte LDS reads);
+//     in the result lane l holds keys 4 * (l / 16) + r of query l % 16.
+//   weighted values, transposed:  O^T[d][q] = sum_key V[key][d] P[key][q]   A = V^T, B = P
+//     K step s of a 16-key sub-tile takes key 4 * (l / 16) + s from lane l: exactly result register s of the score
+//     MFMA, so the softmax weights go from one MFMA into the next without leaving their registers.  A lane's A
+//     operand V[key][4 * (l % 16) + c], c = 0..3, is one 16-byte read serving the four MFMAs that own dims 4 m + c.
+// Streaming softmax per query across the tiles (running maximum shared by the four lane groups of a query through
+// two shuffles, partial sums of the weights kept per lane and added up at the end).
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int HD>
+__global__ __launch_bounds__(256) void attention_prefill_mfma_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride) {
+    constexpr int KT = 64;        // positions per tile
+    constexpr int LD = HD + 4;    // LDS row stride in floats: an odd number of 16-byte chunks, conflict-free operand reads
+    constexpr int QR = HD / 4;    // Q registers per lane = K steps of a score tile
+    constexpr int DT = HD / 16;   // 16 x 16 output tiles per MFMA group
+    static_assert(HD % 16 == 0, "head_dim must be a multiple of 16");
+    __shared__ __align__(16) float ks[KT][LD];
+    __shared__ __align__(16) float vs[KT][LD];
+    const uint32_t h = blockIdx.x;
+    const uint32_t qblocks = (n + 63u) / 64u;
+    const uint32_t j0 = (qblocks - 1u - blockIdx.y) * 64u;  // longest rows first
+    const uint32_t base = a.d_pos ? *a.d_pos : pos0;
+    const uint32_t kv_dim = a.n_kv_heads * HD, kvh = h / (a.n_heads / a.n_kv_heads);
+    const float* kbase = a.k_cache + (size_t)kvh * HD;
+    const float* vbase = a.v_cache + (size_t)kvh * HD;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+    const uint32_t jq = j0 + 16u * wave + l16;           // this lane's query token
+    const uint32_t jl = jq < n ? jq : n - 1u;            // ... clamped for loads
+    const uint32_t pq = base + jl;                       // its position = the last key it sees
+    uint32_t wg_last = base + (j0 + 63u < n ? j0 + 63u : n - 1u);  // last position any query of the workgroup sees
+    if (wg_last >= a.max_seq) wg_last = a.max_seq - 1u;
+    const uint32_t wave_last = min(base + min(j0 + 16u * wave + 15u, n - 1u), wg_last);
+
+    float qr[QR];
+    {
+        const float4* qp = reinterpret_cast<const float4*>(a.q + (size_t)jl * q_stride + (size_t)h * HD + (size_t)g * QR);
+#pragma unroll
+        for (int i = 0; i < QR / 4; i++) {
+            const float4 v = qp[i];
+            qr[4 * i] = v.x * a.scale, qr[4 * i + 1] = v.y * a.scale, qr[4 * i + 2] = v.z * a.scale, qr[4 * i + 3] = v.w * a.scale;
+        }
+    }
+    v4f o[DT];
+#pragma unroll
+    for (int c = 0; c < DT; c++) o[c] = v4f{0.f, 0.f, 0.f, 0.f};
+    float m_run = -__builtin_inff(), l_run = 0.0f;
+
+    for (uint32_t t0 = 0; t0 <= wg_last; t0 += KT) {
+        __syncthreads();  // the previous tile has been consumed
+        {
+            constexpr int C4 = HD / 4, RPP = 256 / C4, NR = KT / RPP;  // float4 columns, rows per pass, passes
+            const uint32_t c4 = tid % C4, r0 = tid / C4;
+            float4 kk[NR], vv[NR];
+#pragma unroll
+            for (int i = 0; i < NR; i++) {
+                const uint32_t key = min(t0 + r0 + i * RPP, wg_last);
+                kk[i] = reinterpret_cast<const float4*>(kbase + (size_t)key * kv_dim)[c4];
+                vv[i] = reinterpret_cast<const float4*>(vbase + (size_t)key * kv_dim)[c4];
+            }
+#pragma unroll
+            for (int i = 0; i < NR; i++) {
+                *reinterpret_cast<float4*>(&ks[r0 + i * RPP][4 * c4]) = kk[i];
+                *reinterpret_cast<float4*>(&vs[r0 + i * RPP][4 * c4]) = vv[i];
+            }
+        }
+        __syncthreads();
+        if (t0 > wave_last) continue;  // every query of this wave ends before the tile (still takes part in the barriers)
+
+        // scores of 4 sub-tiles x 16 keys
+        v4f sc[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) sc[u] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < QR / 4; i++) {
+            float4 kq[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) kq[u] = *reinterpret_cast<const float4*>(&ks[16 * u + l16][g * QR + 4 * i]);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[u].x, qr[4 * i], sc[u], 0, 0, 0);
+                sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[u].y, qr[4 * i + 1], sc[u], 0, 0, 0);
+                sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[u].z, qr[4 * i + 2], sc[u], 0, 0, 0);
+                sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[u].w, qr[4 * i + 3], sc[u], 0, 0, 0);
+            }
+        }
+        // causal mask + tile maximum of this lane's query
+        float tmax = -__builtin_inff();
+        const bool masked_tile = t0 + KT - 1u > base + min(j0 + 16u * wave, n - 1u);  // some key of the tile is past some query of the wave
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (masked_tile && t0 + 16u * u + 4u * g + r > pq) sc[u][r] = -__builtin_inff();
+                tmax = fmaxf(tmax, sc[u][r]);
+            }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const float m_new = fmaxf(m_run, tmax);  // finite: key 0 is visible to every query and lies in the first tile
+        const float alpha = m_run == -__builtin_inff() ? 0.0f : ggml_expf(m_run - m_new);  // first tile: nothing to rescale
+        m_run = m_new;
+        float psum = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float pw = sc[u][r] == -__builtin_inff() ? 0.0f : ggml_expf(sc[u][r] - m_new);
+                sc[u][r] = pw;
+                psum += pw;
+            }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int c = 0; c < DT; c++) o[c] *= alpha;
+        // O^T += V^T P
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int sidx = 0; sidx < 4; sidx++) {
+                const float pv = sc[u][sidx];
+#pragma unroll
+                for (int c4 = 0; c4 < DT / 4; c4++) {
+                    const float4 vq = *reinterpret_cast<const float4*>(&vs[16 * u + 4 * g + sidx][16 * c4 * 4 + 4 * l16]);
+                    o[4 * c4 + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.x, pv, o[4 * c4 + 0], 0, 0, 0);
+                    o[4 * c4 + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.y, pv, o[4 * c4 + 1], 0, 0, 0);
+                    o[4 * c4 + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.z, pv, o[4 * c4 + 2], 0, 0, 0);
+                    o[4 * c4 + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.w, pv, o[4 * c4 + 3], 0, 0, 0);
+                }
+            }
+    }
+    // the weight sums of a query's four lane groups
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+    if (jq < n) {
+        // tile c4*4 + c, register r of lane (l16, g) holds dim 64 * c4 + 4 * (4 * g + r) + c of query l16
+        float* dst = a.out + (size_t)jq * out_stride + (size_t)h * HD;
+#pragma unroll
+        for (int c4 = 0; c4 < DT / 4; c4++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float4 v;
+                v.x = __fdiv_rn(o[4 * c4 + 0][r], l_run), v.y = __fdiv_rn(o[4 * c4 + 1][r], l_run);
+                v.z = __fdiv_rn(o[4 * c4 + 2][r], l_run), v.w = __fdiv_rn(o[4 * c4 + 3][r], l_run);
+                *reinterpret_cast<float4*>(dst + 64 * c4 + 16 * g + 4 * r) = v;
+            }
+    }
+}
+
 // ---- gated short convolution, one step ---------------------------------------------------
 // forward_conv_block's middle (wick/src/model/lfm2.rs:694-726): proj = [b | c | x]; bx = b*x;
 // out = c * (sum_k buffer[k][ch]*w[ch][k] + bx*w[ch][K-1]); the rolling buffer shifts by one slot and takes bx.
@@ -866,6 +1018,10 @@ hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, co
                                     uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L) {
     if (n == 0) return hipSuccess;
     AttentionArgs a{d_q, d_k_cache, d_v_cache, d_out, d_scratch, d_pos, 0u, max_seq, n_heads, n_kv_heads, head_dim, scale};
+    // the matrix-core kernel needs 16-byte aligned rows (q, caches, out) and whole tiles of head dims
+    const bool aligned = q_stride % 4u == 0 && out_stride % 4u == 0 && ((uintptr_t)d_q | (uintptr_t)d_k_cache | (uintptr_t)d_v_cache | (uintptr_t)d_out) % 16u == 0;
+    if (head_dim == 64 && aligned && n >= 16)
+        return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64>, dim3(n_heads, (n + 63u) / 64u), dim3(256), a, pos0, n, q_stride, out_stride);
     const dim3 grid(n_heads, (n + 7u) / 8u), block(256);
     switch (head_dim) {
         case 32: return launch_kernel(L, kFamOther, attention_prefill_kernel<32>, grid, block, a, pos0, n, q_stride, out_stride);
