@@ -60,6 +60,15 @@ int wick_rocm_attention_decode(wick_rocm_ctx *ctx, const float *d_q, const float
                                float *d_scratch, uint32_t seq_len, const uint32_t *d_pos, uint32_t max_seq, uint32_t n_heads,
                                uint32_t n_kv_heads, uint32_t head_dim);
 
+/* Causal attention for the n tokens of a prompt whose K / V rows are already in the caches: pass B of the reference's
+ * batched prefill (wick/src/model/lfm2.rs:1640-1700), i.e. for token j the decode attention above with
+ * seq_len = pos0 + j + 1.  d_q: [n][q_stride] floats (a token's n_heads * head_dim query values first), d_out:
+ * [n][out_stride].  head_dim 32 / 64 / 128 / 256; head_dim 64 with 16-byte aligned rows and n >= 16 runs on the f32
+ * matrix cores (same products, sums in another order). */
+int wick_rocm_attention_prefill(wick_rocm_ctx *ctx, const float *d_q, uint32_t q_stride, const float *d_k_cache, const float *d_v_cache,
+                                float *d_out, uint32_t out_stride, uint32_t pos0, uint32_t n, uint32_t max_seq, uint32_t n_heads,
+                                uint32_t n_kv_heads, uint32_t head_dim);
+
 /* The attention block between the Q/K/V projections and the output projection: what wick_rocm_qk_norm_rope followed
  * by wick_rocm_attention_decode compute (wick/src/model/lfm2.rs:783-1006), bit for bit, with the norm, the rotation and
  * the KV append folded into the attention kernel (workgroups norm and rotate their own query head; those that own the

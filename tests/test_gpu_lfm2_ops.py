@@ -162,6 +162,34 @@ def test_attention_decode(ctx, ops, oracle, n_heads, n_kv, hd, seq):
         b.free()
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,pos0,n,pad", [
+    (4, 2, 64, 0, 16, 0), (4, 4, 64, 0, 63, 4), (8, 2, 64, 5, 130, 0), (4, 1, 64, 100, 64, 8), (2, 2, 64, 0, 200, 0), (16, 8, 64, 61, 67, 0),
+    (4, 2, 64, 0, 9, 0),     # fewer than 16 tokens: the scalar kernel
+    (4, 2, 32, 3, 40, 0), (2, 1, 128, 0, 70, 4),  # head dims without a matrix-core kernel
+])
+def test_attention_prefill(ctx, ops, oracle, n_heads, n_kv, hd, pos0, n, pad):
+    """Causal attention over a prompt (wick/src/model/lfm2.rs:1640-1700): token j == the decode attention with seq_len = pos0 + j + 1.
+    head_dim 64 runs on the f32 matrix cores: same products, sums in tiles of 64 positions."""
+    kv_dim, seq_total = n_kv * hd, pos0 + n
+    max_seq = seq_total + 2
+    q_stride, out_stride = n_heads * hd + 2 * kv_dim + pad, n_heads * hd + pad
+    q = oracle.fill_normal(7 * n + pos0, 1.0, n * q_stride)
+    kc, vc = oracle.fill_normal(n + 1, 1.0, max_seq * kv_dim), oracle.fill_normal(n + 2, 1.0, max_seq * kv_dim)
+    d_q, d_kc, d_vc = ctx.to_device(q), ctx.to_device(kc), ctx.to_device(vc)
+    d_out = ctx.to_device(np.full(n * out_stride, 7.5, np.float32))
+    ops.encode_attention_prefill(d_q, q_stride, d_kc, d_vc, d_out, out_stride, pos0, n, max_seq, n_heads, n_kv, hd)
+    got = d_out.download(np.float32, n * out_stride).reshape(n, out_stride)
+    assert np.all(got[:, n_heads * hd:] == 7.5)  # padding between rows is left alone
+    for j in sorted({0, 1, 15, 16, 17, n // 2, n - 2, n - 1} & set(range(n))) if n > 80 else range(n):
+        seq = pos0 + j + 1
+        ref = L.attention(q[j * q_stride: j * q_stride + n_heads * hd], kc[: seq * kv_dim], vc[: seq * kv_dim], n_heads, n_kv, hd, seq)
+        assert np.allclose(got[j, : n_heads * hd], ref, rtol=0, atol=4e-6 * max(np.abs(ref).max(), 1e-3)), f"token {j}"
+    with pytest.raises(W.RocmError, match="beyond the cache"):
+        ops.encode_attention_prefill(d_q, q_stride, d_kc, d_vc, d_out, out_stride, 3, n, n + 2, n_heads, n_kv, hd)
+    for b in (d_q, d_kc, d_vc, d_out):
+        b.free()
+
+
 @pytest.mark.parametrize("n_heads,n_kv,hd,max_seq,steps", [(4, 2, 64, 300, [0, 1, 2, 63, 64, 65, 130, 299]), (16, 8, 64, 4096, [0, 700, 4095]),
                                                            (4, 4, 32, 64, [0, 5, 63]), (2, 1, 128, 5000, [4100, 4999]), (2, 1, 256, 100, [99]),
                                                            (3, 1, 96, 80, [0, 7, 79])])

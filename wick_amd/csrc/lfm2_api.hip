@@ -72,6 +72,24 @@ int wick_rocm_attention_decode(wick_rocm_ctx* ctx, const float* d_q, const float
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "attention launch");
 }
 
+int wick_rocm_attention_prefill(wick_rocm_ctx* ctx, const float* d_q, uint32_t q_stride, const float* d_k_cache, const float* d_v_cache,
+                                float* d_out, uint32_t out_stride, uint32_t pos0, uint32_t n, uint32_t max_seq, uint32_t n_heads,
+                                uint32_t n_kv_heads, uint32_t head_dim) {
+    WR_ENTER(ctx);
+    if (!d_q || !d_k_cache || !d_v_cache || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention_prefill: null device pointer");
+    if ((head_dim != 32u && head_dim != 64u && head_dim != 128u && head_dim != 256u) || n_heads == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "attention_prefill: head_dim must be 32, 64, 128 or 256, n_kv_heads must divide n_heads");
+    if (q_stride < n_heads * head_dim || out_stride < n_heads * head_dim || q_stride % 4u != 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "attention_prefill: strides must cover n_heads * head_dim (q_stride a multiple of 4)");
+    if (misaligned(d_q, 16) || misaligned(d_k_cache, 16) || misaligned(d_v_cache, 16))
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention_prefill: q and the caches must be 16-byte aligned");
+    if ((uint64_t)pos0 + n > max_seq) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention_prefill: positions beyond the cache");
+    const float scale = 1.0f / sqrtf((float)head_dim);  // wick/src/model/lfm2.rs:862
+    hipError_t e = launch_attention_prefill(d_q, d_k_cache, d_v_cache, d_out, nullptr, pos0, nullptr, n, q_stride, out_stride, max_seq, n_heads,
+                                            n_kv_heads, head_dim, scale, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "attention_prefill launch");
+}
+
 size_t wick_rocm_attention_block_scratch_bytes(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim) {
     return attention_scratch_floats(max_seq, n_heads, head_dim) * sizeof(float);
 }

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "wick_rocm_rope_theta_scale": (_F, [_U32, _F]),
     "wick_rocm_attention_decode": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32]),
     "wick_rocm_attention_scratch_floats": (C.c_size_t, [_U32, _U32, _U32]),
+    "wick_rocm_attention_prefill": (C.c_int, [_P, _P, _U32, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _U32, _U32]),
     "wick_rocm_attention_block_scratch_bytes": (C.c_size_t, [_U32, _U32, _U32]),
     "wick_rocm_attention_block": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32, _F, _F]),
     "wick_rocm_shortconv_step": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32]),
@@ -98,6 +99,12 @@ class Lfm2Ops:
                          d_pos=None) -> None:
         self.ctx._check(self._l.wick_rocm_attention_decode(self.ctx._h, _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(scores), seq_len,
                                                            _ptr(d_pos), max_seq, n_heads, n_kv_heads, head_dim))
+
+    def encode_attention_prefill(self, q, q_stride: int, k_cache, v_cache, out, out_stride: int, pos0: int, n: int, max_seq: int, n_heads: int,
+                                 n_kv_heads: int, head_dim: int) -> None:
+        """Causal attention of n prompt tokens at positions pos0.. over caches that already hold their K / V rows."""
+        self.ctx._check(self._l.wick_rocm_attention_prefill(self.ctx._h, _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(out), out_stride,
+                                                            pos0, n, max_seq, n_heads, n_kv_heads, head_dim))
 
     def encode_attention_block(self, q, k, v, q_norm, k_norm, k_cache, v_cache, out, scratch, pos: int, max_seq: int, head_dim: int,
                                n_heads: int, n_kv_heads: int, eps: float, theta_scale: float, d_pos=None) -> None:
