@@ -162,6 +162,13 @@ int wick_rocm_gemv_q8_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *w
 int wick_rocm_gemm_q8(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_t *d_quants, const float *d_scales,
                       uint32_t n, float *d_y, uint32_t y_stride, int y_layout, int accumulate);
 
+/* The same for 1..3 weights of one dtype and k over the same quantized activations (Q / K / V, gate / up of a prompt
+ * pass: the batched counterpart of encode_gemv_qkv / encode_gemv_gate_up, wick/src/model/metal_lfm2.rs:1043-1119) in
+ * one launch, y_i written like wick_rocm_gemm_q8 writes it (shared stride, layout, accumulate flag); results are those
+ * of one wick_rocm_gemm_q8 call per weight, bit for bit. */
+int wick_rocm_gemm_q8_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *ws, float *const *d_ys, uint32_t count,
+                            const int8_t *d_quants, const float *d_scales, uint32_t n, uint32_t y_stride, int y_layout, int accumulate);
+
 /* The n at and above which wick_rocm_gemm_q8 / wick_rocm_matmul_f32 hand off from the
  * multi-token GEMV to the MFMA GEMM (default 16, the reference's GEMM_MIN_N,
  * wick/src/model/metal_lfm2.rs:18-21); 0 restores the default.  A tuning knob, like

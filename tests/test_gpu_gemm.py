@@ -97,6 +97,40 @@ def test_accumulate(ctx, oracle, dtype, n):
 
 
 @pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+@pytest.mark.parametrize("ms,n,k,layout,acc", [
+    ((256, 128, 128), 200, 512, W.LAYOUT_TOKEN_MAJOR, False),   # Q / K / V into one [n][q|k|v] row
+    ((300, 300), 130, 1024, W.LAYOUT_TOKEN_MAJOR, True),         # gate / up, ragged row tiles, accumulate
+    ((129, 1, 257), 40, 256, W.LAYOUT_TOKEN_MAJOR, False),       # narrow tile
+    ((128, 64), 17, 128, W.LAYOUT_ROW_MAJOR, False),
+    ((64, 96), 5, 256, W.LAYOUT_TOKEN_MAJOR, False),             # below the MFMA hand-off: one call per weight
+])
+def test_gemm_multi_equals_one_launch_per_weight(ctx, oracle, dtype, ms, n, k, layout, acc):
+    """Up to three weights over the same activations in one launch: bit-identical to one launch per weight."""
+    with Problem(ctx, oracle, dtype, ms[0], k, n, seed=sum(ms) + n) as p:
+        ws = [p.w] + [ctx.upload_weight(oracle.synth_weight(dtype, m, k, 50 + i, 0.02), dtype, m, k) for i, m in enumerate(ms[1:])]
+        tm = layout == W.LAYOUT_TOKEN_MAJOR
+        stride = sum(ms) + 3 if tm else n + 1
+        y0 = oracle.fill_normal(9, 1.0, (n if tm else sum(ms)) * stride)
+        d_a, d_b = p.to_device(y0), p.to_device(y0)
+        offs = np.concatenate([[0], np.cumsum(ms)[:-1]])
+        elem = lambda o: int(o) * 4 if tm else int(o) * stride * 4  # byte offset of a weight's first output
+        ya = [d_a.ptr + elem(o) for o in offs]
+        yb = [d_b.ptr + elem(o) for o in offs]
+        ctx.gemm_preq_multi(ws, p.d_s, p.d_q, n, ya, stride, layout=layout, accumulate=acc)
+        for w, y in zip(ws, yb):
+            ctx.gemm_preq(w, p.d_s, p.d_q, n, y, y_stride=stride, layout=layout, accumulate=acc)
+        a, b = d_a.download(np.float32, y0.size), d_b.download(np.float32, y0.size)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        assert not np.array_equal(a, y0)
+        with pytest.raises(W.RocmError, match="share k and dtype"):
+            other = ctx.upload_weight(oracle.synth_weight(dtype, 32, k + 128, 3, 0.02), dtype, 32, k + 128)
+            ws.append(other)
+            ctx.gemm_preq_multi([ws[0], other], p.d_s, p.d_q, n, ya[:2], stride, layout=layout)
+        for w in ws[1:]:
+            w.free()
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
 def test_full_size_prefill_shape(ctx, oracle, dtype):
     """m=6912, n=2002, k=2048 (the LFM2-1.2B ffn_up prefill shape).  The oracle checks a
     band of rows across ALL tokens plus scattered rows; size-independent properties cover

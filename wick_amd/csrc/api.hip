@@ -502,6 +502,36 @@ int wick_rocm_gemm_q8(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_
     return gemm_locked(ctx, w, d_quants, d_scales, n, d_y, y_stride, y_layout, accumulate);
 }
 
+int wick_rocm_gemm_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count, const int8_t* d_quants,
+                            const float* d_scales, uint32_t n, uint32_t y_stride, int y_layout, int accumulate) {
+    WR_ENTER(ctx);
+    if (!ws || !d_ys || count == 0 || count > 3) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemm_q8_multi: 1..3 weights");
+    for (uint32_t i = 0; i < count; i++) {
+        if (int rc = check_weight(ctx, ws[i])) return rc;
+        if (ws[i]->type != ws[0]->type || ws[i]->k != ws[0]->k) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "gemm_q8_multi: weights must share k and dtype");
+    }
+    const wick_rocm_weight* w0 = ws[0];
+    const bool one_launch = count > 1 && w0->type != kTypeQ6_K && n >= ctx->gemm_min_n && w0->k % 128u == 0 && d_quants && d_scales &&
+                            reinterpret_cast<uintptr_t>(d_quants) % 16u == 0 && reinterpret_cast<uintptr_t>(d_scales) % 16u == 0;
+    if (!one_launch) {  // shapes without a batched launch: one call per weight, same results
+        for (uint32_t i = 0; i < count; i++)
+            if (int rc = gemm_locked(ctx, ws[i], d_quants, d_scales, n, d_ys[i], y_stride, y_layout, accumulate)) return rc;
+        return WICK_ROCM_OK;
+    }
+    if (y_layout != WICK_ROCM_LAYOUT_TOKEN_MAJOR && y_layout != WICK_ROCM_LAYOUT_ROW_MAJOR)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "unknown output layout");
+    const uint8_t* wp[3];
+    uint32_t ms[3];
+    for (uint32_t i = 0; i < count; i++) {
+        if (!d_ys[i]) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "null device pointer");
+        if (y_layout == WICK_ROCM_LAYOUT_TOKEN_MAJOR ? y_stride < ws[i]->m : y_stride < n)
+            return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "y_stride smaller than the output extent");
+        wp[i] = static_cast<const uint8_t*>(ws[i]->d), ms[i] = ws[i]->m;
+    }
+    hipError_t e = launch_gemm_mfma_multi(w0->type, wp, ms, count, w0->k, d_quants, d_scales, n, d_ys, y_stride, y_layout, accumulate, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "gemm launch");
+}
+
 int wick_rocm_reserve_scratch(wick_rocm_ctx* ctx, uint32_t max_n, uint32_t max_k) {
     WR_ENTER(ctx);
     if (max_k % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "reserve_scratch: max_k % 32 != 0");

@@ -82,7 +82,24 @@ struct GemmArgs {
     uint32_t row_tiles, tok_tiles;
     int y_row_major;
     int accumulate;
+    // Up to two more weights that share the activations (Q / K / V, gate / up): their row tiles follow the first
+    // weight's in the launch's tile list.  tile_start[i]: first row tile of weight i + 1 (UINT32_MAX: absent).
+    const uint8_t* w_more[2];
+    float* y_more[2];
+    uint32_t m_more[2];
+    uint32_t tile_start[2];
 };
+
+// Makes `a` describe the weight that owns row tile `row_tile` and rebases the tile index to that weight.
+__device__ __forceinline__ void select_weight(GemmArgs& a, uint32_t& row_tile) {
+    const bool second = row_tile >= a.tile_start[0], third = row_tile >= a.tile_start[1];
+    if (second) {
+        a.w = third ? a.w_more[1] : a.w_more[0];
+        a.y = third ? a.y_more[1] : a.y_more[0];
+        a.m = third ? a.m_more[1] : a.m_more[0];
+        row_tile -= third ? a.tile_start[1] : a.tile_start[0];
+    }
+}
 
 // One stage of operands.  Row counts are padded (one 16-byte operand row per
 // plane, two float2 per scale row) so that the stage WRITES, where neighbouring
@@ -335,6 +352,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
     bool valid_tile;
     tile_of_block(blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
     if (!valid_tile) return;  // whole workgroup leaves together
+    select_weight(a, row_tile);
     const uint32_t row0 = row_tile * BM;
     const uint32_t tok0 = tok_tile * BN;
 
@@ -494,6 +512,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     bool valid_tile;
     tile_of_block(blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
     if (!valid_tile) return;  // whole workgroup leaves together
+    select_weight(a, row_tile);
     const uint32_t row0 = row_tile * BM;
     const uint32_t tok0 = tok_tile * BN_NARROW;
 
@@ -586,9 +605,14 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
 }
 
 template <bool DUMP>
-hipError_t launch(int type, GemmArgs& a, const Launch& L) {
+hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0) {
     if (a.m == 0 || a.n == 0) return hipSuccess;
     a.row_tiles = (a.m + BM - 1) / BM;
+    a.tile_start[0] = a.tile_start[1] = UINT32_MAX;
+    for (uint32_t i = 0; i < more; i++) {
+        a.tile_start[i] = a.row_tiles;
+        a.row_tiles += (a.m_more[i] + BM - 1) / BM;
+    }
     // The narrow tile also serves small problems that would leave more than half of the
     // 512 resident workgroup slots (2 per CU) empty with the wide tile: twice the tiles.
     const bool narrow = a.n <= BN_NARROW || a.row_tiles * ((a.n + BN - 1) / BN) <= 256;
@@ -615,6 +639,21 @@ hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k
     a.y_row_major = (y_layout == 1);
     a.accumulate = accumulate;
     return launch<false>(type, a, L);
+}
+
+// The same launch over up to three weights of one type and k that share the activations: outputs y[i] (same stride,
+// layout and accumulate flag), tiles of all weights in one tile list.
+hipError_t launch_gemm_mfma_multi(int type, const uint8_t* const* d_w, const uint32_t* m, uint32_t count, uint32_t k, const int8_t* d_q,
+                                  const float* d_scales, uint32_t n, float* const* d_y, uint32_t y_stride, int y_layout, int accumulate,
+                                  const Launch& L) {
+    if (count == 0 || count > 3) return hipErrorInvalidValue;
+    GemmArgs a{};
+    a.w = d_w[0], a.xq = d_q, a.xs = d_scales, a.y = d_y[0], a.dots = nullptr;
+    a.m = m[0], a.n = n, a.k = k, a.y_stride = y_stride;
+    a.y_row_major = (y_layout == 1);
+    a.accumulate = accumulate;
+    for (uint32_t i = 1; i < count; i++) a.w_more[i - 1] = d_w[i], a.y_more[i - 1] = d_y[i], a.m_more[i - 1] = m[i];
+    return launch<false>(type, a, L, count - 1);
 }
 
 // Parity hook through the matrix-core path: the same loads, unpack, LDS layout and

@@ -349,6 +349,18 @@ int gemm(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const wick_rocm_lfm2* m,
     return wick_rocm_gemm_q8(ctx, w, m->pQ, m->pS, n, y, y_stride, WICK_ROCM_LAYOUT_TOKEN_MAJOR, accumulate);
 }
 
+// The same for projections that share their input (Q / K / V, gate / up): one launch when dtype and k agree.
+int gemm_group(wick_rocm_ctx* ctx, std::initializer_list<const wick_rocm_weight*> ws, std::initializer_list<float*> ys, const wick_rocm_lfm2* m,
+               uint32_t n, uint32_t y_stride) {
+    bool same = true;
+    for (const wick_rocm_weight* w : ws) same = same && w->type == (*ws.begin())->type && w->k == (*ws.begin())->k;
+    if (same) return wick_rocm_gemm_q8_multi(ctx, ws.begin(), ys.begin(), (uint32_t)ws.size(), m->pQ, m->pS, n, y_stride, WICK_ROCM_LAYOUT_TOKEN_MAJOR, 0);
+    auto y = ys.begin();
+    for (const wick_rocm_weight* w : ws)
+        if (int rc = gemm(ctx, w, m, n, *y++, y_stride, 0)) return rc;
+    return WICK_ROCM_OK;
+}
+
 // One pass of a prompt: n <= prefill_cap tokens (already in pTokens) at positions pos0 .. pos0 + n - 1.  The batched form
 // of enqueue_step (prefill_layers_and_logits, wick/src/model/lfm2.rs:1139-2109): projections as GEMMs over the tokens,
 // the short conv per (token, channel) with the rolling state behind it, the KV append per token, causal attention per
@@ -376,7 +388,7 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
         } else {
             const uint32_t kvd = L.n_kv * hd, S = hs + 2 * kvd;  // a token's [q | k | v]
             float *q = m->pA, *k = m->pA + hs, *v = m->pA + hs + kvd;
-            if ((rc = gemm(ctx, L.q, m, n, q, S, 0)) || (rc = gemm(ctx, L.k, m, n, k, S, 0)) || (rc = gemm(ctx, L.v, m, n, v, S, 0))) break;
+            if ((rc = gemm_group(ctx, {L.q, L.k, L.v}, {q, k, v}, m, n, S))) break;
             if ((rc = locked([&] {
                      return launch_qk_norm_rope(q, k, v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, pos0, nullptr, c.max_seq_len, hd, c.n_heads, L.n_kv,
                                                 c.rms_norm_eps, m->theta_scale, ctx->launch(), n, S, S);
@@ -398,7 +410,7 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
         if ((rc = gemm(ctx, L.n_kv == 0 ? L.out_proj : L.o, m, n, m->pX, hs, 1))) break;  // hidden += out projection
         if ((rc = wick_rocm_rmsnorm(ctx, m->pX, L.ffn_norm, m->pN, n, hs, hs, hs, c.rms_norm_eps))) break;
         if ((rc = wick_rocm_quantize_q8_0(ctx, m->pN, n, hs, hs, m->pQ, m->pS))) break;
-        if ((rc = gemm(ctx, L.gate, m, n, m->pGate, inter, 0)) || (rc = gemm(ctx, L.up, m, n, m->pUp, inter, 0))) break;
+        if ((rc = gemm_group(ctx, {L.gate, L.up}, {m->pGate, m->pUp}, m, n, inter))) break;
         if ((rc = wick_rocm_silu_mul(ctx, m->pGate, m->pUp, n * inter))) break;
         if ((rc = wick_rocm_quantize_q8_0(ctx, m->pGate, n, inter, inter, m->pQ, m->pS))) break;
         rc = gemm(ctx, L.down, m, n, m->pX, hs, 1);

@@ -117,6 +117,9 @@ hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                             const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
                             int accumulate, const Launch& L);
+hipError_t launch_gemm_mfma_multi(int type, const uint8_t* const* d_w, const uint32_t* m, uint32_t count, uint32_t k, const int8_t* d_q,
+                                  const float* d_scales, uint32_t n, float* const* d_y, uint32_t y_stride, int y_layout, int accumulate,
+                                  const Launch& L);
 
 // Per-block i32 dots, out[(j*m + i)*nb + b], through the same unpack + v_dot4 code
 // as the GEMV, or through the GEMM's loads / LDS layout / MFMA (k % 256 == 0).

@@ -84,6 +84,7 @@ _SIGNATURES = {
     "wick_rocm_gemv_q8": (C.c_int, [_P, _P, _P, _P, _P, C.c_int]),
     "wick_rocm_gemv_q8_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, _P, C.c_int]),
     "wick_rocm_gemm_q8": (C.c_int, [_P, _P, _P, _P, C.c_uint32, _P, C.c_uint32, C.c_int, C.c_int]),
+    "wick_rocm_gemm_q8_multi": (C.c_int, [_P, _P, _P, C.c_uint32, _P, _P, C.c_uint32, C.c_uint32, C.c_int, C.c_int]),
     "wick_rocm_matmul_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_uint32, C.c_uint32, _P, C.c_size_t, C.c_uint32, C.c_int]),
     "wick_rocm_gemv_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, C.c_size_t, C.c_int]),
     "wick_rocm_gemv_rmsnorm_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, _P, C.c_float, C.c_int]),
@@ -276,6 +277,14 @@ class RocmContext:
             y_stride = n if layout == LAYOUT_ROW_MAJOR else w.m
         self._check(self._lib.wick_rocm_gemm_q8(self._h, w.handle, _ptr(quants), _ptr(scales), n, _ptr(y), y_stride,
                                                 layout, int(accumulate)))
+
+    def gemm_preq_multi(self, ws: Sequence[RocmWeight], scales, quants, n: int, ys, y_stride: int, layout: int = LAYOUT_TOKEN_MAJOR,
+                        accumulate: bool = False) -> None:
+        """1..3 weights over the same quantized activations in one launch (Q / K / V, gate / up of a prompt pass)."""
+        c = len(ws)
+        wa = (_P * c)(*[w.handle for w in ws])
+        ya = (_P * c)(*[_ptr(y) for y in ys])
+        self._check(self._lib.wick_rocm_gemm_q8_multi(self._h, wa, ya, c, _ptr(quants), _ptr(scales), n, y_stride, layout, int(accumulate)))
 
     def block_dots_i32(self, w: RocmWeight, quants, n: int, out) -> None:
         self._check(self._lib.wick_rocm_block_dots_i32(self._h, w.handle, _ptr(quants), n, _ptr(out)))
