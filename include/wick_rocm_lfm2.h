@@ -90,6 +90,16 @@ int wick_rocm_shortconv_step(wick_rocm_ctx *ctx, const float *d_proj, float *d_b
  * (wick/src/backend/cpu.rs:668-673): gate = silu(gate) * up. */
 int wick_rocm_silu_mul(wick_rocm_ctx *ctx, float *d_gate, const float *d_up, uint32_t n);
 
+/* Prompt-pass forms of the two steps in front of a batched projection, without the f32 round trip through memory:
+ * wick_rocm_rmsnorm followed by wick_rocm_quantize_q8_0, and wick_rocm_silu_mul followed by wick_rocm_quantize_q8_0
+ * (quantize_columns after the norm / the gate, wick/src/model/lfm2.rs:1163-1200, 1990-2050), bit for bit.  Outputs in the
+ * split Q8_0 layout of wick_rocm_quantize_q8_0: d_quants [rows][dim] int8, d_scales [rows][dim / 32] f32.  dim % 32 == 0;
+ * rows of d_x (x_stride floats apart, x_stride % 4 == 0), d_weight, d_gate and d_up 16-byte aligned; gate / up contiguous. */
+int wick_rocm_rmsnorm_quantize_q8_0(wick_rocm_ctx *ctx, const float *d_x, const float *d_weight, uint32_t rows, uint32_t dim, uint32_t x_stride,
+                                    float eps, int8_t *d_quants, float *d_scales);
+int wick_rocm_silu_mul_quantize_q8_0(wick_rocm_ctx *ctx, const float *d_gate, const float *d_up, uint32_t rows, uint32_t dim, int8_t *d_quants,
+                                     float *d_scales);
+
 /* argmax_f32 dispatch of forward_greedy (wick/src/model/metal_lfm2.rs:2187-2195) with the tie / NaN rules of
  * cpu_argmax (wick/src/sampler.rs:7-19).  d_out[0] = pick; when given, *d_token = pick and *d_pos += 1. */
 int wick_rocm_argmax(wick_rocm_ctx *ctx, const float *d_logits, uint32_t n, uint32_t *d_out, uint32_t *d_token, uint32_t *d_pos);

@@ -245,3 +245,43 @@ def test_argmax_rules(ctx, ops):
     assert d_tok.download(np.uint32, 1)[0] == 1 and d_pos.download(np.uint32, 1)[0] == 42
     for b in (d_out, d_tok, d_pos, d_x):
         b.free()
+
+
+@pytest.mark.parametrize("rows,dim,pad", [(1, 32, 0), (3, 256, 0), (17, 1024, 8), (5, 4608, 0), (2, 2080, 4)])
+def test_rmsnorm_quantize_equals_the_two_launches(ctx, ops, oracle, rows, dim, pad):
+    """Norm and Q8_0 quantizer in one pass: quants and scale bits of rmsnorm followed by quantize_q8_0, and of the oracle."""
+    stride, eps = dim + pad, 1e-5
+    x = oracle.fill_normal(rows * 3 + dim, 1.5, rows * stride)
+    wt = (1 + 0.3 * oracle.fill_normal(dim, 1.0, dim)).astype(np.float32)
+    d_x, d_w = ctx.to_device(x), ctx.to_device(wt)
+    d_n, d_q1, d_s1 = ctx.alloc(rows * dim * 4), ctx.alloc(rows * dim), ctx.alloc(rows * dim // 32 * 4)
+    d_q2, d_s2 = ctx.alloc(rows * dim), ctx.alloc(rows * dim // 32 * 4)
+    ops.encode_rmsnorm(d_x, d_w, d_n, dim, eps, rows=rows, x_stride=stride, y_stride=dim)
+    ctx.quantize_q8_0(d_n, rows, dim, dim, d_q1, d_s1)
+    ops.rmsnorm_quantize(d_x, d_w, rows, dim, eps, d_q2, d_s2, x_stride=stride)
+    assert np.array_equal(d_q1.download(np.int8, rows * dim), d_q2.download(np.int8, rows * dim))
+    assert np.array_equal(bits(d_s1.download(np.float32, rows * dim // 32)), bits(d_s2.download(np.float32, rows * dim // 32)))
+    normed = np.concatenate([L.rmsnorm(x[r * stride: r * stride + dim], wt, eps) for r in range(rows)])
+    if np.array_equal(bits(normed), bits(d_n.download(np.float32, rows * dim))):  # the f64 sum of squares is taken in another order than the oracle's loop
+        s, q = oracle.quantize_q8_0_batch(normed, rows, dim)
+        assert np.array_equal(q.ravel(), d_q2.download(np.int8, rows * dim))
+    with pytest.raises(W.RocmError):
+        ops.rmsnorm_quantize(d_x, d_w, rows, dim + 8, eps, d_q2, d_s2, x_stride=stride + 8)
+    for b in (d_x, d_w, d_n, d_q1, d_s1, d_q2, d_s2):
+        b.free()
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 32), (4, 256), (9, 4608), (33, 1024)])
+def test_silu_mul_quantize_equals_the_two_launches(ctx, ops, oracle, rows, dim):
+    g, u = oracle.fill_normal(rows + dim, 2.0, rows * dim), oracle.fill_normal(rows + dim + 1, 1.0, rows * dim)
+    d_g, d_u = ctx.to_device(g), ctx.to_device(u)
+    d_q1, d_s1, d_q2, d_s2 = ctx.alloc(rows * dim), ctx.alloc(rows * dim // 32 * 4), ctx.alloc(rows * dim), ctx.alloc(rows * dim // 32 * 4)
+    ops.silu_mul_quantize(d_g, d_u, rows, dim, d_q2, d_s2)
+    ops.silu_mul_inplace(d_g, d_u, rows * dim)
+    ctx.quantize_q8_0(d_g, rows, dim, dim, d_q1, d_s1)
+    assert np.array_equal(d_q1.download(np.int8, rows * dim), d_q2.download(np.int8, rows * dim))
+    assert np.array_equal(bits(d_s1.download(np.float32, rows * dim // 32)), bits(d_s2.download(np.float32, rows * dim // 32)))
+    s, q = oracle.quantize_q8_0_batch(L.silu_mul(g, u), rows, dim)  # silu_mul is bit-exact, so the oracle's quantizer must agree too
+    assert np.array_equal(q.ravel(), d_q2.download(np.int8, rows * dim))
+    for b in (d_g, d_u, d_q1, d_s1, d_q2, d_s2):
+        b.free()

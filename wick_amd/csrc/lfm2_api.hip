@@ -137,6 +137,29 @@ int wick_rocm_silu_mul(wick_rocm_ctx* ctx, float* d_gate, const float* d_up, uin
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "silu_mul launch");
 }
 
+int wick_rocm_rmsnorm_quantize_q8_0(wick_rocm_ctx* ctx, const float* d_x, const float* d_weight, uint32_t rows, uint32_t dim, uint32_t x_stride,
+                                    float eps, int8_t* d_quants, float* d_scales) {
+    WR_ENTER(ctx);
+    if (!d_x || !d_weight || !d_quants || !d_scales) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "rmsnorm_quantize: null device pointer");
+    if (dim == 0 || dim % 32u != 0 || x_stride < dim || x_stride % 4u != 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "rmsnorm_quantize: dim % 32 != 0 or stride < dim or stride % 4 != 0");
+    if (misaligned(d_x, 16) || misaligned(d_weight, 16) || misaligned(d_quants, 4))
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "rmsnorm_quantize: x and weight must be 16-byte aligned");
+    hipError_t e = launch_rmsnorm_quantize(d_x, d_weight, rows, dim, x_stride, eps, d_quants, d_scales, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "rmsnorm_quantize launch");
+}
+
+int wick_rocm_silu_mul_quantize_q8_0(wick_rocm_ctx* ctx, const float* d_gate, const float* d_up, uint32_t rows, uint32_t dim, int8_t* d_quants,
+                                     float* d_scales) {
+    WR_ENTER(ctx);
+    if (!d_gate || !d_up || !d_quants || !d_scales) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "silu_mul_quantize: null device pointer");
+    if (dim % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "silu_mul_quantize: dim % 32 != 0");
+    if (misaligned(d_gate, 16) || misaligned(d_up, 16) || misaligned(d_quants, 4))
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "silu_mul_quantize: gate and up must be 16-byte aligned");
+    hipError_t e = launch_silu_mul_quantize(d_gate, d_up, rows, dim, d_quants, d_scales, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "silu_mul_quantize launch");
+}
+
 int wick_rocm_argmax(wick_rocm_ctx* ctx, const float* d_logits, uint32_t n, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos) {
     WR_ENTER(ctx);
     if (!d_logits || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "argmax: null device pointer");
@@ -183,7 +206,7 @@ struct wick_rocm_lfm2 {
     unsigned long long* d_argmax_partial = nullptr;
     // prompt (prefill) buffers for up to `prefill_cap` tokens, allocated by the first prefill
     uint32_t prefill_cap = 0;
-    float *pX = nullptr, *pN = nullptr, *pA = nullptr, *pG = nullptr, *pGate = nullptr, *pUp = nullptr, *pS = nullptr, *pAttn = nullptr;
+    float *pX = nullptr, *pA = nullptr, *pG = nullptr, *pGate = nullptr, *pUp = nullptr, *pS = nullptr, *pAttn = nullptr;
     int8_t* pQ = nullptr;
     uint32_t* pTokens = nullptr;
     wick_rocm_graph *g_logits = nullptr, *g_greedy = nullptr;
@@ -334,7 +357,7 @@ int ensure_prefill_buffers(wick_rocm_ctx* ctx, wick_rocm_lfm2* m) {
     const size_t P = c.max_seq_len < kPrefillChunk ? c.max_seq_len : kPrefillChunk;
     const size_t hs = c.hidden_size, inter = c.intermediate_size, hd = hs / c.n_heads, wide = hs > inter ? hs : inter;
     int rc;
-    if ((rc = alloc_t(ctx, m, P * hs, &m->pX)) || (rc = alloc_t(ctx, m, P * hs, &m->pN)) || (rc = alloc_t(ctx, m, P * 3 * hs, &m->pA)) ||
+    if ((rc = alloc_t(ctx, m, P * hs, &m->pX)) || (rc = alloc_t(ctx, m, P * 3 * hs, &m->pA)) ||
         (rc = alloc_t(ctx, m, P * hs, &m->pG)) || (rc = alloc_t(ctx, m, P * inter, &m->pGate)) || (rc = alloc_t(ctx, m, P * inter, &m->pUp)) ||
         (rc = alloc_t(ctx, m, P * wide, &m->pQ)) || (rc = alloc_t(ctx, m, P * (wide / 32), &m->pS)) ||
         (rc = alloc_t(ctx, m, attention_prefill_scratch_floats((uint32_t)P, c.n_heads, (uint32_t)hd), &m->pAttn)) ||
@@ -378,8 +401,7 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
                     "embed_rows launch");
     for (uint32_t i = 0; rc == 0 && i < c.n_layers; i++) {
         const LayerWeights& L = m->layers[i];
-        if ((rc = wick_rocm_rmsnorm(ctx, m->pX, L.attn_norm, m->pN, n, hs, hs, hs, c.rms_norm_eps))) break;
-        if ((rc = wick_rocm_quantize_q8_0(ctx, m->pN, n, hs, hs, m->pQ, m->pS))) break;
+        if ((rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.attn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
         if (L.n_kv == 0) {
             if ((rc = gemm(ctx, L.in_proj, m, n, m->pA, 3 * hs, 0))) break;
             if ((rc = locked([&] { return launch_shortconv_seq(m->pA, L.conv_state, L.conv_w, m->pG, hs, c.conv_kernel_size, n, ctx->launch()); },
@@ -408,11 +430,9 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
         }
         if ((rc = wick_rocm_quantize_q8_0(ctx, m->pG, n, hs, hs, m->pQ, m->pS))) break;
         if ((rc = gemm(ctx, L.n_kv == 0 ? L.out_proj : L.o, m, n, m->pX, hs, 1))) break;  // hidden += out projection
-        if ((rc = wick_rocm_rmsnorm(ctx, m->pX, L.ffn_norm, m->pN, n, hs, hs, hs, c.rms_norm_eps))) break;
-        if ((rc = wick_rocm_quantize_q8_0(ctx, m->pN, n, hs, hs, m->pQ, m->pS))) break;
+        if ((rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.ffn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
         if ((rc = gemm_group(ctx, {L.gate, L.up}, {m->pGate, m->pUp}, m, n, inter))) break;
-        if ((rc = wick_rocm_silu_mul(ctx, m->pGate, m->pUp, n * inter))) break;
-        if ((rc = wick_rocm_quantize_q8_0(ctx, m->pGate, n, inter, inter, m->pQ, m->pS))) break;
+        if ((rc = wick_rocm_silu_mul_quantize_q8_0(ctx, m->pGate, m->pUp, n, inter, m->pQ, m->pS))) break;
         rc = gemm(ctx, L.down, m, n, m->pX, hs, 1);
     }
     return rc;

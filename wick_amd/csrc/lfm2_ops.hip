@@ -812,6 +812,64 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(float* __restrict__ gate,
     gate[i] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, ggml_expf(-g))), up[i]);
 }
 
+// ---- normalise / gate and quantize in one pass (prompt passes) -----------------------------------
+// What rmsnorm_kernel followed by the Q8_0 quantizer compute (wick/src/backend/cpu.rs:577-594, wick/src/backend/simd.rs:255-323),
+// bit for bit, without the f32 round trip through memory: the sum of squares is taken over the same elements per thread
+// and in the same order as rmsnorm_kernel does, the normalised values are formed by the same two products, and eight
+// lanes own one 32-element block exactly as in the quantizer.  One block per row; dim % 32 == 0, rows 16-byte aligned.
+__global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const float* __restrict__ x, const float* __restrict__ weight, int8_t* __restrict__ q,
+                                                               float* __restrict__ scales, uint32_t dim, uint32_t x_stride, float eps) {
+    __shared__ double slots[16];
+    const float* xr = x + (size_t)blockIdx.x * x_stride;
+    double s = 0.0;
+    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
+        const double v = (double)xr[i];
+        s += v * v;
+    }
+    const double total = block_sum_f64(s, slots);
+    const float inv_rms = (float)(1.0 / sqrt(total / (double)dim + (double)eps));
+    const uint32_t quads = dim >> 2;
+    for (uint32_t quad0 = 0; quad0 < quads; quad0 += blockDim.x) {  // groups of 8 lanes stay together: quads % 8 == 0
+        const uint32_t quad = quad0 + threadIdx.x;
+        const bool live = quad < quads;
+        const uint32_t qd = live ? quad : 0;
+        const float4 v = reinterpret_cast<const float4*>(xr)[qd];
+        const float4 w = reinterpret_cast<const float4*>(weight)[qd];
+        const float v0 = __fmul_rn(__fmul_rn(v.x, inv_rms), w.x), v1 = __fmul_rn(__fmul_rn(v.y, inv_rms), w.y);
+        const float v2 = __fmul_rn(__fmul_rn(v.z, inv_rms), w.z), v3 = __fmul_rn(__fmul_rn(v.w, inv_rms), w.w);
+        float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+        amax = group_max8(amax);
+        float id;
+        const float scale = q8_scale_and_inverse(amax, id);
+        const uint32_t packed = q8_pack4(v0, v1, v2, v3, id);
+        if (live) {
+            *reinterpret_cast<uint32_t*>(q + (size_t)blockIdx.x * dim + 4u * quad) = packed;
+            if ((quad & 7u) == 0) scales[(size_t)blockIdx.x * (dim >> 5) + (quad >> 3)] = scale;
+        }
+    }
+}
+
+// silu_mul_kernel followed by the quantizer, bit for bit: the gated values go straight into Q8_0 blocks.
+// gate / up: [n][dim] floats, contiguous, 16-byte aligned.
+__global__ __launch_bounds__(256) void silu_mul_quantize_kernel(const float* __restrict__ gate, const float* __restrict__ up, int8_t* __restrict__ q,
+                                                                float* __restrict__ scales, uint64_t total_quads) {
+    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const bool live = t < total_quads;
+    const uint64_t tt = live ? t : 0;
+    const float4 g = reinterpret_cast<const float4*>(gate)[tt];
+    const float4 u = reinterpret_cast<const float4*>(up)[tt];
+    const float v0 = silu_mul(g.x, u.x), v1 = silu_mul(g.y, u.y), v2 = silu_mul(g.z, u.z), v3 = silu_mul(g.w, u.w);
+    float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+    amax = group_max8(amax);
+    float id;
+    const float scale = q8_scale_and_inverse(amax, id);
+    const uint32_t packed = q8_pack4(v0, v1, v2, v3, id);
+    if (live) {
+        reinterpret_cast<uint32_t*>(q)[tt] = packed;
+        if ((tt & 7u) == 0) scales[tt >> 3] = scale;
+    }
+}
+
 // ---- greedy pick ----------------------------------------------------------------------
 // cpu_argmax (wick/src/sampler.rs:7-19): NaN counts as -inf, values order by f32::total_cmp, the LAST of
 // equal maxima wins; bit-exact.  Two small launches (64 blocks, then one wave over their partial keys): a single
@@ -1030,6 +1088,18 @@ hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, co
         case 256: return launch_kernel(L, kFamOther, attention_prefill_kernel<256>, grid, block, a, pos0, n, q_stride, out_stride);
         default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t launch_rmsnorm_quantize(const float* d_x, const float* d_weight, uint32_t rows, uint32_t dim, uint32_t x_stride, float eps, int8_t* d_q,
+                                   float* d_scales, const Launch& L) {
+    if (rows == 0) return hipSuccess;
+    return launch_kernel(L, kFamQuantize, rmsnorm_quantize_kernel, dim3(rows), dim3(256), d_x, d_weight, d_q, d_scales, dim, x_stride, eps);
+}
+
+hipError_t launch_silu_mul_quantize(const float* d_gate, const float* d_up, uint32_t n, uint32_t dim, int8_t* d_q, float* d_scales, const Launch& L) {
+    const uint64_t total = (uint64_t)n * (dim >> 2);
+    if (total == 0) return hipSuccess;
+    return launch_kernel(L, kFamQuantize, silu_mul_quantize_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), d_gate, d_up, d_q, d_scales, total);
 }
 
 hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const Launch& L) {

@@ -167,6 +167,9 @@ hipError_t launch_attention_layer(const float* d_q, const float* d_k, const floa
                                   float theta_scale, float scale, const Launch& L);
 hipError_t launch_shortconv_step(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
                                  uint32_t kernel_size, const Launch& L);
+hipError_t launch_rmsnorm_quantize(const float* d_x, const float* d_weight, uint32_t rows, uint32_t dim, uint32_t x_stride, float eps, int8_t* d_q,
+                                   float* d_scales, const Launch& L);
+hipError_t launch_silu_mul_quantize(const float* d_gate, const float* d_up, uint32_t n, uint32_t dim, int8_t* d_q, float* d_scales, const Launch& L);
 hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const Launch& L);
 // d_history[pos] = pick (pos = *d_pos before it is advanced), when given.  d_partial: scratch of kArgmaxPartials keys, 8-byte aligned;
 // d_x 16-byte aligned.

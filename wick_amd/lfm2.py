@@ -36,6 +36,8 @@ _SIGNATURES = {
     "wick_rocm_shortconv_step": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32]),
     "wick_rocm_silu_mul": (C.c_int, [_P, _P, _P, _U32]),
     "wick_rocm_argmax": (C.c_int, [_P, _P, _U32, _P, _P, _P]),
+    "wick_rocm_rmsnorm_quantize_q8_0": (C.c_int, [_P, _P, _P, _U32, _U32, _U32, _F, _P, _P]),
+    "wick_rocm_silu_mul_quantize_q8_0": (C.c_int, [_P, _P, _P, _U32, _U32, _P, _P]),
     "wick_rocm_lfm2_load": (C.c_int, [_P, _P, _U32, C.POINTER(_P)]),
     "wick_rocm_lfm2_free": (C.c_int, [_P, _P]),
     "wick_rocm_lfm2_get_config": (C.c_int, [_P, C.POINTER(Lfm2Config)]),
@@ -118,6 +120,15 @@ class Lfm2Ops:
 
     def silu_mul_inplace(self, gate, up, n: int) -> None:
         self.ctx._check(self._l.wick_rocm_silu_mul(self.ctx._h, _ptr(gate), _ptr(up), n))
+
+    def rmsnorm_quantize(self, x, weight, rows: int, dim: int, eps: float, quants, scales, x_stride: Optional[int] = None) -> None:
+        """encode_rmsnorm + quantize_q8_0 of `rows` vectors without the f32 round trip."""
+        self.ctx._check(self._l.wick_rocm_rmsnorm_quantize_q8_0(self.ctx._h, _ptr(x), _ptr(weight), rows, dim, x_stride or dim, eps, _ptr(quants),
+                                                                _ptr(scales)))
+
+    def silu_mul_quantize(self, gate, up, rows: int, dim: int, quants, scales) -> None:
+        """silu_mul_inplace + quantize_q8_0 of [rows][dim] gate / up values, the gated f32 values never written."""
+        self.ctx._check(self._l.wick_rocm_silu_mul_quantize_q8_0(self.ctx._h, _ptr(gate), _ptr(up), rows, dim, _ptr(quants), _ptr(scales)))
 
     def argmax(self, logits, n: int, out, d_token=None, d_pos=None) -> None:
         self.ctx._check(self._l.wick_rocm_argmax(self.ctx._h, _ptr(logits), n, _ptr(out), _ptr(d_token), _ptr(d_pos)))
