@@ -418,6 +418,11 @@ int gemv_xform_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, flo
     }
     if (int rc = ensure_scratch(ctx, k, k / 32u, k)) return rc;
     hipError_t e;
+    if (xform == kXformRmsNorm && ws[0]->type == kTypeQ6_K && aligned16(x) && aligned16(d_aux)) {  // norm and quantizer in one launch
+        e = launch_rmsnorm_quantize(x, d_aux, 1, k, k, eps, ctx->scratch_q, ctx->scratch_s, ctx->launch());
+        if (e != hipSuccess) return fail_hip(ctx, e, "rmsnorm_quantize launch");
+        return q6k_gemv_locked(ctx, ws, d_ys, count, ctx->scratch_q, ctx->scratch_s, accumulate);
+    }
     if (xform == kXformRmsNorm) {
         e = launch_rmsnorm(x, d_aux, ctx->scratch_f, 1, k, k, k, eps, ctx->launch());
     } else {

@@ -294,7 +294,8 @@ int gemv_residual(wick_rocm_ctx* ctx, const wick_rocm_weight* w, float* y, const
 int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
     const wick_rocm_lfm2_config& c = m->cfg;
     const uint32_t hs = c.hidden_size, hd = hs / c.n_heads;
-    int rc = wick_rocm_embed_row(ctx, m->embd, 0, m->d_token, m->hidden);
+    // m->hidden already holds the token's embedding row: set_step (or the previous step's greedy pick) looked it up
+    int rc = 0;
     for (uint32_t i = 0; rc == 0 && i < c.n_layers; i++) {
         const LayerWeights& L = m->layers[i];
         if (L.n_kv == 0) {
@@ -317,7 +318,7 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
     if (!greedy) return WICK_ROCM_OK;
     std::lock_guard<std::mutex> lk(ctx->mu);
     hipError_t e = launch_argmax(m->logits, c.vocab_size, m->d_argmax_partial, m->d_pick, m->d_token, m->d_pos, m->d_history, c.max_seq_len,
-                                 ctx->launch());
+                                 ctx->launch(), static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m, c.hidden_size, m->hidden);
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
 }
 
@@ -440,7 +441,8 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
 
 int set_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t token, uint32_t pos) {
     std::lock_guard<std::mutex> lk(ctx->mu);
-    hipError_t e = launch_set_step(m->d_token, token, m->d_pos, pos, ctx->launch());
+    hipError_t e = launch_set_step(m->d_token, token, m->d_pos, pos, ctx->launch(), static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m,
+                                   m->cfg.hidden_size, m->hidden);
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "set_step launch");
 }
 

@@ -926,17 +926,27 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __rest
 }
 
 // Stage 2: one wave merges the partial keys and publishes the pick.
+// An embedding to look the next step's input up in (w null: none): row `token` of w as k floats into `out`.
+struct EmbedArgs {
+    const uint8_t* w;
+    float* out;
+    int type;
+    uint32_t m, k;
+};
+
 __global__ __launch_bounds__(64) void argmax_final_kernel(const unsigned long long* __restrict__ partial, uint32_t blocks, uint32_t n,
                                                           uint32_t* __restrict__ out, uint32_t* __restrict__ d_token, uint32_t* __restrict__ d_pos,
-                                                          uint32_t* __restrict__ d_history, uint32_t history_len) {
+                                                          uint32_t* __restrict__ d_history, uint32_t history_len, EmbedArgs emb) {
     unsigned long long best = threadIdx.x < blocks ? partial[threadIdx.x] : 0ull;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         const unsigned long long o = __shfl_xor(best, off, 64);
         best = o > best ? o : best;
     }
+    const uint32_t pick = n ? (uint32_t)(best & 0xffffffffull) : 0u;  // every lane holds the maximum after the butterfly
+    if (emb.w && pick < emb.m)  // the pick is the next step's token: its embedding row is that step's input
+        for (uint32_t e = threadIdx.x; e < emb.k; e += 64) emb.out[e] = dequant_element(emb.w, emb.type, pick, emb.k, e);
     if (threadIdx.x == 0) {
-        const uint32_t pick = n ? (uint32_t)(best & 0xffffffffull) : 0u;
         out[0] = pick;
         if (d_token) *d_token = pick;
         if (d_pos) {
@@ -947,12 +957,15 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const unsigned long lo
     }
 }
 
-// Sets the device-side token / position of the next step (either may be null).
-__global__ void set_step_kernel(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
+// Sets the device-side token / position of the next step (either may be null) and, when an embedding is given, looks
+// the token's row up as that step's input.
+__global__ __launch_bounds__(256) void set_step_kernel(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, EmbedArgs emb) {
+    if (threadIdx.x == 0) {
         if (d_token) *d_token = token;
         if (d_pos) *d_pos = pos;
     }
+    if (emb.w && token < emb.m)
+        for (uint32_t e = threadIdx.x; e < emb.k; e += blockDim.x) emb.out[e] = dequant_element(emb.w, emb.type, token, emb.k, e);
 }
 
 __global__ void advance_pos_kernel(uint32_t* d_pos) {
@@ -1108,15 +1121,19 @@ hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const L
 }
 
 hipError_t launch_argmax(const float* d_x, uint32_t n, unsigned long long* d_partial, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos,
-                         uint32_t* d_history, uint32_t history_len, const Launch& L) {
+                         uint32_t* d_history, uint32_t history_len, const Launch& L, const uint8_t* d_embd, int embd_type, uint32_t embd_m,
+                         uint32_t embd_k, float* d_embd_out) {
     const uint32_t blocks = n >= 4096u ? kArgmaxBlocks : 1u;
     hipError_t e = launch_kernel(L, kFamOther, argmax_partial_kernel, dim3(blocks), dim3(256), d_x, n, d_partial);
     if (e != hipSuccess) return e;
-    return launch_kernel(L, kFamOther, argmax_final_kernel, dim3(1), dim3(64), d_partial, blocks, n, d_out, d_token, d_pos, d_history, history_len);
+    const EmbedArgs emb{d_embd_out ? d_embd : nullptr, d_embd_out, embd_type, embd_m, embd_k};
+    return launch_kernel(L, kFamOther, argmax_final_kernel, dim3(1), dim3(64), d_partial, blocks, n, d_out, d_token, d_pos, d_history, history_len, emb);
 }
 
-hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L) {
-    return launch_kernel(L, kFamOther, set_step_kernel, dim3(1), dim3(64), d_token, token, d_pos, pos);
+hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L, const uint8_t* d_embd, int embd_type,
+                           uint32_t embd_m, uint32_t embd_k, float* d_embd_out) {
+    const EmbedArgs emb{d_embd_out ? d_embd : nullptr, d_embd_out, embd_type, embd_m, embd_k};
+    return launch_kernel(L, kFamOther, set_step_kernel, dim3(1), dim3(256), d_token, token, d_pos, pos, emb);
 }
 
 hipError_t launch_advance_pos(uint32_t* d_pos, const Launch& L) {

@@ -174,9 +174,12 @@ hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const L
 // d_history[pos] = pick (pos = *d_pos before it is advanced), when given.  d_partial: scratch of kArgmaxPartials keys, 8-byte aligned;
 // d_x 16-byte aligned.
 constexpr uint32_t kArgmaxPartials = 64;
+// d_embd_out non-null: the pick's row of the embedding (d_embd, type, m x k) is written there as the next step's input.
 hipError_t launch_argmax(const float* d_x, uint32_t n, unsigned long long* d_partial, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos,
-                         uint32_t* d_history, uint32_t history_len, const Launch& L);
-hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L);
+                         uint32_t* d_history, uint32_t history_len, const Launch& L, const uint8_t* d_embd = nullptr, int embd_type = 0,
+                         uint32_t embd_m = 0, uint32_t embd_k = 0, float* d_embd_out = nullptr);
+hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L, const uint8_t* d_embd = nullptr,
+                           int embd_type = 0, uint32_t embd_m = 0, uint32_t embd_k = 0, float* d_embd_out = nullptr);
 hipError_t launch_advance_pos(uint32_t* d_pos, const Launch& L);
 
 // n at and above which gemm_q8 uses the MFMA kernel (when k % 256 == 0).
