@@ -293,8 +293,7 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
                     part += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
                 }
             }
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+            part = wave_sum_f64(part);
             if (lane == 0) sq[threadIdx.x >> 6] = part;
             __syncthreads();
             const double total = (sq[0] + sq[1]) + (sq[2] + sq[3]);

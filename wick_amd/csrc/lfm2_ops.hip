@@ -19,12 +19,6 @@ namespace wick_rocm {
 
 namespace {
 
-__device__ __forceinline__ double wave_sum_f64(double v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-
 // Sum over a block of up to 16 waves; every thread gets the total.  `slots` holds 16 doubles.
 __device__ __forceinline__ double block_sum_f64(double v, double* slots) {
     v = wave_sum_f64(v);
@@ -252,24 +246,6 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttentionArgs a) 
 constexpr uint32_t kAttnChunk = 64;       // positions a workgroup handles per pass
 constexpr uint32_t kAttnMaxSplits = 64;   // workgroups per head; contexts beyond 64 * 64 positions make them loop
 
-__device__ __forceinline__ float block_max_f32(float v, float* slots) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
-    __syncthreads();
-    return fmaxf(fmaxf(slots[0], slots[1]), fmaxf(slots[2], slots[3]));
-}
-
-__device__ __forceinline__ float block_sum_f32(float v, float* slots) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
-    __syncthreads();
-    return (slots[0] + slots[1]) + (slots[2] + slots[3]);
-}
-
 // The chunks of workgroup (h, split): scores against q (HD floats, 16-byte aligned, global or LDS), streaming softmax,
 // weighted values; leaves {max, sum, acc[HD]} in the partial record of (h, split).  All 256 threads call it.
 template <int HD>
@@ -284,7 +260,6 @@ __device__ __forceinline__ void attention_chunks(const AttentionArgs& a, uint32_
     static_assert(KROWS >= 1 && KROWS % KB == 0 && VROWS % VB == 0, "chunk does not tile");
     __shared__ float sc[kAttnChunk];
     __shared__ float red[256];
-    __shared__ float slots[4];
     const uint32_t kv_dim = a.n_kv_heads * HD;
     const uint32_t kvh = h / (a.n_heads / a.n_kv_heads);
     const float* kbase = a.k_cache + (size_t)kvh * HD;
@@ -316,11 +291,16 @@ __device__ __forceinline__ void attention_chunks(const AttentionArgs& a, uint32_
             }
         }
         __syncthreads();
-        const float s = tid < kAttnChunk ? sc[tid] : -__builtin_inff();
-        const float m_new = fmaxf(m_run, block_max_f32(s, slots));
-        const float e = tid < nt ? ggml_expf(s - m_new) : 0.0f;
-        if (tid < kAttnChunk) sc[tid] = e;  // every thread read its own score above; positions past the end weigh 0
-        const float l_chunk = block_sum_f32(e, slots);  // its barriers publish sc[]
+        // Every wave takes the chunk's 64 scores (one per lane) and reduces them on its own: no cross-wave exchange,
+        // the exponentials are computed four times over instead.
+        const uint32_t lane = tid & 63u;
+        const float s = sc[lane];
+        const float m_new = fmaxf(m_run, wave_max_f32(s));
+        const float e = lane < nt ? ggml_expf(s - m_new) : 0.0f;  // positions past the end weigh 0
+        const float l_chunk = wave_sum_f32(e);
+        __syncthreads();  // every wave has read the scores
+        if (tid < kAttnChunk) sc[tid] = e;
+        __syncthreads();
         const float corr = ggml_expf(m_run - m_new);    // 0 on the first chunk (m_run = -inf)
         l_run = l_run * corr + l_chunk;
         acc *= corr;
@@ -366,13 +346,9 @@ __device__ __forceinline__ void attention_merge(const AttentionArgs& a, uint32_t
         const bool on = tid < active;
         const float m_i = on ? parts[(size_t)tid * (HD + 2)] : -__builtin_inff();
         const float l_i = on ? parts[(size_t)tid * (HD + 2) + 1] : 0.0f;
-        float m = m_i;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+        const float m = wave_max_f32(m_i);
         const float w = on ? ggml_expf(m_i - m) : 0.0f;
-        float l = l_i * w;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off, 64);
+        const float l = wave_sum_f32(l_i * w);
         wts[tid] = w;
         if (tid == 0) total = l;
     }
@@ -526,15 +502,10 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
         for (uint32_t w2 = 0; w2 < 2; w2++) {  // this wave's two queries: one lane per position of the chunk
             const uint32_t q = 2 * wave + w2;
             const float s = sc[q][lane];
-            float mx = s;
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-            const float m_new = fmaxf(m_run[w2], mx);
+            const float m_new = fmaxf(m_run[w2], wave_max_f32(s));
             // a chunk (or a query slot) with nothing to see keeps -inf: weights 0, nothing rescaled
             const float e = m_new == -__builtin_inff() ? 0.0f : ggml_expf(s - m_new);
-            float l = e;
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off, 64);
+            const float l = wave_sum_f32(e);
             const float c = m_new == -__builtin_inff() ? 1.0f : ggml_expf(m_run[w2] - m_new);
             sc[q][lane] = e;
             l_run[w2] = l_run[w2] * c + l;

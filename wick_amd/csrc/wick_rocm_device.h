@@ -188,6 +188,49 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
+// The same for a double over the whole wave, every lane gets the total: four DPP steps inside the rows of 16 lanes
+// (each moves the two halves of the double), then the four row totals through scalar registers.  A butterfly of
+// 64-bit shuffles costs twelve trips through the LDS crossbar, which is most of an RMSNorm prologue.
+template <int CTRL>
+__device__ __forceinline__ double dpp_add_f64(double v) {
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, 0xf, 0xf, false);
+    return v + __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+    v = dpp_add_f64<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add_f64<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add_f64<0x141>(v);  // row_half_mirror
+    v = dpp_add_f64<0x140>(v);  // row_mirror: every lane of a row holds the row's sum
+    const int lo = __double2loint(v), hi = __double2hiint(v);
+    const double r0 = __hiloint2double(__builtin_amdgcn_readlane(hi, 0), __builtin_amdgcn_readlane(lo, 0));
+    const double r1 = __hiloint2double(__builtin_amdgcn_readlane(hi, 16), __builtin_amdgcn_readlane(lo, 16));
+    const double r2 = __hiloint2double(__builtin_amdgcn_readlane(hi, 32), __builtin_amdgcn_readlane(lo, 32));
+    const double r3 = __hiloint2double(__builtin_amdgcn_readlane(hi, 48), __builtin_amdgcn_readlane(lo, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// f32 sum / maximum over the whole wave, every lane gets the result: DPP inside the rows, row results through scalar
+// registers.
+__device__ __forceinline__ float wave_sum_f32(float v) {
+    v = group_sum<16>(v);
+    const int b = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) {
+    return fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false)));
+}
+__device__ __forceinline__ float wave_max_f32(float v) {
+    v = dpp_max<0xB1>(v), v = dpp_max<0x4E>(v), v = dpp_max<0x141>(v), v = dpp_max<0x140>(v);
+    const int b = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
 __device__ __forceinline__ float bits_f(uint32_t u) { return __uint_as_float(u); }
 
 // ggml_expf (wick/src/backend/cpu.rs:604-652), operation for operation: bit-exact.
