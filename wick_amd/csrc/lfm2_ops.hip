@@ -905,27 +905,34 @@ struct EmbedArgs {
     uint32_t m, k;
 };
 
-__global__ __launch_bounds__(64) void argmax_final_kernel(const unsigned long long* __restrict__ partial, uint32_t blocks, uint32_t n,
-                                                          uint32_t* __restrict__ out, uint32_t* __restrict__ d_token, uint32_t* __restrict__ d_pos,
-                                                          uint32_t* __restrict__ d_history, uint32_t history_len, EmbedArgs emb) {
-    unsigned long long best = threadIdx.x < blocks ? partial[threadIdx.x] : 0ull;
+__global__ __launch_bounds__(256) void argmax_final_kernel(const unsigned long long* __restrict__ partial, uint32_t blocks, uint32_t n,
+                                                           uint32_t* __restrict__ out, uint32_t* __restrict__ d_token, uint32_t* __restrict__ d_pos,
+                                                           uint32_t* __restrict__ d_history, uint32_t history_len, EmbedArgs emb) {
+    __shared__ uint32_t picked;
+    if (threadIdx.x < 64) {  // the first wave reduces the (at most 64) partial keys
+        unsigned long long best = threadIdx.x < blocks ? partial[threadIdx.x] : 0ull;
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const unsigned long long o = __shfl_xor(best, off, 64);
-        best = o > best ? o : best;
-    }
-    const uint32_t pick = n ? (uint32_t)(best & 0xffffffffull) : 0u;  // every lane holds the maximum after the butterfly
-    if (emb.w && pick < emb.m)  // the pick is the next step's token: its embedding row is that step's input
-        for (uint32_t e = threadIdx.x; e < emb.k; e += 64) emb.out[e] = dequant_element(emb.w, emb.type, pick, emb.k, e);
-    if (threadIdx.x == 0) {
-        out[0] = pick;
-        if (d_token) *d_token = pick;
-        if (d_pos) {
-            const uint32_t pos = *d_pos;
-            if (d_history && pos < history_len) d_history[pos] = pick;  // the pick made after the token at `pos`
-            *d_pos = pos + 1u;
+        for (int off = 32; off > 0; off >>= 1) {
+            const unsigned long long o = __shfl_xor(best, off, 64);
+            best = o > best ? o : best;
+        }
+        if (threadIdx.x == 0) {
+            const uint32_t pick = n ? (uint32_t)(best & 0xffffffffull) : 0u;
+            picked = pick;
+            out[0] = pick;
+            if (d_token) *d_token = pick;
+            if (d_pos) {
+                const uint32_t pos = *d_pos;
+                if (d_history && pos < history_len) d_history[pos] = pick;  // the pick made after the token at `pos`
+                *d_pos = pos + 1u;
+            }
         }
     }
+    if (!emb.w) return;
+    __syncthreads();
+    const uint32_t pick = picked;  // the pick is the next step's token: its embedding row is that step's input
+    if (pick < emb.m)
+        for (uint32_t e = threadIdx.x; e < emb.k; e += blockDim.x) emb.out[e] = dequant_element(emb.w, emb.type, pick, emb.k, e);
 }
 
 // Sets the device-side token / position of the next step (either may be null) and, when an embedding is given, looks
@@ -1098,7 +1105,7 @@ hipError_t launch_argmax(const float* d_x, uint32_t n, unsigned long long* d_par
     hipError_t e = launch_kernel(L, kFamOther, argmax_partial_kernel, dim3(blocks), dim3(256), d_x, n, d_partial);
     if (e != hipSuccess) return e;
     const EmbedArgs emb{d_embd_out ? d_embd : nullptr, d_embd_out, embd_type, embd_m, embd_k};
-    return launch_kernel(L, kFamOther, argmax_final_kernel, dim3(1), dim3(64), d_partial, blocks, n, d_out, d_token, d_pos, d_history, history_len, emb);
+    return launch_kernel(L, kFamOther, argmax_final_kernel, dim3(1), dim3(emb.w ? 256 : 64), d_partial, blocks, n, d_out, d_token, d_pos, d_history, history_len, emb);
 }
 
 hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L, const uint8_t* d_embd, int embd_type,
