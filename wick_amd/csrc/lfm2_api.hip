@@ -343,7 +343,12 @@ int step_graph(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy, wick_rocm_gra
 // One step on the context's stream: a replay of the captured graph, or the same launches enqueued one by one.
 int run_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
     // per-dispatch timing cannot see inside a graph: while it is on, steps are enqueued launch by launch
-    if (!m->use_graph || ctx->timer.enabled) return enqueue_step(ctx, m, greedy);
+    bool timing;
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        timing = ctx->timer.enabled;
+    }
+    if (!m->use_graph || timing) return enqueue_step(ctx, m, greedy);
     wick_rocm_graph* g = nullptr;
     if (int rc = step_graph(ctx, m, greedy, &g)) return rc;
     return wick_rocm_graph_launch(ctx, g);
