@@ -254,3 +254,31 @@ def test_long_prompt_runs_in_passes(ctx, oracle, tmp_path):
     check_step(got, want, ref.min_margin, "long prompt")
     check_step(model.forward(9, 2100), ref.forward(9, 2100, state), ref.min_margin, "step after the long prompt")
     model.free()
+
+
+def test_cpp_host_mirror_runs_the_model(ctx, oracle, tmp_path):
+    """The C++ mirror's RocmLfm2Model (statically linked selftest binary) and this binding drive the same library:
+    same greedy tokens from the same GGUF file, and they are the oracle's."""
+    import os
+    import subprocess
+
+    from conftest import ROOT
+
+    exe = os.path.join(ROOT, "wick_amd", "lib", "host_selftest")
+    assert os.path.exists(exe), "host_selftest has not been built (make -C wick_amd/csrc)"
+    kw = dict(hidden=256, inter=256, vocab=256, seed=26)
+    img, cfg, tensors = lfm2_synth.build(oracle, **kw)
+    path = tmp_path / "model.gguf"
+    path.write_bytes(img)
+    out = subprocess.run([exe, str(path)], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0 and "selftest OK" in out.stdout, out.stdout + out.stderr
+    lines = dict(l.split(":", 1) for l in out.stdout.splitlines() if ":" in l)
+    got = [int(t) for t in lines["tokens"].split()]
+    ref, state, tok, want = L.Lfm2Oracle(cfg, tensors), None, 17, []
+    state = ref.new_state()
+    for pos in range(10):
+        tok = L.argmax(ref.forward(tok, pos, state))
+        want.append(tok)
+    assert got == want
+    a, b = lines["prefill"].split()
+    assert a == b

@@ -9,6 +9,8 @@
 //   quantize_to_scratch / _columns    wick/src/model/lfm2.rs:571-612
 //   gemv_with_preq                    wick/src/backend/cpu.rs:334-354
 //   gemm_preq                         wick/src/model/lfm2.rs:539-565
+//   trait Model (forward / forward_prefill / forward_greedy)   wick/src/model/mod.rs:72-323
+//   load_model_metal                  wick/src/model/mod.rs:385-403
 // Errors become exceptions here (anyhow::Result on the Rust side); contract
 // violations the reference asserts on (null buffers, bad strides) are reported the
 // same way instead of aborting.
@@ -21,6 +23,7 @@
 
 #include "../../include/wick_gguf.h"
 #include "../../include/wick_rocm.h"
+#include "../../include/wick_rocm_lfm2.h"
 
 namespace wick {
 
@@ -155,14 +158,64 @@ public:
 
     wick_rocm_ctx* raw() { return ctx_; }
 
-private:
     void check(int rc) {
         if (rc == 0) return;
         char buf[512] = {0};
         wick_rocm_last_error(ctx_, buf, sizeof buf);
         throw BackendError(rc, buf);
     }
+
+private:
     wick_rocm_ctx* ctx_ = nullptr;
+};
+
+// An LFM2 model on the GPU with the `Model` trait's methods (wick/src/model/mod.rs:72-323); what
+// load_model_metal returns for the Metal backend (wick/src/model/mod.rs:385-403).  Owns weights, KV caches,
+// conv state and scratch; the GGUF file may be closed once the constructor has returned.
+class RocmLfm2Model {
+public:
+    RocmLfm2Model(RocmContext& ctx, const GgufFile& gguf, uint32_t context_size) : ctx_(ctx) {
+        ctx_.check(wick_rocm_lfm2_load(ctx_.raw(), gguf.raw(), context_size, &m_));
+        ctx_.check(wick_rocm_lfm2_get_config(m_, &cfg_));
+    }
+    ~RocmLfm2Model() { wick_rocm_lfm2_free(ctx_.raw(), m_); }
+    RocmLfm2Model(const RocmLfm2Model&) = delete;
+    RocmLfm2Model& operator=(const RocmLfm2Model&) = delete;
+
+    const wick_rocm_lfm2_config& config() const { return cfg_; }
+    size_t gpu_memory_bytes() const { return wick_rocm_lfm2_gpu_memory_bytes(m_); }
+    // A fresh InferenceState.
+    void reset() { ctx_.check(wick_rocm_lfm2_reset(ctx_.raw(), m_)); }
+
+    // forward(tokens = [token], pos) -> logits [vocab_size]
+    std::vector<float> forward(uint32_t token, uint32_t pos) {
+        std::vector<float> logits(cfg_.vocab_size);
+        ctx_.check(wick_rocm_lfm2_forward(ctx_.raw(), m_, token, pos, logits.data()));
+        return logits;
+    }
+    // forward_prefill(tokens, start_pos) -> logits of the last token
+    std::vector<float> forward_prefill(const std::vector<uint32_t>& tokens, uint32_t start_pos) {
+        std::vector<float> logits(cfg_.vocab_size);
+        ctx_.check(wick_rocm_lfm2_forward_prefill(ctx_.raw(), m_, tokens.data(), static_cast<uint32_t>(tokens.size()), start_pos, logits.data()));
+        return logits;
+    }
+    // forward_greedy(tokens = [token], pos) -> next token id, picked on the device
+    uint32_t forward_greedy(uint32_t token, uint32_t pos) {
+        uint32_t next = 0;
+        ctx_.check(wick_rocm_lfm2_forward_greedy(ctx_.raw(), m_, token, pos, &next));
+        return next;
+    }
+    // n greedy steps without a host round trip between them
+    std::vector<uint32_t> generate_greedy(uint32_t token, uint32_t pos, uint32_t n) {
+        std::vector<uint32_t> out(n);
+        ctx_.check(wick_rocm_lfm2_generate_greedy(ctx_.raw(), m_, token, pos, n, out.data()));
+        return out;
+    }
+
+private:
+    RocmContext& ctx_;
+    wick_rocm_lfm2* m_ = nullptr;
+    wick_rocm_lfm2_config cfg_{};
 };
 
 }  // namespace wick

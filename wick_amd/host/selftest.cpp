@@ -7,6 +7,10 @@
 //   * encode_gemv (fused quantize) == quantize_columns + gemv_with_preq, bit for bit;
 //   * error statuses instead of aborts.
 // Prints "selftest OK" and exits 0 on success.
+// With a GGUF file as argument it instead loads that LFM2 model through the mirror's RocmLfm2Model and prints
+//   tokens: <ten greedy picks from token 17 at position 0>
+//   prefill: <argmax of forward_prefill over those picks> <argmax of the same tokens fed one by one>
+// for the caller to compare with another binding of the same library.
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -24,8 +28,47 @@ static uint16_t f32_to_f16(float f) {
     return (uint16_t)r;
 }
 
-int main() {
+static size_t argmax(const std::vector<float>& v) {
+    size_t best = 0;
+    for (size_t i = 1; i < v.size(); i++)
+        if (v[i] >= v[best]) best = i;  // the last of equal maxima, as the reference's cpu_argmax picks
+    return best;
+}
+
+static int model_check(const char* path) {
+    wick::RocmContext ctx(0);
+    std::vector<uint32_t> picks;
+    {
+        wick::GgufFile gguf(path);
+        wick::RocmLfm2Model model(ctx, gguf, 64);
+        if (model.config().vocab_size == 0 || model.gpu_memory_bytes() == 0) return 1;
+        picks = model.generate_greedy(17, 0, 10);
+        std::printf("tokens:");
+        for (uint32_t t : picks) std::printf(" %u", t);
+        std::printf("\n");
+        model.reset();
+        uint32_t tok = 17;
+        for (uint32_t pos = 0; pos < 10; pos++) {
+            tok = model.forward_greedy(tok, pos);
+            if (tok != picks[pos]) { std::printf("forward_greedy differs from generate_greedy at %u\n", pos); return 1; }
+        }
+        model.reset();
+        const size_t a = argmax(model.forward_prefill(picks, 0));
+        model.reset();
+        std::vector<float> logits;
+        for (uint32_t pos = 0; pos < picks.size(); pos++) logits = model.forward(picks[pos], pos);
+        std::printf("prefill: %zu %zu\n", a, argmax(logits));
+        bool threw = false;
+        try { model.forward(model.config().vocab_size, 0); } catch (const wick::BackendError& e) { threw = e.status == WICK_ROCM_ERR_INVALID_ARG; }
+        if (!threw) { std::printf("token out of range not reported\n"); return 1; }
+    }
+    std::printf("selftest OK\n");
+    return 0;
+}
+
+int main(int argc, char** argv) {
     try {
+        if (argc > 1) return model_check(argv[1]);
         wick::RocmContext ctx(0);
         // --- closed form ---------------------------------------------------------
         const uint32_t m = 64, k = 32, n = 4;
