@@ -265,16 +265,17 @@ def trace_lfm2_step(ctx, W, O, tokens=32, context=4096):
     return {"tokens": tokens, "start_pos": 1024, "last_pick": int(picks[-1])}
 
 
-def bench_lfm2_step(ctx, W, O, tokens=64, context=4096):
+def bench_lfm2_step(ctx, W, O, tokens=64, context=4096, body=2, embd=14):
     """Whole decode steps of the model handle (embedding, 16 layers with their norms / conv / attention / gates, tied
     LM head, greedy pick), replayed as one graph per token with token and position resident on the device."""
     from wick_amd import gguf as G
     from wick_amd.lfm2 import RocmLfm2Model
 
-    with G.GgufFile.from_bytes(lfm2_350m_image(O)) as g:
+    with G.GgufFile.from_bytes(lfm2_350m_image(O, body=body, embd=embd)) as g:
         model = RocmLfm2Model(ctx, g, context)
     model.generate_greedy(1, 0, 8)  # captures the graph, warms up
-    out = {"model": "LFM2-350M-shaped, Q4_0 body + Q6_K tied embedding, random init", "context": context,
+    names = {2: "Q4_0", 8: "Q8_0", 14: "Q6_K"}
+    out = {"model": f"LFM2-350M-shaped, {names[body]} body + {names[embd]} tied embedding, random init", "context": context,
            "gpu_memory_MB": model.gpu_memory_bytes() / 1e6, "runs": []}
     for start in (0, 1024, context - tokens):  # attention cost grows with the position
         model.reset()
@@ -454,7 +455,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline decode step (+ CPU baseline)")
-    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | copy | probe | cpu")
+    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | lm_head_q6k | lfm2_step | lfm2_step_q8 | lfm2_step_trace | copy | probe | cpu")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -478,6 +479,7 @@ def main():
             "lm_head": lambda: bench_lm_head_sweep(ctx, W, O),
             "lm_head_q6k": lambda: bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024),
             "lfm2_step": lambda: bench_lfm2_step(ctx, W, O),
+            "lfm2_step_q8": lambda: bench_lfm2_step(ctx, W, O, body=8, embd=8),
             "lfm2_step_trace": lambda: trace_lfm2_step(ctx, W, O),
             "copy": lambda: bench_copy(ctx),
             "probe": lambda: bench_probe(ctx),
