@@ -217,10 +217,11 @@ def bench_single_gemv(ctx, W, O, dtype, m, k, launches=200, wb=None):
             "kernel_us": kus, "kernel_GBps": b / kus / 1e3, "kernel_frac_of_hbm_peak": b / kus / 1e3 / HBM_PEAK_GBS}
 
 
-def lfm2_350m_image(O, body=2, embd=14):
+def lfm2_350m_image(O, body=2, embd=14, HS=HS, IS=IS, KV=KV):
     """A randomly initialised LFM2-350M-shaped model as a GGUF image: 16 layers (gated conv except attention at
     2, 5, 8, 10, 12, 14), hidden 1024, FFN 4608, 16 heads / 8 KV heads, vocabulary 65536, Q4_0 body with the tied
-    embedding in Q6_K like the shipped Q4_0 files (tensor names of wick/src/model/lfm2.rs:97-300)."""
+    embedding in Q6_K like the shipped Q4_0 files (tensor names of wick/src/model/lfm2.rs:97-300).  Other hidden / FFN /
+    KV widths give the other sizes of the family (head_dim stays 64)."""
     from wick_amd import gguf as G
 
     attn = {2, 5, 8, 10, 12, 14}
@@ -265,17 +266,17 @@ def trace_lfm2_step(ctx, W, O, tokens=32, context=4096):
     return {"tokens": tokens, "start_pos": 1024, "last_pick": int(picks[-1])}
 
 
-def bench_lfm2_step(ctx, W, O, tokens=64, context=4096, body=2, embd=14):
+def bench_lfm2_step(ctx, W, O, tokens=64, context=4096, body=2, embd=14, dims=None, label="LFM2-350M-shaped"):
     """Whole decode steps of the model handle (embedding, 16 layers with their norms / conv / attention / gates, tied
     LM head, greedy pick), replayed as one graph per token with token and position resident on the device."""
     from wick_amd import gguf as G
     from wick_amd.lfm2 import RocmLfm2Model
 
-    with G.GgufFile.from_bytes(lfm2_350m_image(O, body=body, embd=embd)) as g:
+    with G.GgufFile.from_bytes(lfm2_350m_image(O, body=body, embd=embd, **(dims or {}))) as g:
         model = RocmLfm2Model(ctx, g, context)
     model.generate_greedy(1, 0, 8)  # captures the graph, warms up
     names = {2: "Q4_0", 8: "Q8_0", 14: "Q6_K"}
-    out = {"model": f"LFM2-350M-shaped, {names[body]} body + {names[embd]} tied embedding, random init", "context": context,
+    out = {"model": f"{label}, {names[body]} body + {names[embd]} tied embedding, random init", "context": context,
            "gpu_memory_MB": model.gpu_memory_bytes() / 1e6, "runs": []}
     for start in (0, 1024, context - tokens):  # attention cost grows with the position
         model.reset()
@@ -455,7 +456,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline decode step (+ CPU baseline)")
-    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | lm_head_q6k | lfm2_step | lfm2_step_q8 | lfm2_step_trace | copy | probe | cpu")
+    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | lm_head_q6k | lfm2_step | lfm2_step_q8 | lfm2_step_1p2b | lfm2_step_trace | copy | probe | cpu")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -480,6 +481,8 @@ def main():
             "lm_head_q6k": lambda: bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024),
             "lfm2_step": lambda: bench_lfm2_step(ctx, W, O),
             "lfm2_step_q8": lambda: bench_lfm2_step(ctx, W, O, body=8, embd=8),
+            # the per-layer shapes of BASELINE's LFM2-1.2B call sites: hidden 2048, FFN 6912, 32 heads / 8 KV heads
+            "lfm2_step_1p2b": lambda: bench_lfm2_step(ctx, W, O, dims=dict(HS=2048, IS=6912, KV=512), label="LFM2-1.2B-shaped"),
             "lfm2_step_trace": lambda: trace_lfm2_step(ctx, W, O),
             "copy": lambda: bench_copy(ctx),
             "probe": lambda: bench_probe(ctx),
