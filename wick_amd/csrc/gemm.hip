@@ -617,6 +617,7 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0) {
     // 512 resident workgroup slots (2 per CU) empty with the wide tile: twice the tiles.
     const bool narrow = a.n <= BN_NARROW || a.row_tiles * ((a.n + BN - 1) / BN) <= 256;
     a.tok_tiles = narrow ? (a.n + BN_NARROW - 1) / BN_NARROW : (a.n + BN - 1) / BN;
+    if ((uint64_t)a.row_tiles * a.tok_tiles > 0x7fffff00ull) return hipErrorInvalidValue;  // beyond a launch's grid
     const uint32_t tiles = a.row_tiles * a.tok_tiles;
     const uint32_t blocks = ((tiles + 7u) / 8u) * 8u;  // every XCD gets the same number of slots
     if (narrow) {
