@@ -423,6 +423,22 @@ def bench_copy(ctx, nbytes=256 << 20, reps=10):
     return {"bytes": nbytes, "ms": ms, "GBps_read_plus_write": 2 * nbytes / ms / 1e6}
 
 
+def bench_upload(ctx, nbytes=256 << 20, reps=3):
+    """Host -> device rate of wick_rocm_upload from ordinary (pageable) host memory: what loading a model's weights costs
+    once; no step of the path crosses PCIe afterwards."""
+    host = np.ones(nbytes, np.uint8)
+    d = ctx.alloc(nbytes)
+    d.upload(host)
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        d.upload(host)
+    ctx.sync()
+    dt = (time.perf_counter() - t0) / reps
+    d.free()
+    return {"bytes": nbytes, "ms": dt * 1e3, "GBps": nbytes / dt / 1e9}
+
+
 def cpu_baseline(O, dtype, host_weights, budget_s=12.0):
     """The reference's x86 path for the same step: per call site a serial f32 GEMV
     (wick/src/backend/cpu.rs:293-306; Q8_0 rows would be chunked over threads).  Runs
@@ -456,7 +472,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline decode step (+ CPU baseline)")
-    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | lm_head_q6k | lfm2_step | lfm2_step_q8 | lfm2_step_1p2b | lfm2_step_trace | copy | probe | cpu")
+    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | lm_head_q6k | upload | lfm2_step | lfm2_step_q8 | lfm2_step_1p2b | lfm2_step_trace | copy | probe | cpu")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -485,6 +501,7 @@ def main():
             "lfm2_step_1p2b": lambda: bench_lfm2_step(ctx, W, O, dims=dict(HS=2048, IS=6912, KV=512), label="LFM2-1.2B-shaped"),
             "lfm2_step_trace": lambda: trace_lfm2_step(ctx, W, O),
             "copy": lambda: bench_copy(ctx),
+            "upload": lambda: bench_upload(ctx),
             "probe": lambda: bench_probe(ctx),
         }
         if leg not in one:
