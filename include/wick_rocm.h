@@ -232,11 +232,17 @@ int wick_rocm_reserve_scratch(wick_rocm_ctx *ctx, uint32_t max_n, uint32_t max_k
 
 /* ---- parity hook ----------------------------------------------------------
  * The exact per-block i32 dots the kernels scale and accumulate
- * (wick/src/backend/simd.rs:369-383, 478-492): d_out[(j*m + i)*(k/32) + b].
+ * (wick/src/backend/simd.rs:369-383, 478-492): d_out[(j*m + i)*(k/32) + b], written by the product kernel
+ * that a wick_rocm_gemm_q8 call of the same weight, n and tuning knobs would run (decode GEMV, multi-token GEMV
+ * or int8-MFMA GEMM) with the scaling replaced by a store.
  * For Q6_K weights: the i32 dot of every 16-weight group (wick/src/backend/simd.rs:583-630),
  * d_out[(j*m + i)*(k/16) + g]. */
 int wick_rocm_block_dots_i32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_t *d_quants, uint32_t n,
                              int32_t *d_out);
+/* The same dots as the fused decode GEMV sees them: one f32 activation vector (16-byte aligned) quantized to Q8_0
+ * INSIDE the GEMV kernel (quantize_f32_to_q8_0_neon, wick/src/backend/simd.rs:255-323, then the block dots above),
+ * d_out[i*(k/32) + b].  Only shapes the fused kernel takes (even block count per row, k <= 8192); Q4_0 / Q8_0. */
+int wick_rocm_block_dots_f32_i32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const float *d_x, int32_t *d_out);
 
 /* ---- one submission per token -------------------------------------------
  * The reference's GPU backends encode a whole token into one command buffer and

@@ -145,6 +145,12 @@ int wick_rocm_lfm2_forward(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t t
  * single steps would (up to the rounding of GEMM against GEMV sums) and returns the logits of the LAST token. */
 int wick_rocm_lfm2_forward_prefill(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, const uint32_t *tokens, uint32_t n, uint32_t start_pos,
                                    float *logits);
+/* Model::forward_prefill_chunked (wick/src/model/mod.rs:111-140): the prompt in chunks of `ubatch` tokens (0 = one chunk),
+ * each a wick_rocm_lfm2_forward_prefill of its own; `cancel` (may be null) is read after every chunk and a non-zero value
+ * stops the call there.  *consumed = tokens that made it into the state (0 < consumed <= n for n > 0; 0 and no logits for an
+ * empty prompt); `logits` (may be null) are those of the last processed chunk. */
+int wick_rocm_lfm2_forward_prefill_chunked(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, const uint32_t *tokens, uint32_t n, uint32_t start_pos,
+                                           uint32_t ubatch, const volatile int32_t *cancel, uint32_t *consumed, float *logits);
 /* Model::forward_greedy (wick/src/model/metal_lfm2.rs:2151-2200): same step, the pick is made on the device. */
 int wick_rocm_lfm2_forward_greedy(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t token, uint32_t pos, uint32_t *next_token);
 /* n greedy steps starting with `token` at `pos`, without a host round trip between steps: out_tokens[i] is the

@@ -37,6 +37,10 @@
 #include <string.h>
 
 #define ORC_API __attribute__((visibility("default")))
+/* Rows are independent (the reference itself hands row chunks to a thread pool, par_rows,
+ * wick/src/backend/cpu.rs:222-234), so the row loops may run on several threads without
+ * changing any result. */
+#define ORC_PAR_ROWS _Pragma("omp parallel for schedule(static)")
 
 enum { Q4_0_BLOCK_BYTES = 18, Q8_0_BLOCK_BYTES = 34, QK = 32 };
 enum { ORC_Q4_0 = 2, ORC_Q8_0 = 8 }; /* ggml type ids, wick/src/gguf.rs:36-51 */
@@ -268,6 +272,7 @@ ORC_API int orc_gemv_q8(int ggml_type, const uint8_t *a, const float *x_scales,
     int bb = block_bytes_of(ggml_type);
     if (!bb || k % QK) return -1;
     int64_t nb = k / QK;
+    ORC_PAR_ROWS
     for (int64_t i = 0; i < m; i++)
         y[i] = row_dot_neon_order(ggml_type, a + i * nb * bb, x_scales, x_quants, nb);
     return 0;
@@ -278,6 +283,7 @@ ORC_API int orc_gemv_q8_f64(int ggml_type, const uint8_t *a, const float *x_scal
     int bb = block_bytes_of(ggml_type);
     if (!bb || k % QK) return -1;
     int64_t nb = k / QK;
+    ORC_PAR_ROWS
     for (int64_t i = 0; i < m; i++)
         y[i] = row_dot_f64(ggml_type, a + i * nb * bb, x_scales, x_quants, nb);
     return 0;
@@ -291,6 +297,7 @@ ORC_API int orc_gemm_q8(int ggml_type, const uint8_t *a, const float *b_scales,
     int bb = block_bytes_of(ggml_type);
     if (!bb || k % QK) return -1;
     int64_t nb = k / QK;
+    ORC_PAR_ROWS
     for (int64_t i = 0; i < m; i++)
         for (int64_t j = 0; j < n; j++)
             out[i * n + j] =
@@ -303,6 +310,7 @@ ORC_API int orc_gemm_q8_f64(int ggml_type, const uint8_t *a, const float *b_scal
     int bb = block_bytes_of(ggml_type);
     if (!bb || k % QK) return -1;
     int64_t nb = k / QK;
+    ORC_PAR_ROWS
     for (int64_t i = 0; i < m; i++)
         for (int64_t j = 0; j < n; j++)
             out[i * n + j] = row_dot_f64(ggml_type, a + i * nb * bb, b_scales + j * nb, b_quants + j * k, nb);
@@ -424,6 +432,7 @@ ORC_API int orc_gemv_q6k_q8(const uint8_t *a, const float *x_scales, const int8_
                             int64_t m, int64_t k) {
     if (k % Q6K_SUPER) return -1;
     int64_t nbk = k / Q6K_SUPER;
+    ORC_PAR_ROWS
     for (int64_t i = 0; i < m; i++) {
         volatile float sumf = 0.0f;
         for (int64_t b = 0; b < nbk; b++) {
@@ -451,6 +460,7 @@ ORC_API int orc_gemv_q6k_q8_f64(const uint8_t *a, const float *x_scales, const i
                                 int64_t m, int64_t k) {
     if (k % Q6K_SUPER) return -1;
     int64_t nbk = k / Q6K_SUPER;
+    ORC_PAR_ROWS
     for (int64_t i = 0; i < m; i++) {
         double acc = 0.0;
         for (int64_t b = 0; b < nbk; b++) {
@@ -472,6 +482,7 @@ ORC_API int orc_gemv_q6k_q8_f64(const uint8_t *a, const float *x_scales, const i
  * q = clamp(round(w / (d * scales[g])), -32, 31) + 32. */
 ORC_API void orc_build_q6_k_matrix(const float *values, int64_t m, int64_t k, uint8_t *bytes) {
     int64_t nbk = k / Q6K_SUPER;
+    ORC_PAR_ROWS
     for (int64_t i = 0; i < m; i++)
         for (int64_t b = 0; b < nbk; b++) {
             const float *w = values + i * k + b * Q6K_SUPER;

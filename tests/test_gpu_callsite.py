@@ -252,3 +252,45 @@ def test_gate_and_up_with_the_gate_applied(ctx, oracle, dtype, m, k, norm):
     _close_unless_tie(act, xn, L.silu_mul(L.gemv(dtype, wg, xn, m, k), L.gemv(dtype, wu, xn, m, k)), f"gate_up {dtype} {m}x{k}")
     for b in (hg, hu, d_x, d_nw, d_act, d_g, d_u):
         b.free()
+
+
+def test_a_graph_that_used_the_scratch_goes_stale_when_it_regrows(ctx, oracle):
+    """A captured graph holds the scratch addresses of its launches.  Growing the scratch afterwards frees them, so the
+    graph must refuse to launch (and say why) instead of touching freed memory; graphs that never used the scratch, and
+    graphs captured after the regrow, launch normally."""
+    m, k = 64, 2080  # odd block count: the fused kernel does not take it, so the call quantizes into the context's scratch
+    wb = oracle.synth_weight(W.Q4_0, m, k, 9)
+    w = ctx.upload_weight(wb, W.Q4_0, m, k)
+    x = oracle.fill_normal(2, 1.0, k)
+    d_x, d_y = ctx.to_device(x), ctx.alloc(m * 4)
+    ctx.reserve_scratch(1, 2080)
+    ctx.graph_begin()
+    ctx.encode_gemv(w, d_x, 0, d_y, 0)
+    g_scratch = ctx.graph_end()
+    w2 = ctx.upload_weight(oracle.synth_weight(W.Q4_0, m, 1024, 9), W.Q4_0, m, 1024)
+    d_x2, d_y2 = ctx.to_device(oracle.fill_normal(3, 1.0, 1024)), ctx.alloc(m * 4)
+    ctx.graph_begin()
+    ctx.encode_gemv(w2, d_x2, 0, d_y2, 0)  # fused quantizer: no scratch
+    g_plain = ctx.graph_end()
+    ctx.graph_launch(g_scratch), ctx.graph_launch(g_plain)
+    s, q = oracle.quantize_q8_0(x)
+    assert_f32_parity(d_y.download(np.float32, m), oracle.gemv_q8(W.Q4_0, wb, s, q, m, k), "graph through scratch")
+    # regrow: far more columns than anything before on this context
+    wide = ctx.upload_weight(oracle.synth_weight(W.Q8_0, 32, 8192, 4), W.Q8_0, 32, 8192)
+    d_xw, d_yw = ctx.to_device(oracle.fill_normal(5, 1.0, 5000 * 8192)), ctx.alloc(5000 * 32 * 4)
+    ctx.encode_gemm(wide, d_xw, 0, d_yw, 0, 5000, 8192, 32)
+    with pytest.raises(W.RocmError, match="scratch was regrown") as e:
+        ctx.graph_launch(g_scratch)
+    assert e.value.status == -6
+    ctx.graph_launch(g_plain)  # never touched the scratch: still good
+    ctx.graph_begin()
+    ctx.encode_gemv(w, d_x, 0, d_y, 0)
+    g_again = ctx.graph_end()
+    d_y.upload(np.zeros(m, np.float32))
+    ctx.graph_launch(g_again)
+    assert_f32_parity(d_y.download(np.float32, m), oracle.gemv_q8(W.Q4_0, wb, s, q, m, k), "re-captured graph")
+    for g in (g_scratch, g_plain, g_again):
+        ctx.graph_destroy(g)
+    for b in (d_x, d_y, d_x2, d_y2, d_xw, d_yw):
+        b.free()
+    w.free(), w2.free(), wide.free()

@@ -116,11 +116,13 @@ STREAM_SHAPES = [(1, 64), (9, 128), (33, 192), (100, 256), (1, 512), (3, 512), (
 def test_gemv_streaming_variant(ctx, oracle, dtype, m, k):
     """Both ways of fetching the weights (per-lane loads, whole-line span loads through LDS)
     give the reference's result, pre-quantized and fused-quantizer entry points alike; the
-    fused and the pre-quantized launch of one policy agree bit for bit."""
+    fused and the pre-quantized launch of one policy agree bit for bit, and the parity hook of each
+    (the same kernel with the scaling replaced by a store) writes the oracle's i32 block dots."""
     with Problem(ctx, oracle, dtype, m, k, seed=5 * m + k + dtype) as p:
         ref = oracle.gemv_q8(dtype, p.wb, p.s[0], p.q[0], m, k)
         d_x = p.to_device(p.x)
-        d_y, d_yf = p.alloc(m * 4), p.alloc(m * 4)
+        d_y, d_yf, d_d = p.alloc(m * 4), p.alloc(m * 4), p.alloc(m * (k // 32) * 4)
+        want_dots = oracle.block_dots_i32(dtype, p.wb, p.q, m, 1, k)
         try:
             for direct_max in (1 << 62, 0):
                 ctx.set_gemv_policy(direct_max)
@@ -131,6 +133,16 @@ def test_gemv_streaming_variant(ctx, oracle, dtype, m, k):
                 y, yf = d_y.download(np.float32, m), d_yf.download(np.float32, m)
                 assert_f32_parity(y, ref, f"gemv direct_max={direct_max} {dtype} {m}x{k}")
                 assert np.array_equal(y, yf), "fused quantizer differs from pre-quantized launch"
+                # the raw i32 block dots of THESE kernels (same fetch mode, pre-quantized and fused quantizer), bit for bit
+                for fused in (False, True):
+                    if fused and (k // 32) % 2:
+                        continue  # odd block counts never take the fused kernel
+                    d_d.upload(np.full(m * (k // 32), -1, np.int32))
+                    if fused:
+                        ctx.block_dots_f32_i32(p.w, d_x, d_d)
+                    else:
+                        ctx.block_dots_i32(p.w, p.d_q, 1, d_d)
+                    assert np.array_equal(d_d.download(np.int32, m * (k // 32)).reshape(1, m, -1), want_dots), f"block dots, fused={fused}, direct_max={direct_max}"
         finally:
             ctx.set_gemv_policy(-1)
 
@@ -148,3 +160,26 @@ def test_gemv_streaming_accumulate(ctx, oracle, dtype):
             ctx.set_gemv_policy(-1)
         ref = y0 + oracle.gemv_q8(dtype, p.wb, p.s[0], p.q[0], m, k)
         assert_f32_parity(d_y.download(np.float32, m), ref, "streaming gemv accumulate")
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+def test_block_dots_through_the_product_kernel_at_full_size(ctx, oracle, dtype):
+    """6912 x 2048 (the LFM2-1.2B ffn_up decode shape): the i32 block dots written by the GEMV kernel itself, in the
+    fetch mode the library picks for this size and in the other one, pre-quantized and with the in-kernel quantizer."""
+    m, k = 6912, 2048
+    with Problem(ctx, oracle, dtype, m, k, seed=1234) as p:
+        want = oracle.block_dots_i32(dtype, p.wb, p.q, m, 1, k)
+        d_x, d_d = p.to_device(p.x), p.alloc(m * (k // 32) * 4)
+        try:
+            for policy in (-1, 1 << 62, 0):
+                ctx.set_gemv_policy(policy)
+                for fused in (False, True):
+                    d_d.upload(np.full(m * (k // 32), -1, np.int32))
+                    ctx.block_dots_f32_i32(p.w, d_x, d_d) if fused else ctx.block_dots_i32(p.w, p.d_q, 1, d_d)
+                    assert np.array_equal(d_d.download(np.int32, m * (k // 32)).reshape(1, m, -1), want), (policy, fused)
+        finally:
+            ctx.set_gemv_policy(-1)
+    with Problem(ctx, oracle, W.Q6_K, 8, 256) as p6:
+        with pytest.raises(W.RocmError) as e:
+            ctx.block_dots_f32_i32(p6.w, p6.d_q, p6.d_q)
+        assert e.value.status == -2

@@ -22,10 +22,12 @@ int check_weight(wick_rocm_ctx* ctx, const wick_rocm_weight* w) {
 }
 
 int ensure_scratch(wick_rocm_ctx* ctx, size_t q_bytes, size_t s_floats, size_t f_floats = 0) {
+    if (ctx->capturing) ctx->capture_used_scratch = true;  // the graph being captured will hold these addresses
     if (q_bytes <= ctx->scratch_q_cap && s_floats <= ctx->scratch_s_cap && f_floats <= ctx->scratch_f_cap) return WICK_ROCM_OK;
     if (ctx->capturing)
         return fail(ctx, WICK_ROCM_ERR_STATE, "activation scratch too small during graph capture; call wick_rocm_reserve_scratch first");
     WR_HIP(ctx, hipStreamSynchronize(ctx->stream));  // earlier launches may still read the old scratch
+    ctx->scratch_gen++;  // graphs captured against the old buffers are stale from here on (wick_rocm_graph_launch refuses them)
     if (q_bytes > ctx->scratch_q_cap) {
         if (ctx->scratch_q) WR_HIP(ctx, hipFree(ctx->scratch_q));
         ctx->scratch_q = nullptr, ctx->scratch_q_cap = 0;
@@ -145,14 +147,14 @@ void wick_rocm_ctx_destroy(wick_rocm_ctx* ctx) {
 
 int wick_rocm_last_error(wick_rocm_ctx* ctx, char* buf, size_t buf_len) {
     if (!ctx || !buf || buf_len == 0) return WICK_ROCM_ERR_INVALID_ARG;
-    std::lock_guard<std::mutex> lk(ctx->mu);
+    std::lock_guard<std::recursive_mutex> lk(ctx->mu);
     std::snprintf(buf, buf_len, "%s", ctx->err.c_str());
     return WICK_ROCM_OK;
 }
 
 int wick_rocm_device_info(wick_rocm_ctx* ctx, char* name_buf, size_t name_len, int* compute_units, size_t* hbm_bytes) {
     if (!ctx) return WICK_ROCM_ERR_INVALID_ARG;
-    std::lock_guard<std::mutex> lk(ctx->mu);
+    std::lock_guard<std::recursive_mutex> lk(ctx->mu);
     if (name_buf && name_len) std::snprintf(name_buf, name_len, "%s", ctx->name.c_str());
     if (compute_units) *compute_units = ctx->num_cus;
     if (hbm_bytes) *hbm_bytes = ctx->hbm_bytes;
@@ -274,7 +276,7 @@ int wick_rocm_weight_upload(wick_rocm_ctx* ctx, const void* host_blocks, size_t 
 }
 
 int wick_rocm_weight_from_gguf(wick_rocm_ctx* ctx, const wick_gguf* gguf, const char* tensor_name, wick_rocm_weight** out) {
-    if (!ctx) return WICK_ROCM_ERR_INVALID_ARG;
+    WR_ENTER(ctx);
     if (!gguf || !tensor_name || !out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "weight_from_gguf: null argument");
     uint64_t offset = 0, rows = 0, cols = 0;
     int type = 0;
@@ -584,9 +586,22 @@ int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, cons
     }
     const bool mfma = n >= ctx->gemm_min_n && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
     hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch())
-                        : launch_block_dots_dot4(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch());
+                        : launch_block_dots_gemv(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->num_cus, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "block_dots launch");
     return WICK_ROCM_OK;
+}
+
+int wick_rocm_block_dots_f32_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const float* d_x, int32_t* d_out) {
+    WR_ENTER(ctx);
+    if (int rc = check_weight(ctx, w)) return rc;
+    if (!d_x || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "block_dots_f32: null device pointer");
+    if (w->type == kTypeQ6_K) return fail(ctx, WICK_ROCM_ERR_UNSUPPORTED_DTYPE, "block_dots_f32: Q6_K has no fused-quantizer kernel");
+    GemvBatch b{};
+    b.w[0] = static_cast<const uint8_t*>(w->d), b.row_end[0] = w->m, b.count = 1;
+    if (!pairs_kernel_applies(b, w->k) || reinterpret_cast<uintptr_t>(d_x) % 16u != 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "block_dots_f32: shape not taken by the fused kernel (odd block count, k > 8192 or x not 16-byte aligned)");
+    hipError_t e = launch_block_dots_gemv_f32(w->type, b.w[0], w->m, w->k, d_x, d_out, ctx->num_cus, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "block_dots_f32 launch");
 }
 
 int wick_rocm_graph_begin(wick_rocm_ctx* ctx) {
@@ -595,6 +610,7 @@ int wick_rocm_graph_begin(wick_rocm_ctx* ctx) {
     if (ctx->timer.enabled) return fail(ctx, WICK_ROCM_ERR_STATE, "graph_begin: kernel timing is on");
     WR_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     ctx->capturing = true;
+    ctx->capture_used_scratch = false;
     return WICK_ROCM_OK;
 }
 
@@ -603,16 +619,26 @@ int wick_rocm_graph_end(wick_rocm_ctx* ctx, wick_rocm_graph** out) {
     if (!out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "graph_end: null out pointer");
     *out = nullptr;
     if (!ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "graph_end: no capture in progress");
+    // the capture ends whatever happens next, so that no failure leaves the stream capturing
     ctx->capturing = false;
-    wick_rocm_graph* g = new (std::nothrow) wick_rocm_graph();
-    if (!g) return fail(ctx, WICK_ROCM_ERR_HIP, "out of host memory");
-    hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
-    if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    wick_rocm_graph* g = e == hipSuccess ? new (std::nothrow) wick_rocm_graph() : nullptr;
+    if (e == hipSuccess && !g) {
+        (void)hipGraphDestroy(graph);
+        return fail(ctx, WICK_ROCM_ERR_HIP, "out of host memory");
+    }
+    if (e == hipSuccess) {
+        g->graph = graph;
+        e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    }
     if (e != hipSuccess) {
-        if (g->graph) (void)hipGraphDestroy(g->graph);
+        if (graph) (void)hipGraphDestroy(graph);
         delete g;
         return fail_hip(ctx, e, "graph_end");
     }
+    g->uses_scratch = ctx->capture_used_scratch;
+    g->scratch_gen = ctx->scratch_gen;
     *out = g;
     return WICK_ROCM_OK;
 }
@@ -621,6 +647,9 @@ int wick_rocm_graph_launch(wick_rocm_ctx* ctx, wick_rocm_graph* g) {
     WR_ENTER(ctx);
     if (!g || !g->exec) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "graph_launch: null graph");
     if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "graph_launch during capture");
+    if (graph_is_stale(ctx, g))
+        return fail(ctx, WICK_ROCM_ERR_STATE, "graph_launch: the context's scratch was regrown after this graph was captured (it holds freed addresses); "
+                                              "capture it again, and size the scratch with wick_rocm_reserve_scratch before capturing");
     WR_HIP(ctx, hipGraphLaunch(g->exec, ctx->stream));
     return WICK_ROCM_OK;
 }

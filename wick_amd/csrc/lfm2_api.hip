@@ -1,7 +1,7 @@
 // C ABI of include/wick_rocm_lfm2.h: the decode step's non-matmul operations as entry points, and the
 // LFM2 model handle (weights, KV caches, conv state, scratch, one captured graph per kind of step).
-// Host code only.  The model is a composition of public entry points (it holds its own lock, like the
-// reference's infer_lock, and never the context's).
+// Host code only.  The model is a composition of public entry points; a step, a prompt pass or a capture holds the
+// model's own lock (the reference's infer_lock) and the context's (recursive) lock from start to end.
 #include "../../include/wick_rocm_lfm2.h"
 
 #include <cmath>
@@ -217,7 +217,7 @@ struct wick_rocm_lfm2 {
 namespace {
 
 int ctx_fail(wick_rocm_ctx* ctx, int code, const std::string& what) {
-    std::lock_guard<std::mutex> lk(ctx->mu);
+    std::lock_guard<std::recursive_mutex> lk(ctx->mu);
     return fail(ctx, code, what.c_str());
 }
 
@@ -316,7 +316,7 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
     if (rc) return rc;
     if ((rc = gemv_normed(ctx, {m->embd}, {m->logits}, m->hidden, m->out_norm, c.rms_norm_eps))) return rc;
     if (!greedy) return WICK_ROCM_OK;
-    std::lock_guard<std::mutex> lk(ctx->mu);
+    std::lock_guard<std::recursive_mutex> lk(ctx->mu);
     hipError_t e = launch_argmax(m->logits, c.vocab_size, m->d_argmax_partial, m->d_pick, m->d_token, m->d_pos, m->d_history, c.max_seq_len,
                                  ctx->launch(), static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m, c.hidden_size, m->hidden);
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
@@ -324,6 +324,10 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
 
 int step_graph(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy, wick_rocm_graph** out) {
     wick_rocm_graph*& g = greedy ? m->g_greedy : m->g_logits;
+    if (g && graph_is_stale(ctx, g)) {  // the context's scratch moved since the capture (another model, a wider matmul): capture again
+        wick_rocm_graph_destroy(ctx, g);
+        g = nullptr;
+    }
     if (!g) {
         if (int rc = wick_rocm_graph_begin(ctx)) return rc;
         const int rc = enqueue_step(ctx, m, greedy);
@@ -345,7 +349,7 @@ int run_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
     // per-dispatch timing cannot see inside a graph: while it is on, steps are enqueued launch by launch
     bool timing;
     {
-        std::lock_guard<std::mutex> lk(ctx->mu);
+        std::lock_guard<std::recursive_mutex> lk(ctx->mu);
         timing = ctx->timer.enabled;
     }
     if (!m->use_graph || timing) return enqueue_step(ctx, m, greedy);
@@ -399,7 +403,7 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
     const uint32_t hs = c.hidden_size, hd = hs / c.n_heads, inter = c.intermediate_size;
     const float scale = 1.0f / sqrtf((float)hd);
     auto locked = [&](auto&& launch, const char* what) {
-        std::lock_guard<std::mutex> lk(ctx->mu);
+        std::lock_guard<std::recursive_mutex> lk(ctx->mu);
         const hipError_t e = launch();
         return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, what);
     };
@@ -445,7 +449,7 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
 }
 
 int set_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t token, uint32_t pos) {
-    std::lock_guard<std::mutex> lk(ctx->mu);
+    std::lock_guard<std::recursive_mutex> lk(ctx->mu);
     hipError_t e = launch_set_step(m->d_token, token, m->d_pos, pos, ctx->launch(), static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m,
                                    m->cfg.hidden_size, m->hidden);
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "set_step launch");
@@ -585,6 +589,7 @@ size_t wick_rocm_lfm2_gpu_memory_bytes(const wick_rocm_lfm2* model) { return mod
 int wick_rocm_lfm2_reset(wick_rocm_ctx* ctx, wick_rocm_lfm2* model) {
     if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
     std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);  // nothing else gets onto the context's stream (or into a capture) in between
     const size_t state_floats = (size_t)(model->cfg.conv_kernel_size - 1) * model->cfg.hidden_size;
     if (state_floats) {
         const std::vector<float> zeros(state_floats, 0.0f);
@@ -605,6 +610,7 @@ int wick_rocm_lfm2_set_graph_replay(wick_rocm_lfm2* model, int enabled) {
 int wick_rocm_lfm2_forward(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t token, uint32_t pos, float* logits) {
     if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
     std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);  // nothing else gets onto the context's stream (or into a capture) in between
     if (int rc = check_step(ctx, model, token, pos, 1)) return rc;
     if (int rc = set_step(ctx, model, token, pos)) return rc;
     if (int rc = run_step(ctx, model, false)) return rc;
@@ -616,6 +622,7 @@ int wick_rocm_lfm2_forward_prefill(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, co
     if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
     if (!tokens || n == 0) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 prefill: empty prompt");
     std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);  // nothing else gets onto the context's stream (or into a capture) in between
     const wick_rocm_lfm2_config& c = model->cfg;
     for (uint32_t j = 0; j < n; j++)
         if (tokens[j] >= c.vocab_size) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: token_id out of range");
@@ -634,6 +641,24 @@ int wick_rocm_lfm2_forward_prefill(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, co
     return wick_rocm_sync(ctx);
 }
 
+int wick_rocm_lfm2_forward_prefill_chunked(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
+                                           uint32_t ubatch, const volatile int32_t* cancel, uint32_t* consumed, float* logits) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    if (!consumed) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 prefill: null consumed pointer");
+    *consumed = 0;
+    if (n == 0) return WICK_ROCM_OK;  // the reference's (0, None)
+    if (!tokens) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 prefill: null token pointer");
+    const uint32_t step = ubatch == 0 ? n : ubatch;  // 0 = one chunk covering everything
+    while (*consumed < n) {
+        const uint32_t len = n - *consumed < step ? n - *consumed : step;
+        if (int rc = wick_rocm_lfm2_forward_prefill(ctx, model, tokens + *consumed, len, start_pos + *consumed, logits)) return rc;
+        *consumed += len;
+        // looked at AFTER each chunk, so a call always makes progress by at least one chunk
+        if (cancel && __atomic_load_n(cancel, __ATOMIC_RELAXED) != 0) break;
+    }
+    return WICK_ROCM_OK;
+}
+
 int wick_rocm_lfm2_forward_greedy(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t token, uint32_t pos, uint32_t* next_token) {
     return wick_rocm_lfm2_generate_greedy(ctx, model, token, pos, 1, next_token);
 }
@@ -643,6 +668,7 @@ int wick_rocm_lfm2_generate_greedy(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, ui
     if (!out_tokens) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: null output pointer");
     if (n == 0) return WICK_ROCM_OK;
     std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);  // nothing else gets onto the context's stream (or into a capture) in between
     if (int rc = check_step(ctx, model, token, pos, n)) return rc;
     if (int rc = set_step(ctx, model, token, pos)) return rc;
     for (uint32_t i = 0; i < n; i++)  // the pick of step i is written to the device-side token and position pos + i of the history

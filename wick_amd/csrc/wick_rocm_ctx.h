@@ -13,7 +13,9 @@ using namespace wick_rocm;
 struct wick_rocm_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
-    std::mutex mu;  // serialises calls on this context, like the reference's infer_lock
+    // Serialises calls on this context, like the reference's infer_lock.  Recursive: the model handle holds it for a whole
+    // step or capture while it composes public entry points, which take it again.
+    std::recursive_mutex mu;
     std::string err;
     std::string name;
     int num_cus = 0;
@@ -26,6 +28,10 @@ struct wick_rocm_ctx {
     size_t scratch_s_cap = 0;  // floats
     float* scratch_f = nullptr;  // one transformed f32 activation vector (norm / gate folded into a GEMV that cannot take the fused kernel)
     size_t scratch_f_cap = 0;  // floats
+    // A captured graph has the scratch addresses baked in.  Every regrow bumps the generation; a graph that used the
+    // scratch remembers the generation it was captured under and refuses to launch under another one.
+    uint64_t scratch_gen = 0;
+    bool capture_used_scratch = false;
     uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
     KernelTimer timer;
     int64_t gemv_direct_max_bytes = -1;
@@ -44,7 +50,12 @@ struct wick_rocm_weight {
 struct wick_rocm_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    bool uses_scratch = false;  // some captured launch reads or writes the context's scratch
+    uint64_t scratch_gen = 0;   // ... as it was laid out then
 };
+
+// True when the graph refers to scratch memory that has been freed and reallocated since its capture.
+inline bool graph_is_stale(const wick_rocm_ctx* ctx, const wick_rocm_graph* g) { return g->uses_scratch && g->scratch_gen != ctx->scratch_gen; }
 
 struct wick_rocm_event {
     hipEvent_t ev = nullptr;
@@ -71,7 +82,7 @@ inline int fail_hip(wick_rocm_ctx* ctx, hipError_t e, const char* where) {
 
 // Takes the context lock and makes its device current for the calling thread.
 struct Guard {
-    std::unique_lock<std::mutex> lk;
+    std::unique_lock<std::recursive_mutex> lk;
     hipError_t status;
     explicit Guard(wick_rocm_ctx* ctx) : lk(ctx->mu), status(hipSetDevice(ctx->device)) {}
 };

@@ -113,7 +113,7 @@ hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t
                               const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
                               int accumulate, int num_cus, const Launch& L);
 
-// int8-MFMA GEMM.  Requires k % 256 == 0.
+// int8-MFMA GEMM.  Requires k % 128 == 0.
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                             const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
                             int accumulate, const Launch& L);
@@ -121,14 +121,17 @@ hipError_t launch_gemm_mfma_multi(int type, const uint8_t* const* d_w, const uin
                                   const float* d_scales, uint32_t n, float* const* d_y, uint32_t y_stride, int y_layout, int accumulate,
                                   const Launch& L);
 
-// Per-block i32 dots, out[(j*m + i)*nb + b], through the same unpack + v_dot4 code
-// as the GEMV, or through the GEMM's loads / LDS layout / MFMA (k % 256 == 0).
+// Per-block i32 dots, out[(j*m + i)*nb + b], through the GEMM's loads / LDS layout / MFMA (k % 128 == 0).
 // Register-only instruction-rate probes (probe.hip): shape 0 = v_mfma_i32_32x32x32_i8, 1 = v_mfma_i32_16x16x32_i8,
 // 2 = v_fma_f32.
 hipError_t launch_probe(int shape, uint32_t iters, int num_cus, int* d_sink, double* ops, const Launch& L);
 
-hipError_t launch_block_dots_dot4(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,
-                                  int32_t* d_out, const Launch& L);
+// The same through the decode GEMV's own kernels (gemv_dump.hip): every fetch mode, token count and the fused
+// in-kernel quantizer, exactly as a product launch of that shape would run them.
+hipError_t launch_block_dots_gemv(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n, int32_t* d_out,
+                                  int num_cus, const Launch& L);
+hipError_t launch_block_dots_gemv_f32(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const float* d_x, int32_t* d_out, int num_cus,
+                                      const Launch& L);
 hipError_t launch_block_dots_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n,
                                   int32_t* d_out, const Launch& L);
 
@@ -182,7 +185,7 @@ hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, u
                            int embd_type = 0, uint32_t embd_m = 0, uint32_t embd_k = 0, float* d_embd_out = nullptr);
 hipError_t launch_advance_pos(uint32_t* d_pos, const Launch& L);
 
-// n at and above which gemm_q8 uses the MFMA kernel (when k % 256 == 0).
+// n at and above which gemm_q8 uses the MFMA kernel (when k % 128 == 0).
 constexpr uint32_t kGemmMinN = 16;  // cf. GEMM_MIN_N, wick/src/model/metal_lfm2.rs:18-21
 
 }  // namespace wick_rocm

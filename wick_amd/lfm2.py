@@ -47,6 +47,7 @@ _SIGNATURES = {
     "wick_rocm_lfm2_set_graph_replay": (C.c_int, [_P, C.c_int]),
     "wick_rocm_lfm2_forward": (C.c_int, [_P, _P, _U32, _U32, _P]),
     "wick_rocm_lfm2_forward_prefill": (C.c_int, [_P, _P, _P, _U32, _U32, _P]),
+    "wick_rocm_lfm2_forward_prefill_chunked": (C.c_int, [_P, _P, _P, _U32, _U32, _U32, _P, C.POINTER(_U32), _P]),
     "wick_rocm_lfm2_forward_greedy": (C.c_int, [_P, _P, _U32, _U32, C.POINTER(_U32)]),
     "wick_rocm_lfm2_generate_greedy": (C.c_int, [_P, _P, _U32, _U32, _U32, _P]),
     "wick_rocm_lfm2_logits_device": (_P, [_P]),
@@ -182,6 +183,17 @@ class RocmLfm2Model:
         logits = np.empty(self.config["vocab_size"], np.float32)
         self.ctx._check(self._l.wick_rocm_lfm2_forward_prefill(self.ctx._h, self._h, t.ctypes.data, t.size, start_pos, logits.ctypes.data))
         return logits
+
+    def forward_prefill_chunked(self, tokens, start_pos: int, ubatch: int, cancel=None):
+        """Model::forward_prefill_chunked: (tokens consumed, logits of the last processed chunk or None).  `cancel` is a
+        ctypes.c_int32 another thread may set; it is looked at after every chunk."""
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        logits = np.empty(self.config["vocab_size"], np.float32)
+        consumed = _U32()
+        self.ctx._check(self._l.wick_rocm_lfm2_forward_prefill_chunked(self.ctx._h, self._h, t.ctypes.data, t.size, start_pos, ubatch,
+                                                                       C.addressof(cancel) if cancel is not None else None, C.byref(consumed),
+                                                                       logits.ctypes.data))
+        return consumed.value, (logits if consumed.value else None)
 
     def forward_greedy(self, token: int, pos: int) -> int:
         nxt = _U32()

@@ -92,6 +92,7 @@ _SIGNATURES = {
     "wick_rocm_ffn_gate_up_f32": (C.c_int, [_P, _P, _P, _P, _P, C.c_float, _P]),
     "wick_rocm_reserve_scratch": (C.c_int, [_P, C.c_uint32, C.c_uint32]),
     "wick_rocm_block_dots_i32": (C.c_int, [_P, _P, _P, C.c_uint32, _P]),
+    "wick_rocm_block_dots_f32_i32": (C.c_int, [_P, _P, _P, _P]),
     "wick_rocm_graph_begin": (C.c_int, [_P]),
     "wick_rocm_graph_end": (C.c_int, [_P, C.POINTER(_P)]),
     "wick_rocm_graph_launch": (C.c_int, [_P, _P]),
@@ -288,6 +289,10 @@ class RocmContext:
 
     def block_dots_i32(self, w: RocmWeight, quants, n: int, out) -> None:
         self._check(self._lib.wick_rocm_block_dots_i32(self._h, w.handle, _ptr(quants), n, _ptr(out)))
+
+    def block_dots_f32_i32(self, w: RocmWeight, x, out) -> None:
+        """The block dots of the fused decode GEMV (f32 activation vector quantized inside the kernel)."""
+        self._check(self._lib.wick_rocm_block_dots_f32_i32(self._h, w.handle, _ptr(x), _ptr(out)))
 
     # -- the reference's GPU call-site shape (f32 in, f32 out) -----------------
     def encode_gemv(self, w: RocmWeight, x, x_off_bytes: int, y, y_off_bytes: int, accumulate: bool = False) -> None:
