@@ -191,6 +191,19 @@ int wick_rocm_set_gemv_policy(wick_rocm_ctx *ctx, int64_t direct_max_bytes);
  * Offsets are in bytes like the reference's. */
 int wick_rocm_matmul_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const float *d_x, size_t x_off_bytes, uint32_t n,
                          uint32_t x_stride, float *d_y, size_t y_off_bytes, uint32_t y_stride, int accumulate);
+/* wick_rocm_matmul_f32 for callers that cannot allocate.  It has no counterpart in the reference; it exists for callers
+ * that must not reach hipMalloc / hipFree: code running under HIP graph capture, tight serving loops, harnesses that
+ * forbid allocation.  Same arguments, same kernels and bit-identical results, but the Q8_0-quantized activations go
+ * into a fixed array in device memory that is part of the library's image (4.5 MiB per GPU, held until the process
+ * ends) instead of context scratch that grows on demand.  Limits and rules:
+ *   - n * k <= 4194304 elements (e.g. 2048 tokens x 2048, 512 x 8192); larger calls return WICK_ROCM_ERR_BAD_SHAPE;
+ *   - no hipMalloc, hipFree or other allocating call is made, on any path; with per-dispatch kernel timing on
+ *     (which creates events) the call returns WICK_ROCM_ERR_STATE instead;
+ *   - every call on one GPU uses that GPU's one array, from any context: calls that overlap in time on one GPU race
+ *     (calls on one context's stream are ordered and safe); the array keeps the last call's contents, and nothing in
+ *     it needs clearing, because the quantizer rewrites every byte the matmul reads. */
+int wick_rocm_matmul_f32_noalloc(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const float *d_x, size_t x_off_bytes, uint32_t n,
+                                 uint32_t x_stride, float *d_y, size_t y_off_bytes, uint32_t y_stride, int accumulate);
 /* encode_gemv_qkv / encode_gemv_gate_up (wick/src/model/metal_lfm2.rs:1043-1119):
  * up to four weights sharing k and dtype against ONE f32 activation vector read at
  * d_x + x_off_bytes, y_i (+)= W_i x, in a single launch.  The Q8_0 quantization of x

@@ -156,9 +156,14 @@ class Lfm2Oracle:
     conv_kernel_size, kv_heads_per_layer (0 = gated-conv layer).  `tensors`: GGUF name -> (ggml_type, dims, array),
     quantized weights as raw block bytes (dims [k, m]), norms / conv kernels as float32."""
 
-    def __init__(self, cfg: dict, tensors: dict):
+    def __init__(self, cfg: dict, tensors: dict, jitter_seed=None):
         self.cfg, self.t = cfg, tensors
         self.min_margin = float("inf")  # smallest quantizer_margin over every GEMV input so far
+        # Sensitivity probe: with a seed, every GEMV output is moved by up to 2^-22 of its value (about two ulp), which is
+        # what another order of the f32 block sums does to it -- the order is not part of the contract (rel-L2 1e-5 is).
+        # How far the logits of a jittered run move is how far a correct implementation may sit from this oracle once
+        # activations come near quantizer ties.
+        self.jitter = np.random.default_rng(jitter_seed) if jitter_seed is not None else None
 
     def new_state(self) -> dict:
         c = self.cfg
@@ -174,7 +179,10 @@ class Lfm2Oracle:
     def _gemv(self, name, x):
         gt, dims, data = self.t[name]
         self.min_margin = min(self.min_margin, quantizer_margin(x))
-        return gemv(gt, data, x, dims[1], dims[0])
+        y = gemv(gt, data, x, dims[1], dims[0])
+        if self.jitter is not None:
+            y = (y * (np.float32(1.0) + self.jitter.uniform(-1.0, 1.0, y.size).astype(np.float32) * np.float32(2.0 ** -22))).astype(np.float32)
+        return y
 
     def hidden_after_layers(self, token: int, pos: int, state: dict) -> np.ndarray:
         c = self.cfg

@@ -14,6 +14,14 @@
 #include "wick_rocm_ctx.h"
 #include "../../include/wick_gguf.h"
 
+// Scratch of wick_rocm_matmul_f32_noalloc: the Q8_0-quantized activations (quants, then scales) of one call, in
+// device memory that exists from load time on, one copy per GPU.  `scratch` is a host-side stand-in for the symbol, not a
+// device address: host code only ever uses the address hipGetSymbolAddress returns for the current device
+// (wick_rocm_ctx::noalloc_scratch, looked up in wick_rocm_ctx_create).
+constexpr size_t kNoallocMaxElems = 4u << 20;  // n * k of one call: 4 Mi quants (4 MiB) + 128 Ki scales (512 KiB)
+constexpr size_t kNoallocScratchBytes = kNoallocMaxElems + kNoallocMaxElems / 32 * sizeof(float);
+static __device__ __align__(256) unsigned char scratch[kNoallocScratchBytes];
+
 namespace {
 
 int check_weight(wick_rocm_ctx* ctx, const wick_rocm_weight* w) {
@@ -119,6 +127,14 @@ int wick_rocm_ctx_create(int device_id, wick_rocm_ctx** out) {
         delete ctx;
         return WICK_ROCM_ERR_HIP;
     }
+    // This device's copy of the static scratch array (every GPU has its own, at its own address); the device is current.
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) {
+        (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return WICK_ROCM_ERR_HIP;
+    }
+    ctx->noalloc_scratch = static_cast<unsigned char*>(sym);
     *out = ctx;
     return WICK_ROCM_OK;
 }
@@ -567,6 +583,29 @@ int wick_rocm_matmul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const fl
     if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
     return gemm_locked(ctx, w, ctx->scratch_q, ctx->scratch_s, n, y, n == 1 ? w->m : y_stride,
                        WICK_ROCM_LAYOUT_TOKEN_MAJOR, accumulate);
+}
+
+int wick_rocm_matmul_f32_noalloc(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const float* d_x, size_t x_off_bytes, uint32_t n,
+                                 uint32_t x_stride, float* d_y, size_t y_off_bytes, uint32_t y_stride, int accumulate) {
+    WR_ENTER(ctx);
+    if (int rc = check_weight(ctx, w)) return rc;
+    if (!d_x || !d_y) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "matmul_f32_noalloc: null device pointer");
+    if (n == 0) return WICK_ROCM_OK;
+    if (x_off_bytes % 4u || y_off_bytes % 4u) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "matmul_f32_noalloc: offsets must be multiples of 4");
+    if (n > 1 && (x_stride < w->k || y_stride < w->m))
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "matmul_f32_noalloc: stride smaller than the vector length");
+    if ((uint64_t)n * w->k > kNoallocMaxElems)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "matmul_f32_noalloc: n * k exceeds the static scratch (4194304 elements); use wick_rocm_matmul_f32");
+    if (ctx->timer.enabled) return fail(ctx, WICK_ROCM_ERR_STATE, "matmul_f32_noalloc: per-dispatch kernel timing creates events; switch it off");
+    const float* x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes);
+    float* y = reinterpret_cast<float*>(reinterpret_cast<char*>(d_y) + y_off_bytes);
+    // this device's copy of the static array, never the array's name: quants first, scales behind them
+    int8_t* q = reinterpret_cast<int8_t*>(ctx->noalloc_scratch);
+    float* s = reinterpret_cast<float*>(ctx->noalloc_scratch + kNoallocMaxElems);
+    // Nothing in the scratch has to start at zero: the quantizer writes every byte the matmul reads.
+    hipError_t e = launch_quantize_q8_0(x, n, w->k, n == 1 ? w->k : x_stride, q, s, ctx->launch());
+    if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
+    return gemm_locked(ctx, w, q, s, n, y, n == 1 ? w->m : y_stride, WICK_ROCM_LAYOUT_TOKEN_MAJOR, accumulate);
 }
 
 int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_quants, uint32_t n,

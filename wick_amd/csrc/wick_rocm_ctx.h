@@ -32,6 +32,7 @@ struct wick_rocm_ctx {
     // scratch remembers the generation it was captured under and refuses to launch under another one.
     uint64_t scratch_gen = 0;
     bool capture_used_scratch = false;
+    unsigned char* noalloc_scratch = nullptr;  // this device's address of the static scratch array of wick_rocm_matmul_f32_noalloc
     uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
     KernelTimer timer;
     int64_t gemv_direct_max_bytes = -1;

@@ -86,6 +86,7 @@ _SIGNATURES = {
     "wick_rocm_gemm_q8": (C.c_int, [_P, _P, _P, _P, C.c_uint32, _P, C.c_uint32, C.c_int, C.c_int]),
     "wick_rocm_gemm_q8_multi": (C.c_int, [_P, _P, _P, C.c_uint32, _P, _P, C.c_uint32, C.c_uint32, C.c_int, C.c_int]),
     "wick_rocm_matmul_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_uint32, C.c_uint32, _P, C.c_size_t, C.c_uint32, C.c_int]),
+    "wick_rocm_matmul_f32_noalloc": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_uint32, C.c_uint32, _P, C.c_size_t, C.c_uint32, C.c_int]),
     "wick_rocm_gemv_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, C.c_size_t, C.c_int]),
     "wick_rocm_gemv_rmsnorm_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, _P, C.c_float, C.c_int]),
     "wick_rocm_gemv_silu_mul_f32": (C.c_int, [_P, _P, _P, _P, _P, C.c_int]),
@@ -303,6 +304,12 @@ class RocmContext:
                     accumulate: bool = False) -> None:
         self._check(self._lib.wick_rocm_matmul_f32(self._h, w.handle, _ptr(x), x_off_bytes, n, x_stride, _ptr(y),
                                                    y_off_bytes, y_stride, int(accumulate)))
+
+    def encode_gemm_noalloc(self, w: RocmWeight, x, x_off_bytes: int, y, y_off_bytes: int, n: int, x_stride: int, y_stride: int,
+                            accumulate: bool = False) -> None:
+        """encode_gemm for callers that cannot allocate: quantized activations in the library's static device array."""
+        self._check(self._lib.wick_rocm_matmul_f32_noalloc(self._h, w.handle, _ptr(x), x_off_bytes, n, x_stride, _ptr(y),
+                                                           y_off_bytes, y_stride, int(accumulate)))
 
     def encode_gemv_fused(self, ws: Sequence[RocmWeight], x, x_off_bytes: int, ys, accumulate: bool = False) -> None:
         """encode_gemv_qkv / encode_gemv_gate_up: several weights, one f32 activation, one launch."""
