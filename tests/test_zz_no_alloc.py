@@ -24,7 +24,11 @@ def _both(ctx, oracle, dtype, m, k, n, x_stride, y_stride, seed, accumulate=Fals
     assert not np.array_equal(a, y0)
     # and both are the oracle's result
     s, q = oracle.quantize_q8_0_batch(x, n, k, x_stride)
-    ref = oracle.gemm_q8(dtype, wb, s, q, m, n, k, f64=True) + (y0.reshape(n, y_stride)[:, :m].T if accumulate else 0.0)
+    if dtype == W.Q6_K:  # no batched Q6_K kernel in the reference either: one GEMV per token
+        ref = np.stack([oracle.gemv_q6k_q8(wb, s[j], q[j], m, k) for j in range(n)], axis=1).astype(np.float64)
+    else:
+        ref = oracle.gemm_q8(dtype, wb, s, q, m, n, k, f64=True)
+    ref = ref + (y0.reshape(n, y_stride)[:, :m].T if accumulate else 0.0)
     assert_f32_parity(b.reshape(n, y_stride)[:, :m].T, ref, "no-alloc matmul")
     w.free()
     for buf in (d_x, d_a, d_b):
