@@ -1,25 +1,27 @@
 #!/usr/bin/env python3
 """Benchmark of the block-quantized matmul hot path on one MI355X.
 
-A "step" is one pass of the decode hot path over the LFM2-350M-shaped weight set
-(hidden 1024, 10 short-conv + 6 attention layers, FFN 4608, tied LM head
-65536 x 1024) at n = 1: 93 weight matrices in 65 GEMV launches ({Q,K,V} and
-{gate,up} share one activation and one launch, like the reference's call sites; the
-Q8_0 quantization of the activation runs inside the GEMV kernel), submitted as ONE
-HIP graph per token.  Two distinct device copies of the weight set are alternated
-so every step streams its weights from HBM, not from the 256 MB Infinity Cache.
+Headline (what `value`, `ms_per_step`, `config` and `roofline` describe): the single decode GEMV the HBM target is
+quoted on, Q4_0 6912 x 2048 (LFM2-1.2B ffn_up) against one Q8_0-quantized token.  A "step" is one replay of a HIP graph
+that runs this GEMV once on each of 38 distinct device copies of the weight (303 MB, more than the 256 MB Infinity Cache),
+so every launch streams its 8 MB of weights from HBM.  The launches of a graph are chained on one stream, like the
+GEMVs of a decode step are.  Each replay is bracketed by its own pair of events: mean (= ms_per_step), median, min,
+p10 / p90 over the timed steps are reported.
 
-Prints one JSON line: `value` = algorithmic GEMV bytes per step / step time, plus
-  roofline        the GEMV kernel over the timed steps: algorithmic bytes / summed kernel
-                  execution time (per-dispatch timestamps, the quantity a kernel trace reports)
-  gemm            prefill GEMM leg (Q4_0, m=6912, n=2002, k=2048) with its own roofline
-  gemv_6912x2048  the single-GEMV shape the HBM target is quoted on, HBM-cold
-  decode_step_q8_0, prefill_sites, lm_head_sweep   the other configurations
-  cpu_baseline    the reference's x86 CPU path (f32 per-token GEMV, serial for Q4_0)
-                  timed on this host on a bounded sample of the same step
+Beside it, in the same JSON line:
+  roofline         the GEMV kernel: algorithmic bytes per launch / average launch duration of the timed region
+                   (step time / 38; the kernel runs nowhere else in that region), against 8 TB/s
+  gemv_concurrent  the same launches as INDEPENDENT work on four streams: what the kernel sustains when the gap between
+                   dependent launches is taken out of the picture
+  gemm             the prefill GEMM the matrix-core target is quoted on (Q4_0, m=6912, n=2002, k=2048) with its own
+                   roofline object (per-launch kernel timestamps, median / min over 100 launches)
+  decode_step, decode_step_q8_0, prefill_sites, lm_head_sweep, lm_head_q6_k_65536x1024, lfm2_decode_step
+                   the other configurations (LFM2-350M-shaped decode weight set, the nine LFM2-1.2B prefill call sites at
+                   n = 4096, the 65536 x 2048 head at n = 1 / 4 / 16 / 64, a whole model step)
+  cpu_baseline     the reference's x86 CPU path (f32 per-token GEMV; Q4_0 rows serial, Q8_0 rows over T threads) timed on
+                   this host on bounded samples of the same workloads
 
-`--leg NAME` runs one leg only (used for profiling): decode, decode_q8, gemv, gemm,
-prefill_sites, lm_head, copy, cpu.
+`--leg NAME` runs one leg only (used for profiling; `c1` replays graphs and launches nothing else).
 """
 from __future__ import annotations
 
@@ -137,6 +139,106 @@ def time_graphs(ctx, graphs, steps, warmup):
     ctx.sync()
     ctx.event_destroy(e0), ctx.event_destroy(e1)
     return ms / steps
+
+
+def stats(samples_ms, per=1):
+    """mean / median / min / p10 / p90 of per-step samples, in microseconds per `per` launches."""
+    a = np.asarray(samples_ms, np.float64) * 1e3 / per
+    return {"mean_us": float(a.mean()), "median_us": float(np.median(a)), "min_us": float(a.min()), "p10_us": float(np.percentile(a, 10)),
+            "p90_us": float(np.percentile(a, 90)), "samples": int(a.size)}
+
+
+def time_graph_steps(ctx, graphs, steps, warmup):
+    """Like time_graphs, with an event between consecutive replays: returns (ms per step over the whole timed region,
+    [ms of each step])."""
+    for i in range(warmup):
+        ctx.graph_launch(graphs[i % len(graphs)])
+    ctx.sync()
+    ev = [ctx.event() for _ in range(steps + 1)]
+    ctx.record(ev[0])
+    for i in range(steps):
+        ctx.graph_launch(graphs[i % len(graphs)])
+        ctx.record(ev[i + 1])
+    total = ctx.elapsed_ms(ev[0], ev[steps])
+    each = [ctx.elapsed_ms(ev[i], ev[i + 1]) for i in range(steps)]
+    ctx.sync()
+    for e in ev:
+        ctx.event_destroy(e)
+    return total / steps, each
+
+
+C1 = (6912, 2048)  # LFM2-1.2B ffn_up: the shape the HBM target is quoted on
+
+
+def bench_c1(ctx, W, O, steps, warmup, with_concurrent=True):
+    """Q4_0 6912 x 2048 decode GEMV, HBM-cold: one step = one graph replay = one launch on each of `copies` weight copies."""
+    m, k = C1
+    dtype = W.Q4_0
+    wb = O.synth_weight(dtype, m, k, seed=4242)
+    copies = int(300e6 // wb.nbytes) + 1  # 38: beyond the 256 MB Infinity Cache
+    ws = [ctx.upload_weight(wb, dtype, m, k) for _ in range(copies)]
+    s, q = O.quantize_q8_0(O.fill_normal(3, 1.0, k))
+    d_q, d_s, d_y = ctx.to_device(q), ctx.to_device(s), ctx.alloc(m * 4)
+    ctx.graph_begin()
+    for w in ws:
+        ctx.gemv_with_preq(w, d_s, d_q, d_y)
+    g = ctx.graph_end()
+    ms_step, each = time_graph_steps(ctx, [g], steps, warmup)
+    ctx.graph_destroy(g)
+    b = gemv_bytes(dtype, m, k)
+    res = {"m": m, "k": k, "dtype": dtype, "bytes_per_launch": b, "weight_copies": copies, "launches_per_step": copies, "ms_per_step": ms_step,
+           "per_launch_in_graph": stats(each, copies), "GBps": b * copies / ms_step / 1e6}
+    if with_concurrent:
+        res["concurrent"] = bench_c1_concurrent(ctx, W, ws, d_q, d_s, b, m)
+    for w in ws:
+        w.free()
+    d_q.free(), d_s.free(), d_y.free()
+    return res
+
+
+def bench_c1_concurrent(ctx, W, ws, d_q, d_s, b, m, streams=4, passes=8, reps=12):
+    """The same GEMVs as independent work: `streams` contexts (one stream each, default priority, within the four hardware
+    queues of a process), each replaying a graph over its own share of the weight copies with its own output.  Nothing
+    orders a launch after a launch of another stream, so the time per launch is what the kernel sustains, not the gap
+    between dependent dispatches.  Timed on the host around launch ... sync of all streams (>= 10 ms of GPU work)."""
+    ctxs = [ctx] + [W.RocmContext(0) for _ in range(streams - 1)]
+    graphs, outs, count = [], [], 0
+    for i, c in enumerate(ctxs):
+        mine = ws[i::streams]
+        d_y = c.alloc(m * 4)
+        outs.append(d_y)
+        c.graph_begin()
+        for _ in range(passes):
+            for w in mine:
+                c.gemv_with_preq(w, d_s, d_q, d_y)
+        graphs.append(c.graph_end())
+        count += passes * len(mine)
+
+    def round_trip():
+        for c, g in zip(ctxs, graphs):
+            c.graph_launch(g)
+
+    for _ in range(2):
+        round_trip()
+    for c in ctxs:
+        c.sync()
+    samples = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        for _ in range(4):
+            round_trip()
+        for c in ctxs:
+            c.sync()
+        samples.append((time.perf_counter() - t0) * 1e3 / 4)
+    for c, g, y in zip(ctxs, graphs, outs):
+        c.graph_destroy(g)
+        y.free()
+    for c in ctxs[1:]:
+        c.close()
+    st = stats(samples, count)
+    return {"streams": streams, "launches_per_round": count, "per_launch": st, "GBps_median": b / st["median_us"] / 1e3,
+            "GBps_best": b / st["min_us"] / 1e3, "frac_of_hbm_peak_median": b / st["median_us"] / 1e3 / HBM_PEAK_GBS,
+            "timing": "host clock around 4 rounds of graph launches on every stream + sync of all streams"}
 
 
 def bench_decode(ctx, W, O, dtype, steps, warmup, host_weights, with_unfused=True):
@@ -307,7 +409,7 @@ def bench_lfm2_step(ctx, W, O, tokens=64, context=4096, body=2, embd=14, dims=No
     return out
 
 
-def bench_gemm(ctx, W, O, dtype, m, n, k, reps=20, wb=None, with_quantize=True):
+def bench_gemm(ctx, W, O, dtype, m, n, k, reps=20, wb=None, samples=20):
     wb = O.synth_weight(dtype, m, k, seed=777) if wb is None else wb
     w = ctx.upload_weight(wb, dtype, m, k)
     d_x = ctx.to_device(O.fill_normal(9, 1.0, n * k))
@@ -326,37 +428,80 @@ def bench_gemm(ctx, W, O, dtype, m, n, k, reps=20, wb=None, with_quantize=True):
         run()
     ctx.record(e1)
     ms_both = ctx.elapsed_ms(e0, e1) / reps
-    ctx.kernel_timing_begin()
-    for _ in range(reps):
+    gemm_samples, quant_samples, fam = [], [], "gemm"
+    for _ in range(samples):  # one launch per timing window: a sample per launch (per-dispatch timestamps, the quantity a kernel trace reports)
+        ctx.kernel_timing_begin()
         run()
-    kt = ctx.kernel_timing_end()
+        kt = ctx.kernel_timing_end()
+        fam = "gemm" if kt["gemm"][1] else "gemv"  # small n is served by the multi-token GEMV
+        gemm_samples.append(kt[fam][0])
+        quant_samples.append(kt["quantize"][0])
     ops = 2.0 * m * n * k
-    fam = "gemm" if kt["gemm"][1] else "gemv"  # small n is served by the multi-token GEMV
-    gemm_ms = kt[fam][0] / kt[fam][1]
-    quant_ms = kt["quantize"][0] / kt["quantize"][1]
+    gemm_ms = float(np.mean(gemm_samples))
+    quant_ms = float(np.mean(quant_samples))
     w.free()
     for b in (d_x, d_q, d_s, d_y):
         b.free()
     return {"m": m, "n": n, "k": k, "dtype": dtype, "ops": ops, "kernel_family": fam, "quantize_plus_gemm_ms": ms_both,
             "quantize_plus_gemm_TOPS": ops / ms_both / 1e9, "gemm_kernel_ms": gemm_ms, "gemm_kernel_TOPS": ops / gemm_ms / 1e9,
-            "frac_of_int8_peak": ops / gemm_ms / 1e9 / INT8_PEAK_TOPS,
+            "frac_of_int8_peak": ops / gemm_ms / 1e9 / INT8_PEAK_TOPS, "gemm_kernel_per_launch": stats(gemm_samples),
+            "gemm_kernel_TOPS_median": ops / float(np.median(gemm_samples)) / 1e9, "gemm_kernel_TOPS_best": ops / float(np.min(gemm_samples)) / 1e9,
             "quantize_kernel_ms": quant_ms, "quantize_kernel_GBps": quant_bytes(n, k) / quant_ms / 1e6}
 
 
+def bench_gemm_multi(ctx, W, O, dtype, ms, n, k, blobs, samples=5):
+    """1..3 weights over the same quantized activations in ONE launch (Q | K | V, gate | up of a prompt pass)."""
+    ws = [ctx.upload_weight(b, dtype, m, k) for b, m in zip(blobs, ms)]
+    d_x = ctx.to_device(O.fill_normal(9, 1.0, n * k))
+    stride = sum(ms)
+    d_q, d_s, d_y = ctx.alloc(n * k), ctx.alloc(n * (k // 32) * 4), ctx.alloc(stride * n * 4)
+    ctx.quantize_q8_0(d_x, n, k, k, d_q, d_s)
+    ys = [d_y.ptr + 4 * int(o) for o in np.concatenate([[0], np.cumsum(ms)[:-1]])]
+    run = lambda: ctx.gemm_preq_multi(ws, d_s, d_q, n, ys, stride, layout=W.LAYOUT_TOKEN_MAJOR)
+    for _ in range(2):
+        run()
+    ctx.sync()
+    ts = []
+    for _ in range(samples):
+        ctx.kernel_timing_begin()
+        run()
+        ts.append(ctx.kernel_timing_end()["gemm"][0])
+    for w in ws:
+        w.free()
+    for b in (d_x, d_q, d_s, d_y):
+        b.free()
+    ops = 2.0 * sum(ms) * n * k
+    return {"ops": ops, "gemm_kernel_ms": float(np.mean(ts)), "gemm_kernel_TOPS": ops / float(np.mean(ts)) / 1e9, "per_launch": stats(ts)}
+
+
 def bench_prefill_sites(ctx, W, O, n=4096, dtype=8):
-    """The nine per-layer prefill GEMMs of an LFM2-1.2B-shaped layer at n tokens (Q8_0)."""
+    """The nine per-layer prefill GEMMs of an LFM2-1.2B-shaped layer at n tokens (Q8_0), launched the way the prompt pass
+    launches them (wick_rocm_lfm2_forward_prefill): projections that share their input -- Q | K | V and gate | up -- as one
+    launch over their weights, the others on their own.  K and V alone (512 rows each: half the chip has no tile) are
+    listed too, for reference."""
     hs, is_, kv = 2048, 6912, 512
     sites = [("conv_in", 3 * hs, hs), ("conv_out", hs, hs), ("attn_q", hs, hs), ("attn_k", kv, hs), ("attn_v", kv, hs),
              ("attn_o", hs, hs), ("ffn_gate", is_, hs), ("ffn_up", is_, hs), ("ffn_down", hs, is_)]
-    blobs = synth_many(O, [(dtype, m, k, 300 + i) for i, (_, m, k) in enumerate(sites)])
+    blobs = dict(zip([s_[0] for s_ in sites], synth_many(O, [(dtype, m, k, 300 + i) for i, (_, m, k) in enumerate(sites)])))
+    dims = {name: (m, k) for name, m, k in sites}
+    launches = [("conv_in",), ("conv_out",), ("attn_q", "attn_k", "attn_v"), ("attn_o",), ("ffn_gate", "ffn_up"), ("ffn_down",)]
     out, tot_ops, tot_ms = [], 0.0, 0.0
-    for (name, m, k), wb in zip(sites, blobs):
-        r = bench_gemm(ctx, W, O, dtype, m, n, k, reps=5, wb=wb)
-        out.append({"site": name, "m": m, "k": k, "gemm_kernel_ms": r["gemm_kernel_ms"], "TOPS": r["gemm_kernel_TOPS"],
-                    "frac_of_int8_peak": r["frac_of_int8_peak"]})
+    for group in launches:
+        ms, k = [dims[g][0] for g in group], dims[group[0]][1]
+        if len(group) == 1:
+            r = bench_gemm(ctx, W, O, dtype, ms[0], n, k, reps=3, wb=blobs[group[0]], samples=5)
+        else:
+            r = bench_gemm_multi(ctx, W, O, dtype, ms, n, k, [blobs[g] for g in group])
+        out.append({"launch": "+".join(group), "m": ms, "k": k, "gemm_kernel_ms": r["gemm_kernel_ms"], "TOPS": r["gemm_kernel_TOPS"],
+                    "frac_of_int8_peak": r["gemm_kernel_TOPS"] / INT8_PEAK_TOPS})
         tot_ops += r["ops"]
         tot_ms += r["gemm_kernel_ms"]
-    return {"n": n, "dtype": dtype, "sites": out, "total_ops": tot_ops, "total_gemm_ms": tot_ms, "TOPS": tot_ops / tot_ms / 1e9}
+    alone = []
+    for name in ("attn_k", "attn_v"):
+        r = bench_gemm(ctx, W, O, dtype, dims[name][0], n, dims[name][1], reps=3, wb=blobs[name], samples=5)
+        alone.append({"site": name, "m": dims[name][0], "gemm_kernel_ms": r["gemm_kernel_ms"], "TOPS": r["gemm_kernel_TOPS"]})
+    return {"n": n, "dtype": dtype, "launches": out, "k_v_on_their_own": alone, "total_ops": tot_ops, "total_gemm_ms": tot_ms,
+            "TOPS": tot_ops / tot_ms / 1e9}
 
 
 def bench_lm_head_sweep(ctx, W, O, dtype=8, m=65536, k=2048, ns=(1, 4, 16, 64)):
@@ -439,40 +584,88 @@ def bench_upload(ctx, nbytes=256 << 20, reps=3):
     return {"bytes": nbytes, "ms": dt * 1e3, "GBps": nbytes / dt / 1e9}
 
 
-def cpu_baseline(O, dtype, host_weights, budget_s=12.0):
-    """The reference's x86 path for the same step: per call site a serial f32 GEMV
-    (wick/src/backend/cpu.rs:293-306; Q8_0 rows would be chunked over threads).  Runs
-    whole steps until ~budget_s of CPU time, at least one."""
+def cpu_model_name():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(O, W):
+    """The reference's x86 path (what it executes on this host: f32 per-block AVX2 dots restated in C, the integer kernels
+    being aarch64-only), timed on bounded samples of the benchmark's workloads:
+      headline   the single Q4_0 6912 x 2048 GEMV: rows serial on ONE core (wick/src/backend/cpu.rs:293-306)
+      legs       the Q4_0 decode step (serial), the Q8_0 decode step with rows split over T threads
+                 (wick/src/backend/cpu.rs:222-234, 401-420), the prefill GEMM as a loop of per-token GEMVs
+                 (wick/src/model/lfm2.rs:2111-2169) on a 64-token subset, scaled to 2002 tokens."""
+    threads = os.cpu_count() or 1
+    m, k = C1
+    wb = O.synth_weight(W.Q4_0, m, k, seed=4242)
+    x = O.fill_normal(3, 1.0, k)
+    b = gemv_bytes(W.Q4_0, m, k)
+    O.x86_gemv_f32(W.Q4_0, wb, x, m, k)
+    t0, reps = time.perf_counter(), 0
+    while time.perf_counter() - t0 < 4.0:
+        O.x86_gemv_f32(W.Q4_0, wb, x, m, k)
+        reps += 1
+    dt = time.perf_counter() - t0
+    out = {"value": b * reps / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port", "cpu": cpu_model_name(), "host_threads": threads,
+           "sample": f"{reps} GEMVs of the headline shape (Q4_0 {m} x {k}, {b * reps / 1e6:.0f} MB) in {dt:.1f} s on one core: the reference runs "
+                     "Q4_0 rows serially on x86; f32 per-block AVX2 path restated in C (its integer kernels are aarch64-only)",
+           "us_per_gemv": dt / reps * 1e6, "legs": {}}
     sites = decode_call_sites()
     xs = {HS: O.fill_normal(1, 1.0, HS), IS: O.fill_normal(2, 1.0, IS)}
-    threads = os.cpu_count() or 1
-    gbytes = sum(gemv_bytes(dtype, m, k) for _, ms, k in sites for m in ms)
-    used = 1
+    for dtype, name, budget in ((W.Q4_0, "decode_step_q4_0_serial", 6.0), (W.Q8_0, "decode_step_q8_0_threaded", 4.0)):
+        host_weights = synth_decode_weights(O, dtype)
+        gbytes = sum(gemv_bytes(dtype, mm, kk) for _, ms, kk in sites for mm in ms)
+        used, steps, t0 = 1, 0, time.perf_counter()
+        while True:
+            for sname, ms, kk in sites:
+                for blob, mm in zip(host_weights[sname], ms):
+                    _, u = O.x86_gemv_f32(dtype, blob, xs[kk], mm, kk, threads=threads)
+                    used = max(used, u)
+            steps += 1
+            if time.perf_counter() - t0 >= budget:
+                break
+        dt = time.perf_counter() - t0
+        out["legs"][name] = {"value": gbytes * steps / dt / 1e9, "unit": "GB/s", "cores": used, "ms_per_step": dt / steps * 1e3,
+                             "sample": f"{steps} full LFM2-350M-shaped decode steps ({gbytes * steps / 1e6:.0f} MB of GEMV work) in {dt:.1f} s"}
+        del host_weights
+    mm, n, kk, sub = 6912, 2002, 2048, 64
+    wb = O.synth_weight(W.Q4_0, mm, kk, seed=777)
+    xsub = O.fill_normal(9, 1.0, sub * kk)
     t0 = time.perf_counter()
-    steps = 0
-    while True:
-        for name, ms, k in sites:
-            for b, m in zip(host_weights[name], ms):
-                _, u = O.x86_gemv_f32(dtype, b, xs[k], m, k, threads=threads)
-                used = max(used, u)
-        steps += 1
-        if time.perf_counter() - t0 >= budget_s:
-            break
+    _, used = O.x86_prefill_f32(W.Q4_0, wb, xsub, mm, sub, kk, threads=threads)
     dt = time.perf_counter() - t0
-    return {"value": gbytes * steps / dt / 1e9, "unit": "GB/s", "cores": used, "kind": "port",
-            "sample": f"{steps} full decode steps ({gbytes * steps / 1e6:.0f} MB of GEMV work) in {dt:.1f} s; x86 f32 per-block AVX2 path "
-                      "restated in C (the reference's integer kernels are aarch64-only)",
-            "ms_per_step": dt / steps * 1e3}
+    out["legs"]["prefill_gemm_q4_0_6912x2002x2048"] = {
+        "value": 2.0 * mm * sub * kk / dt / 1e12, "unit": "TOP/s", "cores": used, "ms_scaled_to_2002_tokens": dt * 1e3 * n / sub,
+        "sample": f"{sub} of the 2002 tokens as a loop of per-token f32 GEMVs ({dt:.2f} s), scaled linearly to the whole prompt"}
+    return out
+
+
+def profile_figure(name, key):
+    """A `key: number` line of a committed profile summary (profiles/<name>), or None: the counter-derived figures of the
+    JSON line are read from the file they were measured into instead of being repeated here."""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", name)):
+            if line.strip().startswith(key + ":"):
+                return float(line.split(":", 1)[1].split()[0])
+    except (OSError, ValueError):
+        pass
+    return None
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=100, help="timed graph replays of the headline GEMV (38 launches each)")
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--skip-extra", action="store_true", help="only the headline decode step (+ CPU baseline)")
-    ap.add_argument("--leg", default="all", help="all | decode | decode_q8 | gemv | gemm | prefill_sites | lm_head | lm_head_q6k | upload | lfm2_step | lfm2_step_q8 | lfm2_step_1p2b | lfm2_step_trace | copy | probe | cpu")
+    ap.add_argument("--skip-extra", action="store_true", help="only the headline GEMV, the GEMM (+ CPU baseline)")
+    ap.add_argument("--leg", default="all", help="all | c1 | gemm | decode | decode_q8 | gemv | prefill_sites | lm_head | lm_head_q6k | upload | lfm2_step | lfm2_step_q8 | lfm2_step_1p2b | lfm2_step_trace | copy | probe | cpu")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -483,15 +676,18 @@ def main():
 
     leg = args.leg
     if leg == "cpu":
-        print(json.dumps({"cpu_baseline": cpu_baseline(O, W.Q4_0, synth_decode_weights(O, W.Q4_0))}))
+        print(json.dumps({"cpu_baseline": cpu_baseline(O, W)}))
         return
     ctx = W.RocmContext(0)
     if leg != "all":
         one = {
+            # graph replays only (warm-up included): every gemv_pairs_kernel dispatch a kernel tracer sees belongs to the timed workload
+            "c1": lambda: bench_c1(ctx, W, O, args.steps, args.warmup, with_concurrent=False),
+            "c1_concurrent": lambda: bench_c1(ctx, W, O, args.steps, args.warmup),
             "decode": lambda: bench_decode(ctx, W, O, W.Q4_0, args.steps, args.warmup, synth_decode_weights(O, W.Q4_0), with_unfused=False),
             "decode_q8": lambda: bench_decode(ctx, W, O, W.Q8_0, args.steps, args.warmup, synth_decode_weights(O, W.Q8_0), with_unfused=False),
             "gemv": lambda: bench_single_gemv(ctx, W, O, W.Q4_0, 6912, 2048),
-            "gemm": lambda: bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048),
+            "gemm": lambda: bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048, samples=100),
             "prefill_sites": lambda: bench_prefill_sites(ctx, W, O),
             "lm_head": lambda: bench_lm_head_sweep(ctx, W, O),
             "lm_head_q6k": lambda: bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024),
@@ -511,70 +707,75 @@ def main():
         ctx.close()
         return
 
-    dtype = W.Q4_0
-    host_weights = synth_decode_weights(O, dtype)
-    dec = bench_decode(ctx, W, O, dtype, args.steps, args.warmup, host_weights)
-
+    c1 = bench_c1(ctx, W, O, args.steps, args.warmup)
+    avg_launch_us = c1["ms_per_step"] * 1e3 / c1["launches_per_step"]
+    achieved = c1["bytes_per_launch"] / avg_launch_us / 1e3  # GB/s
+    c1_profile = "gemv_q4_0_6912x2048_hbm_cold.txt"
     out = {
         "metric": "Q4_0 GEMV GB/s (% HBM peak) + prefill int8 GEMM TOPS (% MFMA peak)",
-        "value": dec["step_GBps"],
+        "value": c1["GBps"],
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": dec["ms_per_step"],
+        "ms_per_step": c1["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "i8",
         "data": "synthetic",
         "config": {
-            "workload": "LFM2-350M-shaped decode-step weight set, Q4_0 weights x Q8_0 activations, n=1: 93 GEMVs in 65 launches, "
-                        "each quantizing its f32 activation in-kernel; one HIP graph per step, two weight copies alternated (HBM-cold)",
+            "workload": "single decode GEMV, LFM2-1.2B ffn_up shape: Q4_0 weight 6912 x 2048 x one Q8_0-quantized token (n = 1), HBM-cold; "
+                        f"one step = one HIP-graph replay = {c1['launches_per_step']} chained launches, one per distinct device copy of the weight "
+                        "(303 MB, beyond the 256 MB Infinity Cache)",
             "device": ctx.device_name,
-            "value_definition": "algorithmic GEMV bytes per step (weights + Q8_0 activations + f32 outputs) / step time, activation quantization included in the time",
+            "value_definition": "algorithmic GEMV bytes per step (38 x (weights + Q8_0 activation + f32 output) = 38 x 7 992 448 B) / step time",
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_pairs_kernel (all instantiations of the step, fused quantizer)",
-            "achieved": dec["gemv_kernel_GBps"],
+            "kernel": "gemv_pairs_kernel<Q4_0> (pre-quantized activation, span loads)",
+            "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": dec["gemv_kernel_GBps"] / HBM_PEAK_GBS,
-            # HBM bytes per launch (average over the 65 launches of a step) from the calibrated FETCH_SIZE / WRITE_SIZE passes
-            # recorded in profiles/decode_step_lfm2_350m_q4_0.txt: mean over all GEMV dispatches of the step, 3.21 MB read + 0.02 MB written
-            "traffic": 3.23e6,
-            "traffic_source": "profiles/decode_step_lfm2_350m_q4_0.txt (rocprofv3 --pmc FETCH_SIZE x2.0, WRITE_SIZE x1.0; copy-calibrated)",
-            "bytes_per_launch_avg": dec["gemv_bytes_per_step"] / dec["gemv_launches_per_step"],
-            "avg_launch_us": dec["gemv_kernel_avg_us"],
-            "note": "per-dispatch timestamps include a fixed dispatch cost per launch; in the graph the same launches average "
-                    f"{dec['us_per_launch_in_graph']:.2f} us each",
+            "frac": achieved / HBM_PEAK_GBS,
+            "bytes_per_launch": c1["bytes_per_launch"],
+            "avg_launch_us": avg_launch_us,
+            "avg_launch_definition": "timed region / launches in it: kernel execution + the gap to the next dependent launch, an upper bound of the "
+                                     "kernel's own duration (the kernel trace of `bench.py --leg c1` in the profile gives the duration alone)",
+            "per_launch": c1["per_launch_in_graph"],
+            "frac_best_step": c1["bytes_per_launch"] / c1["per_launch_in_graph"]["min_us"] / 1e3 / HBM_PEAK_GBS,
+            # HBM bytes per launch from the copy-calibrated FETCH_SIZE / WRITE_SIZE passes recorded in the profile summary
+            "traffic": profile_figure(c1_profile, "traffic_bytes_per_launch"),
+            "traffic_source": "profiles/" + c1_profile,
         },
-        "decode_step": dec,
+        "gemv_6912x2048": c1,
     }
+    if "concurrent" in c1:
+        out["gemv_concurrent"] = c1.pop("concurrent")
+
+    gemm_profile = "gemm_q4_0_6912x2002x2048.txt"
+    g = bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048, samples=100)
+    g["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma_kernel<Q4_0>", "achieved": g["gemm_kernel_TOPS"], "peak": INT8_PEAK_TOPS,
+                     "unit": "TOP/s", "frac": g["gemm_kernel_TOPS"] / INT8_PEAK_TOPS, "frac_median": g["gemm_kernel_TOPS_median"] / INT8_PEAK_TOPS,
+                     "frac_best": g["gemm_kernel_TOPS_best"] / INT8_PEAK_TOPS, "avg_launch_us": g["gemm_kernel_ms"] * 1e3,
+                     "traffic": profile_figure(gemm_profile, "traffic_bytes_per_launch"), "traffic_source": "profiles/" + gemm_profile}
+    out["gemm"] = g
 
     if not args.skip_extra:
-        out["gemv_6912x2048"] = bench_single_gemv(ctx, W, O, W.Q4_0, 6912, 2048)
-        g = bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048)
-        g["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma_kernel<Q4_0>", "achieved": g["gemm_kernel_TOPS"], "peak": INT8_PEAK_TOPS,
-                         "unit": "TOP/s", "frac": g["gemm_kernel_TOPS"] / INT8_PEAK_TOPS,
-                         # 88.97 MB read + 55.39 MB written per launch (algorithmic 12.57 + 55.35 MB), profiles/gemm_q4_0_6912x2002x2048.txt
-                         "traffic": 144.4e6, "traffic_source": "profiles/gemm_q4_0_6912x2002x2048.txt"}
-        out["gemm"] = g
         out["measured_ceilings"] = bench_probe(ctx)
-        g["roofline"]["frac_of_measured_mfma_ceiling"] = g["gemm_kernel_TOPS"] / out["measured_ceilings"]["mfma_i32_32x32x32_i8"]["value"]
-        del host_weights  # the CPU leg regenerates what it needs; keep host memory low
-        dq = bench_decode(ctx, W, O, W.Q8_0, max(10, args.steps // 2), args.warmup, synth_decode_weights(O, W.Q8_0), with_unfused=False)
+        g["roofline"]["frac_of_measured_block_loop_ceiling"] = g["gemm_kernel_TOPS"] / out["measured_ceilings"]["block_loop_2xmfma32_plus_64_scaling_fma"]["value"]
+        dec = bench_decode(ctx, W, O, W.Q4_0, 50, args.warmup, synth_decode_weights(O, W.Q4_0))
+        out["decode_step"] = dec
+        dq = bench_decode(ctx, W, O, W.Q8_0, 25, args.warmup, synth_decode_weights(O, W.Q8_0), with_unfused=False)
         out["decode_step_q8_0"] = dq
         out["prefill_sites"] = bench_prefill_sites(ctx, W, O)
         out["lm_head_sweep"] = bench_lm_head_sweep(ctx, W, O)
         # shipped LFM2 Q4_0 files keep the tied embedding / LM head in Q6_K (wick/src/model/metal_lfm2.rs:175-180)
         out["lm_head_q6_k_65536x1024"] = bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024)
         out["lfm2_decode_step"] = bench_lfm2_step(ctx, W, O)
-        host_weights = None
     ctx.close()
     if not args.skip_cpu:
-        out["cpu_baseline"] = cpu_baseline(O, dtype, host_weights or synth_decode_weights(O, dtype))
+        out["cpu_baseline"] = cpu_baseline(O, W)
     print(json.dumps(out))
 
 
