@@ -85,6 +85,23 @@ int wick_rocm_attention_block(wick_rocm_ctx *ctx, float *d_q, float *d_k, const 
  * ((kernel_size-1) * hidden floats, updated in place), d_conv_weight [hidden][kernel_size]; d_out = c * conv(b*x). */
 int wick_rocm_shortconv_step(wick_rocm_ctx *ctx, const float *d_proj, float *d_buffer, const float *d_conv_weight, float *d_out,
                              uint32_t hidden, uint32_t kernel_size);
+/* The same convolution folded into the launches on either side of it, two launches instead of three per gated-conv layer
+ * (the Metal path fuses its dispatches the same way, e.g. encode_gemv_rmsnorm_gate_up, wick/src/model/metal_lfm2.rs:1157-1186):
+ *   wick_rocm_shortconv_out_proj_f32        y (+)= W_out * quantize(c * conv(b * x)): the out projection computes the gated
+ *                                           convolution in its prologue from d_proj, the conv weight and the rolling state,
+ *                                           which it only READS (every workgroup needs the old state);
+ *   wick_rocm_ffn_gate_up_conv_advance_f32  wick_rocm_ffn_gate_up_f32 of the same layer, whose first workgroups also advance
+ *                                           the rolling state by this token (slot s <- slot s + 1, last slot <- b * x).
+ * Called in this order, y, d_act and the state are bit-identical to wick_rocm_shortconv_step + wick_rocm_matmul_f32(accumulate)
+ * + wick_rocm_ffn_gate_up_f32.  Shapes: kernel size 3, hidden <= 2048 (even block count), Q4_0 / Q8_0 weights the one-launch
+ * kernels take, 16-byte aligned buffers; wick_rocm_shortconv_fusable says so beforehand (1 / 0), the calls themselves return
+ * WICK_ROCM_ERR_BAD_SHAPE otherwise (no silent fallback: the two halves only make sense together). */
+int wick_rocm_shortconv_fusable(const wick_rocm_weight *w_out, const wick_rocm_weight *w_gate, const wick_rocm_weight *w_up, uint32_t kernel_size);
+int wick_rocm_shortconv_out_proj_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w_out, const float *d_proj, const float *d_buffer,
+                                     const float *d_conv_weight, uint32_t kernel_size, float *d_y, int accumulate);
+int wick_rocm_ffn_gate_up_conv_advance_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w_gate, const wick_rocm_weight *w_up, const float *d_x,
+                                           const float *d_norm_weight, float eps, float *d_act, const float *d_proj, float *d_buffer,
+                                           uint32_t hidden, uint32_t kernel_size);
 
 /* encode_elementwise(silu_mul_inplace) (wick/src/model/metal_lfm2.rs:1701-1715) = cpu::silu_mul_inplace
  * (wick/src/backend/cpu.rs:668-673): gate = silu(gate) * up. */

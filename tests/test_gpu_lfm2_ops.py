@@ -285,3 +285,49 @@ def test_silu_mul_quantize_equals_the_two_launches(ctx, ops, oracle, rows, dim):
     assert np.array_equal(q.ravel(), d_q2.download(np.int8, rows * dim))
     for b in (d_g, d_u, d_q1, d_s1, d_q2, d_s2):
         b.free()
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+@pytest.mark.parametrize("hidden,inter", [(256, 512), (1024, 4608), (2048, 1024), (192, 320)])
+def test_shortconv_folded_into_its_neighbours(ctx, ops, oracle, dtype, hidden, inter):
+    """Two launches instead of three per gated-conv layer: the convolution in the out projection's prologue (state read only),
+    the state advance in the gate / up launch.  Hidden state, gate output and conv state after three tokens are bit-identical
+    to shortconv_step + out projection (accumulate) + gate / up, and the conv output is the oracle's."""
+    K, eps = 3, float(np.float32(1e-5))
+    w_out = ctx.upload_weight(oracle.synth_weight(dtype, hidden, hidden, 61), dtype, hidden, hidden)
+    w_gate = ctx.upload_weight(oracle.synth_weight(dtype, inter, hidden, 62), dtype, inter, hidden)
+    w_up = ctx.upload_weight(oracle.synth_weight(dtype, inter, hidden, 63), dtype, inter, hidden)
+    assert ops.shortconv_fusable(w_out, w_gate, w_up, K)
+    assert not ops.shortconv_fusable(w_out, w_gate, w_up, 4)
+    rng = np.random.default_rng(hidden + inter)
+    conv_w = rng.standard_normal(hidden * K).astype(np.float32)
+    norm_w = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    d_cw, d_nw = ctx.to_device(conv_w), ctx.to_device(norm_w)
+    state0 = rng.standard_normal((K - 1) * hidden).astype(np.float32)
+    h0 = rng.standard_normal(hidden).astype(np.float32)
+    bufs = {name: (ctx.to_device(state0), ctx.to_device(h0), ctx.alloc(inter * 4)) for name in ("fused", "plain")}
+    d_proj, d_gated = ctx.alloc(3 * hidden * 4), ctx.alloc(hidden * 4)
+    ref_buf = state0.copy()
+    for step in range(3):
+        proj = rng.standard_normal(3 * hidden).astype(np.float32)
+        d_proj.upload(proj)
+        st, hid, act = bufs["fused"]
+        ops.encode_shortconv_out_proj(w_out, d_proj, st, d_cw, K, hid, accumulate=True)
+        ops.encode_ffn_gate_up_conv_advance(w_gate, w_up, hid, d_nw, eps, act, d_proj, st, hidden, K)
+        st, hid, act = bufs["plain"]
+        ops.encode_conv1d_fused(d_proj, st, d_cw, d_gated, hidden, K)
+        ctx.encode_gemv(w_out, d_gated, 0, hid, 0, accumulate=True)
+        ctx.encode_ffn_gate_up(w_gate, w_up, hid, d_nw, eps, act)
+        want_gated = L.shortconv_step(proj, ref_buf, conv_w, hidden, K)
+        assert np.array_equal(d_gated.download(np.float32, hidden).view(np.uint32), want_gated.view(np.uint32))
+        for i, n in enumerate(((K - 1) * hidden, hidden, inter)):
+            a, b = bufs["fused"][i].download(np.uint32, n), bufs["plain"][i].download(np.uint32, n)
+            assert np.array_equal(a, b), f"step {step}: {('conv state', 'hidden', 'gate output')[i]} differs"
+        assert np.array_equal(bufs["fused"][0].download(np.float32, (K - 1) * hidden).view(np.uint32), ref_buf.view(np.uint32))
+    with pytest.raises(W.RocmError, match="kernel size 3") as e:
+        ops.encode_shortconv_out_proj(w_out, d_proj, bufs["fused"][0], d_cw, 4, bufs["fused"][1])
+    assert e.value.status == -3
+    for w in (w_out, w_gate, w_up):
+        w.free()
+    for b in (d_cw, d_nw, d_proj, d_gated) + bufs["fused"] + bufs["plain"]:
+        b.free()

@@ -472,6 +472,18 @@ int wick_rocm_gemv_silu_mul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, c
     return gemv_xform_locked(ctx, ws, ys, 1, d_gate, kXformSiluMul, d_up, 0.0f, accumulate);
 }
 
+namespace {
+
+const auto aligned16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16u == 0; };
+
+// Whether the one-launch gate / up kernel takes these weights (lock held or not: reads handles only).
+bool gate_up_fused(const wick_rocm_weight* w_gate, const wick_rocm_weight* w_up) {
+    return w_gate->type == w_up->type && w_gate->type != kTypeQ6_K && w_gate->m == w_up->m && w_gate->k == w_up->k &&
+           gated_kernel_applies(static_cast<const uint8_t*>(w_gate->d), static_cast<const uint8_t*>(w_up->d), w_gate->k);
+}
+
+}  // namespace
+
 int wick_rocm_ffn_gate_up_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w_gate, const wick_rocm_weight* w_up, const float* d_x,
                               const float* d_norm_weight, float eps, float* d_act) {
     WR_ENTER(ctx);
@@ -480,10 +492,8 @@ int wick_rocm_ffn_gate_up_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w_gate
     if (!d_x || !d_act) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "ffn_gate_up: null device pointer");
     if (w_gate->m != w_up->m || w_gate->k != w_up->k) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "ffn_gate_up: gate and up must have one shape");
     const uint32_t m = w_gate->m, k = w_gate->k;
-    const auto aligned16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16u == 0; };
     const auto *g = static_cast<const uint8_t*>(w_gate->d), *u = static_cast<const uint8_t*>(w_up->d);
-    if (w_gate->type == w_up->type && w_gate->type != kTypeQ6_K && gated_kernel_applies(g, u, k) && aligned16(d_x) &&
-        (!d_norm_weight || aligned16(d_norm_weight))) {
+    if (gate_up_fused(w_gate, w_up) && aligned16(d_x) && (!d_norm_weight || aligned16(d_norm_weight))) {
         hipError_t e = launch_gemv_gated_f32(w_gate->type, g, u, m, k, d_x, d_act, ctx->num_cus, ctx->launch(),
                                              d_norm_weight ? kXformRmsNorm : kXformNone, d_norm_weight, eps);
         return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "gated gemv launch");
@@ -501,6 +511,45 @@ int wick_rocm_ffn_gate_up_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w_gate
     }
     hipError_t e = launch_silu_mul(d_act, up_out, m, ctx->launch());
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "silu_mul launch");
+}
+
+int wick_rocm_shortconv_fusable(const wick_rocm_weight* w_out, const wick_rocm_weight* w_gate, const wick_rocm_weight* w_up, uint32_t kernel_size) {
+    if (!w_out || !w_gate || !w_up || !w_out->d || !w_gate->d || !w_up->d) return 0;
+    return w_out->type != kTypeQ6_K && w_out->k % 4u == 0 &&
+           shortconv_kernel_applies(static_cast<const uint8_t*>(w_out->d), w_out->k, kernel_size) && gate_up_fused(w_gate, w_up);
+}
+
+int wick_rocm_shortconv_out_proj_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w_out, const float* d_proj, const float* d_buffer,
+                                     const float* d_conv_weight, uint32_t kernel_size, float* d_y, int accumulate) {
+    WR_ENTER(ctx);
+    if (int rc = check_weight(ctx, w_out)) return rc;
+    if (!d_proj || !d_buffer || !d_conv_weight || !d_y) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "shortconv_out_proj: null device pointer");
+    if (w_out->type == kTypeQ6_K || !shortconv_kernel_applies(static_cast<const uint8_t*>(w_out->d), w_out->k, kernel_size))
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "shortconv_out_proj: needs kernel size 3, hidden <= 2048 with an even block count and a Q4_0 / Q8_0 weight; "
+                                                  "use wick_rocm_shortconv_step + wick_rocm_matmul_f32");
+    if (!aligned16(d_proj) || !aligned16(d_buffer) || !aligned16(d_conv_weight))
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "shortconv_out_proj: proj, buffer and conv weight must be 16-byte aligned");
+    hipError_t e = launch_gemv_shortconv_f32(w_out->type, static_cast<const uint8_t*>(w_out->d), w_out->m, w_out->k, d_proj, d_buffer, d_conv_weight,
+                                             d_y, accumulate, ctx->num_cus, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "shortconv gemv launch");
+}
+
+int wick_rocm_ffn_gate_up_conv_advance_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w_gate, const wick_rocm_weight* w_up, const float* d_x,
+                                           const float* d_norm_weight, float eps, float* d_act, const float* d_proj, float* d_buffer,
+                                           uint32_t hidden, uint32_t kernel_size) {
+    WR_ENTER(ctx);
+    if (int rc = check_weight(ctx, w_gate)) return rc;
+    if (int rc = check_weight(ctx, w_up)) return rc;
+    if (!d_x || !d_act || !d_proj || !d_buffer) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "ffn_gate_up_conv_advance: null device pointer");
+    if (!gate_up_fused(w_gate, w_up) || hidden == 0 || hidden % 4u != 0 || kernel_size < 2)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "ffn_gate_up_conv_advance: shapes the one-launch gate / up kernel does not take (or hidden % 4 != 0, kernel size < 2); "
+                                                  "use wick_rocm_shortconv_step and wick_rocm_ffn_gate_up_f32");
+    if (!aligned16(d_x) || (d_norm_weight && !aligned16(d_norm_weight)) || !aligned16(d_proj) || !aligned16(d_buffer))
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "ffn_gate_up_conv_advance: x, norm weight, proj and buffer must be 16-byte aligned");
+    hipError_t e = launch_gemv_gated_f32(w_gate->type, static_cast<const uint8_t*>(w_gate->d), static_cast<const uint8_t*>(w_up->d), w_gate->m, w_gate->k, d_x,
+                                         d_act, ctx->num_cus, ctx->launch(), d_norm_weight ? kXformRmsNorm : kXformNone, d_norm_weight, eps, d_buffer, d_proj,
+                                         hidden, kernel_size);
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "gated gemv launch");
 }
 
 int wick_rocm_gemv_f32_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count,

@@ -31,8 +31,27 @@ bool gated_kernel_applies(const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32
 }
 
 // out[r] = silu(W_gate[r] . x') * (W_up[r] . x'), x' = xform(x) quantized to Q8_0, in one launch.
+bool shortconv_kernel_applies(const uint8_t* d_w, uint32_t k, uint32_t kernel_size) {
+    const uint32_t nb = k >> 5;
+    return kernel_size == 3 && k <= (uint32_t)kConvMaxK && nb % 2u == 0 && reinterpret_cast<uintptr_t>(d_w) % 4u == 0;
+}
+
+hipError_t launch_gemv_shortconv_f32(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const float* d_proj, const float* d_state,
+                                     const float* d_conv_w, float* d_y, int accumulate, int num_cus, const Launch& L) {
+    GemvArgs a{};
+    a.batch.w[0] = d_w, a.batch.y[0] = d_y, a.batch.row_end[0] = m, a.batch.count = 1;
+    a.xf = d_proj;
+    a.xform = kXformShortConv, a.xaux = d_conv_w, a.xaux2 = d_state;
+    a.x_stride = k;
+    a.k = k;
+    a.n = 1;
+    a.accumulate = accumulate;
+    return type == kTypeQ4_0 ? dispatch<2, 1, true>(a, num_cus, L) : dispatch<8, 1, true>(a, num_cus, L);
+}
+
 hipError_t launch_gemv_gated_f32(int type, const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t m, uint32_t k, const float* d_x,
-                                 float* d_out, int num_cus, const Launch& L, int xform, const float* d_aux, float eps) {
+                                 float* d_out, int num_cus, const Launch& L, int xform, const float* d_aux, float eps, float* conv_state,
+                                 const float* conv_proj, uint32_t conv_hidden, uint32_t conv_kernel) {
     GemvArgs a{};
     a.batch.w[0] = d_w_gate, a.batch.w[1] = d_w_up;
     a.batch.y[0] = d_out;
@@ -40,6 +59,7 @@ hipError_t launch_gemv_gated_f32(int type, const uint8_t* d_w_gate, const uint8_
     a.batch.count = 1;  // the waves are laid out over the rows of one weight; each handles both
     a.xf = d_x;
     a.xform = xform, a.xaux = d_aux, a.eps = eps, a.gated = 1;
+    a.conv_state = conv_state, a.conv_proj = conv_proj, a.conv_hidden = conv_hidden, a.conv_kernel = conv_kernel;
     a.x_stride = k;
     a.k = k;
     a.n = 1;

@@ -37,7 +37,13 @@ struct GemvArgs {
     const int8_t* xq;   // [n][k]      (pre-quantized activations)
     const float* xs;    // [n][k/32]
     const float* xf;    // [n][x_stride] f32 activations, quantized in-kernel (FUSEQ variants)
-    const float* xaux;  // FUSEQ with a transform: RMSNorm weights [k] / the "up" vector [k]
+    const float* xaux;  // FUSEQ with a transform: RMSNorm weights [k] / the "up" vector [k] / the conv kernel [k][3]
+    const float* xaux2; // kXformShortConv: the rolling conv state [2][k] (read only)
+    // GATED with a side job: the rolling state of the layer's short convolution is advanced by the first workgroups
+    // (conv_state[s] <- conv_state[s + 1], last slot <- b * x of conv_proj = [b | c | x]); null: no side job
+    float* conv_state;
+    const float* conv_proj;
+    uint32_t conv_hidden, conv_kernel;
     float eps;          // RMSNorm epsilon
     int32_t* dots;      // parity hook (DUMP variants): raw i32 block dots, [token][row][block], instead of y
     int xform;          // kXformNone / kXformRmsNorm / kXformSiluMul (host-side selector of the kernel variant)
@@ -63,6 +69,7 @@ struct ActRegs {
 // FUSEQ workgroups have four waves that quantize the activation vector together.
 constexpr int kFusedWaves = 4;
 constexpr int kFusedMaxK = 8192;
+constexpr int kConvMaxK = 2048;  // kXformShortConv: eight operands per quad instead of two
 
 // How a lane gets its pair (MODE):
 //   kDirect    each lane loads its own 36 / 68 bytes (two / four 16-byte loads + one dword);
@@ -81,6 +88,10 @@ enum { kDirect = 0, kDirectNT = 1, kSpan = 2 };
 //                  encode_gemv_rmsnorm_gate_up (wick/src/model/metal_lfm2.rs:1157-1186);
 //   kXformSiluMul  silu(x) * up (cpu::silu_mul_inplace, wick/src/backend/cpu.rs:668-673) in front of the FFN's
 //                  down projection.
+//   kXformShortConv  the gated short convolution of a decode step (forward_conv_block's middle, wick/src/model/lfm2.rs:694-726)
+//                  in front of its out projection: x = [b | c | x'] (3k floats), out = c * (s0 w0 + s1 w1 + (b x') w2)
+//                  with the rolling state s0, s1 READ ONLY -- many workgroups read it, so it is advanced by a later
+//                  launch (the side job of the gate / up kernel).  Kernel size 3, k <= 2048.
 // Every workgroup redoes the transform on the whole vector (k <= 8192 floats, a few per thread): cheaper than a
 // launch of its own.
 
@@ -120,9 +131,11 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
         FUSEQ ? blockIdx.x * kFusedWaves + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) : blockIdx.x;
     // The f32 activations are requested first of all (fused variant): they need only two
     // scalars of the argument block, and everything below overlaps with their latency.
-    constexpr int kQuadRounds = kFusedMaxK / 4 / (64 * kFusedWaves);  // 8
+    constexpr int kQuadRounds = XF == kXformShortConv ? kConvMaxK / 4 / (64 * kFusedWaves)  // 2: eight operands per quad
+                                                      : kFusedMaxK / 4 / (64 * kFusedWaves);  // 8
     float4 xv[FUSEQ ? kQuadRounds : 1];
-    float4 av[XF != kXformNone ? kQuadRounds : 1];  // the transform's second operand, same quads
+    float4 av[XF != kXformNone && XF != kXformShortConv ? kQuadRounds : 1];  // the transform's second operand, same quads
+    float4 cv[XF == kXformShortConv ? kQuadRounds : 1][7];  // conv operands: c, x', state 0, state 1, three quads of the kernel (xv holds b)
     if constexpr (FUSEQ) {
         const uint32_t quads = p_k >> 2;
 #pragma unroll
@@ -133,7 +146,18 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
             if (i > 0 && i * 64 * kFusedWaves >= quads) break;
             xv[i] = reinterpret_cast<const float4*>(p_x)[min(quad, quads - 1)];
         }
-        if constexpr (XF != kXformNone) {
+        if constexpr (XF == kXformShortConv) {
+            const float4 *px = reinterpret_cast<const float4*>(p_x), *st = reinterpret_cast<const float4*>(a.xaux2),
+                         *cw = reinterpret_cast<const float4*>(a.xaux);
+#pragma unroll
+            for (int i = 0; i < kQuadRounds; i++) {
+                if (i > 0 && i * 64 * kFusedWaves >= quads) break;
+                const uint32_t quad = min(threadIdx.x + i * 64 * kFusedWaves, quads - 1);
+                cv[i][0] = px[quads + quad], cv[i][1] = px[2 * quads + quad];
+                cv[i][2] = st[quad], cv[i][3] = st[quads + quad];
+                cv[i][4] = cw[3 * quad], cv[i][5] = cw[3 * quad + 1], cv[i][6] = cw[3 * quad + 2];  // [channel][tap] of four channels
+            }
+        } else if constexpr (XF != kXformNone) {
             const float4* aux = reinterpret_cast<const float4*>(a.xaux);
 #pragma unroll
             for (int i = 0; i < kQuadRounds; i++) {
@@ -145,6 +169,22 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
         // keep the compiler from moving the weight loads in front of these
         asm volatile("" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
+    }
+
+    if constexpr (GATED) {
+        // Side job of the FFN's gate / up launch in a gated-conv layer: advance the layer's rolling conv state.  The out
+        // projection before this launch has read the old state; nothing reads it again before the next token.  One thread
+        // per four channels, slots ascending, exactly what shortconv_step_kernel does to the state.
+        if (a.conv_state != nullptr && blockIdx.x * (64u * kFusedWaves) < (a.conv_hidden >> 2)) {
+            const uint32_t cq = a.conv_hidden >> 2, d_conv = a.conv_kernel - 1;
+            const float4* pj = reinterpret_cast<const float4*>(a.conv_proj);
+            float4* st = reinterpret_cast<float4*>(a.conv_state);
+            for (uint32_t q = blockIdx.x * (64u * kFusedWaves) + threadIdx.x; q < cq; q += gridDim.x * (64u * kFusedWaves)) {  // any grid covers every channel
+                const float4 b = pj[q], x = pj[2 * cq + q];
+                for (uint32_t s_ = 1; s_ < d_conv; s_++) st[(size_t)(s_ - 1) * cq + q] = st[(size_t)s_ * cq + q];
+                st[(size_t)(d_conv - 1) * cq + q] = make_float4(__fmul_rn(b.x, x.x), __fmul_rn(b.y, x.y), __fmul_rn(b.z, x.z), __fmul_rn(b.w, x.w));
+            }
+        }
     }
 
     // Which weight of the batch this wave works on.  Every per-weight field is copied out of
@@ -284,6 +324,28 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
                 if (i * 64 * kFusedWaves < quads) {
                     xv[i].x = silu_mul(xv[i].x, av[i].x), xv[i].y = silu_mul(xv[i].y, av[i].y);
                     xv[i].z = silu_mul(xv[i].z, av[i].z), xv[i].w = silu_mul(xv[i].w, av[i].w);
+                }
+            }
+        }
+        if constexpr (XF == kXformShortConv) {
+            // per channel, the operations and their order are shortconv_step_kernel's: bit-identical
+#pragma unroll
+            for (int i = 0; i < kQuadRounds; i++) {
+                if (i * 64 * kFusedWaves < quads) {
+                    const float w[12] = {cv[i][4].x, cv[i][4].y, cv[i][4].z, cv[i][4].w, cv[i][5].x, cv[i][5].y,
+                                         cv[i][5].z, cv[i][5].w, cv[i][6].x, cv[i][6].y, cv[i][6].z, cv[i][6].w};
+                    const float b[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w}, c[4] = {cv[i][0].x, cv[i][0].y, cv[i][0].z, cv[i][0].w};
+                    const float xx[4] = {cv[i][1].x, cv[i][1].y, cv[i][1].z, cv[i][1].w};
+                    const float s0[4] = {cv[i][2].x, cv[i][2].y, cv[i][2].z, cv[i][2].w}, s1[4] = {cv[i][3].x, cv[i][3].y, cv[i][3].z, cv[i][3].w};
+                    float o[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float sum = __fadd_rn(0.0f, __fmul_rn(s0[j], w[3 * j]));
+                        sum = __fadd_rn(sum, __fmul_rn(s1[j], w[3 * j + 1]));
+                        sum = __fadd_rn(sum, __fmul_rn(__fmul_rn(b[j], xx[j]), w[3 * j + 2]));
+                        o[j] = __fmul_rn(c[j], sum);
+                    }
+                    xv[i] = make_float4(o[0], o[1], o[2], o[3]);
                 }
             }
         }
@@ -552,6 +614,14 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
             if (multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSmall, XF>);
             return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall, XF>);
         };
+        if (a.xform == kXformShortConv) {  // k <= 2048: rows of at most 32 pairs; one weight
+            if constexpr (LPR <= 32 && NCHUNK == 1) {
+                if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan, kXformShortConv>);
+                return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall, kXformShortConv>);
+            } else {
+                return hipErrorInvalidValue;  // shortconv_kernel_applies() keeps such shapes away
+            }
+        }
         if (a.xform == kXformRmsNorm) return with_xform(std::integral_constant<int, kXformRmsNorm>{});
         if (a.xform == kXformSiluMul) return with_xform(std::integral_constant<int, kXformSiluMul>{});
         return with_xform(std::integral_constant<int, kXformNone>{});

@@ -186,6 +186,7 @@ struct LayerWeights {
     wick_rocm_weight *gate = nullptr, *up = nullptr, *down = nullptr;
     float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr, *conv_w = nullptr;
     float *k_cache = nullptr, *v_cache = nullptr, *conv_state = nullptr;
+    bool conv_fused = false;  // gated-conv layer whose convolution rides in its out projection and gate / up launches
 };
 
 }  // namespace
@@ -300,8 +301,12 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
         const LayerWeights& L = m->layers[i];
         if (L.n_kv == 0) {
             if ((rc = gemv_normed(ctx, {L.in_proj}, {m->proj}, m->hidden, L.attn_norm, c.rms_norm_eps))) break;
-            if ((rc = wick_rocm_shortconv_step(ctx, m->proj, L.conv_state, L.conv_w, m->gated, hs, c.conv_kernel_size))) break;
-            if ((rc = gemv_residual(ctx, L.out_proj, m->hidden, m->gated))) break;
+            if (L.conv_fused) {  // the convolution in the out projection's prologue, its state advance in the gate / up launch below
+                if ((rc = wick_rocm_shortconv_out_proj_f32(ctx, L.out_proj, m->proj, L.conv_state, L.conv_w, c.conv_kernel_size, m->hidden, 1))) break;
+            } else {
+                if ((rc = wick_rocm_shortconv_step(ctx, m->proj, L.conv_state, L.conv_w, m->gated, hs, c.conv_kernel_size))) break;
+                if ((rc = gemv_residual(ctx, L.out_proj, m->hidden, m->gated))) break;
+            }
         } else {
             if ((rc = gemv_normed(ctx, {L.q, L.k, L.v}, {m->q, m->k, m->v}, m->hidden, L.attn_norm, c.rms_norm_eps))) break;
             if ((rc = wick_rocm_attention_block(ctx, m->q, m->k, m->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, m->attn, m->scores, 0, m->d_pos,
@@ -310,7 +315,12 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
             if ((rc = gemv_residual(ctx, L.o, m->hidden, m->attn))) break;
         }
         // gate = silu(W_gate n(hidden)) * (W_up n(hidden)); hidden += W_down gate
-        if ((rc = wick_rocm_ffn_gate_up_f32(ctx, L.gate, L.up, m->hidden, L.ffn_norm, c.rms_norm_eps, m->gate))) break;
+        if (L.conv_fused)
+            rc = wick_rocm_ffn_gate_up_conv_advance_f32(ctx, L.gate, L.up, m->hidden, L.ffn_norm, c.rms_norm_eps, m->gate, m->proj, L.conv_state, hs,
+                                                        c.conv_kernel_size);
+        else
+            rc = wick_rocm_ffn_gate_up_f32(ctx, L.gate, L.up, m->hidden, L.ffn_norm, c.rms_norm_eps, m->gate);
+        if (rc) break;
         rc = gemv_residual(ctx, L.down, m->hidden, m->gate);
     }
     if (rc) return rc;
@@ -544,6 +554,8 @@ int wick_rocm_lfm2_load(wick_rocm_ctx* ctx, const wick_gguf* g, uint32_t context
         if ((rc = upload_weight(ctx, m, g, p + "ffn_gate.weight", inter, hs, &L.gate))) return bail(rc);
         if ((rc = upload_weight(ctx, m, g, p + "ffn_up.weight", inter, hs, &L.up))) return bail(rc);
         if ((rc = upload_weight(ctx, m, g, p + "ffn_down.weight", hs, inter, &L.down))) return bail(rc);
+        L.conv_fused = L.n_kv == 0 && L.conv_state && reinterpret_cast<uintptr_t>(L.conv_state) % 16u == 0 && reinterpret_cast<uintptr_t>(L.conv_w) % 16u == 0 &&
+                       wick_rocm_shortconv_fusable(L.out_proj, L.gate, L.up, c.conv_kernel_size) != 0;
     }
     if ((rc = upload_f32(ctx, m, g, "token_embd_norm.weight", hs, &m->out_norm))) return bail(rc);
     if ((rc = upload_weight(ctx, m, g, "token_embd.weight", c.vocab_size, hs, &m->embd))) return bail(rc);

@@ -87,7 +87,7 @@ hipError_t launch_gemv(int type, const GemvBatch& batch, uint32_t k, const int8_
 // kernel).  Only when pairs_kernel_applies() and d_x is 16-byte aligned.
 bool pairs_kernel_applies(const GemvBatch& batch, uint32_t k);
 // xform: what is done to x before it is quantized (d_aux: the RMSNorm weights / the "up" vector, k floats, 16-byte aligned).
-enum { kXformNone = 0, kXformRmsNorm = 1, kXformSiluMul = 2 };
+enum { kXformNone = 0, kXformRmsNorm = 1, kXformSiluMul = 2, kXformShortConv = 3 };
 hipError_t launch_gemv_f32(int type, const GemvBatch& batch, uint32_t k, const float* d_x, int accumulate, int num_cus,
                            const Launch& L, int xform = kXformNone, const float* d_aux = nullptr, float eps = 0.0f);
 
@@ -95,9 +95,19 @@ hipError_t launch_gemv_f32(int type, const GemvBatch& batch, uint32_t k, const f
 // x' = xform(x) quantized to Q8_0 (xform: none or RMSNorm).  Only when gated_kernel_applies() (even block count,
 // k <= 4096, 4-byte aligned weights) and d_x / d_aux are 16-byte aligned.
 bool gated_kernel_applies(const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t k);
+// conv_state non-null: the first workgroups also advance that rolling short-conv state by one token (slot s <- slot s + 1, last
+// slot <- b * x of conv_proj = [b | c | x], conv_hidden floats each, conv_hidden % 4 == 0, 16-byte aligned): what
+// launch_shortconv_step does to the state, for a layer whose conv output went through launch_gemv_shortconv_f32.
 hipError_t launch_gemv_gated_f32(int type, const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t m, uint32_t k, const float* d_x,
                                  float* d_out, int num_cus, const Launch& L, int xform = kXformNone, const float* d_aux = nullptr,
-                                 float eps = 0.0f);
+                                 float eps = 0.0f, float* conv_state = nullptr, const float* conv_proj = nullptr, uint32_t conv_hidden = 0,
+                                 uint32_t conv_kernel = 0);
+// y (+)= W * quantize(c * conv(b * x)) for d_proj = [b | c | x] (k floats each), the rolling state d_state ([2][k], read only) and
+// the conv kernel d_conv_w ([k][3]): the gated short convolution folded into its out projection.  Only when
+// shortconv_kernel_applies() (kernel size 3, k <= 2048, even block count) and all pointers are 16-byte aligned.
+bool shortconv_kernel_applies(const uint8_t* d_w, uint32_t k, uint32_t kernel_size);
+hipError_t launch_gemv_shortconv_f32(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const float* d_proj, const float* d_state,
+                                     const float* d_conv_w, float* d_y, int accumulate, int num_cus, const Launch& L);
 
 // Q6_K decode GEMV, one token (gemv_q6k.hip).  k % 256 == 0, k <= 8192; the weight allocation is padded by
 // 16 bytes; y[row * y_row_stride].  launch_group_dots_q6k is its parity hook: out[i * (k/16) + g] = exact i32 dot of 16-weight group g.

@@ -44,6 +44,9 @@ _SIGNATURES = {
     "wick_rocm_lfm2_layer_kv_heads": (C.c_int, [_P, _U32, C.POINTER(_U32)]),
     "wick_rocm_lfm2_gpu_memory_bytes": (C.c_size_t, [_P]),
     "wick_rocm_lfm2_reset": (C.c_int, [_P, _P]),
+    "wick_rocm_shortconv_fusable": (C.c_int, [_P, _P, _P, _U32]),
+    "wick_rocm_shortconv_out_proj_f32": (C.c_int, [_P, _P, _P, _P, _P, _U32, _P, C.c_int]),
+    "wick_rocm_ffn_gate_up_conv_advance_f32": (C.c_int, [_P, _P, _P, _P, _P, C.c_float, _P, _P, _P, _U32, _U32]),
     "wick_rocm_lfm2_set_graph_replay": (C.c_int, [_P, C.c_int]),
     "wick_rocm_lfm2_forward": (C.c_int, [_P, _P, _U32, _U32, _P]),
     "wick_rocm_lfm2_forward_prefill": (C.c_int, [_P, _P, _P, _U32, _U32, _P]),
@@ -108,6 +111,20 @@ class Lfm2Ops:
         """Causal attention of n prompt tokens at positions pos0.. over caches that already hold their K / V rows."""
         self.ctx._check(self._l.wick_rocm_attention_prefill(self.ctx._h, _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(out), out_stride,
                                                             pos0, n, max_seq, n_heads, n_kv_heads, head_dim))
+
+    def shortconv_fusable(self, w_out: RocmWeight, w_gate: RocmWeight, w_up: RocmWeight, kernel_size: int) -> bool:
+        return bool(self._l.wick_rocm_shortconv_fusable(w_out.handle, w_gate.handle, w_up.handle, kernel_size))
+
+    def encode_shortconv_out_proj(self, w_out: RocmWeight, proj, buffer, conv_weight, kernel_size: int, y, accumulate: bool = False) -> None:
+        """y (+)= W_out quantize(c * conv(b * x)): the gated short convolution in the out projection's prologue (state read only)."""
+        self.ctx._check(self._l.wick_rocm_shortconv_out_proj_f32(self.ctx._h, w_out.handle, _ptr(proj), _ptr(buffer), _ptr(conv_weight), kernel_size,
+                                                                 _ptr(y), int(accumulate)))
+
+    def encode_ffn_gate_up_conv_advance(self, w_gate: RocmWeight, w_up: RocmWeight, x, norm_weight, eps: float, act, proj, buffer, hidden: int,
+                                        kernel_size: int) -> None:
+        """encode_ffn_gate_up + the conv state of the same layer advanced by this token, in one launch."""
+        self.ctx._check(self._l.wick_rocm_ffn_gate_up_conv_advance_f32(self.ctx._h, w_gate.handle, w_up.handle, _ptr(x), _ptr(norm_weight), eps, _ptr(act),
+                                                                       _ptr(proj), _ptr(buffer), hidden, kernel_size))
 
     def encode_attention_block(self, q, k, v, q_norm, k_norm, k_cache, v_cache, out, scratch, pos: int, max_seq: int, head_dim: int,
                                n_heads: int, n_kv_heads: int, eps: float, theta_scale: float, d_pos=None) -> None:
