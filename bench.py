@@ -372,7 +372,22 @@ def trace_lfm2_step(ctx, W, O, tokens=32, context=4096):
     return {"tokens": tokens, "start_pos": 1024, "last_pick": int(picks[-1])}
 
 
-def bench_lfm2_step(ctx, W, O, tokens=64, context=4096, body=2, embd=14, dims=None, label="LFM2-350M-shaped"):
+def trace_lfm2_prefill(ctx, W, O, n=2002, context=4096):
+    """One warm prompt pass of n tokens, for a kernel tracer (eager launches only)."""
+    from wick_amd import gguf as G
+    from wick_amd.lfm2 import RocmLfm2Model
+
+    with G.GgufFile.from_bytes(lfm2_350m_image(O)) as g:
+        model = RocmLfm2Model(ctx, g, context)
+    toks = np.random.default_rng(n).integers(0, VOCAB, n)
+    for _ in range(2):
+        model.reset()
+        logits = model.forward_prefill(toks, 0)
+    model.free()
+    return {"prompt_tokens": n, "passes": 2, "argmax": int(np.argmax(logits))}
+
+
+def bench_lfm2_step(ctx, W, O, tokens=64, context=4096, body=2, embd=14, dims=None, label="LFM2-350M-shaped", kernel_times=True):
     """Whole decode steps of the model handle (embedding, 16 layers with their norms / conv / attention / gates, tied
     LM head, greedy pick), replayed as one graph per token with token and position resident on the device."""
     from wick_amd import gguf as G
@@ -395,12 +410,21 @@ def bench_lfm2_step(ctx, W, O, tokens=64, context=4096, body=2, embd=14, dims=No
     for n in (512, 2002):
         toks = np.random.default_rng(n).integers(0, VOCAB, n)
         model.reset()
-        model.forward_prefill(toks[:64], 0)  # buffers allocated, kernels warm
+        model.forward_prefill(toks, 0)  # buffers sized for this prompt, kernels warm
+        ts = []
+        for _ in range(7):
+            model.reset()
+            t0 = time.perf_counter()
+            model.forward_prefill(toks, 0)  # tokens up, the batched pass, the last token's logits down
+            ts.append(time.perf_counter() - t0)
+        dt = float(np.median(ts))
+        out["prefill"].append({"prompt_tokens": n, "ms": dt * 1e3, "ms_min": min(ts) * 1e3, "samples": len(ts), "tokens_per_s": n / dt})
+    if kernel_times:
+        ctx.kernel_timing_begin()
         model.reset()
-        t0 = time.perf_counter()
         model.forward_prefill(toks, 0)
-        dt = time.perf_counter() - t0
-        out["prefill"].append({"prompt_tokens": n, "ms": dt * 1e3, "tokens_per_s": n / dt})
+        kt = ctx.kernel_timing_end()
+        out["prefill_kernel_time_2002"] = {fam: {"us": ms * 1e3, "launches": n} for fam, (ms, n) in kt.items() if n}
     # where the time goes: the same steps enqueued one by one with per-dispatch timestamps
     model.set_graph_replay(False)
     model.reset()
@@ -701,6 +725,7 @@ def main():
             # the per-layer shapes of BASELINE's LFM2-1.2B call sites: hidden 2048, FFN 6912, 32 heads / 8 KV heads
             "lfm2_step_1p2b": lambda: bench_lfm2_step(ctx, W, O, dims=dict(HS=2048, IS=6912, KV=512), label="LFM2-1.2B-shaped"),
             "lfm2_step_trace": lambda: trace_lfm2_step(ctx, W, O),
+            "lfm2_prefill_trace": lambda: trace_lfm2_prefill(ctx, W, O),
             "copy": lambda: bench_copy(ctx),
             "upload": lambda: bench_upload(ctx),
             "probe": lambda: bench_probe(ctx),

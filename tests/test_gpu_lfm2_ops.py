@@ -164,6 +164,7 @@ def test_attention_decode(ctx, ops, oracle, n_heads, n_kv, hd, seq):
 
 @pytest.mark.parametrize("n_heads,n_kv,hd,pos0,n,pad", [
     (4, 2, 64, 0, 16, 0), (4, 4, 64, 0, 63, 4), (8, 2, 64, 5, 130, 0), (4, 1, 64, 100, 64, 8), (2, 2, 64, 0, 200, 0), (16, 8, 64, 61, 67, 0),
+    (4, 2, 64, 37, 450, 0), (2, 1, 64, 0, 1000, 0),  # 8 and 16 blocks of 64 queries, taken in (long, short) pairs
     (4, 2, 64, 0, 9, 0),     # fewer than 16 tokens: the scalar kernel
     (4, 2, 32, 3, 40, 0), (2, 1, 128, 0, 70, 4),  # head dims without a matrix-core kernel
 ])
@@ -180,7 +181,7 @@ def test_attention_prefill(ctx, ops, oracle, n_heads, n_kv, hd, pos0, n, pad):
     ops.encode_attention_prefill(d_q, q_stride, d_kc, d_vc, d_out, out_stride, pos0, n, max_seq, n_heads, n_kv, hd)
     got = d_out.download(np.float32, n * out_stride).reshape(n, out_stride)
     assert np.all(got[:, n_heads * hd:] == 7.5)  # padding between rows is left alone
-    for j in sorted({0, 1, 15, 16, 17, n // 2, n - 2, n - 1} & set(range(n))) if n > 80 else range(n):
+    for j in sorted({0, 1, 15, 16, 17, 63, 64, 65, 127, 128, n // 2, n - 65, n - 64, n - 2, n - 1} & set(range(n))) if n > 80 else range(n):
         seq = pos0 + j + 1
         ref = L.attention(q[j * q_stride: j * q_stride + n_heads * hd], kc[: seq * kv_dim], vc[: seq * kv_dim], n_heads, n_kv, hd, seq)
         assert np.allclose(got[j, : n_heads * hd], ref, rtol=0, atol=4e-6 * max(np.abs(ref).max(), 1e-3)), f"token {j}"

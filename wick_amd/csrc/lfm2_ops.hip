@@ -551,8 +551,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
 }
 
 // The same causal attention on the f32 matrix cores (v_mfma_f32_16x16x4_f32: exact f32 products, f32 sums; only the
-// order of the sums differs from the scalar kernel above).  A workgroup = 4 waves = 64 consecutive queries of one head,
-// 16 per wave; it walks the cache in tiles of 64 positions that all four waves share through LDS.
+// order of the sums differs from the scalar kernel above).  Four waves = 64 consecutive queries of one head, 16 per
+// wave; they walk the cache in tiles of 64 positions shared through LDS.
 //   scores, transposed:  S^T[key][q] = sum_d K[key][d] Q[q][d]   A = K (keys are the M rows), B = Q^T
 //     lane l feeds key l % 16 and query l % 16 at head dims (l / 16) * HD/4 + s, s = 0 .. HD/4 - 1 (the order of the
 //     K steps is free as long as both operands agree, so a lane's dims are contiguous: 16-byte LDS reads);
@@ -563,29 +563,38 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
 //     operand V[key][4 * (l % 16) + c], c = 0..3, is one 16-byte read serving the four MFMAs that own dims 4 m + c.
 // Streaming softmax per query across the tiles (running maximum shared by the four lane groups of a query through
 // two shuffles, partial sums of the weights kept per lane and added up at the end).
+// Causal work grows with the query's position, so with HALVES == 2 a workgroup of eight waves takes two blocks of 64
+// queries: block (last - y) on waves 0-3 and block y on waves 4-7.  Every workgroup then covers the same number of
+// (wave, tile) steps, a SIMD's two waves share one copy of each K/V tile, and the short block's waves drop out of
+// the arithmetic (not the barriers) once their queries are past.  The next tile's K/V rows are fetched into
+// registers while the current one is being multiplied.
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <int HD>
-__global__ __launch_bounds__(256) void attention_prefill_mfma_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride) {
+template <int HD, int HALVES>
+__global__ __launch_bounds__(256 * HALVES) void attention_prefill_mfma_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride) {
+    constexpr int NT = 256 * HALVES;
     constexpr int KT = 64;        // positions per tile
     constexpr int LD = HD + 4;    // LDS row stride in floats: an odd number of 16-byte chunks, conflict-free operand reads
     constexpr int QR = HD / 4;    // Q registers per lane = K steps of a score tile
     constexpr int DT = HD / 16;   // 16 x 16 output tiles per MFMA group
     static_assert(HD % 16 == 0, "head_dim must be a multiple of 16");
-    __shared__ __align__(16) float ks[KT][LD];
-    __shared__ __align__(16) float vs[KT][LD];
+    __shared__ __align__(16) float ks[2][KT][LD];
+    __shared__ __align__(16) float vs[2][KT][LD];
     const uint32_t h = blockIdx.x;
     const uint32_t qblocks = (n + 63u) / 64u;
-    const uint32_t j0 = (qblocks - 1u - blockIdx.y) * 64u;  // longest rows first
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = (tid >> 6) & 3u, half = tid >> 8, l16 = lane & 15u, g = lane >> 4;
+    const uint32_t qb_long = qblocks - 1u - blockIdx.y;  // longest rows first
+    const uint32_t qb = half == 0 ? qb_long : blockIdx.y;
+    const bool active = half == 0 || qb != qb_long;      // an odd count leaves the middle block without a partner
+    const uint32_t j0 = qb * 64u;
     const uint32_t base = a.d_pos ? *a.d_pos : pos0;
     const uint32_t kv_dim = a.n_kv_heads * HD, kvh = h / (a.n_heads / a.n_kv_heads);
     const float* kbase = a.k_cache + (size_t)kvh * HD;
     const float* vbase = a.v_cache + (size_t)kvh * HD;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
     const uint32_t jq = j0 + 16u * wave + l16;           // this lane's query token
     const uint32_t jl = jq < n ? jq : n - 1u;            // ... clamped for loads
     const uint32_t pq = base + jl;                       // its position = the last key it sees
-    uint32_t wg_last = base + (j0 + 63u < n ? j0 + 63u : n - 1u);  // last position any query of the workgroup sees
+    uint32_t wg_last = base + (qb_long * 64u + 63u < n ? qb_long * 64u + 63u : n - 1u);  // last position any query of the workgroup sees
     if (wg_last >= a.max_seq) wg_last = a.max_seq - 1u;
     const uint32_t wave_last = min(base + min(j0 + 16u * wave + 15u, n - 1u), wg_last);
 
@@ -603,91 +612,120 @@ __global__ __launch_bounds__(256) void attention_prefill_mfma_kernel(AttentionAr
     for (int c = 0; c < DT; c++) o[c] = v4f{0.f, 0.f, 0.f, 0.f};
     float m_run = -__builtin_inff(), l_run = 0.0f;
 
-    for (uint32_t t0 = 0; t0 <= wg_last; t0 += KT) {
-        __syncthreads();  // the previous tile has been consumed
-        {
-            constexpr int C4 = HD / 4, RPP = 256 / C4, NR = KT / RPP;  // float4 columns, rows per pass, passes
-            const uint32_t c4 = tid % C4, r0 = tid / C4;
-            float4 kk[NR], vv[NR];
+    constexpr int C4 = HD / 4, RPP = NT / C4, NR = KT / RPP;  // float4 columns, rows per pass, passes
+    const uint32_t c4 = tid % C4, r0 = tid / C4;
+    float4 kk[NR], vv[NR];
+    auto fetch_tile = [&](uint32_t t0) {
 #pragma unroll
-            for (int i = 0; i < NR; i++) {
-                const uint32_t key = min(t0 + r0 + i * RPP, wg_last);
-                kk[i] = reinterpret_cast<const float4*>(kbase + (size_t)key * kv_dim)[c4];
-                vv[i] = reinterpret_cast<const float4*>(vbase + (size_t)key * kv_dim)[c4];
-            }
+        for (int i = 0; i < NR; i++) {
+            const uint32_t key = min(t0 + r0 + i * RPP, wg_last);
+            kk[i] = reinterpret_cast<const float4*>(kbase + (size_t)key * kv_dim)[c4];
+            vv[i] = reinterpret_cast<const float4*>(vbase + (size_t)key * kv_dim)[c4];
+        }
+    };
+    auto store_tile = [&](int buf) {
 #pragma unroll
-            for (int i = 0; i < NR; i++) {
-                *reinterpret_cast<float4*>(&ks[r0 + i * RPP][4 * c4]) = kk[i];
-                *reinterpret_cast<float4*>(&vs[r0 + i * RPP][4 * c4]) = vv[i];
+        for (int i = 0; i < NR; i++) {
+            *reinterpret_cast<float4*>(&ks[buf][r0 + i * RPP][4 * c4]) = kk[i];
+            *reinterpret_cast<float4*>(&vs[buf][r0 + i * RPP][4 * c4]) = vv[i];
+        }
+    };
+    // Two tiles in LDS: tile t+1 is written (and tile t+2 requested) after the arithmetic of tile t, into the buffer
+    // that tile t-1 left -- one barrier per tile, and no wave waits for global memory before it multiplies.
+    fetch_tile(0);
+    store_tile(0);
+    if (KT <= wg_last) fetch_tile(KT);
+    __syncthreads();
+    int cur = 0;
+    for (uint32_t t0 = 0; t0 <= wg_last; t0 += KT, cur ^= 1) {
+        if (active && t0 <= wave_last) {  // else: every query of this wave ends before the tile (it still stages tiles and meets the barriers)
+            const float (*ks_t)[LD] = ks[cur];
+            const float (*vs_t)[LD] = vs[cur];
+            // scores of 4 sub-tiles x 16 keys.  The four accumulators take turns so that no MFMA waits for the one before it,
+            // and the operands of the next 16 MFMAs are read while the current 16 run (the fences keep that order).
+            v4f sc[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) sc[u] = v4f{0.f, 0.f, 0.f, 0.f};
+            float4 kq[2][4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) kq[0][u] = *reinterpret_cast<const float4*>(&ks_t[16 * u + l16][g * QR]);
+#pragma unroll
+            for (int i = 0; i < QR / 4; i++) {
+                if (i + 1 < QR / 4) {
+#pragma unroll
+                    for (int u = 0; u < 4; u++) kq[(i + 1) & 1][u] = *reinterpret_cast<const float4*>(&ks_t[16 * u + l16][g * QR + 4 * (i + 1)]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < 4; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].x, qr[4 * i], sc[u], 0, 0, 0);
+#pragma unroll
+                for (int u = 0; u < 4; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].y, qr[4 * i + 1], sc[u], 0, 0, 0);
+#pragma unroll
+                for (int u = 0; u < 4; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].z, qr[4 * i + 2], sc[u], 0, 0, 0);
+#pragma unroll
+                for (int u = 0; u < 4; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].w, qr[4 * i + 3], sc[u], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
+            // causal mask + tile maximum of this lane's query
+            float tmax = -__builtin_inff();
+            const bool masked_tile = t0 + KT - 1u > base + min(j0 + 16u * wave, n - 1u);  // some key of the tile is past some query of the wave
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (masked_tile && t0 + 16u * u + 4u * g + r > pq) sc[u][r] = -__builtin_inff();
+                    tmax = fmaxf(tmax, sc[u][r]);
+                }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+            const float m_new = fmaxf(m_run, tmax);  // finite: key 0 is visible to every query and lies in the first tile
+            const float alpha = ggml_expf_nonpos(m_run - m_new);  // first tile: exp(-inf) = 0, nothing to rescale
+            m_run = m_new;
+            float psum = 0.0f;
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float pw = ggml_expf_nonpos(sc[u][r] - m_new);  // masked keys: exp(-inf) = 0
+                    sc[u][r] = pw;
+                    psum += pw;
+                }
+            l_run = l_run * alpha + psum;
+#pragma unroll
+            for (int c = 0; c < DT; c++) o[c] *= alpha;
+            // O^T += V^T P, the V reads four keys ahead of their MFMAs (sched_group_barrier: 0x100 = LDS read, 0x008 = MFMA)
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int sidx = 0; sidx < 4; sidx++) {
+                    const float pv = sc[u][sidx];
+#pragma unroll
+                    for (int c4 = 0; c4 < DT / 4; c4++) {
+                        const float4 vq = *reinterpret_cast<const float4*>(&vs_t[16 * u + 4 * g + sidx][16 * c4 * 4 + 4 * l16]);
+                        o[4 * c4 + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.x, pv, o[4 * c4 + 0], 0, 0, 0);
+                        o[4 * c4 + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.y, pv, o[4 * c4 + 1], 0, 0, 0);
+                        o[4 * c4 + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.z, pv, o[4 * c4 + 2], 0, 0, 0);
+                        o[4 * c4 + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.w, pv, o[4 * c4 + 3], 0, 0, 0);
+                    }
+                }
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+            for (int i = 0; i < 4 * DT - 4; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+        }
+        if (t0 + KT <= wg_last) {
+            store_tile(cur ^ 1);
+            if (t0 + 2 * KT <= wg_last) fetch_tile(t0 + 2 * KT);
         }
         __syncthreads();
-        if (t0 > wave_last) continue;  // every query of this wave ends before the tile (still takes part in the barriers)
-
-        // scores of 4 sub-tiles x 16 keys
-        v4f sc[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) sc[u] = v4f{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int i = 0; i < QR / 4; i++) {
-            float4 kq[4];
-#pragma unroll
-            for (int u = 0; u < 4; u++) kq[u] = *reinterpret_cast<const float4*>(&ks[16 * u + l16][g * QR + 4 * i]);
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[u].x, qr[4 * i], sc[u], 0, 0, 0);
-                sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[u].y, qr[4 * i + 1], sc[u], 0, 0, 0);
-                sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[u].z, qr[4 * i + 2], sc[u], 0, 0, 0);
-                sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[u].w, qr[4 * i + 3], sc[u], 0, 0, 0);
-            }
-        }
-        // causal mask + tile maximum of this lane's query
-        float tmax = -__builtin_inff();
-        const bool masked_tile = t0 + KT - 1u > base + min(j0 + 16u * wave, n - 1u);  // some key of the tile is past some query of the wave
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                if (masked_tile && t0 + 16u * u + 4u * g + r > pq) sc[u][r] = -__builtin_inff();
-                tmax = fmaxf(tmax, sc[u][r]);
-            }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-        const float m_new = fmaxf(m_run, tmax);  // finite: key 0 is visible to every query and lies in the first tile
-        const float alpha = m_run == -__builtin_inff() ? 0.0f : ggml_expf(m_run - m_new);  // first tile: nothing to rescale
-        m_run = m_new;
-        float psum = 0.0f;
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const float pw = sc[u][r] == -__builtin_inff() ? 0.0f : ggml_expf(sc[u][r] - m_new);
-                sc[u][r] = pw;
-                psum += pw;
-            }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int c = 0; c < DT; c++) o[c] *= alpha;
-        // O^T += V^T P
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-#pragma unroll
-            for (int sidx = 0; sidx < 4; sidx++) {
-                const float pv = sc[u][sidx];
-#pragma unroll
-                for (int c4 = 0; c4 < DT / 4; c4++) {
-                    const float4 vq = *reinterpret_cast<const float4*>(&vs[16 * u + 4 * g + sidx][16 * c4 * 4 + 4 * l16]);
-                    o[4 * c4 + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.x, pv, o[4 * c4 + 0], 0, 0, 0);
-                    o[4 * c4 + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.y, pv, o[4 * c4 + 1], 0, 0, 0);
-                    o[4 * c4 + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.z, pv, o[4 * c4 + 2], 0, 0, 0);
-                    o[4 * c4 + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.w, pv, o[4 * c4 + 3], 0, 0, 0);
-                }
-            }
     }
     // the weight sums of a query's four lane groups
     l_run += __shfl_xor(l_run, 16);
     l_run += __shfl_xor(l_run, 32);
-    if (jq < n) {
+    if (active && jq < n) {
         // tile c4*4 + c, register r of lane (l16, g) holds dim 64 * c4 + 4 * (4 * g + r) + c of query l16
         float* dst = a.out + (size_t)jq * out_stride + (size_t)h * HD;
 #pragma unroll
@@ -1069,8 +1107,11 @@ hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, co
     AttentionArgs a{d_q, d_k_cache, d_v_cache, d_out, d_scratch, d_pos, 0u, max_seq, n_heads, n_kv_heads, head_dim, scale};
     // the matrix-core kernel needs 16-byte aligned rows (q, caches, out) and whole tiles of head dims
     const bool aligned = q_stride % 4u == 0 && out_stride % 4u == 0 && ((uintptr_t)d_q | (uintptr_t)d_k_cache | (uintptr_t)d_v_cache | (uintptr_t)d_out) % 16u == 0;
-    if (head_dim == 64 && aligned && n >= 16)
-        return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64>, dim3(n_heads, (n + 63u) / 64u), dim3(256), a, pos0, n, q_stride, out_stride);
+    if (head_dim == 64 && aligned && n >= 16) {
+        const uint32_t qblocks = (n + 63u) / 64u;
+        if (qblocks == 1) return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 1>, dim3(n_heads, 1), dim3(256), a, pos0, n, q_stride, out_stride);
+        return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(512), a, pos0, n, q_stride, out_stride);
+    }
     const dim3 grid(n_heads, (n + 7u) / 8u), block(256);
     switch (head_dim) {
         case 32: return launch_kernel(L, kFamOther, attention_prefill_kernel<32>, grid, block, a, pos0, n, q_stride, out_stride);
