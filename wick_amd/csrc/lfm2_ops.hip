@@ -111,9 +111,18 @@ struct QkNormRopeArgs {
     uint32_t q_stride, kv_stride;  // floats between consecutive tokens of q / of k and v (a prompt: blockIdx.y = token, position pos + token)
 };
 
+// The rotation of pair i at position pos: angle = pos * theta_scale^i, the power by repeated multiplication as in the
+// reference.
+__device__ __forceinline__ void rope_sincos(uint32_t pos, uint32_t i, float theta_scale, float& sn, float& cs) {
+    float theta = (float)pos;
+    for (uint32_t j = 0; j < i; j++) theta = __fmul_rn(theta, theta_scale);
+    sincosf(theta, &sn, &cs);
+}
+
 // RMSNorm + RoPE of one head by the calling wave: dst[] (and dst2[], when given) receive the result; src may equal dst.
+// sn_tab / cs_tab: the position's sines and cosines per pair when the caller has them already (else computed here).
 __device__ __forceinline__ void norm_rope_head(const float* src, const float* w, uint32_t hd, uint32_t pos, float eps, float theta_scale,
-                                               float* dst, float* dst2) {
+                                               float* dst, float* dst2, const float* sn_tab = nullptr, const float* cs_tab = nullptr) {
     const uint32_t lane = threadIdx.x & 63u, half = hd >> 1;
     double s = 0.0;
     for (uint32_t i = lane; i < hd; i += 64) {
@@ -122,10 +131,9 @@ __device__ __forceinline__ void norm_rope_head(const float* src, const float* w,
     }
     const float inv_rms = (float)(1.0 / sqrt(wave_sum_f64(s) / (double)hd + (double)eps));
     for (uint32_t i = lane; i < half; i += 64) {
-        float theta = (float)pos;
-        for (uint32_t j = 0; j < i; j++) theta = __fmul_rn(theta, theta_scale);
         float sn, cs;
-        sincosf(theta, &sn, &cs);
+        if (sn_tab) sn = sn_tab[i], cs = cs_tab[i];
+        else rope_sincos(pos, i, theta_scale, sn, cs);
         const float x0 = __fmul_rn(__fmul_rn(src[i], inv_rms), w[i]);
         const float x1 = __fmul_rn(__fmul_rn(src[i + half], inv_rms), w[i + half]);
         const float r0 = __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn));
@@ -135,21 +143,38 @@ __device__ __forceinline__ void norm_rope_head(const float* src, const float* w,
     }
 }
 
-__global__ __launch_bounds__(64) void qk_norm_rope_kernel(QkNormRopeArgs a) {
-    const uint32_t tok = blockIdx.y;
-    const uint32_t pos = (a.d_pos ? *a.d_pos : a.pos) + tok;
-    const bool is_q = blockIdx.x < a.n_heads;
-    const uint32_t h = is_q ? blockIdx.x : blockIdx.x - a.n_heads;
+__device__ __forceinline__ void qk_norm_rope_one_head(const QkNormRopeArgs& a, uint32_t tok, uint32_t pos, uint32_t hh, const float* sn_tab,
+                                                      const float* cs_tab) {
+    const bool is_q = hh < a.n_heads;
+    const uint32_t h = is_q ? hh : hh - a.n_heads;
     const uint32_t hd = a.head_dim, kv_dim = a.n_kv_heads * hd;
     float* head = (is_q ? a.q + (size_t)tok * a.q_stride : a.k + (size_t)tok * a.kv_stride) + (size_t)h * hd;
     const bool store = !is_q && pos < a.max_seq;  // the host checks a by-value pos; a device-side pos past the cache is dropped
     norm_rope_head(head, is_q ? a.q_norm : a.k_norm, hd, pos, a.eps, a.theta_scale, head,
-                   store ? a.k_cache + (size_t)pos * kv_dim + (size_t)h * hd : nullptr);
+                   store ? a.k_cache + (size_t)pos * kv_dim + (size_t)h * hd : nullptr, sn_tab, cs_tab);
     if (store) {
         const float* vh = a.v + (size_t)tok * a.kv_stride + (size_t)h * hd;
         float* vc = a.v_cache + (size_t)pos * kv_dim + (size_t)h * hd;
-        for (uint32_t i = threadIdx.x; i < hd; i += 64) vc[i] = vh[i];
+        for (uint32_t i = threadIdx.x & 63u; i < hd; i += 64) vc[i] = vh[i];
     }
+}
+
+__global__ __launch_bounds__(64) void qk_norm_rope_kernel(QkNormRopeArgs a) {
+    const uint32_t tok = blockIdx.y;
+    const uint32_t pos = (a.d_pos ? *a.d_pos : a.pos) + tok;
+    qk_norm_rope_one_head(a, tok, pos, blockIdx.x, nullptr, nullptr);
+}
+
+// The same for the tokens of a prompt: one workgroup per token works out the position's sines and cosines once (every
+// head of the token uses the same ones) and its four waves share the heads.  Same operations per element: bit-identical.
+constexpr uint32_t kRopeTableMax = 128;  // pairs = head_dim / 2
+__global__ __launch_bounds__(256) void qk_norm_rope_tokens_kernel(QkNormRopeArgs a) {
+    __shared__ float sn_tab[kRopeTableMax], cs_tab[kRopeTableMax];
+    const uint32_t tok = blockIdx.x;
+    const uint32_t pos = (a.d_pos ? *a.d_pos : a.pos) + tok;
+    for (uint32_t i = threadIdx.x; i < (a.head_dim >> 1); i += 256) rope_sincos(pos, i, a.theta_scale, sn_tab[i], cs_tab[i]);
+    __syncthreads();
+    for (uint32_t hh = threadIdx.x >> 6; hh < a.n_heads + a.n_kv_heads; hh += 4) qk_norm_rope_one_head(a, tok, pos, hh, sn_tab, cs_tab);
 }
 
 // ---- decode attention -----------------------------------------------------------------
@@ -563,26 +588,37 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
 //     operand V[key][4 * (l % 16) + c], c = 0..3, is one 16-byte read serving the four MFMAs that own dims 4 m + c.
 // Streaming softmax per query across the tiles (running maximum shared by the four lane groups of a query through
 // two shuffles, partial sums of the weights kept per lane and added up at the end).
-// Causal work grows with the query's position, so with HALVES == 2 a workgroup of eight waves takes two blocks of 64
-// queries: block (last - y) on waves 0-3 and block y on waves 4-7.  Every workgroup then covers the same number of
-// (wave, tile) steps, a SIMD's two waves share one copy of each K/V tile, and the short block's waves drop out of
-// the arithmetic (not the barriers) once their queries are past.  The next tile's K/V rows are fetched into
-// registers while the current one is being multiplied.
+// Causal work grows with the query's position, so with HALVES == 2 a workgroup takes two blocks of 64 queries, block
+// (last - y) and block y: every workgroup then covers the same number of (wave, tile) steps and the two blocks share
+// one copy of each K/V tile; the short block's waves drop out of the arithmetic (not the barriers) once their
+// queries are past.  Each block of 64 queries is served by 4 x KSPLIT waves: with KSPLIT == 2 a second wave per 16
+// queries takes the upper 32 keys of every tile with a softmax state of its own, and the two states are merged at the
+// end through LDS -- four waves per SIMD while both blocks run and two when only the long one is left, so that one
+// wave's exp / rescale work overlaps another's MFMAs.  The next tile's K/V rows are fetched into registers while the
+// current one is being multiplied.
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <int HD, int HALVES>
-__global__ __launch_bounds__(256 * HALVES) void attention_prefill_mfma_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride) {
-    constexpr int NT = 256 * HALVES;
+template <int HD, int HALVES, int KSPLIT>
+__global__ __launch_bounds__(256 * HALVES * KSPLIT) void attention_prefill_mfma_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride) {
+    constexpr int NT = 256 * HALVES * KSPLIT;
     constexpr int KT = 64;        // positions per tile
+    constexpr int NU = 4 / KSPLIT;  // 16-key sub-tiles of a tile per wave
     constexpr int LD = HD + 4;    // LDS row stride in floats: an odd number of 16-byte chunks, conflict-free operand reads
     constexpr int QR = HD / 4;    // Q registers per lane = K steps of a score tile
     constexpr int DT = HD / 16;   // 16 x 16 output tiles per MFMA group
     static_assert(HD % 16 == 0, "head_dim must be a multiple of 16");
-    __shared__ __align__(16) float ks[2][KT][LD];
-    __shared__ __align__(16) float vs[2][KT][LD];
+    static_assert(KSPLIT == 1 || KSPLIT == 2, "one or two waves per 16 queries");
+    __shared__ __align__(16) float kv_tiles[2][2][KT][LD];  // [K | V][buffer][position][dim]
+    float (*ks)[KT][LD] = kv_tiles[0];
+    float (*vs)[KT][LD] = kv_tiles[1];
     const uint32_t h = blockIdx.x;
     const uint32_t qblocks = (n + 63u) / 64u;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = (tid >> 6) & 3u, half = tid >> 8, l16 = lane & 15u, g = lane >> 4;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
+    const uint32_t wave_id = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t wave = wave_id & 3u;                    // 16-query group of the block (= the SIMD, so a SIMD's waves share it)
+    const uint32_t ksp = (wave_id >> 2) & (KSPLIT - 1u);   // which keys of a tile: sub-tiles NU * ksp ..
+    const uint32_t half = wave_id / (4u * KSPLIT);         // which block of the pair
+    const uint32_t u0 = NU * ksp;
     const uint32_t qb_long = qblocks - 1u - blockIdx.y;  // longest rows first
     const uint32_t qb = half == 0 ? qb_long : blockIdx.y;
     const bool active = half == 0 || qb != qb_long;      // an odd count leaves the middle block without a partner
@@ -638,55 +674,58 @@ __global__ __launch_bounds__(256 * HALVES) void attention_prefill_mfma_kernel(At
     __syncthreads();
     int cur = 0;
     for (uint32_t t0 = 0; t0 <= wg_last; t0 += KT, cur ^= 1) {
-        if (active && t0 <= wave_last) {  // else: every query of this wave ends before the tile (it still stages tiles and meets the barriers)
-            const float (*ks_t)[LD] = ks[cur];
-            const float (*vs_t)[LD] = vs[cur];
-            // scores of 4 sub-tiles x 16 keys.  The four accumulators take turns so that no MFMA waits for the one before it,
-            // and the operands of the next 16 MFMAs are read while the current 16 run (the fences keep that order).
-            v4f sc[4];
+        if (active && t0 + 16u * u0 <= wave_last) {  // else: every query of this wave ends before its keys of the tile (it still stages tiles and meets the barriers)
+            const float (*ks_t)[LD] = ks[cur] + 16u * u0;  // this wave's keys of the tile
+            const float (*vs_t)[LD] = vs[cur] + 16u * u0;
+            const uint32_t key0 = t0 + 16u * u0;
+            // scores of NU sub-tiles x 16 keys.  The accumulators take turns so that no MFMA waits for the one before it,
+            // and the operands of the next group of MFMAs are read while the current group runs (the fences keep that order).
+            v4f sc[NU];
 #pragma unroll
-            for (int u = 0; u < 4; u++) sc[u] = v4f{0.f, 0.f, 0.f, 0.f};
-            float4 kq[2][4];
+            for (int u = 0; u < NU; u++) sc[u] = v4f{0.f, 0.f, 0.f, 0.f};
+            float4 kq[2][NU];
 #pragma unroll
-            for (int u = 0; u < 4; u++) kq[0][u] = *reinterpret_cast<const float4*>(&ks_t[16 * u + l16][g * QR]);
+            for (int u = 0; u < NU; u++) kq[0][u] = *reinterpret_cast<const float4*>(&ks_t[16 * u + l16][g * QR]);
 #pragma unroll
             for (int i = 0; i < QR / 4; i++) {
                 if (i + 1 < QR / 4) {
 #pragma unroll
-                    for (int u = 0; u < 4; u++) kq[(i + 1) & 1][u] = *reinterpret_cast<const float4*>(&ks_t[16 * u + l16][g * QR + 4 * (i + 1)]);
+                    for (int u = 0; u < NU; u++) kq[(i + 1) & 1][u] = *reinterpret_cast<const float4*>(&ks_t[16 * u + l16][g * QR + 4 * (i + 1)]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int u = 0; u < 4; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].x, qr[4 * i], sc[u], 0, 0, 0);
+                for (int u = 0; u < NU; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].x, qr[4 * i], sc[u], 0, 0, 0);
 #pragma unroll
-                for (int u = 0; u < 4; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].y, qr[4 * i + 1], sc[u], 0, 0, 0);
+                for (int u = 0; u < NU; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].y, qr[4 * i + 1], sc[u], 0, 0, 0);
 #pragma unroll
-                for (int u = 0; u < 4; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].z, qr[4 * i + 2], sc[u], 0, 0, 0);
+                for (int u = 0; u < NU; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].z, qr[4 * i + 2], sc[u], 0, 0, 0);
 #pragma unroll
-                for (int u = 0; u < 4; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].w, qr[4 * i + 3], sc[u], 0, 0, 0);
+                for (int u = 0; u < NU; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].w, qr[4 * i + 3], sc[u], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // causal mask + tile maximum of this lane's query
             float tmax = -__builtin_inff();
-            const bool masked_tile = t0 + KT - 1u > base + min(j0 + 16u * wave, n - 1u);  // some key of the tile is past some query of the wave
+            const bool masked_tile = key0 + 16u * NU - 1u > base + min(j0 + 16u * wave, n - 1u);  // some key of these is past some query of the wave
 #pragma unroll
-            for (int u = 0; u < 4; u++)
+            for (int u = 0; u < NU; u++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    if (masked_tile && t0 + 16u * u + 4u * g + r > pq) sc[u][r] = -__builtin_inff();
+                    if (masked_tile && key0 + 16u * u + 4u * g + r > pq) sc[u][r] = -__builtin_inff();
                     tmax = fmaxf(tmax, sc[u][r]);
                 }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-            const float m_new = fmaxf(m_run, tmax);  // finite: key 0 is visible to every query and lies in the first tile
-            const float alpha = ggml_expf_nonpos(m_run - m_new);  // first tile: exp(-inf) = 0, nothing to rescale
+            const float m_new = fmaxf(m_run, tmax);
+            // a query that has seen no key yet (only in a wave that takes the upper keys) keeps weights and sums at 0
+            const float m_sub = m_new == -__builtin_inff() ? 0.0f : m_new;
+            const float alpha = ggml_expf_nonpos(m_run - m_sub);  // first keys: exp(-inf) = 0, nothing to rescale
             m_run = m_new;
             float psum = 0.0f;
 #pragma unroll
-            for (int u = 0; u < 4; u++)
+            for (int u = 0; u < NU; u++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const float pw = ggml_expf_nonpos(sc[u][r] - m_new);  // masked keys: exp(-inf) = 0
+                    const float pw = ggml_expf_nonpos(sc[u][r] - m_sub);  // masked keys: exp(-inf) = 0
                     sc[u][r] = pw;
                     psum += pw;
                 }
@@ -695,7 +734,7 @@ __global__ __launch_bounds__(256 * HALVES) void attention_prefill_mfma_kernel(At
             for (int c = 0; c < DT; c++) o[c] *= alpha;
             // O^T += V^T P, the V reads four keys ahead of their MFMAs (sched_group_barrier: 0x100 = LDS read, 0x008 = MFMA)
 #pragma unroll
-            for (int u = 0; u < 4; u++)
+            for (int u = 0; u < NU; u++)
 #pragma unroll
                 for (int sidx = 0; sidx < 4; sidx++) {
                     const float pv = sc[u][sidx];
@@ -710,7 +749,7 @@ __global__ __launch_bounds__(256 * HALVES) void attention_prefill_mfma_kernel(At
                 }
             __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-            for (int i = 0; i < 4 * DT - 4; i++) {
+            for (int i = 0; i < NU * DT - 4; i++) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             }
@@ -725,6 +764,30 @@ __global__ __launch_bounds__(256 * HALVES) void attention_prefill_mfma_kernel(At
     // the weight sums of a query's four lane groups
     l_run += __shfl_xor(l_run, 16);
     l_run += __shfl_xor(l_run, 32);
+    if constexpr (KSPLIT == 2) {
+        // the upper-key waves hand (maximum, weight sum, weighted values) to their partners through the tile buffers,
+        // which nobody reads any more (the loop ends on a barrier)
+        constexpr int NS = 2 + 4 * DT;  // floats per lane
+        static_assert(sizeof(kv_tiles) >= sizeof(float) * NS * 64 * 4 * HALVES, "tile buffers hold the partner states");
+        float* xch = &kv_tiles[0][0][0][0] + (size_t)(half * 4u + wave) * NS * 64u + lane;
+        if (ksp == 1) {
+            xch[0] = m_run, xch[64] = l_run;
+#pragma unroll
+            for (int c = 0; c < DT; c++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) xch[(2 + 4 * c + r) * 64] = o[c][r];
+        }
+        __syncthreads();
+        if (ksp == 1) return;
+        const float m_b = xch[0], l_b = xch[64];
+        const float m_all = fmaxf(m_run, m_b);  // finite: key 0 is visible to every query and belongs to this wave
+        const float fa = ggml_expf_nonpos(m_run - m_all), fb = ggml_expf_nonpos(m_b - m_all);  // fb = 0 if the partner saw no key
+        l_run = l_run * fa + l_b * fb;
+#pragma unroll
+        for (int c = 0; c < DT; c++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) o[c][r] = o[c][r] * fa + xch[(2 + 4 * c + r) * 64] * fb;
+    }
     if (active && jq < n) {
         // tile c4*4 + c, register r of lane (l16, g) holds dim 64 * c4 + 4 * (4 * g + r) + c of query l16
         float* dst = a.out + (size_t)jq * out_stride + (size_t)h * HD;
@@ -1009,6 +1072,7 @@ hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const f
     if (n_tokens == 0) return hipSuccess;
     QkNormRopeArgs a{d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, d_pos, pos, max_seq, head_dim, n_heads, n_kv_heads, eps, theta_scale,
                      q_stride, kv_stride};
+    if (n_tokens > 1 && head_dim / 2 <= kRopeTableMax) return launch_kernel(L, kFamOther, qk_norm_rope_tokens_kernel, dim3(n_tokens), dim3(256), a);
     return launch_kernel(L, kFamOther, qk_norm_rope_kernel, dim3(n_heads + n_kv_heads, n_tokens), dim3(64), a);
 }
 
@@ -1109,8 +1173,8 @@ hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, co
     const bool aligned = q_stride % 4u == 0 && out_stride % 4u == 0 && ((uintptr_t)d_q | (uintptr_t)d_k_cache | (uintptr_t)d_v_cache | (uintptr_t)d_out) % 16u == 0;
     if (head_dim == 64 && aligned && n >= 16) {
         const uint32_t qblocks = (n + 63u) / 64u;
-        if (qblocks == 1) return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 1>, dim3(n_heads, 1), dim3(256), a, pos0, n, q_stride, out_stride);
-        return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(512), a, pos0, n, q_stride, out_stride);
+        if (qblocks == 1) return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 1, 2>, dim3(n_heads, 1), dim3(512), a, pos0, n, q_stride, out_stride);
+        return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 2, 2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride, out_stride);
     }
     const dim3 grid(n_heads, (n + 7u) / 8u), block(256);
     switch (head_dim) {
