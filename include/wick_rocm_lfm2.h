@@ -49,6 +49,14 @@ int wick_rocm_qk_norm_rope(wick_rocm_ctx *ctx, float *d_q, float *d_k, const flo
                            uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale);
 float wick_rocm_rope_theta_scale(uint32_t head_dim, float freq_base);
 
+/* The same for the n tokens of a prompt at positions pos0 .. pos0 + n - 1: pass A of the reference's batched prefill
+ * (QK norm, RoPE and the cache append per token, wick/src/model/lfm2.rs:1557-1620).  Token j's query heads start at
+ * d_q + j * q_stride, its key and value heads at d_k / d_v + j * kv_stride (floats).  Bit-identical to n calls of
+ * wick_rocm_qk_norm_rope. */
+int wick_rocm_qk_norm_rope_tokens(wick_rocm_ctx *ctx, float *d_q, uint32_t q_stride, float *d_k, const float *d_v, uint32_t kv_stride,
+                                  const float *d_q_norm, const float *d_k_norm, float *d_k_cache, float *d_v_cache, uint32_t pos0, uint32_t n,
+                                  uint32_t max_seq, uint32_t head_dim, uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale);
+
 /* encode_attention (wick/src/model/metal_lfm2.rs:1736-1867) = attn_scores + softmax_inplace + attn_values per
  * query head (wick/src/model/lfm2.rs:984-1006) over cache rows [0, seq_len) (seq_len = *d_pos + 1 when d_pos is
  * given), grouped-query: head h reads KV head h / (n_heads / n_kv_heads).  d_scratch holds

@@ -126,6 +126,43 @@ def test_qk_norm_rope_and_append(ctx, ops, oracle, n_heads, n_kv, hd, pos):
         b.free()
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,pos0,n,pad", [(16, 8, 64, 0, 40, 0), (4, 2, 64, 4000, 96, 8), (3, 1, 128, 7, 5, 0), (2, 2, 256, 100, 3, 4),
+                                                        (5, 5, 32, 0, 1, 0)])
+def test_qk_norm_rope_of_a_prompt(ctx, ops, oracle, n_heads, n_kv, hd, pos0, n, pad):
+    """Pass A of the batched prefill (wick/src/model/lfm2.rs:1557-1620): one launch for the n tokens == n single-token launches, bit for bit
+    (the prompt kernel shares a position's sin / cos between the heads; same operations per element)."""
+    max_seq, eps, base = 4096, 1e-5, 1_000_000.0
+    kv_dim = n_kv * hd
+    q_stride, kv_stride = n_heads * hd + 2 * kv_dim + pad, n_heads * hd + 2 * kv_dim + pad  # one [q | k | v] row per token, like the prompt pass
+    rows = oracle.fill_normal(11 + n, 1.0, n * q_stride)
+    qn, kn = 1 + 0.2 * oracle.fill_normal(4, 1.0, hd), 1 + 0.2 * oracle.fill_normal(5, 1.0, hd)
+    d_qn, d_kn = ctx.to_device(qn), ctx.to_device(kn)
+    ts = rope_theta_scale(hd, base)
+    out = []
+    for batched in (True, False):
+        d_rows = ctx.to_device(rows)
+        d_kc, d_vc = ctx.to_device(np.full(max_seq * kv_dim, 7.0, np.float32)), ctx.to_device(np.full(max_seq * kv_dim, 7.0, np.float32))
+        q_ptr, k_ptr, v_ptr = d_rows.ptr, d_rows.ptr + 4 * n_heads * hd, d_rows.ptr + 4 * (n_heads * hd + kv_dim)
+        if batched:
+            ops.encode_qk_norm_rope_tokens(q_ptr, q_stride, k_ptr, v_ptr, kv_stride, d_qn, d_kn, d_kc, d_vc, pos0, n, max_seq, hd, n_heads, n_kv, eps, ts)
+        else:
+            for j in range(n):
+                o = 4 * j * q_stride
+                ops.encode_qk_norm_rope(q_ptr + o, k_ptr + o, v_ptr + o, d_qn, d_kn, d_kc, d_vc, pos0 + j, max_seq, hd, n_heads, n_kv, eps, ts)
+        out.append((d_rows.download(np.float32, n * q_stride), d_kc.download(np.float32, max_seq * kv_dim), d_vc.download(np.float32, max_seq * kv_dim)))
+        for b in (d_rows, d_kc, d_vc):
+            b.free()
+    for a, b in zip(*out):
+        assert np.array_equal(bits(a), bits(b))
+    got = out[0][0].reshape(n, q_stride)
+    assert np.array_equal(bits(got[:, n_heads * hd + kv_dim:]), bits(rows.reshape(n, q_stride)[:, n_heads * hd + kv_dim:]))  # v and the padding untouched
+    kc = out[0][1].reshape(max_seq, kv_dim)
+    assert np.array_equal(bits(kc[pos0:pos0 + n]), bits(got[:, n_heads * hd: n_heads * hd + kv_dim])) and (kc[:pos0] == 7.0).all() and (kc[pos0 + n:] == 7.0).all()
+    with pytest.raises(W.RocmError, match="beyond the cache"):
+        ops.encode_qk_norm_rope_tokens(d_qn, q_stride, d_qn, d_qn, kv_stride, d_qn, d_kn, d_qn, d_qn, max_seq - n + 1, n, max_seq, hd, n_heads, n_kv, eps, ts)
+    d_qn.free(), d_kn.free()
+
+
 # contexts of <= 256 positions (and head_dim 96) run the one-workgroup kernel, longer ones the sequence-split kernel;
 # 20000 positions make every workgroup walk several chunks
 @pytest.mark.parametrize("n_heads,n_kv,hd,seq", [(4, 2, 64, 1), (16, 8, 64, 10), (16, 8, 64, 253), (16, 8, 64, 257), (8, 2, 64, 1500), (4, 4, 32, 33),

@@ -57,6 +57,22 @@ int wick_rocm_qk_norm_rope(wick_rocm_ctx* ctx, float* d_q, float* d_k, const flo
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "qk_norm_rope launch");
 }
 
+int wick_rocm_qk_norm_rope_tokens(wick_rocm_ctx* ctx, float* d_q, uint32_t q_stride, float* d_k, const float* d_v, uint32_t kv_stride,
+                                  const float* d_q_norm, const float* d_k_norm, float* d_k_cache, float* d_v_cache, uint32_t pos0, uint32_t n,
+                                  uint32_t max_seq, uint32_t head_dim, uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale) {
+    WR_ENTER(ctx);
+    if (!d_q || !d_k || !d_v || !d_q_norm || !d_k_norm || !d_k_cache || !d_v_cache)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "qk_norm_rope_tokens: null device pointer");
+    if (head_dim == 0 || head_dim % 2u != 0 || head_dim > 256u || n_heads == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "qk_norm_rope_tokens: head_dim must be even and <= 256, n_kv_heads must divide n_heads");
+    if (q_stride < n_heads * head_dim || kv_stride < n_kv_heads * head_dim)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "qk_norm_rope_tokens: strides must cover a token's heads");
+    if ((uint64_t)pos0 + n > max_seq) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "qk_norm_rope_tokens: positions beyond the cache");
+    hipError_t e = launch_qk_norm_rope(d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, pos0, nullptr, max_seq, head_dim, n_heads, n_kv_heads,
+                                       eps, theta_scale, ctx->launch(), n, q_stride, kv_stride);
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "qk_norm_rope_tokens launch");
+}
+
 int wick_rocm_attention_decode(wick_rocm_ctx* ctx, const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out,
                                float* d_scores, uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
                                uint32_t head_dim) {

@@ -27,6 +27,7 @@ _SIGNATURES = {
     "wick_rocm_embed_row": (C.c_int, [_P, _P, _U32, _P, _P]),
     "wick_rocm_rmsnorm": (C.c_int, [_P, _P, _P, _P, _U32, _U32, _U32, _U32, _F]),
     "wick_rocm_qk_norm_rope": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32, _F, _F]),
+    "wick_rocm_qk_norm_rope_tokens": (C.c_int, [_P, _P, _U32, _P, _P, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _U32, _F, _F]),
     "wick_rocm_rope_theta_scale": (_F, [_U32, _F]),
     "wick_rocm_attention_decode": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32]),
     "wick_rocm_attention_scratch_floats": (C.c_size_t, [_U32, _U32, _U32]),
@@ -100,6 +101,13 @@ class Lfm2Ops:
                             n_kv_heads: int, eps: float, theta_scale: float, d_pos=None) -> None:
         self.ctx._check(self._l.wick_rocm_qk_norm_rope(self.ctx._h, _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(k_cache),
                                                        _ptr(v_cache), pos, _ptr(d_pos), max_seq, head_dim, n_heads, n_kv_heads, eps, theta_scale))
+
+    def encode_qk_norm_rope_tokens(self, q, q_stride: int, k, v, kv_stride: int, q_norm, k_norm, k_cache, v_cache, pos0: int, n: int, max_seq: int,
+                                   head_dim: int, n_heads: int, n_kv_heads: int, eps: float, theta_scale: float) -> None:
+        """encode_qk_norm_rope for the n tokens of a prompt at positions pos0.. (token j's heads at j * stride floats)."""
+        self.ctx._check(self._l.wick_rocm_qk_norm_rope_tokens(self.ctx._h, _ptr(q), q_stride, _ptr(k), _ptr(v), kv_stride, _ptr(q_norm), _ptr(k_norm),
+                                                              _ptr(k_cache), _ptr(v_cache), pos0, n, max_seq, head_dim, n_heads, n_kv_heads, eps,
+                                                              theta_scale))
 
     def encode_attention(self, q, k_cache, v_cache, out, scores, seq_len: int, max_seq: int, n_heads: int, n_kv_heads: int, head_dim: int,
                          d_pos=None) -> None:
