@@ -77,6 +77,15 @@ int wick_rocm_attention_prefill(wick_rocm_ctx *ctx, const float *d_q, uint32_t q
                                 float *d_out, uint32_t out_stride, uint32_t pos0, uint32_t n, uint32_t max_seq, uint32_t n_heads,
                                 uint32_t n_kv_heads, uint32_t head_dim);
 
+/* The same with the result written as Q8_0 blocks ([n][n_heads * head_dim] quants, [n][n_heads * head_dim / 32] scales), which is
+ * what the output projection reads (the reference quantizes that input inside its GEMM call, wick/src/model/lfm2.rs:571-592):
+ * bit-identical to wick_rocm_attention_prefill + wick_rocm_quantize_q8_0, one launch and one float round trip less.  Only where
+ * the matrix-core kernel runs (head_dim 64, n >= 16, 16-byte aligned q and caches, q_stride % 4 == 0): WICK_ROCM_ERR_BAD_SHAPE
+ * otherwise. */
+int wick_rocm_attention_prefill_quantize_q8_0(wick_rocm_ctx *ctx, const float *d_q, uint32_t q_stride, const float *d_k_cache,
+                                              const float *d_v_cache, int8_t *d_out_q, float *d_out_scales, uint32_t pos0, uint32_t n,
+                                              uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim);
+
 /* The attention block between the Q/K/V projections and the output projection: what wick_rocm_qk_norm_rope followed
  * by wick_rocm_attention_decode compute (wick/src/model/lfm2.rs:783-1006), bit for bit, with the norm, the rotation and
  * the KV append folded into the attention kernel (workgroups norm and rotate their own query head; those that own the
@@ -93,6 +102,16 @@ int wick_rocm_attention_block(wick_rocm_ctx *ctx, float *d_q, float *d_k, const 
  * ((kernel_size-1) * hidden floats, updated in place), d_conv_weight [hidden][kernel_size]; d_out = c * conv(b*x). */
 int wick_rocm_shortconv_step(wick_rocm_ctx *ctx, const float *d_proj, float *d_buffer, const float *d_conv_weight, float *d_out,
                              uint32_t hidden, uint32_t kernel_size);
+/* The gated short convolution for the n tokens of a prompt (the sequential core of the reference's batched prefill,
+ * wick/src/model/lfm2.rs:1306-1350): d_proj [n][3 * hidden] = a token's [b | c | x], d_out [n][hidden]; token j sees the gated
+ * inputs b*x of tokens j-(K-1) .. j, those before the prompt from the rolling state, which is brought up to date afterwards.
+ * Bit-identical to n calls of wick_rocm_shortconv_step.  The _quantize_q8_0 form writes the result as Q8_0 blocks for the out
+ * projection instead ([n][hidden] quants, [n][hidden / 32] scales; bit-identical to the float form + wick_rocm_quantize_q8_0;
+ * hidden % 32 == 0 and 16-byte aligned buffers, WICK_ROCM_ERR_BAD_SHAPE otherwise). */
+int wick_rocm_shortconv_seq(wick_rocm_ctx *ctx, const float *d_proj, float *d_buffer, const float *d_conv_weight, float *d_out,
+                            uint32_t hidden, uint32_t kernel_size, uint32_t n);
+int wick_rocm_shortconv_seq_quantize_q8_0(wick_rocm_ctx *ctx, const float *d_proj, float *d_buffer, const float *d_conv_weight,
+                                          int8_t *d_out_q, float *d_out_scales, uint32_t hidden, uint32_t kernel_size, uint32_t n);
 /* The same convolution folded into the launches on either side of it, two launches instead of three per gated-conv layer
  * (the Metal path fuses its dispatches the same way, e.g. encode_gemv_rmsnorm_gate_up, wick/src/model/metal_lfm2.rs:1157-1186):
  *   wick_rocm_shortconv_out_proj_f32        y (+)= W_out * quantize(c * conv(b * x)): the out projection computes the gated

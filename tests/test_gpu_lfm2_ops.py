@@ -97,6 +97,50 @@ def test_shortconv_steps_bit_exact(ctx, ops, oracle, hidden, kernel):
         b.free()
 
 
+@pytest.mark.parametrize("hidden,kernel,n,start", [(1024, 3, 70, 0), (96, 3, 5, 2), (320, 4, 9, 1), (64, 2, 3, 0), (128, 1, 4, 0), (1024, 3, 1, 3),
+                                                   (300, 3, 6, 0)])
+def test_shortconv_of_a_prompt(ctx, ops, oracle, hidden, kernel, n, start):
+    """The convolution of n prompt tokens at once (wick/src/model/lfm2.rs:1306-1350) == n single steps, bit for bit, state included
+    (`start` single steps first, so the rolling state is not all zero); its quantizing form == the float form + the Q8_0 quantizer."""
+    w = oracle.fill_normal(kernel, 0.5, hidden * kernel)
+    d_w = ctx.to_device(w)
+    ref_buf = np.zeros((kernel - 1) * hidden, np.float32)
+    d_buf = ctx.to_device(np.zeros(max(kernel - 1, 1) * hidden, np.float32))
+    d_out1 = ctx.alloc(hidden * 4)
+    for step in range(start):
+        proj = oracle.fill_normal(50 + step, 1.0, 3 * hidden)
+        d_p = ctx.to_device(proj)
+        ops.encode_conv1d_fused(d_p, d_buf, d_w, d_out1, hidden, kernel)
+        L.shortconv_step(proj, ref_buf, w, hidden, kernel)
+        d_p.free()
+    state0 = d_buf.download(np.float32, max(kernel - 1, 1) * hidden)
+    projs = oracle.fill_normal(200 + n, 1.0, n * 3 * hidden)
+    want = np.stack([L.shortconv_step(projs[j * 3 * hidden:(j + 1) * 3 * hidden], ref_buf, w, hidden, kernel) for j in range(n)])
+    d_projs, d_out = ctx.to_device(projs), ctx.alloc(n * hidden * 4)
+    ops.encode_conv1d_seq(d_projs, d_buf, d_w, d_out, hidden, kernel, n)
+    got = d_out.download(np.float32, n * hidden).reshape(n, hidden)
+    assert np.array_equal(bits(got), bits(want))
+    if kernel > 1:
+        assert np.array_equal(bits(d_buf.download(np.float32, (kernel - 1) * hidden)), bits(ref_buf))
+    d_q, d_s = ctx.alloc(n * hidden), ctx.alloc(n * (hidden // 32 + 1) * 4)
+    if hidden % 32 == 0:
+        d_buf2 = ctx.to_device(state0)
+        ops.encode_conv1d_seq_quantize(d_projs, d_buf2, d_w, d_q, d_s, hidden, kernel, n)
+        fq, fs = d_q.download(np.int8, n * hidden), d_s.download(np.float32, n * (hidden // 32))
+        ctx.quantize_q8_0(d_out, n, hidden, hidden, d_q, d_s)
+        assert np.array_equal(fq, d_q.download(np.int8, n * hidden)) and np.array_equal(bits(fs), bits(d_s.download(np.float32, n * (hidden // 32))))
+        rs, rq = oracle.quantize_q8_0_batch(want.reshape(-1), n, hidden)
+        assert np.array_equal(fq, rq.reshape(-1)) and np.array_equal(bits(fs), bits(rs.reshape(-1)))
+        if kernel > 1:
+            assert np.array_equal(bits(d_buf2.download(np.float32, (kernel - 1) * hidden)), bits(ref_buf))
+        d_buf2.free()
+    else:
+        with pytest.raises(W.RocmError, match="hidden % 32"):
+            ops.encode_conv1d_seq_quantize(d_projs, d_buf, d_w, d_q, d_s, hidden, kernel, n)
+    for b in (d_w, d_buf, d_out1, d_projs, d_out, d_q, d_s):
+        b.free()
+
+
 @pytest.mark.parametrize("n_heads,n_kv,hd,pos", [(4, 2, 64, 0), (16, 8, 64, 5), (8, 8, 32, 300), (4, 1, 128, 4095), (2, 2, 256, 17)])
 def test_qk_norm_rope_and_append(ctx, ops, oracle, n_heads, n_kv, hd, pos):
     max_seq, eps, base = 4096, 1e-5, 1_000_000.0
@@ -225,6 +269,29 @@ def test_attention_prefill(ctx, ops, oracle, n_heads, n_kv, hd, pos0, n, pad):
     with pytest.raises(W.RocmError, match="beyond the cache"):
         ops.encode_attention_prefill(d_q, q_stride, d_kc, d_vc, d_out, out_stride, 3, n, n + 2, n_heads, n_kv, hd)
     for b in (d_q, d_kc, d_vc, d_out):
+        b.free()
+
+
+@pytest.mark.parametrize("n_heads,n_kv,pos0,n", [(4, 2, 0, 16), (16, 8, 61, 67), (2, 1, 0, 200), (4, 4, 37, 450)])
+def test_attention_prefill_quantizing_epilogue(ctx, ops, oracle, n_heads, n_kv, pos0, n):
+    """The prompt attention writing Q8_0 blocks (the out projection's input) == the float result + the quantizer, bit for bit."""
+    hd = 64
+    kv_dim, max_seq = n_kv * hd, pos0 + n + 2
+    q_stride, hs = n_heads * hd + 2 * kv_dim, n_heads * hd
+    q = oracle.fill_normal(7 * n + pos0, 1.0, n * q_stride)
+    kc, vc = oracle.fill_normal(n + 1, 1.0, max_seq * kv_dim), oracle.fill_normal(n + 2, 1.0, max_seq * kv_dim)
+    d_q, d_kc, d_vc = ctx.to_device(q), ctx.to_device(kc), ctx.to_device(vc)
+    d_out, d_oq, d_os = ctx.alloc(n * hs * 4), ctx.to_device(np.full(n * hs, 99, np.int8)), ctx.alloc(n * (hs // 32) * 4)
+    ops.encode_attention_prefill_quantize(d_q, q_stride, d_kc, d_vc, d_oq, d_os, pos0, n, max_seq, n_heads, n_kv, hd)
+    fq, fs = d_oq.download(np.int8, n * hs), d_os.download(np.float32, n * (hs // 32))
+    ops.encode_attention_prefill(d_q, q_stride, d_kc, d_vc, d_out, hs, pos0, n, max_seq, n_heads, n_kv, hd)
+    ctx.quantize_q8_0(d_out, n, hs, hs, d_oq, d_os)
+    assert np.array_equal(fq, d_oq.download(np.int8, n * hs)) and np.array_equal(bits(fs), bits(d_os.download(np.float32, n * (hs // 32))))
+    with pytest.raises(W.RocmError, match="head_dim 64"):
+        ops.encode_attention_prefill_quantize(d_q, q_stride, d_kc, d_vc, d_oq, d_os, pos0, 8, max_seq, n_heads, n_kv, hd)
+    with pytest.raises(W.RocmError, match="beyond the cache"):
+        ops.encode_attention_prefill_quantize(d_q, q_stride, d_kc, d_vc, d_oq, d_os, 3, n, n + 2, n_heads, n_kv, hd)
+    for b in (d_q, d_kc, d_vc, d_out, d_oq, d_os):
         b.free()
 
 

@@ -106,6 +106,45 @@ int wick_rocm_attention_prefill(wick_rocm_ctx* ctx, const float* d_q, uint32_t q
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "attention_prefill launch");
 }
 
+int wick_rocm_attention_prefill_quantize_q8_0(wick_rocm_ctx* ctx, const float* d_q, uint32_t q_stride, const float* d_k_cache, const float* d_v_cache,
+                                              int8_t* d_out_q, float* d_out_scales, uint32_t pos0, uint32_t n, uint32_t max_seq, uint32_t n_heads,
+                                              uint32_t n_kv_heads, uint32_t head_dim) {
+    WR_ENTER(ctx);
+    if (!d_q || !d_k_cache || !d_v_cache || !d_out_q || !d_out_scales)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention_prefill_quantize: null device pointer");
+    if (n_heads == 0 || n_kv_heads == 0 || n_heads % n_kv_heads != 0 || q_stride < n_heads * head_dim)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "attention_prefill_quantize: n_kv_heads must divide n_heads, q_stride must cover n_heads * head_dim");
+    if (!attention_prefill_quantize_applies(d_q, d_k_cache, d_v_cache, n, q_stride, head_dim) || misaligned(d_out_q, 4))
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE,
+                    "attention_prefill_quantize: needs head_dim 64, n >= 16, q_stride % 4 == 0 and 16-byte aligned q and caches (use attention_prefill + quantize_q8_0)");
+    if ((uint64_t)pos0 + n > max_seq) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention_prefill_quantize: positions beyond the cache");
+    const float scale = 1.0f / sqrtf((float)head_dim);  // wick/src/model/lfm2.rs:862
+    hipError_t e = launch_attention_prefill(d_q, d_k_cache, d_v_cache, nullptr, nullptr, pos0, nullptr, n, q_stride, 0, max_seq, n_heads, n_kv_heads,
+                                            head_dim, scale, ctx->launch(), d_out_q, d_out_scales);
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "attention_prefill_quantize launch");
+}
+
+int wick_rocm_shortconv_seq(wick_rocm_ctx* ctx, const float* d_proj, float* d_buffer, const float* d_conv_weight, float* d_out, uint32_t hidden,
+                            uint32_t kernel_size, uint32_t n) {
+    WR_ENTER(ctx);
+    if (!d_proj || !d_buffer || !d_conv_weight || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "shortconv_seq: null device pointer");
+    if (hidden == 0 || kernel_size == 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "shortconv_seq: hidden and kernel_size must be > 0");
+    hipError_t e = launch_shortconv_seq(d_proj, d_buffer, d_conv_weight, d_out, hidden, kernel_size, n, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "shortconv_seq launch");
+}
+
+int wick_rocm_shortconv_seq_quantize_q8_0(wick_rocm_ctx* ctx, const float* d_proj, float* d_buffer, const float* d_conv_weight, int8_t* d_out_q,
+                                          float* d_out_scales, uint32_t hidden, uint32_t kernel_size, uint32_t n) {
+    WR_ENTER(ctx);
+    if (!d_proj || !d_buffer || !d_conv_weight || !d_out_q || !d_out_scales)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "shortconv_seq_quantize: null device pointer");
+    if (hidden == 0 || kernel_size == 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "shortconv_seq_quantize: hidden and kernel_size must be > 0");
+    if (!shortconv_seq_quantize_applies(d_proj, d_buffer, hidden) || misaligned(d_out_q, 4))
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "shortconv_seq_quantize: needs hidden % 32 == 0 and 16-byte aligned buffers (use shortconv_seq + quantize_q8_0)");
+    hipError_t e = launch_shortconv_seq_quantize(d_proj, d_buffer, d_conv_weight, d_out_q, d_out_scales, hidden, kernel_size, n, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "shortconv_seq_quantize launch");
+}
+
 size_t wick_rocm_attention_block_scratch_bytes(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim) {
     return attention_scratch_floats(max_seq, n_heads, head_dim) * sizeof(float);
 }
@@ -438,10 +477,14 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
     for (uint32_t i = 0; rc == 0 && i < c.n_layers; i++) {
         const LayerWeights& L = m->layers[i];
         if ((rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.attn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
+        bool quantized = false;
         if (L.n_kv == 0) {
             if ((rc = gemm(ctx, L.in_proj, m, n, m->pA, 3 * hs, 0))) break;
-            if ((rc = locked([&] { return launch_shortconv_seq(m->pA, L.conv_state, L.conv_w, m->pG, hs, c.conv_kernel_size, n, ctx->launch()); },
-                             "shortconv_seq launch")))
+            quantized = shortconv_seq_quantize_applies(m->pA, L.conv_state, hs);
+            if ((rc = locked([&] {
+                     return quantized ? launch_shortconv_seq_quantize(m->pA, L.conv_state, L.conv_w, m->pQ, m->pS, hs, c.conv_kernel_size, n, ctx->launch())
+                                      : launch_shortconv_seq(m->pA, L.conv_state, L.conv_w, m->pG, hs, c.conv_kernel_size, n, ctx->launch());
+                 }, "shortconv_seq launch")))
                 break;
         } else {
             const uint32_t kvd = L.n_kv * hd, S = hs + 2 * kvd;  // a token's [q | k | v]
@@ -453,9 +496,10 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
                  }, "qk_norm_rope launch")))
                 break;
             if (attention_layer_applies(hd)) {
+                quantized = attention_prefill_quantize_applies(q, L.k_cache, L.v_cache, n, S, hd);
                 rc = locked([&] {
                     return launch_attention_prefill(q, L.k_cache, L.v_cache, m->pG, m->pAttn, pos0, nullptr, n, S, hs, c.max_seq_len, c.n_heads, L.n_kv, hd,
-                                                    scale, ctx->launch());
+                                                    scale, ctx->launch(), quantized ? m->pQ : nullptr, quantized ? m->pS : nullptr);
                 }, "attention_prefill launch");
             } else {  // head dims without a batched kernel: the decode kernel, token by token
                 for (uint32_t j = 0; rc == 0 && j < n; j++)
@@ -464,7 +508,8 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
             }
             if (rc) break;
         }
-        if ((rc = wick_rocm_quantize_q8_0(ctx, m->pG, n, hs, hs, m->pQ, m->pS))) break;
+        // the out projection's input: already Q8_0 blocks when its producer wrote them itself
+        if (!quantized && (rc = wick_rocm_quantize_q8_0(ctx, m->pG, n, hs, hs, m->pQ, m->pS))) break;
         if ((rc = gemm(ctx, L.n_kv == 0 ? L.out_proj : L.o, m, n, m->pX, hs, 1))) break;  // hidden += out projection
         if ((rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.ffn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
         if ((rc = gemm_group(ctx, {L.gate, L.up}, {m->pGate, m->pUp}, m, n, inter))) break;

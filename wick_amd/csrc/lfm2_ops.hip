@@ -599,7 +599,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 template <int HD, int HALVES, int KSPLIT>
-__global__ __launch_bounds__(256 * HALVES * KSPLIT) void attention_prefill_mfma_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride) {
+__global__ __launch_bounds__(256 * HALVES * KSPLIT) void attention_prefill_mfma_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride,
+                                                                                        int8_t* q_out, float* s_out) {
     constexpr int NT = 256 * HALVES * KSPLIT;
     constexpr int KT = 64;        // positions per tile
     constexpr int NU = 4 / KSPLIT;  // 16-key sub-tiles of a tile per wave
@@ -788,6 +789,30 @@ __global__ __launch_bounds__(256 * HALVES * KSPLIT) void attention_prefill_mfma_
 #pragma unroll
             for (int r = 0; r < 4; r++) o[c][r] = o[c][r] * fa + xch[(2 + 4 * c + r) * 64] * fb;
     }
+    if (q_out) {
+        // Q8_0 blocks of the result instead of floats (what the output projection consumes): a lane holds 16 consecutive
+        // dims of its query, two neighbouring lane groups one 32-dim block.  Rows are n_heads * HD wide, no padding.
+        static_assert(HD == 64, "the quantizing epilogue is written for one 64-dim head = two blocks");
+        float v[4][4];
+        float amax = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                v[r][c] = __fdiv_rn(o[c][r], l_run);
+                amax = fmaxf(amax, fabsf(v[r][c]));
+            }
+        amax = fmaxf(amax, __shfl_xor(amax, 16));
+        float id;
+        const float scale = q8_scale_and_inverse(amax, id);
+        if (active && jq < n) {
+            const size_t row = (size_t)jq * a.n_heads * HD + (size_t)h * HD;
+#pragma unroll
+            for (int r = 0; r < 4; r++) reinterpret_cast<uint32_t*>(q_out + row + 16 * g)[r] = q8_pack4(v[r][0], v[r][1], v[r][2], v[r][3], id);
+            if ((g & 1u) == 0) s_out[(row >> 5) + (g >> 1)] = scale;
+        }
+        return;
+    }
     if (active && jq < n) {
         // tile c4*4 + c, register r of lane (l16, g) holds dim 64 * c4 + 4 * (4 * g + r) + c of query l16
         float* dst = a.out + (size_t)jq * out_stride + (size_t)h * HD;
@@ -854,6 +879,54 @@ __global__ __launch_bounds__(256) void shortconv_seq_kernel(const float* __restr
     const float* p = proj + (size_t)j * 3 * hidden;
     sum = __fadd_rn(sum, __fmul_rn(__fmul_rn(p[ch], p[2 * hidden + ch]), w[d_conv]));
     out[(size_t)j * hidden + ch] = __fmul_rn(p[hidden + ch], sum);
+}
+
+// shortconv_seq_kernel followed by the Q8_0 quantizer, bit for bit: a thread takes four consecutive channels of one
+// token (16-byte loads), eight threads one 32-channel block, and the gated convolution goes straight into Q8_0 blocks
+// for the out projection -- the f32 result never touches memory.  hidden % 32 == 0, 16-byte aligned buffers.
+__global__ __launch_bounds__(256) void shortconv_seq_quantize_kernel(const float* __restrict__ proj, const float* __restrict__ buffer,
+                                                                     const float* __restrict__ conv_w, int8_t* __restrict__ q,
+                                                                     float* __restrict__ scales, uint32_t hidden, uint32_t kernel_size,
+                                                                     uint64_t total_quads) {
+    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const bool live = t < total_quads;
+    const uint64_t tt = live ? t : 0;
+    const uint32_t qpr = hidden >> 2;
+    const uint32_t j = (uint32_t)(tt / qpr), c0 = 4u * (uint32_t)(tt % qpr);
+    const uint32_t d_conv = kernel_size - 1;
+    const float* w = conv_w + (size_t)c0 * kernel_size;
+    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t k = 0; k < d_conv; k++) {
+        const int src = (int)j - (int)d_conv + (int)k;  // token of this tap, < 0: before the prompt
+        float tap[4];
+        if (src < 0) {
+            const float4 s4 = *reinterpret_cast<const float4*>(buffer + (size_t)(src + (int)d_conv) * hidden + c0);
+            tap[0] = s4.x, tap[1] = s4.y, tap[2] = s4.z, tap[3] = s4.w;
+        } else {
+            const float* p = proj + (size_t)src * 3 * hidden;
+            const float4 b = *reinterpret_cast<const float4*>(p + c0), x = *reinterpret_cast<const float4*>(p + 2 * hidden + c0);
+            tap[0] = __fmul_rn(b.x, x.x), tap[1] = __fmul_rn(b.y, x.y), tap[2] = __fmul_rn(b.z, x.z), tap[3] = __fmul_rn(b.w, x.w);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) sum[i] = __fadd_rn(sum[i], __fmul_rn(tap[i], w[(size_t)i * kernel_size + k]));
+    }
+    const float* p = proj + (size_t)j * 3 * hidden;
+    const float4 b = *reinterpret_cast<const float4*>(p + c0), c = *reinterpret_cast<const float4*>(p + hidden + c0),
+                 x = *reinterpret_cast<const float4*>(p + 2 * hidden + c0);
+    const float bx[4] = {__fmul_rn(b.x, x.x), __fmul_rn(b.y, x.y), __fmul_rn(b.z, x.z), __fmul_rn(b.w, x.w)};
+    const float cc[4] = {c.x, c.y, c.z, c.w};
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[i] = __fmul_rn(cc[i], __fadd_rn(sum[i], __fmul_rn(bx[i], w[(size_t)i * kernel_size + d_conv])));
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    amax = group_max8(amax);
+    float id;
+    const float scale = q8_scale_and_inverse(amax, id);
+    const uint32_t packed = q8_pack4(v[0], v[1], v[2], v[3], id);
+    if (live) {
+        reinterpret_cast<uint32_t*>(q)[tt] = packed;
+        if ((tt & 7u) == 0) scales[tt >> 3] = scale;
+    }
 }
 
 // New rolling state after n prompt tokens: slot s holds b*x of token n - (K-1) + s (an old slot when that is negative).
@@ -1162,19 +1235,48 @@ hipError_t launch_shortconv_seq(const float* d_proj, float* d_buffer, const floa
     return launch_kernel(L, kFamOther, shortconv_state_kernel, dim3(blocks), dim3(256), d_proj, d_buffer, hidden, kernel_size, n);
 }
 
+bool shortconv_seq_quantize_applies(const float* d_proj, const float* d_buffer, uint32_t hidden) {
+    return hidden % 32u == 0 && ((uintptr_t)d_proj | (uintptr_t)d_buffer) % 16u == 0;
+}
+
+// The convolution of n tokens written as Q8_0 blocks ([n][hidden] quants, [n][hidden / 32] scales), then the state.
+hipError_t launch_shortconv_seq_quantize(const float* d_proj, float* d_buffer, const float* d_conv_w, int8_t* d_q, float* d_scales, uint32_t hidden,
+                                         uint32_t kernel_size, uint32_t n, const Launch& L) {
+    if (n == 0) return hipSuccess;
+    if (!shortconv_seq_quantize_applies(d_proj, d_buffer, hidden)) return hipErrorInvalidValue;
+    const uint64_t total = (uint64_t)n * (hidden >> 2);
+    hipError_t e = launch_kernel(L, kFamQuantize, shortconv_seq_quantize_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), d_proj,
+                                 static_cast<const float*>(d_buffer), d_conv_w, d_q, d_scales, hidden, kernel_size, total);
+    if (e != hipSuccess || kernel_size < 2) return e;
+    return launch_kernel(L, kFamOther, shortconv_state_kernel, dim3((hidden + 255u) / 256u), dim3(256), d_proj, d_buffer, hidden, kernel_size, n);
+}
+
 size_t attention_prefill_scratch_floats(uint32_t, uint32_t, uint32_t) { return 4; }  // the kernel keeps everything on chip
 
+bool attention_prefill_quantize_applies(const float* d_q, const float* d_k_cache, const float* d_v_cache, uint32_t n, uint32_t q_stride,
+                                        uint32_t head_dim) {
+    return head_dim == 64 && n >= 16 && q_stride % 4u == 0 && ((uintptr_t)d_q | (uintptr_t)d_k_cache | (uintptr_t)d_v_cache) % 16u == 0;
+}
+
+// d_q8 / d_q8_scales given (attention_prefill_quantize_applies): the result is written as Q8_0 blocks, rows of
+// n_heads * head_dim quants, bit-identical to quantizing the float result; d_out is not written then.
 hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scratch,
                                     uint32_t pos0, const uint32_t* d_pos, uint32_t n, uint32_t q_stride, uint32_t out_stride, uint32_t max_seq,
-                                    uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L) {
+                                    uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L, int8_t* d_q8,
+                                    float* d_q8_scales) {
     if (n == 0) return hipSuccess;
     AttentionArgs a{d_q, d_k_cache, d_v_cache, d_out, d_scratch, d_pos, 0u, max_seq, n_heads, n_kv_heads, head_dim, scale};
     // the matrix-core kernel needs 16-byte aligned rows (q, caches, out) and whole tiles of head dims
-    const bool aligned = q_stride % 4u == 0 && out_stride % 4u == 0 && ((uintptr_t)d_q | (uintptr_t)d_k_cache | (uintptr_t)d_v_cache | (uintptr_t)d_out) % 16u == 0;
+    const bool aligned = q_stride % 4u == 0 && ((uintptr_t)d_q | (uintptr_t)d_k_cache | (uintptr_t)d_v_cache) % 16u == 0 &&
+                         (d_q8 || (out_stride % 4u == 0 && (uintptr_t)d_out % 16u == 0));
+    if (d_q8 && !(aligned && attention_prefill_quantize_applies(d_q, d_k_cache, d_v_cache, n, q_stride, head_dim))) return hipErrorInvalidValue;
     if (head_dim == 64 && aligned && n >= 16) {
         const uint32_t qblocks = (n + 63u) / 64u;
-        if (qblocks == 1) return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 1, 2>, dim3(n_heads, 1), dim3(512), a, pos0, n, q_stride, out_stride);
-        return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 2, 2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride, out_stride);
+        if (qblocks == 1)
+            return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 1, 2>, dim3(n_heads, 1), dim3(512), a, pos0, n, q_stride, out_stride, d_q8,
+                                 d_q8_scales);
+        return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 2, 2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride,
+                             out_stride, d_q8, d_q8_scales);
     }
     const dim3 grid(n_heads, (n + 7u) / 8u), block(256);
     switch (head_dim) {

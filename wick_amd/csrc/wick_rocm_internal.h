@@ -164,7 +164,14 @@ hipError_t launch_shortconv_seq(const float* d_proj, float* d_buffer, const floa
 size_t attention_prefill_scratch_floats(uint32_t n, uint32_t n_heads, uint32_t head_dim);
 hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scratch,
                                     uint32_t pos0, const uint32_t* d_pos, uint32_t n, uint32_t q_stride, uint32_t out_stride, uint32_t max_seq,
-                                    uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L);
+                                    uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L, int8_t* d_q8 = nullptr,
+                                    float* d_q8_scales = nullptr);
+// The two producers of an out projection's input written directly as Q8_0 blocks (no float result in memory).
+bool attention_prefill_quantize_applies(const float* d_q, const float* d_k_cache, const float* d_v_cache, uint32_t n, uint32_t q_stride,
+                                        uint32_t head_dim);
+bool shortconv_seq_quantize_applies(const float* d_proj, const float* d_buffer, uint32_t hidden);
+hipError_t launch_shortconv_seq_quantize(const float* d_proj, float* d_buffer, const float* d_conv_w, int8_t* d_q, float* d_scales, uint32_t hidden,
+                                         uint32_t kernel_size, uint32_t n, const Launch& L);
 // d_scores is scratch of attention_scratch_floats(max_seq, n_heads, head_dim) floats.
 uint32_t attention_splits(uint32_t max_seq);
 size_t attention_scratch_floats(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim);

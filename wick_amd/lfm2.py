@@ -27,6 +27,9 @@ _SIGNATURES = {
     "wick_rocm_embed_row": (C.c_int, [_P, _P, _U32, _P, _P]),
     "wick_rocm_rmsnorm": (C.c_int, [_P, _P, _P, _P, _U32, _U32, _U32, _U32, _F]),
     "wick_rocm_qk_norm_rope": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32, _F, _F]),
+    "wick_rocm_attention_prefill_quantize_q8_0": (C.c_int, [_P, _P, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _U32]),
+    "wick_rocm_shortconv_seq": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32, _U32]),
+    "wick_rocm_shortconv_seq_quantize_q8_0": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _U32, _U32]),
     "wick_rocm_qk_norm_rope_tokens": (C.c_int, [_P, _P, _U32, _P, _P, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _U32, _F, _F]),
     "wick_rocm_rope_theta_scale": (_F, [_U32, _F]),
     "wick_rocm_attention_decode": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32]),
@@ -119,6 +122,21 @@ class Lfm2Ops:
         """Causal attention of n prompt tokens at positions pos0.. over caches that already hold their K / V rows."""
         self.ctx._check(self._l.wick_rocm_attention_prefill(self.ctx._h, _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(out), out_stride,
                                                             pos0, n, max_seq, n_heads, n_kv_heads, head_dim))
+
+    def encode_attention_prefill_quantize(self, q, q_stride: int, k_cache, v_cache, out_q, out_scales, pos0: int, n: int, max_seq: int, n_heads: int,
+                                          n_kv_heads: int, head_dim: int) -> None:
+        """encode_attention_prefill with the result written as Q8_0 blocks (the out projection's input)."""
+        self.ctx._check(self._l.wick_rocm_attention_prefill_quantize_q8_0(self.ctx._h, _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(out_q),
+                                                                          _ptr(out_scales), pos0, n, max_seq, n_heads, n_kv_heads, head_dim))
+
+    def encode_conv1d_seq(self, proj, buffer, conv_weight, out, hidden: int, kernel_size: int, n: int) -> None:
+        """The gated short convolution of n prompt tokens (proj [n][3*hidden] -> out [n][hidden]), then the rolling state."""
+        self.ctx._check(self._l.wick_rocm_shortconv_seq(self.ctx._h, _ptr(proj), _ptr(buffer), _ptr(conv_weight), _ptr(out), hidden, kernel_size, n))
+
+    def encode_conv1d_seq_quantize(self, proj, buffer, conv_weight, out_q, out_scales, hidden: int, kernel_size: int, n: int) -> None:
+        """encode_conv1d_seq with the result written as Q8_0 blocks."""
+        self.ctx._check(self._l.wick_rocm_shortconv_seq_quantize_q8_0(self.ctx._h, _ptr(proj), _ptr(buffer), _ptr(conv_weight), _ptr(out_q),
+                                                                      _ptr(out_scales), hidden, kernel_size, n))
 
     def shortconv_fusable(self, w_out: RocmWeight, w_gate: RocmWeight, w_up: RocmWeight, kernel_size: int) -> bool:
         return bool(self._l.wick_rocm_shortconv_fusable(w_out.handle, w_gate.handle, w_up.handle, kernel_size))
