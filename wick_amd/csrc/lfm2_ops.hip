@@ -177,6 +177,54 @@ __global__ __launch_bounds__(256) void qk_norm_rope_tokens_kernel(QkNormRopeArgs
     for (uint32_t hh = threadIdx.x >> 6; hh < a.n_heads + a.n_kv_heads; hh += 4) qk_norm_rope_one_head(a, tok, pos, hh, sn_tab, cs_tab);
 }
 
+// head_dim 64: a lane owns one element of a head, so a wave keeps up to six heads in flight -- all their loads first,
+// then the arithmetic, then the stores: one memory round trip per wave instead of one per head.  The rotation partner
+// (element i +- 32) comes through a lane exchange of the normalised value.  Same operations per element: bit-identical.
+__global__ __launch_bounds__(256) void qk_norm_rope_tokens64_kernel(QkNormRopeArgs a) {
+    constexpr uint32_t HD = 64, HB = 6;
+    __shared__ float sn_tab[HD / 2], cs_tab[HD / 2];
+    const uint32_t tok = blockIdx.x, lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t pos = (a.d_pos ? *a.d_pos : a.pos) + tok;
+    if (threadIdx.x < HD / 2) rope_sincos(pos, threadIdx.x, a.theta_scale, sn_tab[threadIdx.x], cs_tab[threadIdx.x]);
+    const uint32_t heads = a.n_heads + a.n_kv_heads, kv_dim = a.n_kv_heads * HD;
+    const bool store = pos < a.max_seq;  // the host checks a by-value pos; a device-side pos past the cache is dropped
+    const float wq = a.q_norm[lane], wk = a.k_norm[lane];
+    for (uint32_t first = 0; first < heads; first += 4u * HB) {  // the same number of trips for every wave: there is a barrier inside
+        const uint32_t hh0 = first + wave;
+        float v[HB], vv[HB];
+        float* head[HB];
+#pragma unroll
+        for (uint32_t t = 0; t < HB; t++) {
+            const uint32_t hh = hh0 + 4u * t;
+            const bool is_q = hh < a.n_heads;
+            const uint32_t h = is_q ? hh : hh - a.n_heads;
+            head[t] = hh < heads ? (is_q ? a.q + (size_t)tok * a.q_stride : a.k + (size_t)tok * a.kv_stride) + (size_t)h * HD : nullptr;
+            v[t] = head[t] ? head[t][lane] : 0.0f;
+            vv[t] = head[t] && !is_q ? a.v[(size_t)tok * a.kv_stride + (size_t)h * HD + lane] : 0.0f;
+        }
+        __syncthreads();  // the table (first trip; later trips find it published already)
+        const float sn = sn_tab[lane & 31u], cs = cs_tab[lane & 31u];
+#pragma unroll
+        for (uint32_t t = 0; t < HB; t++) {
+            const uint32_t hh = hh0 + 4u * t;  // wave-uniform
+            if (hh >= heads) break;
+            const bool is_q = hh < a.n_heads;
+            const double sq = (double)v[t] * (double)v[t];
+            const float inv_rms = (float)(1.0 / sqrt(wave_sum_f64(sq) / (double)HD + (double)a.eps));
+            const float xn = __fmul_rn(__fmul_rn(v[t], inv_rms), is_q ? wq : wk);
+            const float other = __shfl_xor(xn, 32);
+            // lanes 0-31 hold x0 and write r0 = x0 cs - x1 sn; lanes 32-63 hold x1 and write r1 = x0 sn + x1 cs
+            const float r = lane < 32u ? __fsub_rn(__fmul_rn(xn, cs), __fmul_rn(other, sn)) : __fadd_rn(__fmul_rn(other, sn), __fmul_rn(xn, cs));
+            head[t][lane] = r;
+            if (!is_q && store) {
+                const size_t at = (size_t)pos * kv_dim + (size_t)(hh - a.n_heads) * HD + lane;
+                a.k_cache[at] = r;
+                a.v_cache[at] = vv[t];
+            }
+        }
+    }
+}
+
 // ---- decode attention -----------------------------------------------------------------
 // forward_attn_block's tail (wick/src/model/lfm2.rs:984-1006) = attn_scores -> softmax_inplace -> attn_values
 // (cpu.rs:1346-1355, 715-731, 1391-1401), one 256-thread block per query head over positions [0, seq_len).
@@ -1145,6 +1193,7 @@ hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const f
     if (n_tokens == 0) return hipSuccess;
     QkNormRopeArgs a{d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, d_pos, pos, max_seq, head_dim, n_heads, n_kv_heads, eps, theta_scale,
                      q_stride, kv_stride};
+    if (n_tokens > 1 && head_dim == 64) return launch_kernel(L, kFamOther, qk_norm_rope_tokens64_kernel, dim3(n_tokens), dim3(256), a);
     if (n_tokens > 1 && head_dim / 2 <= kRopeTableMax) return launch_kernel(L, kFamOther, qk_norm_rope_tokens_kernel, dim3(n_tokens), dim3(256), a);
     return launch_kernel(L, kFamOther, qk_norm_rope_kernel, dim3(n_heads + n_kv_heads, n_tokens), dim3(64), a);
 }
