@@ -144,6 +144,19 @@ int wick_rocm_rmsnorm_quantize_q8_0(wick_rocm_ctx *ctx, const float *d_x, const 
 int wick_rocm_silu_mul_quantize_q8_0(wick_rocm_ctx *ctx, const float *d_gate, const float *d_up, uint32_t rows, uint32_t dim, int8_t *d_quants,
                                      float *d_scales);
 
+/* The feed-forward block's gate and up projections over n prompt tokens with the SiLU gate and the Q8_0 quantizer of the
+ * down projection's input in the GEMM's epilogue (wick/src/model/lfm2.rs:2025-2090: gemm_preq(ffn_gate), gemm_preq(ffn_up),
+ * silu_mul_inplace, quantize_columns): d_out_quants [n][m] int8, d_out_scales [n][m / 32] f32, bit-identical to
+ * wick_rocm_gemm_q8_multi + wick_rocm_silu_mul_quantize_q8_0; the two float projections (2 * n * m * 4 bytes) are never written.
+ * d_quants / d_scales: the n quantized activation rows (wick_rocm_quantize_q8_0 layout).  Only where the wide matrix-core tile
+ * runs: both weights Q4_0 or both Q8_0 with the same m and k, m % 32 == 0, k % 128 == 0, n > 64 and more than 256 tiles of
+ * 64 rows x 128 tokens; wick_rocm_ffn_gate_up_silu_quantize_applies says so beforehand (1 / 0), the call returns
+ * WICK_ROCM_ERR_BAD_SHAPE otherwise. */
+int wick_rocm_ffn_gate_up_silu_quantize_applies(const wick_rocm_weight *w_gate, const wick_rocm_weight *w_up, uint32_t n);
+int wick_rocm_ffn_gate_up_silu_quantize_q8(wick_rocm_ctx *ctx, const wick_rocm_weight *w_gate, const wick_rocm_weight *w_up,
+                                           const int8_t *d_quants, const float *d_scales, uint32_t n, int8_t *d_out_quants,
+                                           float *d_out_scales);
+
 /* argmax_f32 dispatch of forward_greedy (wick/src/model/metal_lfm2.rs:2187-2195) with the tie / NaN rules of
  * cpu_argmax (wick/src/sampler.rs:7-19).  d_out[0] = pick; when given, *d_token = pick and *d_pos += 1. */
 int wick_rocm_argmax(wick_rocm_ctx *ctx, const float *d_logits, uint32_t n, uint32_t *d_out, uint32_t *d_token, uint32_t *d_pos);

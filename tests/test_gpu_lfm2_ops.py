@@ -436,3 +436,36 @@ def test_shortconv_folded_into_its_neighbours(ctx, ops, oracle, dtype, hidden, i
         w.free()
     for b in (d_cw, d_nw, d_proj, d_gated) + bufs["fused"] + bufs["plain"]:
         b.free()
+
+
+@pytest.mark.parametrize("dtype,m,k,n", [(W.Q4_0, 4608, 1024, 2002), (W.Q8_0, 2080, 256, 1100), (W.Q4_0, 2048, 128, 1153)])
+def test_gate_up_gemm_with_gate_and_quantizer_in_its_epilogue(ctx, ops, oracle, dtype, m, k, n):
+    """gemm_preq(ffn_gate), gemm_preq(ffn_up), silu_mul_inplace and quantize_columns of the batched prefill
+    (wick/src/model/lfm2.rs:2025-2090) as one launch: quants and scales bit-identical to the three-launch sequence, which the
+    other tests hold against the oracle; a sampled band is checked against the oracle directly as well."""
+    wg, wu = oracle.synth_weight(dtype, m, k, seed=31), oracle.synth_weight(dtype, m, k, seed=32)
+    d_wg, d_wu = ctx.upload_weight(wg, dtype, m, k), ctx.upload_weight(wu, dtype, m, k)
+    xs, xq = oracle.quantize_q8_0_batch(oracle.fill_normal(5, 1.0, n * k), n, k)
+    d_xq, d_xs = ctx.to_device(xq), ctx.to_device(xs)
+    assert ops.ffn_gate_up_silu_quantize_applies(d_wg, d_wu, n)
+    d_oq, d_os = ctx.to_device(np.full(n * m, 99, np.int8)), ctx.alloc(n * (m // 32) * 4)
+    ops.encode_ffn_gate_up_silu_quantize(d_wg, d_wu, d_xs, d_xq, n, d_oq, d_os)
+    fq, fs = d_oq.download(np.int8, n * m), d_os.download(np.float32, n * (m // 32))
+    d_g, d_u = ctx.alloc(n * m * 4), ctx.alloc(n * m * 4)
+    ctx.gemm_preq_multi([d_wg, d_wu], d_xs, d_xq, n, [d_g, d_u], m)
+    ops.silu_mul_quantize(d_g, d_u, n, m, d_oq, d_os)
+    assert np.array_equal(fq, d_oq.download(np.int8, n * m)) and np.array_equal(bits(fs), bits(d_os.download(np.float32, n * (m // 32))))
+    # the oracle on a few tokens: its own GEMV route, gate and quantizer (f32 sums in another order: a quant may differ by one
+    # where a value sits on a rounding tie, never more)
+    for j in (0, n // 2, n - 1):
+        g = oracle.gemv_q8(dtype, wg, xs[j], xq[j], m, k)
+        u = oracle.gemv_q8(dtype, wu, xs[j], xq[j], m, k)
+        rs, rq = oracle.quantize_q8_0_batch(L.silu_mul(g, u), 1, m)
+        got = fq.reshape(n, m)[j].astype(np.int32)
+        assert np.abs(got - rq.reshape(-1).astype(np.int32)).max() <= 1 and np.allclose(fs.reshape(n, m // 32)[j], rs.reshape(-1), rtol=2e-3)
+    assert not ops.ffn_gate_up_silu_quantize_applies(d_wg, d_wu, 64)
+    with pytest.raises(W.RocmError, match="ffn_gate_up_silu_quantize"):
+        ops.encode_ffn_gate_up_silu_quantize(d_wg, d_wu, d_xs, d_xq, 64, d_oq, d_os)
+    for b in (d_xq, d_xs, d_oq, d_os, d_g, d_u):
+        b.free()
+    d_wg.free(), d_wu.free()

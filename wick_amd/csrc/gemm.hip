@@ -88,6 +88,10 @@ struct GemmArgs {
     float* y_more[2];
     uint32_t m_more[2];
     uint32_t tile_start[2];
+    // Gated feed-forward launch (GATED kernels only): w = gate, w_up = up, the output is the Q8_0-quantized silu(gate) * up.
+    const uint8_t* w_up;
+    int8_t* q_out;   // [n][m]
+    float* s_out;    // [n][m / 32]
 };
 
 // Makes `a` describe the weight that owns row tile `row_tile` and rebases the tile index to that weight.
@@ -162,15 +166,25 @@ __device__ __forceinline__ void dma_activations(const GemmArgs& a, StageT<NTOK>&
 //   weights      256 pairs   = 128 rows x 2 pairs             : threads 0..255, row = t >> 1, pair = t & 1
 //   activations  direct-to-LDS, see dma_activations
 //   token scales one float4 (4 blocks) per token               : threads 256..256+NTOK-1, token = t - 256
-template <int TYPE, int NTOK>
+// GATED: the tile's 128 operand rows are 64 output rows of the gate weight and the same 64 of the up weight, laid out so
+// that every wave (64 operand rows = four 16-row MFMA tiles) holds {gate rows A, gate rows B, up rows A, up rows B} of
+// the same 32 output rows: the SiLU gate and a whole Q8_0 block of its result then sit in one wave's registers.
+template <int TYPE, int NTOK, bool GATED = false>
 __device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uint32_t tok0, uint32_t kb0,
                                            StageRegs<TYPE>& r) {
     using PT = PairTraits<TYPE>;
     const uint32_t t = threadIdx.x;
     const uint32_t nb = a.k >> 5;
     if (t < 2 * BM) {
-        const uint32_t row = min(row0 + (t >> 1), a.m - 1);
-        const uint8_t* p = a.w + ((size_t)row * nb + kb0 + 2 * (t & 1u)) * (PT::BYTES / 2);
+        const uint32_t lr = t >> 1;  // operand row of the tile
+        uint32_t row = row0 + lr;
+        const uint8_t* w = a.w;
+        if constexpr (GATED) {
+            row = row0 + 32u * (lr >> 6) + 16u * ((lr >> 4) & 1u) + (lr & 15u);
+            w = (lr >> 5) & 1u ? a.w_up : a.w;
+        }
+        row = min(row, a.m - 1);
+        const uint8_t* p = w + ((size_t)row * nb + kb0 + 2 * (t & 1u)) * (PT::BYTES / 2);
         load_pair<PT::DWORDS>(p, r.w);
     } else if (t < 2 * BM + NTOK && a.xs) {  // xs is null only for the parity hook, which never scales
         const uint32_t tok = min(tok0 + (t - 2 * BM), a.n - 1);
@@ -345,15 +359,25 @@ __device__ __forceinline__ void tile_of_block(uint32_t bid, uint32_t row_tiles, 
     tok_tile = sc * S + t2 % w;
 }
 
-template <int TYPE, bool DUMP>
+// Maximum over the 16 lanes of a DPP row (lanes that share lane / 16); every lane of the row ends with it.
+__device__ __forceinline__ float row_max16(float v) {
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false)));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false)));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false)));  // row_half_mirror
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false)));  // row_mirror
+    return v;
+}
+
+template <int TYPE, bool DUMP, bool GATED = false>
 __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
+    static_assert(!(DUMP && GATED), "the parity hook dumps plain projections");
     __shared__ Smem sm;
     uint32_t row_tile, tok_tile;
     bool valid_tile;
     tile_of_block(blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
     if (!valid_tile) return;  // whole workgroup leaves together
-    select_weight(a, row_tile);
-    const uint32_t row0 = row_tile * BM;
+    if constexpr (!GATED) select_weight(a, row_tile);
+    const uint32_t row0 = row_tile * (GATED ? BM / 2 : BM);  // GATED: 64 output rows per tile, see load_stage
     const uint32_t tok0 = tok_tile * BN;
 
     const uint32_t lane = threadIdx.x & 63u;
@@ -378,7 +402,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
 
     StageRegs<TYPE> regs;
     dma_activations(a, sm.st[0], tok0, 0);
-    load_stage<TYPE, BN>(a, row0, tok0, 0, regs);
+    load_stage<TYPE, BN, GATED>(a, row0, tok0, 0, regs);
     store_stage<TYPE, BN>(sm.st[0], regs);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
     __syncthreads();
@@ -389,7 +413,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
             // the other LDS stage was last read in stage st-1 and every wave has passed the
             // barrier that ended it, so it can be refilled from here on
             dma_activations(a, sm.st[(st + 1) & 1u], tok0, (st + 1) * KB);
-            load_stage<TYPE, BN>(a, row0, tok0, (st + 1) * KB, regs);
+            load_stage<TYPE, BN, GATED>(a, row0, tok0, (st + 1) * KB, regs);
         }
 
         // 8 MFMA tiles per block, software-pipelined by hand: four result buffers, the matrix
@@ -449,7 +473,30 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
         __syncthreads();
     }
 
-    if constexpr (!DUMP) {
+    if constexpr (GATED) {
+        // silu(gate) * up and the Q8_0 quantizer on the wave's registers, element for element what silu_mul_quantize_kernel
+        // computes from the two float results: row tiles 0 / 1 are gate rows A / B, 2 / 3 the same rows of up; the 16 lanes
+        // of a DPP row hold the 16 rows of a tile for the same four tokens, so one row reduction gives a block's maximum.
+        static_assert(RT == 4, "two gate and two up row tiles per wave");
+        const uint32_t rbase = row0 + (wrow0 >> 1);  // first of this wave's 32 output rows = one Q8_0 block
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t tok = tok0 + wtok0 + 16 * tt + 4 * kq + r;
+                const float ha = silu_mul(acc[tt][0][r], acc[tt][2][r]), hb = silu_mul(acc[tt][1][r], acc[tt][3][r]);
+                const float amax = row_max16(fmaxf(fabsf(ha), fabsf(hb)));
+                float id;
+                const float scale = q8_scale_and_inverse(amax, id);
+                const int qa = (int)__builtin_rintf(__fmul_rn(ha, id)), qb = (int)__builtin_rintf(__fmul_rn(hb, id));
+                if (tok < a.n && rbase < a.m) {  // m % 32 == 0: a block is inside the matrix or not at all
+                    int8_t* dst = a.q_out + (size_t)tok * a.m + rbase;
+                    dst[l16] = (int8_t)qa;
+                    dst[16 + l16] = (int8_t)qb;
+                    if (l16 == 0) a.s_out[(size_t)tok * (a.m >> 5) + (rbase >> 5)] = scale;
+                }
+            }
+    } else if constexpr (!DUMP) {
 #pragma unroll
         for (int tt = 0; tt < TT; tt++)
 #pragma unroll
@@ -655,6 +702,30 @@ hipError_t launch_gemm_mfma_multi(int type, const uint8_t* const* d_w, const uin
     a.accumulate = accumulate;
     for (uint32_t i = 1; i < count; i++) a.w_more[i - 1] = d_w[i], a.y_more[i - 1] = d_y[i], a.m_more[i - 1] = m[i];
     return launch<false>(type, a, L, count - 1);
+}
+
+// Gate and up projection of a feed-forward block over n tokens in one launch whose epilogue applies the SiLU gate and
+// quantizes: out = Q8_0(silu(W_gate x) * (W_up x)), [n][m] quants + [n][m / 32] scales, bit-identical to the two
+// projections + silu_mul_quantize_kernel.  The float projections (2 * n * m * 4 bytes) are never written.
+bool gemm_gated_applies(uint32_t m, uint32_t n, uint32_t k) {
+    // wide tiles only (the narrow kernel's waves own 16 rows: no block in one wave), and enough of them to fill the chip
+    return m % 32u == 0 && k % 128u == 0 && n > BN_NARROW && (uint64_t)((m + 63u) / 64u) * ((n + BN - 1) / BN) > 256u;
+}
+
+hipError_t launch_gemm_mfma_gated(int type, const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t m, uint32_t k, const int8_t* d_q,
+                                  const float* d_scales, uint32_t n, int8_t* d_out_q, float* d_out_scales, const Launch& L) {
+    if (m == 0 || n == 0) return hipSuccess;
+    if (!gemm_gated_applies(m, n, k)) return hipErrorInvalidValue;
+    GemmArgs a{};
+    a.w = d_w_gate, a.w_up = d_w_up, a.xq = d_q, a.xs = d_scales, a.q_out = d_out_q, a.s_out = d_out_scales;
+    a.m = m, a.n = n, a.k = k;
+    a.row_tiles = (m + 63u) / 64u;
+    a.tok_tiles = (n + BN - 1) / BN;
+    a.tile_start[0] = a.tile_start[1] = UINT32_MAX;
+    if ((uint64_t)a.row_tiles * a.tok_tiles > 0x7fffff00ull) return hipErrorInvalidValue;
+    const uint32_t blocks = ((a.row_tiles * a.tok_tiles + 7u) / 8u) * 8u;
+    if (type == kTypeQ4_0) return launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, false, true>, dim3(blocks), dim3(THREADS), a);
+    return launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, false, true>, dim3(blocks), dim3(THREADS), a);
 }
 
 // Parity hook through the matrix-core path: the same loads, unpack, LDS layout and

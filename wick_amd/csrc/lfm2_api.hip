@@ -124,6 +124,27 @@ int wick_rocm_attention_prefill_quantize_q8_0(wick_rocm_ctx* ctx, const float* d
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "attention_prefill_quantize launch");
 }
 
+int wick_rocm_ffn_gate_up_silu_quantize_applies(const wick_rocm_weight* w_gate, const wick_rocm_weight* w_up, uint32_t n) {
+    if (!w_gate || !w_up || !w_gate->d || !w_up->d) return 0;
+    if (w_gate->type != w_up->type || (w_gate->type != kTypeQ4_0 && w_gate->type != kTypeQ8_0)) return 0;
+    if (w_gate->m != w_up->m || w_gate->k != w_up->k) return 0;
+    return gemm_gated_applies(w_gate->m, n, w_gate->k) ? 1 : 0;
+}
+
+int wick_rocm_ffn_gate_up_silu_quantize_q8(wick_rocm_ctx* ctx, const wick_rocm_weight* w_gate, const wick_rocm_weight* w_up, const int8_t* d_quants,
+                                           const float* d_scales, uint32_t n, int8_t* d_out_quants, float* d_out_scales) {
+    WR_ENTER(ctx);
+    if (!w_gate || !w_up || !d_quants || !d_scales || !d_out_quants || !d_out_scales)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "ffn_gate_up_silu_quantize: null argument");
+    if (!wick_rocm_ffn_gate_up_silu_quantize_applies(w_gate, w_up, n) || misaligned(d_quants, 16) || misaligned(d_scales, 16))
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE,
+                    "ffn_gate_up_silu_quantize: needs two Q4_0 or two Q8_0 weights of one shape, m % 32 == 0, k % 128 == 0, n > 64, more than 256 "
+                    "tiles and 16-byte aligned activations (use gemm_q8_multi + silu_mul_quantize_q8_0)");
+    hipError_t e = launch_gemm_mfma_gated(w_gate->type, static_cast<const uint8_t*>(w_gate->d), static_cast<const uint8_t*>(w_up->d), w_gate->m, w_gate->k,
+                                          d_quants, d_scales, n, d_out_quants, d_out_scales, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "ffn_gate_up_silu_quantize launch");
+}
+
 int wick_rocm_shortconv_seq(wick_rocm_ctx* ctx, const float* d_proj, float* d_buffer, const float* d_conv_weight, float* d_out, uint32_t hidden,
                             uint32_t kernel_size, uint32_t n) {
     WR_ENTER(ctx);
@@ -262,8 +283,8 @@ struct wick_rocm_lfm2 {
     unsigned long long* d_argmax_partial = nullptr;
     // prompt (prefill) buffers for up to `prefill_cap` tokens, allocated by the first prefill
     uint32_t prefill_cap = 0;
-    float *pX = nullptr, *pA = nullptr, *pG = nullptr, *pGate = nullptr, *pUp = nullptr, *pS = nullptr, *pAttn = nullptr;
-    int8_t* pQ = nullptr;
+    float *pX = nullptr, *pA = nullptr, *pG = nullptr, *pGate = nullptr, *pUp = nullptr, *pS = nullptr, *pS2 = nullptr, *pAttn = nullptr;
+    int8_t *pQ = nullptr, *pQ2 = nullptr;
     uint32_t* pTokens = nullptr;
     wick_rocm_graph *g_logits = nullptr, *g_greedy = nullptr;
     bool use_graph = true;
@@ -435,6 +456,7 @@ int ensure_prefill_buffers(wick_rocm_ctx* ctx, wick_rocm_lfm2* m) {
     if ((rc = alloc_t(ctx, m, P * hs, &m->pX)) || (rc = alloc_t(ctx, m, P * 3 * hs, &m->pA)) ||
         (rc = alloc_t(ctx, m, P * hs, &m->pG)) || (rc = alloc_t(ctx, m, P * inter, &m->pGate)) || (rc = alloc_t(ctx, m, P * inter, &m->pUp)) ||
         (rc = alloc_t(ctx, m, P * wide, &m->pQ)) || (rc = alloc_t(ctx, m, P * (wide / 32), &m->pS)) ||
+        (rc = alloc_t(ctx, m, P * inter, &m->pQ2)) || (rc = alloc_t(ctx, m, P * (inter / 32), &m->pS2)) ||
         (rc = alloc_t(ctx, m, attention_prefill_scratch_floats((uint32_t)P, c.n_heads, (uint32_t)hd), &m->pAttn)) ||
         (rc = alloc_t(ctx, m, P, &m->pTokens)))
         return rc;
@@ -512,6 +534,12 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
         if (!quantized && (rc = wick_rocm_quantize_q8_0(ctx, m->pG, n, hs, hs, m->pQ, m->pS))) break;
         if ((rc = gemm(ctx, L.n_kv == 0 ? L.out_proj : L.o, m, n, m->pX, hs, 1))) break;  // hidden += out projection
         if ((rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.ffn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
+        if (wick_rocm_ffn_gate_up_silu_quantize_applies(L.gate, L.up, n)) {
+            // gate, up, SiLU gate and the down projection's quantizer in one launch; its output cannot overwrite its own input
+            if ((rc = wick_rocm_ffn_gate_up_silu_quantize_q8(ctx, L.gate, L.up, m->pQ, m->pS, n, m->pQ2, m->pS2))) break;
+            rc = wick_rocm_gemm_q8(ctx, L.down, m->pQ2, m->pS2, n, m->pX, hs, WICK_ROCM_LAYOUT_TOKEN_MAJOR, 1);
+            continue;
+        }
         if ((rc = gemm_group(ctx, {L.gate, L.up}, {m->pGate, m->pUp}, m, n, inter))) break;
         if ((rc = wick_rocm_silu_mul_quantize_q8_0(ctx, m->pGate, m->pUp, n, inter, m->pQ, m->pS))) break;
         rc = gemm(ctx, L.down, m, n, m->pX, hs, 1);

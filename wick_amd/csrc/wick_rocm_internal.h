@@ -130,6 +130,10 @@ hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k
 hipError_t launch_gemm_mfma_multi(int type, const uint8_t* const* d_w, const uint32_t* m, uint32_t count, uint32_t k, const int8_t* d_q,
                                   const float* d_scales, uint32_t n, float* const* d_y, uint32_t y_stride, int y_layout, int accumulate,
                                   const Launch& L);
+// out = Q8_0(silu(W_gate x) * (W_up x)) over n tokens in one launch (wide tiles only: gemm_gated_applies).
+bool gemm_gated_applies(uint32_t m, uint32_t n, uint32_t k);
+hipError_t launch_gemm_mfma_gated(int type, const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t m, uint32_t k, const int8_t* d_q,
+                                  const float* d_scales, uint32_t n, int8_t* d_out_q, float* d_out_scales, const Launch& L);
 
 // Per-block i32 dots, out[(j*m + i)*nb + b], through the GEMM's loads / LDS layout / MFMA (k % 128 == 0).
 // Register-only instruction-rate probes (probe.hip): shape 0 = v_mfma_i32_32x32x32_i8, 1 = v_mfma_i32_16x16x32_i8,

@@ -30,6 +30,8 @@ _SIGNATURES = {
     "wick_rocm_attention_prefill_quantize_q8_0": (C.c_int, [_P, _P, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _U32]),
     "wick_rocm_shortconv_seq": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32, _U32]),
     "wick_rocm_shortconv_seq_quantize_q8_0": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _U32, _U32]),
+    "wick_rocm_ffn_gate_up_silu_quantize_applies": (C.c_int, [_P, _P, _U32]),
+    "wick_rocm_ffn_gate_up_silu_quantize_q8": (C.c_int, [_P, _P, _P, _P, _P, _U32, _P, _P]),
     "wick_rocm_qk_norm_rope_tokens": (C.c_int, [_P, _P, _U32, _P, _P, _U32, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _U32, _F, _F]),
     "wick_rocm_rope_theta_scale": (_F, [_U32, _F]),
     "wick_rocm_attention_decode": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _P, _U32, _U32, _U32, _U32]),
@@ -137,6 +139,14 @@ class Lfm2Ops:
         """encode_conv1d_seq with the result written as Q8_0 blocks."""
         self.ctx._check(self._l.wick_rocm_shortconv_seq_quantize_q8_0(self.ctx._h, _ptr(proj), _ptr(buffer), _ptr(conv_weight), _ptr(out_q),
                                                                       _ptr(out_scales), hidden, kernel_size, n))
+
+    def ffn_gate_up_silu_quantize_applies(self, w_gate: RocmWeight, w_up: RocmWeight, n: int) -> bool:
+        return bool(self._l.wick_rocm_ffn_gate_up_silu_quantize_applies(w_gate.handle, w_up.handle, n))
+
+    def encode_ffn_gate_up_silu_quantize(self, w_gate: RocmWeight, w_up: RocmWeight, scales, quants, n: int, out_q, out_scales) -> None:
+        """Q8_0(silu(W_gate x) * (W_up x)) for n quantized activation rows: gate / up GEMM with the gate and the quantizer in its epilogue."""
+        self.ctx._check(self._l.wick_rocm_ffn_gate_up_silu_quantize_q8(self.ctx._h, w_gate.handle, w_up.handle, _ptr(quants), _ptr(scales), n,
+                                                                       _ptr(out_q), _ptr(out_scales)))
 
     def shortconv_fusable(self, w_out: RocmWeight, w_gate: RocmWeight, w_up: RocmWeight, kernel_size: int) -> bool:
         return bool(self._l.wick_rocm_shortconv_fusable(w_out.handle, w_gate.handle, w_up.handle, kernel_size))
