@@ -528,8 +528,49 @@ def bench_prefill_sites(ctx, W, O, n=4096, dtype=8):
     for name in ("attn_k", "attn_v"):
         r = bench_gemm(ctx, W, O, dtype, dims[name][0], n, dims[name][1], reps=3, wb=blobs[name], samples=5)
         alone.append({"site": name, "m": dims[name][0], "gemm_kernel_ms": r["gemm_kernel_ms"], "TOPS": r["gemm_kernel_TOPS"]})
-    return {"n": n, "dtype": dtype, "launches": out, "k_v_on_their_own": alone, "total_ops": tot_ops, "total_gemm_ms": tot_ms,
-            "TOPS": tot_ops / tot_ms / 1e9}
+    res = {"n": n, "dtype": dtype, "launches": out, "k_v_on_their_own": alone, "total_ops": tot_ops, "total_gemm_ms": tot_ms,
+           "TOPS": tot_ops / tot_ms / 1e9}
+    res["ffn_gate_up_to_q8"] = [bench_gate_up_fused(ctx, W, O, dtype, is_, hs, n, blobs["ffn_gate"], blobs["ffn_up"]),
+                                bench_gate_up_fused(ctx, W, O, W.Q4_0, 4608, 1024, 2002), bench_gate_up_fused(ctx, W, O, W.Q8_0, 4608, 1024, 2002),
+                                bench_gate_up_fused(ctx, W, O, W.Q4_0, 6912, 2048, 2002), bench_gate_up_fused(ctx, W, O, W.Q4_0, 6912, 1024, 2002),
+                                bench_gate_up_fused(ctx, W, O, W.Q4_0, 4608, 2048, 2002), bench_gate_up_fused(ctx, W, O, W.Q4_0, 4608, 2048, 1024)]
+    return res
+
+
+def bench_gate_up_fused(ctx, W, O, dtype, m, k, n, wg=None, wu=None, reps=5):
+    """gate | up of a prompt pass up to the down projection's Q8_0 input: one GEMM launch over both weights + the SiLU gate /
+    quantizer kernel, against the GEMM whose epilogue gates and quantizes (same bits).  Per-dispatch timestamps, median."""
+    from wick_amd.lfm2 import Lfm2Ops
+    ops = Lfm2Ops(ctx)
+    wg = O.synth_weight(dtype, m, k, seed=41) if wg is None else wg
+    wu = O.synth_weight(dtype, m, k, seed=42) if wu is None else wu
+    d_wg, d_wu = ctx.upload_weight(wg, dtype, m, k), ctx.upload_weight(wu, dtype, m, k)
+    s, q = O.quantize_q8_0_batch(O.fill_normal(9, 1.0, n * k), n, k)
+    d_q, d_s = ctx.to_device(q), ctx.to_device(s)
+    d_g, d_u, d_oq, d_os = ctx.alloc(n * m * 4), ctx.alloc(n * m * 4), ctx.alloc(n * m), ctx.alloc(n * (m // 32) * 4)
+
+    def separate():
+        ctx.gemm_preq_multi([d_wg, d_wu], d_s, d_q, n, [d_g, d_u], m)
+        ops.silu_mul_quantize(d_g, d_u, n, m, d_oq, d_os)
+
+    def fused():
+        ops.encode_ffn_gate_up_silu_quantize(d_wg, d_wu, d_s, d_q, n, d_oq, d_os)
+
+    out = {"dtype": dtype, "m": m, "k": k, "n": n}
+    for name, fn in (("separate_us", separate), ("fused_us", fused)):
+        fn()
+        ts = []
+        for _ in range(reps):
+            ctx.kernel_timing_begin()
+            fn()
+            kt = ctx.kernel_timing_end()
+            ts.append(sum(ms for ms, cnt in kt.values()) * 1e3)
+            out[name.replace("_us", "_gemm_us")] = kt["gemm"][0] * 1e3
+        out[name] = float(np.median(ts))
+    for b in (d_q, d_s, d_g, d_u, d_oq, d_os):
+        b.free()
+    d_wg.free(), d_wu.free()
+    return out
 
 
 def bench_lm_head_sweep(ctx, W, O, dtype=8, m=65536, k=2048, ns=(1, 4, 16, 64)):
