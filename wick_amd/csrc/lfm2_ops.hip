@@ -876,6 +876,256 @@ __global__ __launch_bounds__(256 * HALVES * KSPLIT) void attention_prefill_mfma_
     }
 }
 
+// The same launch layout with the two matrix products on the f16 matrix cores at f32 accuracy: every f32 operand x is
+// split into hi = f16(x) and lo = f16(x - hi) (22-23 significant bits together) and a product a * b is taken as
+// a_hi b_hi + a_hi b_lo + a_lo b_hi, each an exact f16 x f16 product accumulated in f32 by v_mfma_f32_16x16x32_f16 (the
+// dropped a_lo b_lo term is below 2^-22 of the product).  Three MFMAs of K = 32 in 16 cycles each replace eight f32 MFMAs
+// of K = 4 in 32 cycles each: the matrix time drops by a factor of five and the kernel becomes bound by the softmax's
+// vector work.  K tiles sit in LDS as f16 hi / lo rows, V tiles transposed ([dim][key]) so that the second product's A
+// operand (V^T: 8 keys of one dim per lane) is two 8-byte reads; the softmax weights are scaled by 2^12 before the
+// split (exact, undone at the end) so that small weights keep their bits in f16.  Slot j of lane group g stands for
+// key 4 g + j of the wave's first 16-key sub-tile (j < 4) or of its second (j >= 4) in both operands of the second
+// product, which is again exactly how the first product leaves the weights in the registers.
+#ifndef WICK_PROMPT_ATTENTION_F16X3
+#define WICK_PROMPT_ATTENTION_F16X3 1
+#endif
+constexpr bool kPromptAttentionF16x3 = WICK_PROMPT_ATTENTION_F16X3 != 0;
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void split_f16(float x, _Float16& hi, _Float16& lo) {
+    hi = (_Float16)x;
+    lo = (_Float16)(x - (float)hi);
+}
+
+template <int HALVES>
+__global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride,
+                                                                                int8_t* q_out, float* s_out) {
+    constexpr int HD = 64, KT = 64, NT = 512 * HALVES;
+    constexpr int LDH = 72;  // f16 per LDS row: 64 + 8 (144 bytes: 16-byte aligned rows, conflict-free operand reads)
+    constexpr float kPScale = 4096.0f;
+    __shared__ __align__(16) _Float16 kbuf[2][2][KT][LDH];  // [buffer][hi | lo][key][dim]
+    __shared__ __align__(16) _Float16 vbuf[2][2][HD][LDH];  // [buffer][hi | lo][dim][key]
+    const uint32_t h = blockIdx.x;
+    const uint32_t qblocks = (n + 63u) / 64u;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
+    const uint32_t wave_id = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t wave = wave_id & 3u, ksp = (wave_id >> 2) & 1u, half = wave_id >> 3;
+    const uint32_t qb_long = qblocks - 1u - blockIdx.y;
+    const uint32_t qb = half == 0 ? qb_long : blockIdx.y;
+    const bool active = half == 0 || qb != qb_long;
+    const uint32_t j0 = qb * 64u;
+    const uint32_t base = a.d_pos ? *a.d_pos : pos0;
+    const uint32_t kv_dim = a.n_kv_heads * HD, kvh = h / (a.n_heads / a.n_kv_heads);
+    const float* kbase = a.k_cache + (size_t)kvh * HD;
+    const float* vbase = a.v_cache + (size_t)kvh * HD;
+    const uint32_t jq = j0 + 16u * wave + l16;
+    const uint32_t jl = jq < n ? jq : n - 1u;
+    const uint32_t pq = base + jl;
+    uint32_t wg_last = base + (qb_long * 64u + 63u < n ? qb_long * 64u + 63u : n - 1u);
+    if (wg_last >= a.max_seq) wg_last = a.max_seq - 1u;
+    const uint32_t wave_last = min(base + min(j0 + 16u * wave + 15u, n - 1u), wg_last);
+
+    // this lane's query, dims 32 s + 8 g .. + 7 of slab s, scaled and split
+    h8 qh[2], ql[2];
+    {
+        const float* qp = a.q + (size_t)jl * q_stride + (size_t)h * HD + 8u * g;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const float4 v0 = *reinterpret_cast<const float4*>(qp + 32 * s), v1 = *reinterpret_cast<const float4*>(qp + 32 * s + 4);
+            const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                _Float16 hi, lo;
+                split_f16(f[i] * a.scale, hi, lo);
+                qh[s][i] = hi, ql[s][i] = lo;
+            }
+        }
+    }
+    v4f o[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) o[c] = v4f{0.f, 0.f, 0.f, 0.f};
+    float m_run = -__builtin_inff(), l_run = 0.0f;
+
+    constexpr int C4 = HD / 4, RPP = NT / C4, NR = KT / RPP;
+    const uint32_t c4 = tid % C4, r0 = tid / C4;
+    float4 kk[NR], vv[NR];
+    auto fetch_tile = [&](uint32_t t0) {
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            const uint32_t key = min(t0 + r0 + i * RPP, wg_last);
+            kk[i] = reinterpret_cast<const float4*>(kbase + (size_t)key * kv_dim)[c4];
+            vv[i] = reinterpret_cast<const float4*>(vbase + (size_t)key * kv_dim)[c4];
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            const uint32_t key = r0 + i * RPP;
+            const float kf[4] = {kk[i].x, kk[i].y, kk[i].z, kk[i].w}, vf[4] = {vv[i].x, vv[i].y, vv[i].z, vv[i].w};
+            h4 khi, klo;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                _Float16 hi, lo;
+                split_f16(kf[j], hi, lo);
+                khi[j] = hi, klo[j] = lo;
+                split_f16(vf[j], hi, lo);
+                vbuf[buf][0][4 * c4 + j][key] = hi;
+                vbuf[buf][1][4 * c4 + j][key] = lo;
+            }
+            *reinterpret_cast<h4*>(&kbuf[buf][0][key][4 * c4]) = khi;
+            *reinterpret_cast<h4*>(&kbuf[buf][1][key][4 * c4]) = klo;
+        }
+    };
+    fetch_tile(0);
+    store_tile(0);
+    if (KT <= wg_last) fetch_tile(KT);
+    __syncthreads();
+    int cur = 0;
+    for (uint32_t t0 = 0; t0 <= wg_last; t0 += KT, cur ^= 1) {
+        const uint32_t key0 = t0 + 32u * ksp;  // this wave's 32 keys of the tile
+        if (active && key0 <= wave_last) {
+            // scores: 2 sub-tiles of 16 keys x 2 slabs of 32 dims x 3 products
+            v4f sc[2] = {v4f{0.f, 0.f, 0.f, 0.f}, v4f{0.f, 0.f, 0.f, 0.f}};
+            h8 kh[2][2], kl[2][2];  // [slab][sub-tile]
+#pragma unroll
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    kh[s][u] = *reinterpret_cast<const h8*>(&kbuf[cur][0][32u * ksp + 16 * u + l16][32 * s + 8 * g]);
+                    kl[s][u] = *reinterpret_cast<const h8*>(&kbuf[cur][1][32u * ksp + 16 * u + l16][32 * s + 8 * g]);
+                }
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+#pragma unroll
+                for (int u = 0; u < 2; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kl[s][u], qh[s], sc[u], 0, 0, 0);
+#pragma unroll
+                for (int u = 0; u < 2; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh[s][u], ql[s], sc[u], 0, 0, 0);
+#pragma unroll
+                for (int u = 0; u < 2; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh[s][u], qh[s], sc[u], 0, 0, 0);
+            }
+            // the V operands of the second product are on their way while the softmax runs
+            h8 vh[4], vl[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const h4 a0 = *reinterpret_cast<const h4*>(&vbuf[cur][0][16 * c + l16][32u * ksp + 4 * g]);
+                const h4 a1 = *reinterpret_cast<const h4*>(&vbuf[cur][0][16 * c + l16][32u * ksp + 16 + 4 * g]);
+                const h4 b0 = *reinterpret_cast<const h4*>(&vbuf[cur][1][16 * c + l16][32u * ksp + 4 * g]);
+                const h4 b1 = *reinterpret_cast<const h4*>(&vbuf[cur][1][16 * c + l16][32u * ksp + 16 + 4 * g]);
+                vh[c] = h8{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                vl[c] = h8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+            }
+            float tmax = -__builtin_inff();
+            const bool masked_tile = key0 + 31u > base + min(j0 + 16u * wave, n - 1u);
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (masked_tile && key0 + 16u * u + 4u * g + r > pq) sc[u][r] = -__builtin_inff();
+                    tmax = fmaxf(tmax, sc[u][r]);
+                }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+            const float m_new = fmaxf(m_run, tmax);
+            const float m_sub = m_new == -__builtin_inff() ? 0.0f : m_new;
+            const float alpha = ggml_expf_nonpos(m_run - m_sub);
+            m_run = m_new;
+            float psum = 0.0f;
+            h8 ph, pl;
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float pw = ggml_expf_nonpos(sc[u][r] - m_sub);
+                    psum += pw;
+                    _Float16 hi, lo;
+                    split_f16(pw * kPScale, hi, lo);
+                    ph[4 * u + r] = hi, pl[4 * u + r] = lo;
+                }
+            l_run = l_run * alpha + psum;
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[c] *= alpha;
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vl[c], ph, o[c], 0, 0, 0);
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vh[c], pl, o[c], 0, 0, 0);
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vh[c], ph, o[c], 0, 0, 0);
+        }
+        if (t0 + KT <= wg_last) {
+            store_tile(cur ^ 1);
+            if (t0 + 2 * KT <= wg_last) fetch_tile(t0 + 2 * KT);
+        }
+        __syncthreads();
+    }
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+    {
+        // the upper-key waves hand (maximum, weight sum, weighted values) to their partners through the K buffers
+        constexpr int NS = 18;
+        static_assert(sizeof(kbuf) >= sizeof(float) * NS * 64 * 4 * HALVES, "K buffers hold the partner states");
+        float* xch = reinterpret_cast<float*>(&kbuf[0][0][0][0]) + (size_t)(half * 4u + wave) * NS * 64u + lane;
+        if (ksp == 1) {
+            xch[0] = m_run, xch[64] = l_run;
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) xch[(2 + 4 * c + r) * 64] = o[c][r];
+        }
+        __syncthreads();
+        if (ksp == 1) return;
+        const float m_b = xch[0], l_b = xch[64];
+        const float m_all = fmaxf(m_run, m_b);
+        const float fa = ggml_expf_nonpos(m_run - m_all), fb = ggml_expf_nonpos(m_b - m_all);
+        l_run = l_run * fa + l_b * fb;
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) o[c][r] = (o[c][r] * fa + xch[(2 + 4 * c + r) * 64] * fb) * (1.0f / kPScale);
+    }
+    // register r of tile c holds dim 16 c + 4 g + r of query l16
+    if (q_out) {
+        float v[4][4];
+        float amax[2] = {0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                v[c][r] = __fdiv_rn(o[c][r], l_run);
+                amax[c >> 1] = fmaxf(amax[c >> 1], fabsf(v[c][r]));
+            }
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            amax[b] = fmaxf(amax[b], __shfl_xor(amax[b], 16));
+            amax[b] = fmaxf(amax[b], __shfl_xor(amax[b], 32));
+        }
+        if (active && jq < n) {
+            const size_t row = (size_t)jq * a.n_heads * HD + (size_t)h * HD;
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                float id;
+                const float scale = q8_scale_and_inverse(amax[b], id);
+#pragma unroll
+                for (int cc = 0; cc < 2; cc++) {
+                    const int c = 2 * b + cc;
+                    *reinterpret_cast<uint32_t*>(q_out + row + 16 * c + 4 * g) = q8_pack4(v[c][0], v[c][1], v[c][2], v[c][3], id);
+                }
+                if (g == 0) s_out[(row >> 5) + b] = scale;
+            }
+        }
+        return;
+    }
+    if (active && jq < n) {
+        float* dst = a.out + (size_t)jq * out_stride + (size_t)h * HD;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            float4 v;
+            v.x = __fdiv_rn(o[c][0], l_run), v.y = __fdiv_rn(o[c][1], l_run), v.z = __fdiv_rn(o[c][2], l_run), v.w = __fdiv_rn(o[c][3], l_run);
+            *reinterpret_cast<float4*>(dst + 16 * c + 4 * g) = v;
+        }
+    }
+}
+
 // ---- gated short convolution, one step ---------------------------------------------------
 // forward_conv_block's middle (wick/src/model/lfm2.rs:694-726): proj = [b | c | x]; bx = b*x;
 // out = c * (sum_k buffer[k][ch]*w[ch][k] + bx*w[ch][K-1]); the rolling buffer shifts by one slot and takes bx.
@@ -1321,6 +1571,13 @@ hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, co
     if (d_q8 && !(aligned && attention_prefill_quantize_applies(d_q, d_k_cache, d_v_cache, n, q_stride, head_dim))) return hipErrorInvalidValue;
     if (head_dim == 64 && aligned && n >= 16) {
         const uint32_t qblocks = (n + 63u) / 64u;
+        if (kPromptAttentionF16x3) {
+            if (qblocks == 1)
+                return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<1>, dim3(n_heads, 1), dim3(512), a, pos0, n, q_stride, out_stride, d_q8,
+                                     d_q8_scales);
+            return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride,
+                                 out_stride, d_q8, d_q8_scales);
+        }
         if (qblocks == 1)
             return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 1, 2>, dim3(n_heads, 1), dim3(512), a, pos0, n, q_stride, out_stride, d_q8,
                                  d_q8_scales);
