@@ -71,8 +71,9 @@ int wick_rocm_attention_decode(wick_rocm_ctx *ctx, const float *d_q, const float
 /* Causal attention for the n tokens of a prompt whose K / V rows are already in the caches: pass B of the reference's
  * batched prefill (wick/src/model/lfm2.rs:1640-1700), i.e. for token j the decode attention above with
  * seq_len = pos0 + j + 1.  d_q: [n][q_stride] floats (a token's n_heads * head_dim query values first), d_out:
- * [n][out_stride].  head_dim 32 / 64 / 128 / 256; head_dim 64 with 16-byte aligned rows and n >= 16 runs on the f32
- * matrix cores (same products, sums in another order). */
+ * [n][out_stride].  head_dim 32 / 64 / 128 / 256; head_dim 64 with 16-byte aligned rows and n >= 16 runs on the matrix
+ * cores with every f32 operand split into two f16 halves and three exact-product MFMAs per product (f32 accuracy: measured
+ * rel-L2 2e-7 against an f64 evaluation; sums in another order than the reference's loops). */
 int wick_rocm_attention_prefill(wick_rocm_ctx *ctx, const float *d_q, uint32_t q_stride, const float *d_k_cache, const float *d_v_cache,
                                 float *d_out, uint32_t out_stride, uint32_t pos0, uint32_t n, uint32_t max_seq, uint32_t n_heads,
                                 uint32_t n_kv_heads, uint32_t head_dim);

@@ -251,7 +251,8 @@ def test_attention_decode(ctx, ops, oracle, n_heads, n_kv, hd, seq):
 ])
 def test_attention_prefill(ctx, ops, oracle, n_heads, n_kv, hd, pos0, n, pad):
     """Causal attention over a prompt (wick/src/model/lfm2.rs:1640-1700): token j == the decode attention with seq_len = pos0 + j + 1.
-    head_dim 64 runs on the f32 matrix cores: same products, sums in tiles of 64 positions."""
+    head_dim 64 runs on the matrix cores (f32 operands as f16 hi + lo, three exact-product MFMAs per product), sums in tiles of 64
+    positions."""
     kv_dim, seq_total = n_kv * hd, pos0 + n
     max_seq = seq_total + 2
     q_stride, out_stride = n_heads * hd + 2 * kv_dim + pad, n_heads * hd + pad

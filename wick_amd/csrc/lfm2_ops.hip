@@ -623,260 +623,28 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
     }
 }
 
-// The same causal attention on the f32 matrix cores (v_mfma_f32_16x16x4_f32: exact f32 products, f32 sums; only the
-// order of the sums differs from the scalar kernel above).  Four waves = 64 consecutive queries of one head, 16 per
-// wave; they walk the cache in tiles of 64 positions shared through LDS.
-//   scores, transposed:  S^T[key][q] = sum_d K[key][d] Q[q][d]   A = K (keys are the M rows), B = Q^T
-//     lane l feeds key l % 16 and query l % 16 at head dims (l / 16) * HD/4 + s, s = 0 .. HD/4 - 1 (the order of the
-//     K steps is free as long as both operands agree, so a lane's dims are contiguous: 16-byte LDS reads);
-//     in the result lane l holds keys 4 * (l / 16) + r of query l % 16.
-//   weighted values, transposed:  O^T[d][q] = sum_key V[key][d] P[key][q]   A = V^T, B = P
-//     K step s of a 16-key sub-tile takes key 4 * (l / 16) + s from lane l: exactly result register s of the score
-//     MFMA, so the softmax weights go from one MFMA into the next without leaving their registers.  A lane's A
-//     operand V[key][4 * (l % 16) + c], c = 0..3, is one 16-byte read serving the four MFMAs that own dims 4 m + c.
-// Streaming softmax per query across the tiles (running maximum shared by the four lane groups of a query through
-// two shuffles, partial sums of the weights kept per lane and added up at the end).
+// The same causal attention on the matrix cores, head_dim 64.  Sixteen queries of one head per wave; the cache is walked in
+// tiles of 64 positions that a workgroup's waves share through LDS.
+//   scores, transposed:  S^T[key][q] = sum_d K[key][d] Q[q][d]   A = K (keys are the M rows), B = Q^T;
+//     in the 16 x 16 result lane l holds keys 4 * (l / 16) + r of query l % 16.
+//   weighted values, transposed:  O^T[d][q] = sum_key V[key][d] P[key][q]   A = V^T, B = P: the B operand wants, per lane,
+//     consecutive K-steps (= keys) of one query -- exactly what the score MFMA left in the lane's registers, so the softmax
+//     weights go from one product into the next without leaving their registers (the order of an MFMA's K steps is free as
+//     long as both operands agree on it).
+// Streaming softmax per query across the tiles (running maximum shared by the four lane groups of a query, partial sums of
+// the weights kept per lane and added up at the end).
 // Causal work grows with the query's position, so with HALVES == 2 a workgroup takes two blocks of 64 queries, block
 // (last - y) and block y: every workgroup then covers the same number of (wave, tile) steps and the two blocks share
 // one copy of each K/V tile; the short block's waves drop out of the arithmetic (not the barriers) once their
-// queries are past.  Each block of 64 queries is served by 4 x KSPLIT waves: with KSPLIT == 2 a second wave per 16
-// queries takes the upper 32 keys of every tile with a softmax state of its own, and the two states are merged at the
-// end through LDS -- four waves per SIMD while both blocks run and two when only the long one is left, so that one
-// wave's exp / rescale work overlaps another's MFMAs.  The next tile's K/V rows are fetched into registers while the
-// current one is being multiplied.
+// queries are past.  Each block of 64 queries is served by 8 waves: a second wave per 16 queries takes the upper 32
+// keys of every tile with a softmax state of its own, and the two states are merged at the end through LDS -- four
+// waves per SIMD while both blocks run and two when only the long one is left, so that one wave's exp / rescale work
+// overlaps another's MFMAs.  Two tiles sit in LDS: tile t+1 is written (and tile t+2 requested) after the arithmetic
+// of tile t, into the buffer that tile t-1 left -- one barrier per tile, and no wave waits for global memory before it
+// multiplies.
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <int HD, int HALVES, int KSPLIT>
-__global__ __launch_bounds__(256 * HALVES * KSPLIT) void attention_prefill_mfma_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride,
-                                                                                        int8_t* q_out, float* s_out) {
-    constexpr int NT = 256 * HALVES * KSPLIT;
-    constexpr int KT = 64;        // positions per tile
-    constexpr int NU = 4 / KSPLIT;  // 16-key sub-tiles of a tile per wave
-    constexpr int LD = HD + 4;    // LDS row stride in floats: an odd number of 16-byte chunks, conflict-free operand reads
-    constexpr int QR = HD / 4;    // Q registers per lane = K steps of a score tile
-    constexpr int DT = HD / 16;   // 16 x 16 output tiles per MFMA group
-    static_assert(HD % 16 == 0, "head_dim must be a multiple of 16");
-    static_assert(KSPLIT == 1 || KSPLIT == 2, "one or two waves per 16 queries");
-    __shared__ __align__(16) float kv_tiles[2][2][KT][LD];  // [K | V][buffer][position][dim]
-    float (*ks)[KT][LD] = kv_tiles[0];
-    float (*vs)[KT][LD] = kv_tiles[1];
-    const uint32_t h = blockIdx.x;
-    const uint32_t qblocks = (n + 63u) / 64u;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
-    const uint32_t wave_id = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t wave = wave_id & 3u;                    // 16-query group of the block (= the SIMD, so a SIMD's waves share it)
-    const uint32_t ksp = (wave_id >> 2) & (KSPLIT - 1u);   // which keys of a tile: sub-tiles NU * ksp ..
-    const uint32_t half = wave_id / (4u * KSPLIT);         // which block of the pair
-    const uint32_t u0 = NU * ksp;
-    const uint32_t qb_long = qblocks - 1u - blockIdx.y;  // longest rows first
-    const uint32_t qb = half == 0 ? qb_long : blockIdx.y;
-    const bool active = half == 0 || qb != qb_long;      // an odd count leaves the middle block without a partner
-    const uint32_t j0 = qb * 64u;
-    const uint32_t base = a.d_pos ? *a.d_pos : pos0;
-    const uint32_t kv_dim = a.n_kv_heads * HD, kvh = h / (a.n_heads / a.n_kv_heads);
-    const float* kbase = a.k_cache + (size_t)kvh * HD;
-    const float* vbase = a.v_cache + (size_t)kvh * HD;
-    const uint32_t jq = j0 + 16u * wave + l16;           // this lane's query token
-    const uint32_t jl = jq < n ? jq : n - 1u;            // ... clamped for loads
-    const uint32_t pq = base + jl;                       // its position = the last key it sees
-    uint32_t wg_last = base + (qb_long * 64u + 63u < n ? qb_long * 64u + 63u : n - 1u);  // last position any query of the workgroup sees
-    if (wg_last >= a.max_seq) wg_last = a.max_seq - 1u;
-    const uint32_t wave_last = min(base + min(j0 + 16u * wave + 15u, n - 1u), wg_last);
-
-    float qr[QR];
-    {
-        const float4* qp = reinterpret_cast<const float4*>(a.q + (size_t)jl * q_stride + (size_t)h * HD + (size_t)g * QR);
-#pragma unroll
-        for (int i = 0; i < QR / 4; i++) {
-            const float4 v = qp[i];
-            qr[4 * i] = v.x * a.scale, qr[4 * i + 1] = v.y * a.scale, qr[4 * i + 2] = v.z * a.scale, qr[4 * i + 3] = v.w * a.scale;
-        }
-    }
-    v4f o[DT];
-#pragma unroll
-    for (int c = 0; c < DT; c++) o[c] = v4f{0.f, 0.f, 0.f, 0.f};
-    float m_run = -__builtin_inff(), l_run = 0.0f;
-
-    constexpr int C4 = HD / 4, RPP = NT / C4, NR = KT / RPP;  // float4 columns, rows per pass, passes
-    const uint32_t c4 = tid % C4, r0 = tid / C4;
-    float4 kk[NR], vv[NR];
-    auto fetch_tile = [&](uint32_t t0) {
-#pragma unroll
-        for (int i = 0; i < NR; i++) {
-            const uint32_t key = min(t0 + r0 + i * RPP, wg_last);
-            kk[i] = reinterpret_cast<const float4*>(kbase + (size_t)key * kv_dim)[c4];
-            vv[i] = reinterpret_cast<const float4*>(vbase + (size_t)key * kv_dim)[c4];
-        }
-    };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < NR; i++) {
-            *reinterpret_cast<float4*>(&ks[buf][r0 + i * RPP][4 * c4]) = kk[i];
-            *reinterpret_cast<float4*>(&vs[buf][r0 + i * RPP][4 * c4]) = vv[i];
-        }
-    };
-    // Two tiles in LDS: tile t+1 is written (and tile t+2 requested) after the arithmetic of tile t, into the buffer
-    // that tile t-1 left -- one barrier per tile, and no wave waits for global memory before it multiplies.
-    fetch_tile(0);
-    store_tile(0);
-    if (KT <= wg_last) fetch_tile(KT);
-    __syncthreads();
-    int cur = 0;
-    for (uint32_t t0 = 0; t0 <= wg_last; t0 += KT, cur ^= 1) {
-        if (active && t0 + 16u * u0 <= wave_last) {  // else: every query of this wave ends before its keys of the tile (it still stages tiles and meets the barriers)
-            const float (*ks_t)[LD] = ks[cur] + 16u * u0;  // this wave's keys of the tile
-            const float (*vs_t)[LD] = vs[cur] + 16u * u0;
-            const uint32_t key0 = t0 + 16u * u0;
-            // scores of NU sub-tiles x 16 keys.  The accumulators take turns so that no MFMA waits for the one before it,
-            // and the operands of the next group of MFMAs are read while the current group runs (the fences keep that order).
-            v4f sc[NU];
-#pragma unroll
-            for (int u = 0; u < NU; u++) sc[u] = v4f{0.f, 0.f, 0.f, 0.f};
-            float4 kq[2][NU];
-#pragma unroll
-            for (int u = 0; u < NU; u++) kq[0][u] = *reinterpret_cast<const float4*>(&ks_t[16 * u + l16][g * QR]);
-#pragma unroll
-            for (int i = 0; i < QR / 4; i++) {
-                if (i + 1 < QR / 4) {
-#pragma unroll
-                    for (int u = 0; u < NU; u++) kq[(i + 1) & 1][u] = *reinterpret_cast<const float4*>(&ks_t[16 * u + l16][g * QR + 4 * (i + 1)]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int u = 0; u < NU; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].x, qr[4 * i], sc[u], 0, 0, 0);
-#pragma unroll
-                for (int u = 0; u < NU; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].y, qr[4 * i + 1], sc[u], 0, 0, 0);
-#pragma unroll
-                for (int u = 0; u < NU; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].z, qr[4 * i + 2], sc[u], 0, 0, 0);
-#pragma unroll
-                for (int u = 0; u < NU; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[i & 1][u].w, qr[4 * i + 3], sc[u], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // causal mask + tile maximum of this lane's query
-            float tmax = -__builtin_inff();
-            const bool masked_tile = key0 + 16u * NU - 1u > base + min(j0 + 16u * wave, n - 1u);  // some key of these is past some query of the wave
-#pragma unroll
-            for (int u = 0; u < NU; u++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    if (masked_tile && key0 + 16u * u + 4u * g + r > pq) sc[u][r] = -__builtin_inff();
-                    tmax = fmaxf(tmax, sc[u][r]);
-                }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-            const float m_new = fmaxf(m_run, tmax);
-            // a query that has seen no key yet (only in a wave that takes the upper keys) keeps weights and sums at 0
-            const float m_sub = m_new == -__builtin_inff() ? 0.0f : m_new;
-            const float alpha = ggml_expf_nonpos(m_run - m_sub);  // first keys: exp(-inf) = 0, nothing to rescale
-            m_run = m_new;
-            float psum = 0.0f;
-#pragma unroll
-            for (int u = 0; u < NU; u++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const float pw = ggml_expf_nonpos(sc[u][r] - m_sub);  // masked keys: exp(-inf) = 0
-                    sc[u][r] = pw;
-                    psum += pw;
-                }
-            l_run = l_run * alpha + psum;
-#pragma unroll
-            for (int c = 0; c < DT; c++) o[c] *= alpha;
-            // O^T += V^T P, the V reads four keys ahead of their MFMAs (sched_group_barrier: 0x100 = LDS read, 0x008 = MFMA)
-#pragma unroll
-            for (int u = 0; u < NU; u++)
-#pragma unroll
-                for (int sidx = 0; sidx < 4; sidx++) {
-                    const float pv = sc[u][sidx];
-#pragma unroll
-                    for (int c4 = 0; c4 < DT / 4; c4++) {
-                        const float4 vq = *reinterpret_cast<const float4*>(&vs_t[16 * u + 4 * g + sidx][16 * c4 * 4 + 4 * l16]);
-                        o[4 * c4 + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.x, pv, o[4 * c4 + 0], 0, 0, 0);
-                        o[4 * c4 + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.y, pv, o[4 * c4 + 1], 0, 0, 0);
-                        o[4 * c4 + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.z, pv, o[4 * c4 + 2], 0, 0, 0);
-                        o[4 * c4 + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq.w, pv, o[4 * c4 + 3], 0, 0, 0);
-                    }
-                }
-            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-            for (int i = 0; i < NU * DT - 4; i++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
-        }
-        if (t0 + KT <= wg_last) {
-            store_tile(cur ^ 1);
-            if (t0 + 2 * KT <= wg_last) fetch_tile(t0 + 2 * KT);
-        }
-        __syncthreads();
-    }
-    // the weight sums of a query's four lane groups
-    l_run += __shfl_xor(l_run, 16);
-    l_run += __shfl_xor(l_run, 32);
-    if constexpr (KSPLIT == 2) {
-        // the upper-key waves hand (maximum, weight sum, weighted values) to their partners through the tile buffers,
-        // which nobody reads any more (the loop ends on a barrier)
-        constexpr int NS = 2 + 4 * DT;  // floats per lane
-        static_assert(sizeof(kv_tiles) >= sizeof(float) * NS * 64 * 4 * HALVES, "tile buffers hold the partner states");
-        float* xch = &kv_tiles[0][0][0][0] + (size_t)(half * 4u + wave) * NS * 64u + lane;
-        if (ksp == 1) {
-            xch[0] = m_run, xch[64] = l_run;
-#pragma unroll
-            for (int c = 0; c < DT; c++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) xch[(2 + 4 * c + r) * 64] = o[c][r];
-        }
-        __syncthreads();
-        if (ksp == 1) return;
-        const float m_b = xch[0], l_b = xch[64];
-        const float m_all = fmaxf(m_run, m_b);  // finite: key 0 is visible to every query and belongs to this wave
-        const float fa = ggml_expf_nonpos(m_run - m_all), fb = ggml_expf_nonpos(m_b - m_all);  // fb = 0 if the partner saw no key
-        l_run = l_run * fa + l_b * fb;
-#pragma unroll
-        for (int c = 0; c < DT; c++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) o[c][r] = o[c][r] * fa + xch[(2 + 4 * c + r) * 64] * fb;
-    }
-    if (q_out) {
-        // Q8_0 blocks of the result instead of floats (what the output projection consumes): a lane holds 16 consecutive
-        // dims of its query, two neighbouring lane groups one 32-dim block.  Rows are n_heads * HD wide, no padding.
-        static_assert(HD == 64, "the quantizing epilogue is written for one 64-dim head = two blocks");
-        float v[4][4];
-        float amax = 0.0f;
-#pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                v[r][c] = __fdiv_rn(o[c][r], l_run);
-                amax = fmaxf(amax, fabsf(v[r][c]));
-            }
-        amax = fmaxf(amax, __shfl_xor(amax, 16));
-        float id;
-        const float scale = q8_scale_and_inverse(amax, id);
-        if (active && jq < n) {
-            const size_t row = (size_t)jq * a.n_heads * HD + (size_t)h * HD;
-#pragma unroll
-            for (int r = 0; r < 4; r++) reinterpret_cast<uint32_t*>(q_out + row + 16 * g)[r] = q8_pack4(v[r][0], v[r][1], v[r][2], v[r][3], id);
-            if ((g & 1u) == 0) s_out[(row >> 5) + (g >> 1)] = scale;
-        }
-        return;
-    }
-    if (active && jq < n) {
-        // tile c4*4 + c, register r of lane (l16, g) holds dim 64 * c4 + 4 * (4 * g + r) + c of query l16
-        float* dst = a.out + (size_t)jq * out_stride + (size_t)h * HD;
-#pragma unroll
-        for (int c4 = 0; c4 < DT / 4; c4++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                float4 v;
-                v.x = __fdiv_rn(o[4 * c4 + 0][r], l_run), v.y = __fdiv_rn(o[4 * c4 + 1][r], l_run);
-                v.z = __fdiv_rn(o[4 * c4 + 2][r], l_run), v.w = __fdiv_rn(o[4 * c4 + 3][r], l_run);
-                *reinterpret_cast<float4*>(dst + 64 * c4 + 16 * g + 4 * r) = v;
-            }
-    }
-}
-
-// The same launch layout with the two matrix products on the f16 matrix cores at f32 accuracy: every f32 operand x is
+// Both products run on the f16 matrix cores at f32 accuracy: every f32 operand x is
 // split into hi = f16(x) and lo = f16(x - hi) (22-23 significant bits together) and a product a * b is taken as
 // a_hi b_hi + a_hi b_lo + a_lo b_hi, each an exact f16 x f16 product accumulated in f32 by v_mfma_f32_16x16x32_f16 (the
 // dropped a_lo b_lo term is below 2^-22 of the product).  Three MFMAs of K = 32 in 16 cycles each replace eight f32 MFMAs
@@ -886,10 +654,6 @@ __global__ __launch_bounds__(256 * HALVES * KSPLIT) void attention_prefill_mfma_
 // split (exact, undone at the end) so that small weights keep their bits in f16.  Slot j of lane group g stands for
 // key 4 g + j of the wave's first 16-key sub-tile (j < 4) or of its second (j >= 4) in both operands of the second
 // product, which is again exactly how the first product leaves the weights in the registers.
-#ifndef WICK_PROMPT_ATTENTION_F16X3
-#define WICK_PROMPT_ATTENTION_F16X3 1
-#endif
-constexpr bool kPromptAttentionF16x3 = WICK_PROMPT_ATTENTION_F16X3 != 0;
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 
@@ -898,14 +662,35 @@ __device__ __forceinline__ void split_f16(float x, _Float16& hi, _Float16& lo) {
     lo = (_Float16)(x - (float)hi);
 }
 
+// Reductions over the four lane groups of a query (lanes l, l ^ 16, l ^ 32, l ^ 48) with gfx950's row / half swaps: swapping a
+// register with a copy of itself leaves the two partners' values in the pair, so their maximum (or sum) needs no select
+// and no trip through the LDS crossbar.  Every lane ends with the result.
+__device__ __forceinline__ float groups_max(float v) {
+    const uint32_t b = __float_as_uint(v);
+    auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    const uint32_t c = __float_as_uint(v);
+    auto q = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+    return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
+__device__ __forceinline__ float groups_sum(float v) {
+    const uint32_t b = __float_as_uint(v);
+    auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    const uint32_t c = __float_as_uint(v);
+    auto q = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+    return __uint_as_float(q[0]) + __uint_as_float(q[1]);
+}
+
 template <int HALVES>
 __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride,
                                                                                 int8_t* q_out, float* s_out) {
     constexpr int HD = 64, KT = 64, NT = 512 * HALVES;
-    constexpr int LDH = 72;  // f16 per LDS row: 64 + 8 (144 bytes: 16-byte aligned rows, conflict-free operand reads)
+    constexpr int LDH = 72;  // f16 per K row: 64 + 8 (144 bytes: 16-byte aligned rows, conflict-free 16-byte operand reads)
+    constexpr int LDV = 68;  // f16 per V^T row: 64 + 4 (136 bytes: 8-byte aligned rows; 64 rows' 8-byte writes cover all banks twice)
     constexpr float kPScale = 4096.0f;
     __shared__ __align__(16) _Float16 kbuf[2][2][KT][LDH];  // [buffer][hi | lo][key][dim]
-    __shared__ __align__(16) _Float16 vbuf[2][2][HD][LDH];  // [buffer][hi | lo][dim][key]
+    __shared__ __align__(16) _Float16 vbuf[2][2][HD][LDV];  // [buffer][hi | lo][dim][key]
     const uint32_t h = blockIdx.x;
     const uint32_t qblocks = (n + 63u) / 64u;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
@@ -958,23 +743,39 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
             vv[i] = reinterpret_cast<const float4*>(vbase + (size_t)key * kv_dim)[c4];
         }
     };
+    // A thread holds one key x four dims of K and of V.  K rows go to LDS as they are; V is transposed on the way: the four
+    // lane groups of a wave hold four consecutive keys of the same dims, so a 4 x 4 transpose across them (two rounds of
+    // row / half swaps on {hi, lo} pairs packed into one register) leaves every lane with four keys of one dim = one
+    // 8-byte write per half, instead of eight conflicting 2-byte writes.
     auto store_tile = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < NR; i++) {
             const uint32_t key = r0 + i * RPP;
             const float kf[4] = {kk[i].x, kk[i].y, kk[i].z, kk[i].w}, vf[4] = {vv[i].x, vv[i].y, vv[i].z, vv[i].w};
             h4 khi, klo;
+            uint32_t vp[4];  // V of this key: dim j as {hi, lo}
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 _Float16 hi, lo;
                 split_f16(kf[j], hi, lo);
                 khi[j] = hi, klo[j] = lo;
                 split_f16(vf[j], hi, lo);
-                vbuf[buf][0][4 * c4 + j][key] = hi;
-                vbuf[buf][1][4 * c4 + j][key] = lo;
+                vp[j] = (uint32_t)__builtin_bit_cast(uint16_t, hi) | ((uint32_t)__builtin_bit_cast(uint16_t, lo) << 16);
             }
             *reinterpret_cast<h4*>(&kbuf[buf][0][key][4 * c4]) = khi;
             *reinterpret_cast<h4*>(&kbuf[buf][1][key][4 * c4]) = klo;
+            // transpose M[g][j] (g = lane group = key, j = register = dim) in 2 x 2 blocks, then the blocks themselves
+            auto s01 = __builtin_amdgcn_permlane16_swap(vp[0], vp[1], false, false);
+            auto s23 = __builtin_amdgcn_permlane16_swap(vp[2], vp[3], false, false);
+            auto t02 = __builtin_amdgcn_permlane32_swap(s01[0], s23[0], false, false);
+            auto t13 = __builtin_amdgcn_permlane32_swap(s01[1], s23[1], false, false);
+            const uint32_t w[4] = {t02[0], t13[0], t02[1], t13[1]};  // this lane's dim 4 c4 + g, keys (key & ~3) + 0 .. 3
+            uint2 vhi, vlo;
+            vhi.x = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u), vhi.y = __builtin_amdgcn_perm(w[3], w[2], 0x05040100u);
+            vlo.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u), vlo.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
+            const uint32_t key4 = key & ~3u;
+            *reinterpret_cast<uint2*>(&vbuf[buf][0][4 * c4 + g][key4]) = vhi;
+            *reinterpret_cast<uint2*>(&vbuf[buf][1][4 * c4 + g][key4]) = vlo;
         }
     };
     fetch_tile(0);
@@ -1024,8 +825,7 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
                     if (masked_tile && key0 + 16u * u + 4u * g + r > pq) sc[u][r] = -__builtin_inff();
                     tmax = fmaxf(tmax, sc[u][r]);
                 }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+            tmax = groups_max(tmax);
             const float m_new = fmaxf(m_run, tmax);
             const float m_sub = m_new == -__builtin_inff() ? 0.0f : m_new;
             const float alpha = ggml_expf_nonpos(m_run - m_sub);
@@ -1058,8 +858,7 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
         }
         __syncthreads();
     }
-    l_run += __shfl_xor(l_run, 16);
-    l_run += __shfl_xor(l_run, 32);
+    l_run = groups_sum(l_run);
     {
         // the upper-key waves hand (maximum, weight sum, weighted values) to their partners through the K buffers
         constexpr int NS = 18;
@@ -1096,8 +895,7 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
             }
 #pragma unroll
         for (int b = 0; b < 2; b++) {
-            amax[b] = fmaxf(amax[b], __shfl_xor(amax[b], 16));
-            amax[b] = fmaxf(amax[b], __shfl_xor(amax[b], 32));
+            amax[b] = groups_max(amax[b]);
         }
         if (active && jq < n) {
             const size_t row = (size_t)jq * a.n_heads * HD + (size_t)h * HD;
@@ -1571,17 +1369,10 @@ hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, co
     if (d_q8 && !(aligned && attention_prefill_quantize_applies(d_q, d_k_cache, d_v_cache, n, q_stride, head_dim))) return hipErrorInvalidValue;
     if (head_dim == 64 && aligned && n >= 16) {
         const uint32_t qblocks = (n + 63u) / 64u;
-        if (kPromptAttentionF16x3) {
-            if (qblocks == 1)
-                return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<1>, dim3(n_heads, 1), dim3(512), a, pos0, n, q_stride, out_stride, d_q8,
-                                     d_q8_scales);
-            return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride,
-                                 out_stride, d_q8, d_q8_scales);
-        }
         if (qblocks == 1)
-            return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 1, 2>, dim3(n_heads, 1), dim3(512), a, pos0, n, q_stride, out_stride, d_q8,
+            return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<1>, dim3(n_heads, 1), dim3(512), a, pos0, n, q_stride, out_stride, d_q8,
                                  d_q8_scales);
-        return launch_kernel(L, kFamOther, attention_prefill_mfma_kernel<64, 2, 2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride,
+        return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride,
                              out_stride, d_q8, d_q8_scales);
     }
     const dim3 grid(n_heads, (n + 7u) / 8u), block(256);
