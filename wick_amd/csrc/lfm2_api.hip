@@ -534,10 +534,11 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
         if (!quantized && (rc = wick_rocm_quantize_q8_0(ctx, m->pG, n, hs, hs, m->pQ, m->pS))) break;
         if ((rc = gemm(ctx, L.n_kv == 0 ? L.out_proj : L.o, m, n, m->pX, hs, 1))) break;  // hidden += out projection
         if ((rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.ffn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
-        if (L.gate->type == kTypeQ4_0 && wick_rocm_ffn_gate_up_silu_quantize_applies(L.gate, L.up, n)) {
+        if (L.gate->type == kTypeQ4_0 && L.gate->k <= 1024 && wick_rocm_ffn_gate_up_silu_quantize_applies(L.gate, L.up, n)) {
             // gate, up, SiLU gate and the down projection's quantizer in one launch; its output cannot overwrite its own input.
-            // (Q4_0 only: measured 1-6 % faster than GEMM + gate kernel there, 11 % slower with Q8_0 weights, whose kernel is
-            // two registers over its budget.)
+            // (Where it pays, measured on one GPU against GEMM + gate kernel: Q4_0 with k = 1024 6-7 % faster; k = 2048 2-8 %
+            // slower -- the epilogue's exp / divide work sits on the vector ALU that bounds the GEMM; Q8_0, whose kernel is
+            // two registers over its budget, 11 % slower.)
             if ((rc = wick_rocm_ffn_gate_up_silu_quantize_q8(ctx, L.gate, L.up, m->pQ, m->pS, n, m->pQ2, m->pS2))) break;
             rc = wick_rocm_gemm_q8(ctx, L.down, m->pQ2, m->pS2, n, m->pX, hs, WICK_ROCM_LAYOUT_TOKEN_MAJOR, 1);
             continue;
