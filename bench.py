@@ -763,7 +763,7 @@ def main():
             "lm_head_q6k": lambda: bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024),
             "lfm2_step": lambda: bench_lfm2_step(ctx, W, O),
             "lfm2_step_q8": lambda: bench_lfm2_step(ctx, W, O, body=8, embd=8),
-            # the per-layer shapes of BASELINE's LFM2-1.2B call sites: hidden 2048, FFN 6912, 32 heads / 8 KV heads
+            # the per-layer shapes of an LFM2-1.2B: hidden 2048, FFN 6912, 32 heads / 8 KV heads
             "lfm2_step_1p2b": lambda: bench_lfm2_step(ctx, W, O, dims=dict(HS=2048, IS=6912, KV=512), label="LFM2-1.2B-shaped"),
             "lfm2_step_trace": lambda: trace_lfm2_step(ctx, W, O),
             "lfm2_prefill_trace": lambda: trace_lfm2_prefill(ctx, W, O),

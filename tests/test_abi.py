@@ -90,12 +90,12 @@ def test_product_path_does_not_import_the_oracle():
 
 
 def _documented_build():
-    """The unit lists and flags of the build.rs that INTEGRATION.md shows a maintainer."""
+    """The unit lists and flags of the build.rs shown to a maintainer in the integration notes at the repository root."""
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     lists = {}
     for name in ("HIP_UNITS", "PRELOAD_UNITS", "CPP_UNITS", "HIP_FLAGS", "PRELOAD_FLAGS", "CPP_FLAGS"):
         m = re.search(r"const " + name + r": &\[&str\] = &\[(.*?)\];", text, flags=re.S)
-        assert m, f"INTEGRATION.md: build.rs has no {name}"
+        assert m, f"the documented build.rs has no {name}"
         lists[name] = re.findall(r'"([^"]*)"', m.group(1))
     return lists
 
