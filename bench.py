@@ -734,8 +734,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline GEMV, the GEMM (+ CPU baseline)")
+    ap.add_argument("--prompt-tokens", type=int, default=2002, help="lfm2_prefill_trace: tokens of the traced prompt pass")
     ap.add_argument("--graph-only", action="store_true", help="decode legs: graph replays only, no eager launches (for kernel tracers)")
-    ap.add_argument("--leg", default="all", help="all | c1 | gemm | decode | decode_q8 | gemv | prefill_sites | lm_head | lm_head_q6k | upload | lfm2_step | lfm2_step_q8 | lfm2_step_1p2b | lfm2_step_trace | copy | probe | cpu")
+    ap.add_argument("--leg", default="all", help="all | c1 | gemm | decode | decode_q8 | gemv | prefill_sites | lm_head | lm_head_q6k | upload | lfm2_step | lfm2_step_q8 | lfm2_step_1p2b | lfm2_step_trace | lfm2_prefill_trace | copy | probe | cpu")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -766,7 +767,7 @@ def main():
             # the per-layer shapes of an LFM2-1.2B: hidden 2048, FFN 6912, 32 heads / 8 KV heads
             "lfm2_step_1p2b": lambda: bench_lfm2_step(ctx, W, O, dims=dict(HS=2048, IS=6912, KV=512), label="LFM2-1.2B-shaped"),
             "lfm2_step_trace": lambda: trace_lfm2_step(ctx, W, O),
-            "lfm2_prefill_trace": lambda: trace_lfm2_prefill(ctx, W, O),
+            "lfm2_prefill_trace": lambda: trace_lfm2_prefill(ctx, W, O, n=args.prompt_tokens),
             "copy": lambda: bench_copy(ctx),
             "upload": lambda: bench_upload(ctx),
             "probe": lambda: bench_probe(ctx),

@@ -175,6 +175,13 @@ int wick_rocm_gemm_q8_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *w
  * the reference's WICK_Q4_FAST / WICK_SPLITS switches (wick/src/backend/cpu.rs:23-27). */
 int wick_rocm_set_gemm_min_n(wick_rocm_ctx *ctx, uint32_t min_n);
 
+/* A GEMM launch that would leave at least half of the CUs without a tile while walking a long K (few tokens x few rows x
+ * k >= 2048: the down projection of a short prompt) is split over K in up to max_splits shares (1, 2, 4, 8): the shares' sums go
+ * to context scratch and a second small launch adds them up in a fixed order -- deterministic, but not the same low-order bits
+ * as the unsplit sum (both inside the f32 bar).  max_splits = 1 switches it off, 0 restores the default (8).  A tuning knob like
+ * the one above; wick_rocm_matmul_f32_noalloc never splits. */
+int wick_rocm_set_gemm_max_k_splits(wick_rocm_ctx *ctx, uint32_t max_splits);
+
 /* How the single-token GEMV fetches its weights, by bytes of weights in one launch: below
  * direct_max_bytes every lane loads its own block pair; from there on a wave loads whole
  * cache lines and redistributes them through LDS.  Negative = the built-in default (3 MiB

@@ -168,3 +168,43 @@ def test_argument_errors(ctx, oracle):
             ctx.gemm_preq(p.w, p.d_s, p.d_q, 20, d_y, y_stride=64, layout=5)
         assert e.value.status == -1
         ctx.gemm_preq(p.w, p.d_s, p.d_q, 0, d_y, y_stride=64, layout=W.LAYOUT_TOKEN_MAJOR)  # n = 0: no-op
+
+
+@pytest.mark.parametrize("dtype,m,n,k,layout,accumulate", [
+    (W.Q4_0, 1024, 512, 4608, "token", True),    # the down projection of a 512-token prompt: 64 tiles, 4 shares
+    (W.Q8_0, 1024, 100, 2048, "token", False),   # 16 tiles, 4 shares of 4 stages
+    (W.Q4_0, 300, 70, 4608, "row", True),        # ragged rows and tokens, 8 shares, row-major output
+    (W.Q8_0, 2048, 640, 6912, "token", False),   # 160 tiles: no split (would pass 256)
+    (W.Q4_0, 1024, 2002, 4608, "token", False),  # 256 tiles: no split
+])
+def test_gemm_split_over_k(ctx, oracle, dtype, m, n, k, layout, accumulate):
+    """GEMM launches with few tiles and a long K walk K in shares (one workgroup per tile and share, a second launch adds the
+    shares in a fixed order): held against the oracle like every other launch, equal to the unsplit launch to a few 1e-7,
+    and the same bits on every run."""
+    wb = oracle.synth_weight(dtype, m, k, seed=77)
+    w = ctx.upload_weight(wb, dtype, m, k)
+    s, q = oracle.quantize_q8_0_batch(oracle.fill_normal(5, 1.0, n * k), n, k)
+    d_q, d_s = ctx.to_device(q), ctx.to_device(s)
+    lay = W.LAYOUT_TOKEN_MAJOR if layout == "token" else W.LAYOUT_ROW_MAJOR
+    stride = (m + 8) if layout == "token" else (n + 4)
+    size = n * stride if layout == "token" else m * stride
+    y0 = oracle.fill_normal(6, 1.0, size)
+    outs = []
+    for splits in (0, 0, 1):  # default twice, then switched off
+        ctx.set_gemm_max_k_splits(splits)
+        d_y = ctx.to_device(y0)
+        ctx.gemm_preq(w, d_s, d_q, n, d_y, y_stride=stride, layout=lay, accumulate=accumulate)
+        y = d_y.download(np.float32, size)
+        outs.append((y.reshape(n, stride)[:, :m].T if layout == "token" else y.reshape(m, stride)[:, :n]).copy())
+        pad = y.reshape(n, stride)[:, m:] if layout == "token" else y.reshape(m, stride)[:, n:]
+        assert np.array_equal(pad, (y0.reshape(n, stride)[:, m:] if layout == "token" else y0.reshape(m, stride)[:, n:]))
+        d_y.free()
+    ctx.set_gemm_max_k_splits(0)
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    ref = oracle.gemm_q8(dtype, wb, s, q, m, n, k, f64=True)
+    if accumulate:
+        ref = ref + (y0.reshape(n, stride)[:, :m].T if layout == "token" else y0.reshape(m, stride)[:, :n])
+    assert_f32_parity(outs[0], ref, "split GEMM")
+    assert_f32_parity(outs[2], ref, "unsplit GEMM")
+    assert np.linalg.norm(outs[0].astype(np.float64) - outs[2]) <= 1e-6 * np.linalg.norm(outs[2])
+    w.free(), d_q.free(), d_s.free()

@@ -58,8 +58,10 @@ int ensure_scratch(wick_rocm_ctx* ctx, size_t q_bytes, size_t s_floats, size_t f
 }
 
 // Routing shared by wick_rocm_gemm_q8 and wick_rocm_matmul_f32 (lock already held).
+// may_split: the call may take the K-split launch pair, whose partial sums live in context scratch (never the entry point
+// that must not allocate, never during a capture that has not reserved the room).
 int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q, const float* d_s, uint32_t n,
-                float* d_y, uint32_t y_stride, int y_layout, int accumulate) {
+                float* d_y, uint32_t y_stride, int y_layout, int accumulate, bool may_split = true) {
     if (!d_q || !d_s || !d_y) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "null device pointer");
     if (n == 0) return WICK_ROCM_OK;
     if (y_layout != WICK_ROCM_LAYOUT_TOKEN_MAJOR && y_layout != WICK_ROCM_LAYOUT_ROW_MAJOR)
@@ -79,10 +81,16 @@ int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q
     const bool mfma_ok = (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_q) % 16u == 0) &&
                          (reinterpret_cast<uintptr_t>(d_s) % 16u == 0);
     hipError_t e;
-    if (n >= ctx->gemm_min_n && mfma_ok)
+    if (n >= ctx->gemm_min_n && mfma_ok) {
+        uint32_t splits = may_split && ctx->gemm_max_splits > 1 ? gemm_split_k(w->m, n, w->k, ctx->gemm_max_splits) : 1u;
+        if (splits > 1) {
+            const size_t floats = (size_t)splits * n * w->m;
+            if (ctx->capturing && floats > ctx->scratch_f_cap) splits = 1;  // no room reserved: the unsplit launch, same result to the f32 bar
+            else if (int rc = ensure_scratch(ctx, 0, 0, floats)) return rc;
+        }
         e = launch_gemm_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
-                             y_layout, accumulate, ctx->launch());
-    else
+                             y_layout, accumulate, ctx->launch(), splits, splits > 1 ? ctx->scratch_f : nullptr);
+    } else
         e = launch_gemv_tokens(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
                                y_layout, accumulate, ctx->num_cus, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "gemm launch");
@@ -239,6 +247,12 @@ int wick_rocm_probe_rate(wick_rocm_ctx* ctx, int shape, uint32_t iters, double* 
 int wick_rocm_set_gemv_policy(wick_rocm_ctx* ctx, int64_t direct_max_bytes) {
     WR_ENTER(ctx);
     ctx->gemv_direct_max_bytes = direct_max_bytes < 0 ? -1 : direct_max_bytes;
+    return WICK_ROCM_OK;
+}
+
+int wick_rocm_set_gemm_max_k_splits(wick_rocm_ctx* ctx, uint32_t max_splits) {
+    WR_ENTER(ctx);
+    ctx->gemm_max_splits = max_splits == 0 ? kGemmMaxSplits : (max_splits > 8 ? 8u : max_splits);
     return WICK_ROCM_OK;
 }
 
@@ -654,7 +668,7 @@ int wick_rocm_matmul_f32_noalloc(wick_rocm_ctx* ctx, const wick_rocm_weight* w, 
     // Nothing in the scratch has to start at zero: the quantizer writes every byte the matmul reads.
     hipError_t e = launch_quantize_q8_0(x, n, w->k, n == 1 ? w->k : x_stride, q, s, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "quantize_q8_0 launch");
-    return gemm_locked(ctx, w, q, s, n, y, n == 1 ? w->m : y_stride, WICK_ROCM_LAYOUT_TOKEN_MAJOR, accumulate);
+    return gemm_locked(ctx, w, q, s, n, y, n == 1 ? w->m : y_stride, WICK_ROCM_LAYOUT_TOKEN_MAJOR, accumulate, /*may_split=*/false);
 }
 
 int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_quants, uint32_t n,

@@ -92,6 +92,10 @@ struct GemmArgs {
     const uint8_t* w_up;
     int8_t* q_out;   // [n][m]
     float* s_out;    // [n][m / 32]
+    // K split of a narrow launch with few tiles: workgroup (tile, split) walks its share of the stages and leaves its sums
+    // in partial[split][n][m]; gemm_splitk_reduce_kernel adds the shares up in a fixed order.  ksplit <= 1: off.
+    uint32_t ksplit;
+    float* partial;
 };
 
 // Makes `a` describe the weight that owns row tile `row_tile` and rebases the tile index to that weight.
@@ -557,7 +561,9 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     __shared__ SmemT<BN_NARROW> sm;
     uint32_t row_tile, tok_tile;
     bool valid_tile;
-    tile_of_block(blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
+    const uint32_t ksplit = DUMP || a.ksplit < 2 ? 1u : a.ksplit;
+    const uint32_t split = ksplit > 1 ? blockIdx.x % ksplit : 0u;  // the splits of a tile are neighbours: different XCDs, same time
+    tile_of_block(ksplit > 1 ? blockIdx.x / ksplit : blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
     if (!valid_tile) return;  // whole workgroup leaves together
     select_weight(a, row_tile);
     const uint32_t row0 = row_tile * BM;
@@ -569,7 +575,11 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     const uint32_t kq = lane >> 4;      // which 8-byte quarter of the block this lane feeds
     const uint32_t wrow0 = wave * 16;   // wave's rows within the tile
     const uint32_t nb = a.k >> 5;
-    const uint32_t stages = nb / KB;
+    // this workgroup's stages: [first, first + stages)
+    const uint32_t all_stages = nb / KB;
+    const uint32_t per_split = (all_stages + ksplit - 1) / ksplit;
+    const uint32_t first = split * per_split;
+    const uint32_t stages = min(all_stages, first + per_split) - first;  // >= 1: the host splits only where every share is
 
     float acc[4][4];
 #pragma unroll
@@ -581,8 +591,8 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     asm volatile("" : "+v"(cbias));
 
     StageRegs<TYPE> regs;
-    dma_activations(a, sm.st[0], tok0, 0);
-    load_stage<TYPE, BN_NARROW>(a, row0, tok0, 0, regs);
+    dma_activations(a, sm.st[0], tok0, first * KB);
+    load_stage<TYPE, BN_NARROW>(a, row0, tok0, first * KB, regs);
     store_stage<TYPE, BN_NARROW>(sm.st[0], regs);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
     __syncthreads();
@@ -590,8 +600,8 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     for (uint32_t st = 0; st < stages; st++) {
         const StageT<BN_NARROW>& s = sm.st[st & 1u];
         if (st + 1 < stages) {
-            dma_activations(a, sm.st[(st + 1) & 1u], tok0, (st + 1) * KB);
-            load_stage<TYPE, BN_NARROW>(a, row0, tok0, (st + 1) * KB, regs);
+            dma_activations(a, sm.st[(st + 1) & 1u], tok0, (first + st + 1) * KB);
+            load_stage<TYPE, BN_NARROW>(a, row0, tok0, (first + st + 1) * KB, regs);
         }
 
         LaneAddr la;  // block 0 of this stage's buffer
@@ -613,7 +623,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
             la.wt += adv ? kOffWt : 0;
             la.dws += adv ? kOffDws : 0;
             la.dxf += adv ? kOffDxfNarrow : 0;
-            const uint32_t row = row0 + wrow0 + l16, tok = tok0 + 4 * kq, blk = st * KB + b;
+            const uint32_t row = row0 + wrow0 + l16, tok = tok0 + 4 * kq, blk = (first + st) * KB + b;
             v4i d[4];
             lds_wait<5>(mt);  // the five scale reads issued after the matrices may still be in flight
 #pragma unroll
@@ -644,11 +654,40 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
             for (int r = 0; r < 4; r++) {
                 const uint32_t tok = tok0 + 16 * tt + 4 * kq + r;
                 if (row < a.m && tok < a.n) {
-                    float* dst = a.y_row_major ? a.y + (size_t)row * a.y_stride + tok : a.y + (size_t)tok * a.y_stride + row;
-                    *dst = a.accumulate ? *dst + acc[tt][r] : acc[tt][r];
+                    if (ksplit > 1) {
+                        a.partial[((size_t)split * a.n + tok) * a.m + row] = acc[tt][r];
+                    } else {
+                        float* dst = a.y_row_major ? a.y + (size_t)row * a.y_stride + tok : a.y + (size_t)tok * a.y_stride + row;
+                        *dst = a.accumulate ? *dst + acc[tt][r] : acc[tt][r];
+                    }
                 }
             }
     }
+}
+
+// y (+)= partial[0] + partial[1] + ... in that order, element by element (token-major partials [split][n][m]).
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial, uint32_t splits, uint32_t n, uint32_t m,
+                                                                 float* __restrict__ y, uint32_t y_stride, int y_row_major, int accumulate) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, total = (size_t)n * m;
+    if (i >= total) return;
+    float sum = partial[i];
+    for (uint32_t s_ = 1; s_ < splits; s_++) sum += partial[(size_t)s_ * total + i];
+    const uint32_t tok = (uint32_t)(i / m), row = (uint32_t)(i % m);
+    float* dst = y_row_major ? y + (size_t)row * y_stride + tok : y + (size_t)tok * y_stride + row;
+    *dst = accumulate ? *dst + sum : sum;
+}
+
+// How many ways a single-weight launch is split over K: only narrow launches that leave at least half of the CUs without
+// a tile, with K long enough (>= 16 stages) that the shorter walk pays for the second launch, every share >= 4 stages.
+uint32_t split_k_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits) {
+    const uint32_t row_tiles = (m + BM - 1) / BM;
+    const bool narrow = n <= BN_NARROW || row_tiles * ((n + BN - 1) / BN) <= 256;
+    if (!narrow) return 1;
+    const uint32_t tiles = row_tiles * ((n + BN_NARROW - 1) / BN_NARROW), stages = (k >> 5) / KB;
+    if (stages < 16) return 1;
+    uint32_t s_ = 1;
+    while (2 * s_ <= max_splits && tiles * 2 * s_ <= 256 && stages / (2 * s_) >= 4) s_ *= 2;
+    return s_;
 }
 
 template <bool DUMP>
@@ -668,6 +707,15 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0) {
     const uint32_t tiles = a.row_tiles * a.tok_tiles;
     const uint32_t blocks = ((tiles + 7u) / 8u) * 8u;  // every XCD gets the same number of slots
     if (narrow) {
+        if (!DUMP && a.ksplit > 1) {
+            const uint32_t split_blocks = ((tiles * a.ksplit + 7u) / 8u) * 8u;
+            hipError_t e = type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(split_blocks), dim3(THREADS), a)
+                                             : launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(split_blocks), dim3(THREADS), a);
+            if (e != hipSuccess) return e;
+            const size_t total = (size_t)a.n * a.m;
+            return launch_kernel(L, kFamGemm, gemm_splitk_reduce_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256),
+                                 static_cast<const float*>(a.partial), a.ksplit, a.n, a.m, a.y, a.y_stride, a.y_row_major, a.accumulate);
+        }
         if (type == kTypeQ4_0) return launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
         return launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
     }
@@ -678,14 +726,21 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0) {
 
 }  // namespace
 
+uint32_t gemm_split_k(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits) { return split_k_factor(m, n, k, max_splits); }
+
+// splits > 1 (= gemm_split_k(m, n, k, ...)) with d_partial holding splits * n * m floats: the K-split launch pair.
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                             const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
-                            int accumulate, const Launch& L) {
+                            int accumulate, const Launch& L, uint32_t splits, float* d_partial) {
     GemmArgs a{};
     a.w = d_w, a.xq = d_q, a.xs = d_scales, a.y = d_y, a.dots = nullptr;
     a.m = m, a.n = n, a.k = k, a.y_stride = y_stride;
     a.y_row_major = (y_layout == 1);
     a.accumulate = accumulate;
+    if (splits > 1 && d_partial) {
+        if (splits != split_k_factor(m, n, k, splits)) return hipErrorInvalidValue;  // the shape does not carry that split
+        a.ksplit = splits, a.partial = d_partial;
+    }
     return launch<false>(type, a, L);
 }
 

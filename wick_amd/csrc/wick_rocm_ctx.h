@@ -34,6 +34,7 @@ struct wick_rocm_ctx {
     bool capture_used_scratch = false;
     unsigned char* noalloc_scratch = nullptr;  // this device's address of the static scratch array of wick_rocm_matmul_f32_noalloc
     uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
+    uint32_t gemm_max_splits = kGemmMaxSplits;  // K split of GEMM launches with few tiles (1: off)
     KernelTimer timer;
     int64_t gemv_direct_max_bytes = -1;
     unsigned long long* argmax_partial = nullptr;  // kArgmaxPartials keys for wick_rocm_argmax

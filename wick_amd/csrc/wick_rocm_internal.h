@@ -126,7 +126,9 @@ hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t
 // int8-MFMA GEMM.  Requires k % 128 == 0.
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                             const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
-                            int accumulate, const Launch& L);
+                            int accumulate, const Launch& L, uint32_t splits = 1, float* d_partial = nullptr);
+// Ways (1, 2, 4 or 8, at most max_splits) the launch above may be split over K: > 1 only for launches of few tiles and long K.
+uint32_t gemm_split_k(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits);
 hipError_t launch_gemm_mfma_multi(int type, const uint8_t* const* d_w, const uint32_t* m, uint32_t count, uint32_t k, const int8_t* d_q,
                                   const float* d_scales, uint32_t n, float* const* d_y, uint32_t y_stride, int y_layout, int accumulate,
                                   const Launch& L);
@@ -208,5 +210,6 @@ hipError_t launch_advance_pos(uint32_t* d_pos, const Launch& L);
 
 // n at and above which gemm_q8 uses the MFMA kernel (when k % 128 == 0).
 constexpr uint32_t kGemmMinN = 16;  // cf. GEMM_MIN_N, wick/src/model/metal_lfm2.rs:18-21
+constexpr uint32_t kGemmMaxSplits = 8;  // most K shares of a GEMM launch with few tiles
 
 }  // namespace wick_rocm

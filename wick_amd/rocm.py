@@ -73,6 +73,7 @@ _SIGNATURES = {
     "wick_rocm_sync": (C.c_int, [_P]),
     "wick_rocm_copy": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_set_gemm_min_n": (C.c_int, [_P, C.c_uint32]),
+    "wick_rocm_set_gemm_max_k_splits": (C.c_int, [_P, C.c_uint32]),
     "wick_rocm_set_gemv_policy": (C.c_int, [_P, C.c_int64]),
     "wick_rocm_probe_rate": (C.c_int, [_P, C.c_int, C.c_uint32, C.POINTER(C.c_double)]),
     "wick_rocm_weight_upload": (C.c_int, [_P, _P, C.c_size_t, C.c_int, C.c_uint32, C.c_uint32, C.POINTER(_P)]),
@@ -237,6 +238,10 @@ class RocmContext:
 
     def set_gemm_min_n(self, min_n: int) -> None:
         self._check(self._lib.wick_rocm_set_gemm_min_n(self._h, min_n))
+
+    def set_gemm_max_k_splits(self, max_splits: int) -> None:
+        """Most K shares of a GEMM launch with few tiles and long K (1: never split, 0: the default)."""
+        self._check(self._lib.wick_rocm_set_gemm_max_k_splits(self._h, max_splits))
 
     def alloc(self, nbytes: int) -> DeviceBuffer:
         return DeviceBuffer(self, nbytes)
