@@ -57,6 +57,17 @@ int wick_rocm_qk_norm_rope_tokens(wick_rocm_ctx *ctx, float *d_q, uint32_t q_str
                                   const float *d_q_norm, const float *d_k_norm, float *d_k_cache, float *d_v_cache, uint32_t pos0, uint32_t n,
                                   uint32_t max_seq, uint32_t head_dim, uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale);
 
+/* One attention layer's part of the n_keep context shift (InferenceState::shift_kv_with_rope, wick/src/kv_cache.rs:601-700;
+ * Metal: encode_kv_shift_layers, wick/src/model/metal_lfm2.rs:2657-2761): rows [n_keep, n_keep + shift) of both caches
+ * ([>= seq_len][n_kv_heads*head_dim] floats) are dropped, the rows behind them move down by `shift`, and every key head that
+ * moved is rotated by -shift positions (apply_rope_delta_to_head, wick/src/backend/cpu.rs:2174-2187), so that it reads as if it
+ * had been rotated for its new row.  Values move unchanged.  Rows from seq_len - shift on are left as they were; the caller's
+ * seq_len becomes seq_len - shift.  d_scratch holds wick_rocm_kv_shift_scratch_floats(...) floats (may be null when
+ * n_keep + shift == seq_len: nothing moves).  shift > 0, n_keep + shift <= seq_len.  Not available inside a graph capture. */
+size_t wick_rocm_kv_shift_scratch_floats(uint32_t seq_len, uint32_t n_keep, uint32_t shift, uint32_t n_kv_heads, uint32_t head_dim);
+int wick_rocm_kv_shift(wick_rocm_ctx *ctx, float *d_k_cache, float *d_v_cache, float *d_scratch, uint32_t seq_len, uint32_t n_keep,
+                       uint32_t shift, uint32_t n_kv_heads, uint32_t head_dim, float theta_scale);
+
 /* encode_attention (wick/src/model/metal_lfm2.rs:1736-1867) = attn_scores + softmax_inplace + attn_values per
  * query head (wick/src/model/lfm2.rs:984-1006) over cache rows [0, seq_len) (seq_len = *d_pos + 1 when d_pos is
  * given), grouped-query: head h reads KV head h / (n_heads / n_kv_heads).  d_scratch holds
@@ -205,6 +216,11 @@ int wick_rocm_lfm2_forward(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t t
  * single steps would (up to the rounding of GEMM against GEMV sums) and returns the logits of the LAST token. */
 int wick_rocm_lfm2_forward_prefill(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, const uint32_t *tokens, uint32_t n, uint32_t start_pos,
                                    float *logits);
+/* Model::forward_prefill_from_embeddings (wick/src/model/lfm2.rs:2452-2487, wick/src/model/metal_lfm2.rs:2426-2464): the same
+ * passes over n frames given as hidden-size vectors (frame j at embeddings[j * hidden_size], host memory) instead of token ids;
+ * logits of the LAST frame. */
+int wick_rocm_lfm2_forward_prefill_from_embeddings(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, const float *embeddings, uint32_t n,
+                                                   uint32_t start_pos, float *logits);
 /* Model::forward_prefill_chunked (wick/src/model/mod.rs:111-140): the prompt in chunks of `ubatch` tokens (0 = one chunk),
  * each a wick_rocm_lfm2_forward_prefill of its own; `cancel` (may be null) is read after every chunk and a non-zero value
  * stops the call there.  *consumed = tokens that made it into the state (0 < consumed <= n for n > 0; 0 and no logits for an
@@ -217,6 +233,34 @@ int wick_rocm_lfm2_forward_greedy(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uin
  * pick after step i (which is also step i+1's input). */
 int wick_rocm_lfm2_generate_greedy(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t token, uint32_t pos, uint32_t n,
                                    uint32_t *out_tokens);
+/* The embedding-input steps of the audio / soft-token paths (Model::supports_embedding_input is true for this backend).
+ * forward_from_embedding (wick/src/model/lfm2.rs:2295-2323): a step whose input is `embedding` ([hidden_size] floats, host
+ * memory) instead of a token's embedding row -> logits.
+ * forward_embedding (:2325-2337, wick/src/model/metal_lfm2.rs:2204-2250): a token step that stops after the output norm ->
+ * `hidden` ([hidden_size] floats, host memory; may be null), no LM head.
+ * forward_hidden_from_embedding (:2339-2349): both at once. */
+int wick_rocm_lfm2_forward_from_embedding(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, const float *embedding, uint32_t pos, float *logits);
+int wick_rocm_lfm2_forward_embedding(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t token, uint32_t pos, float *hidden);
+int wick_rocm_lfm2_forward_hidden_from_embedding(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, const float *embedding, uint32_t pos,
+                                                 float *hidden);
+
+/* Model::snapshot_state / restore_state (wick/src/model/mod.rs:301-315; snapshot_state_locked / restore_state_locked,
+ * wick/src/model/metal_lfm2.rs:2535-2634): the model's state after seq_len positions as host bytes, layer by layer in model
+ * order -- an attention layer contributes its key rows [0, seq_len) then its value rows [0, seq_len) (f32, [seq_len][kv_dim];
+ * LayerSnapshot::Attention's k_data, v_data), a gated-conv layer its rolling buffer ((conv_kernel_size - 1) * hidden_size f32;
+ * LayerSnapshot::Conv's buffer).  wick_rocm_lfm2_layer_state_bytes gives one layer's share (an attention layer's is split
+ * evenly between keys and values), wick_rocm_lfm2_state_bytes the total; `nbytes` must equal it.  The position count itself
+ * stays with the caller (StateSnapshot::seq_len), as `pos` does in the step calls. */
+size_t wick_rocm_lfm2_layer_state_bytes(const wick_rocm_lfm2 *model, uint32_t layer, uint32_t seq_len);
+size_t wick_rocm_lfm2_state_bytes(const wick_rocm_lfm2 *model, uint32_t seq_len);
+int wick_rocm_lfm2_snapshot_state(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t seq_len, void *out, size_t nbytes);
+int wick_rocm_lfm2_restore_state(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t seq_len, const void *in, size_t nbytes);
+
+/* Model::shift_kv (wick/src/model/lfm2.rs:2507-2516, wick/src/model/metal_lfm2.rs:2473-2531; supports_kv_shift is true for
+ * this backend): wick_rocm_kv_shift on every attention layer of a state of seq_len positions; gated-conv layers keep their
+ * rolling buffer.  The next step's position is seq_len - shift.  Waits for the shift. */
+int wick_rocm_lfm2_shift_kv(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model, uint32_t seq_len, uint32_t n_keep, uint32_t shift);
+
 /* The logits of the last step on the device ([vocab_size] floats). */
 const float *wick_rocm_lfm2_logits_device(const wick_rocm_lfm2 *model);
 

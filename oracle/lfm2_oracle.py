@@ -63,6 +63,21 @@ def rope(q, k, pos: int, n_heads: int, n_kv_heads: int, head_dim: int, freq_base
     return q2, k2
 
 
+def rope_delta(head, delta_pos: int, head_dim: int, freq_base: float) -> np.ndarray:
+    h = _c(head, np.float32).copy()
+    ops().orc_rope_delta(_p(h), C.c_int32(delta_pos), C.c_int64(head_dim), C.c_float(freq_base))
+    return h
+
+
+def shift_kv(k_cache, v_cache, seq_len: int, n_keep: int, shift: int, n_kv_heads: int, head_dim: int, freq_base: float):
+    """The caches of one attention layer ([>= seq_len][n_kv_heads * head_dim]) after dropping rows [n_keep, n_keep + shift)."""
+    assert shift > 0 and n_keep + shift <= seq_len
+    k2, v2 = _c(k_cache, np.float32).copy(), _c(v_cache, np.float32).copy()
+    ops().orc_shift_kv(_p(k2), _p(v2), C.c_int64(seq_len), C.c_int64(n_keep), C.c_int64(shift), C.c_int64(n_kv_heads), C.c_int64(head_dim),
+                       C.c_float(freq_base))
+    return k2, v2
+
+
 def rope_theta_scale(head_dim: int, freq_base: float) -> float:
     return float(ops().orc_rope_theta_scale(head_dim, C.c_float(freq_base)))
 
@@ -184,11 +199,17 @@ class Lfm2Oracle:
             y = (y * (np.float32(1.0) + self.jitter.uniform(-1.0, 1.0, y.size).astype(np.float32) * np.float32(2.0 ** -22))).astype(np.float32)
         return y
 
-    def hidden_after_layers(self, token: int, pos: int, state: dict) -> np.ndarray:
+    def hidden_after_layers(self, token, pos: int, state: dict, embedding=None) -> np.ndarray:
+        """run_layers (wick/src/model/lfm2.rs:1020-1124) on the token's embedding row, or on `embedding` when given
+        (forward_embedding / forward_hidden_from_embedding, :2325-2349): the hidden state after the output norm."""
         c = self.cfg
         hs, eps = c["hidden_size"], c["rms_norm_eps"]
-        gt, dims, data = self.t["token_embd.weight"]
-        hidden = embed_row(gt, data, token, dims[0])
+        if embedding is None:
+            gt, dims, data = self.t["token_embd.weight"]
+            hidden = embed_row(gt, data, token, dims[0])
+        else:
+            hidden = _c(embedding, np.float32).copy()
+            assert hidden.size == hs
         for i, n_kv in enumerate(c["kv_heads_per_layer"]):
             normed = rmsnorm(hidden, self._f32(f"blk.{i}.attn_norm.weight"), eps)
             if n_kv == 0:
@@ -222,3 +243,23 @@ class Lfm2Oracle:
         """Logits of one decode step (tied embedding as LM head, wick/src/model/lfm2.rs:2258-2289)."""
         hidden = self.hidden_after_layers(token, pos, state)
         return self._gemv("token_embd.weight", hidden)
+
+    def forward_from_embedding(self, embedding, pos: int, state: dict) -> np.ndarray:
+        """Logits of one step whose input is a hidden-size vector instead of a token (wick/src/model/lfm2.rs:2295-2323)."""
+        return self._gemv("token_embd.weight", self.hidden_after_layers(None, pos, state, embedding))
+
+    def shift_kv(self, state: dict, n_keep: int, shift: int) -> None:
+        """Lfm2Model::shift_kv (wick/src/model/lfm2.rs:2507-2516): every attention layer drops cache rows [n_keep, n_keep + shift)
+        and re-rotates the keys behind them; conv layers are left alone; seq_len shrinks by `shift`."""
+        c = self.cfg
+        hd, seq = c["hidden_size"] // c["n_heads"], state["seq_len"]
+        assert shift > 0 and n_keep + shift <= seq
+        for n_kv, ls in zip(c["kv_heads_per_layer"], state["layers"]):
+            if n_kv == 0 or not ls["k"]:
+                continue
+            assert len(ls["k"]) == seq
+            k, v = shift_kv(np.concatenate(ls["k"]), np.concatenate(ls["v"]), seq, n_keep, shift, n_kv, hd, c["rope_theta"])
+            kvd = n_kv * hd
+            ls["k"] = [k[t * kvd:(t + 1) * kvd].copy() for t in range(seq - shift)]
+            ls["v"] = [v[t * kvd:(t + 1) * kvd].copy() for t in range(seq - shift)]
+        state["seq_len"] = seq - shift

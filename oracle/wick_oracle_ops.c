@@ -19,6 +19,14 @@
  *   orc_rope           pos = 0 is the identity (cpu.rs:2783-2797); closed form
  *                      theta_i = pos * base^(-2 i / d) in float64; norm of every pair preserved;
  *                      R(p + q) = R(q) R(p)
+ *   orc_rope_delta     the reference's own checks (wick/tests/n_keep_shift.rs:47-91): a head rotated for
+ *                      p_old and then by p_new - p_old equals the head rotated for p_new within 1e-3
+ *                      on the same 25 position pairs and inputs, delta 0 is the identity; for
+ *                      delta >= 0 bit-equal to orc_rope at pos = delta
+ *   orc_shift_kv       the reference's closed-form case (wick/tests/n_keep_shift.rs:138-236: caches filled
+ *                      with raw heads rotated for their row, 24 rows, n_keep 5, shift 7): kept rows
+ *                      byte-identical, moved keys within 1e-3 of a fresh rotation for the new row, moved
+ *                      value rows bit-equal to their old rows; numpy restatement of the row move
  *   orc_attn_scores /  the reference's own inputs (cpu.rs:2910-3003) against numpy matmul;
  *   orc_attn_values    seq_len = 0 leaves the output untouched / zero (cpu.rs:3005-3010)
  *   orc_shortconv_step identity kernel reproduces b*x*c; numpy restatement over several steps
@@ -110,6 +118,32 @@ static void rope_head(float* head, int64_t pos, int64_t head_dim, float freq_bas
 ORC_API void orc_rope(float* q, float* k, int64_t pos, int64_t n_heads, int64_t n_kv_heads, int64_t head_dim, float freq_base) {
     for (int64_t h = 0; h < n_heads; h++) rope_head(q + h * head_dim, pos, head_dim, freq_base);
     for (int64_t h = 0; h < n_kv_heads; h++) rope_head(k + h * head_dim, pos, head_dim, freq_base);
+}
+
+/* apply_rope_delta_to_head, wick/src/backend/cpu.rs:2174-2187: the same pairs and theta schedule from a signed start angle. */
+ORC_API void orc_rope_delta(float* head, int32_t delta_pos, int64_t head_dim, float freq_base) {
+    const int64_t half = head_dim / 2;
+    const float theta_scale = powf(freq_base, -2.0f / (float)head_dim);
+    float theta = (float)delta_pos;
+    for (int64_t i = 0; i < half; i++) {
+        const float s = sinf(theta), c = cosf(theta);
+        const float x0 = head[i], x1 = head[i + half];
+        head[i] = x0 * c - x1 * s;
+        head[i + half] = x0 * s + x1 * c;
+        theta *= theta_scale;
+    }
+}
+
+/* InferenceState::shift_kv_with_rope for one attention layer, wick/src/kv_cache.rs:601-700: rows [n_keep, n_keep + shift) of
+ * both caches ([seq_len][n_kv_heads * head_dim]) are dropped, the rows behind them move down by `shift`, and every key head
+ * that moved is rotated by -shift positions.  The caller's seq_len becomes seq_len - shift; rows past it are left as they are. */
+ORC_API void orc_shift_kv(float* k_cache, float* v_cache, int64_t seq_len, int64_t n_keep, int64_t shift, int64_t n_kv_heads, int64_t head_dim,
+                          float freq_base) {
+    const int64_t kv_dim = n_kv_heads * head_dim, new_len = seq_len - shift;
+    memmove(k_cache + n_keep * kv_dim, k_cache + (n_keep + shift) * kv_dim, (size_t)((new_len - n_keep) * kv_dim) * sizeof(float));
+    memmove(v_cache + n_keep * kv_dim, v_cache + (n_keep + shift) * kv_dim, (size_t)((new_len - n_keep) * kv_dim) * sizeof(float));
+    for (int64_t t = n_keep; t < new_len; t++)
+        for (int64_t h = 0; h < n_kv_heads; h++) orc_rope_delta(k_cache + t * kv_dim + h * head_dim, -(int32_t)shift, head_dim, freq_base);
 }
 
 /* The f32 theta_scale the reference derives from freq_base (cpu.rs:2150), for callers that hand it to the device. */

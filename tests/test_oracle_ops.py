@@ -86,6 +86,58 @@ def test_rope_identity_closed_form_and_composition():
     assert L.rope_theta_scale(64, 1_000_000.0) == np.float32(np.float32(1_000_000.0) ** np.float32(-2.0 / 64))
 
 
+def _rope_head(head, pos, hd, base):
+    return L.rope(head, np.zeros(hd, np.float32), pos, 1, 1, hd, base)[0]
+
+
+def test_rope_delta_on_the_reference_cases():
+    hd, base = 64, 10_000.0  # wick/tests/n_keep_shift.rs:47-78: the same position pairs and head values
+    raw = (np.arange(hd) * 0.01).astype(np.float32)
+    for p_old in (0, 1, 7, 64, 2048):
+        for p_new in (0, 1, 5, 63, 2000):
+            via = L.rope_delta(_rope_head(raw, p_old, hd, base), p_new - p_old, hd, base)
+            assert np.abs(via - _rope_head(raw, p_new, hd, base)).max() < 1e-3, (p_old, p_new)
+    orig = (np.arange(32) * 0.1 + 1.0).astype(np.float32)  # wick/tests/n_keep_shift.rs:80-91
+    assert np.abs(L.rope_delta(orig, 0, 32, base) - orig).max() < 1e-5
+    assert np.array_equal(L.rope_delta(orig, 0, 32, base), orig)  # cos 0 = 1, sin 0 = 0 exactly
+    # a non-negative delta walks the very same angles as a rotation for that position
+    rng = np.random.default_rng(11)
+    h = rng.standard_normal(hd).astype(np.float32)
+    for d in (1, 5, 777):
+        assert np.array_equal(L.rope_delta(h, d, hd, 1_000_000.0), _rope_head(h, d, hd, 1_000_000.0))
+    # a negative delta is the inverse rotation: closed form in float64, and there-and-back returns the head
+    for d in (-1, -7, -300):
+        theta = d * np.float64(1_000_000.0) ** (-2.0 * np.arange(hd // 2) / hd)
+        x = h.reshape(2, hd // 2).astype(np.float64)
+        ref = np.concatenate([x[0] * np.cos(theta) - x[1] * np.sin(theta), x[0] * np.sin(theta) + x[1] * np.cos(theta)])
+        assert np.allclose(L.rope_delta(h, d, hd, 1_000_000.0), ref, atol=2e-6 * max(-d, 8))
+        assert np.allclose(L.rope_delta(L.rope_delta(h, d, hd, 1_000_000.0), -d, hd, 1_000_000.0), h, atol=1e-5)
+
+
+def test_shift_kv_on_the_reference_case():
+    hd, base, seq, n_keep, shift = 16, 10_000.0, 24, 5, 7  # wick/tests/n_keep_shift.rs:138-236
+    for layer, n_kv in enumerate((4, 2)):
+        kvd = n_kv * hd
+        raw = np.array([[layer + 0.1 * h + 0.01 * d for d in range(hd)] for h in range(n_kv)], np.float32)
+        k = np.stack([np.concatenate([_rope_head(raw[h], t, hd, base) for h in range(n_kv)]) for t in range(seq)])
+        v = np.stack([(raw + np.float32(0.001) * np.float32(t)).astype(np.float32).ravel() for t in range(seq)])
+        k2, v2 = L.shift_kv(k.ravel(), v.ravel(), seq, n_keep, shift, n_kv, hd, base)
+        k2, v2 = k2.reshape(seq, kvd), v2.reshape(seq, kvd)
+        assert np.array_equal(k2[:n_keep], k[:n_keep]) and np.array_equal(v2[:n_keep], v[:n_keep])  # kept rows untouched
+        for t_new in range(n_keep, seq - shift):
+            fresh = np.concatenate([_rope_head(raw[h], t_new, hd, base) for h in range(n_kv)])
+            assert np.abs(k2[t_new] - fresh).max() < 1e-3
+            assert np.array_equal(v2[t_new], v[t_new + shift])  # the row kept its identity
+        # the row move itself, restated: keys are the old rows rotated back by `shift`
+        for t_new in (n_keep, seq - shift - 1):
+            for h in range(n_kv):
+                assert np.array_equal(k2[t_new, h * hd:(h + 1) * hd], L.rope_delta(k[t_new + shift, h * hd:(h + 1) * hd], -shift, hd, base))
+    # dropping everything behind n_keep leaves the kept rows and nothing to rotate
+    k = np.arange(6 * 8, dtype=np.float32)
+    k2, v2 = L.shift_kv(k, k + 1, 6, 2, 4, 1, 8, base)
+    assert np.array_equal(k2[:16], k[:16]) and np.array_equal(v2[:16], k[:16] + 1)
+
+
 def test_attention_helpers_on_the_reference_inputs():
     hd, kv_dim, seq = 64, 128, 10  # cpu.rs:2910-2925
     q = ((np.arange(hd) - 32.0) * 0.05).astype(np.float32)

@@ -73,6 +73,25 @@ int wick_rocm_qk_norm_rope_tokens(wick_rocm_ctx* ctx, float* d_q, uint32_t q_str
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "qk_norm_rope_tokens launch");
 }
 
+size_t wick_rocm_kv_shift_scratch_floats(uint32_t seq_len, uint32_t n_keep, uint32_t shift, uint32_t n_kv_heads, uint32_t head_dim) {
+    if ((uint64_t)n_keep + shift > seq_len) return 0;
+    return 2 * (size_t)(seq_len - n_keep - shift) * n_kv_heads * head_dim;
+}
+
+int wick_rocm_kv_shift(wick_rocm_ctx* ctx, float* d_k_cache, float* d_v_cache, float* d_scratch, uint32_t seq_len, uint32_t n_keep, uint32_t shift,
+                       uint32_t n_kv_heads, uint32_t head_dim, float theta_scale) {
+    WR_ENTER(ctx);
+    if (!d_k_cache || !d_v_cache) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "kv_shift: null device pointer");
+    if (shift == 0) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "kv_shift: shift must be > 0");
+    if ((uint64_t)n_keep + shift > seq_len) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "kv_shift: shift range out of bounds (n_keep + shift > seq_len)");
+    if (head_dim == 0 || head_dim % 2u != 0 || head_dim > 256u || n_kv_heads == 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "kv_shift: head_dim must be even and <= 256, n_kv_heads > 0");
+    if (seq_len - n_keep - shift != 0 && !d_scratch) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "kv_shift: null scratch pointer");
+    if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "kv_shift: not available inside a graph capture");
+    hipError_t e = launch_kv_shift(d_k_cache, d_v_cache, d_scratch, seq_len, n_keep, shift, n_kv_heads, head_dim, theta_scale, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "kv_shift launch");
+}
+
 int wick_rocm_attention_decode(wick_rocm_ctx* ctx, const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out,
                                float* d_scores, uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
                                uint32_t head_dim) {
@@ -286,12 +305,17 @@ struct wick_rocm_lfm2 {
     float *pX = nullptr, *pA = nullptr, *pG = nullptr, *pGate = nullptr, *pUp = nullptr, *pS = nullptr, *pS2 = nullptr, *pAttn = nullptr;
     int8_t *pQ = nullptr, *pQ2 = nullptr;
     uint32_t* pTokens = nullptr;
-    wick_rocm_graph *g_logits = nullptr, *g_greedy = nullptr;
+    float* shift_stage = nullptr;  // staging rows of a context shift, allocated by the first one
+    wick_rocm_graph* g_step[3] = {nullptr, nullptr, nullptr};  // one captured step per StepMode
     bool use_graph = true;
     std::mutex mu;
 };
 
 namespace {
+
+// What a step ends with: the tied LM head's logits, the greedy pick on top of them, or only the hidden state after the
+// output norm (forward_embedding / forward_hidden_from_embedding, wick/src/model/lfm2.rs:2325-2349).
+enum StepMode { kStepLogits = 0, kStepGreedy = 1, kStepHidden = 2 };
 
 int ctx_fail(wick_rocm_ctx* ctx, int code, const std::string& what) {
     std::lock_guard<std::recursive_mutex> lk(ctx->mu);
@@ -339,8 +363,8 @@ int upload_weight(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, const wick_gguf* g, con
 
 void release(wick_rocm_ctx* ctx, wick_rocm_lfm2* m) {
     wick_rocm_sync(ctx);
-    if (m->g_logits) wick_rocm_graph_destroy(ctx, m->g_logits);
-    if (m->g_greedy) wick_rocm_graph_destroy(ctx, m->g_greedy);
+    for (wick_rocm_graph* g : m->g_step)
+        if (g) wick_rocm_graph_destroy(ctx, g);
     for (wick_rocm_weight* w : m->weights) wick_rocm_weight_free(ctx, w);
     for (void* b : m->buffers) wick_rocm_buffer_free(ctx, b);
     delete m;
@@ -368,7 +392,7 @@ int gemv_residual(wick_rocm_ctx* ctx, const wick_rocm_weight* w, float* y, const
 
 // Enqueues one decode step that reads token / pos from the device: run_layers + the tied LM head
 // (wick/src/model/lfm2.rs:1020-1124, 2258-2289), optionally the greedy pick.
-int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
+int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, StepMode mode) {
     const wick_rocm_lfm2_config& c = m->cfg;
     const uint32_t hs = c.hidden_size, hd = hs / c.n_heads;
     // m->hidden already holds the token's embedding row: set_step (or the previous step's greedy pick) looked it up
@@ -400,23 +424,24 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
         rc = gemv_residual(ctx, L.down, m->hidden, m->gate);
     }
     if (rc) return rc;
+    if (mode == kStepHidden) return wick_rocm_rmsnorm(ctx, m->hidden, m->out_norm, m->gated, 1, hs, hs, hs, c.rms_norm_eps);  // m->gated is free here
     if ((rc = gemv_normed(ctx, {m->embd}, {m->logits}, m->hidden, m->out_norm, c.rms_norm_eps))) return rc;
-    if (!greedy) return WICK_ROCM_OK;
+    if (mode != kStepGreedy) return WICK_ROCM_OK;
     std::lock_guard<std::recursive_mutex> lk(ctx->mu);
     hipError_t e = launch_argmax(m->logits, c.vocab_size, m->d_argmax_partial, m->d_pick, m->d_token, m->d_pos, m->d_history, c.max_seq_len,
                                  ctx->launch(), static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m, c.hidden_size, m->hidden);
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
 }
 
-int step_graph(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy, wick_rocm_graph** out) {
-    wick_rocm_graph*& g = greedy ? m->g_greedy : m->g_logits;
+int step_graph(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, StepMode mode, wick_rocm_graph** out) {
+    wick_rocm_graph*& g = m->g_step[mode];
     if (g && graph_is_stale(ctx, g)) {  // the context's scratch moved since the capture (another model, a wider matmul): capture again
         wick_rocm_graph_destroy(ctx, g);
         g = nullptr;
     }
     if (!g) {
         if (int rc = wick_rocm_graph_begin(ctx)) return rc;
-        const int rc = enqueue_step(ctx, m, greedy);
+        const int rc = enqueue_step(ctx, m, mode);
         wick_rocm_graph* captured = nullptr;
         const int rc_end = wick_rocm_graph_end(ctx, &captured);  // always end the capture
         if (rc) {
@@ -431,16 +456,16 @@ int step_graph(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy, wick_rocm_gra
 }
 
 // One step on the context's stream: a replay of the captured graph, or the same launches enqueued one by one.
-int run_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, bool greedy) {
+int run_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, StepMode mode) {
     // per-dispatch timing cannot see inside a graph: while it is on, steps are enqueued launch by launch
     bool timing;
     {
         std::lock_guard<std::recursive_mutex> lk(ctx->mu);
         timing = ctx->timer.enabled;
     }
-    if (!m->use_graph || timing) return enqueue_step(ctx, m, greedy);
+    if (!m->use_graph || timing) return enqueue_step(ctx, m, mode);
     wick_rocm_graph* g = nullptr;
-    if (int rc = step_graph(ctx, m, greedy, &g)) return rc;
+    if (int rc = step_graph(ctx, m, mode, &g)) return rc;
     return wick_rocm_graph_launch(ctx, g);
 }
 
@@ -485,7 +510,7 @@ int gemm_group(wick_rocm_ctx* ctx, std::initializer_list<const wick_rocm_weight*
 // of enqueue_step (prefill_layers_and_logits, wick/src/model/lfm2.rs:1139-2109): projections as GEMMs over the tokens,
 // the short conv per (token, channel) with the rolling state behind it, the KV append per token, causal attention per
 // (head, token).
-int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint32_t pos0) {
+int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint32_t pos0, bool lookup = true) {
     const wick_rocm_lfm2_config& c = m->cfg;
     const uint32_t hs = c.hidden_size, hd = hs / c.n_heads, inter = c.intermediate_size;
     const float scale = 1.0f / sqrtf((float)hd);
@@ -494,8 +519,10 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
         const hipError_t e = launch();
         return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, what);
     };
-    int rc = locked([&] { return launch_embed_rows(static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m, hs, m->pTokens, n, m->pX, ctx->launch()); },
-                    "embed_rows launch");
+    // the pass's input rows: the tokens' embedding rows, or what the caller put into pX (a prompt given as embeddings)
+    int rc = !lookup ? WICK_ROCM_OK
+                     : locked([&] { return launch_embed_rows(static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m, hs, m->pTokens, n, m->pX, ctx->launch()); },
+                              "embed_rows launch");
     for (uint32_t i = 0; rc == 0 && i < c.n_layers; i++) {
         const LayerWeights& L = m->layers[i];
         if ((rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.attn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
@@ -560,6 +587,23 @@ int set_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t token, uint32_t pos
 int check_step(wick_rocm_ctx* ctx, const wick_rocm_lfm2* m, uint32_t token, uint32_t pos, uint32_t n) {
     if (token >= m->cfg.vocab_size) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: token_id out of range");
     if ((uint64_t)pos + n > m->cfg.max_seq_len) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: position beyond the context size");
+    return WICK_ROCM_OK;
+}
+
+// Walks the layers' state in snapshot order and hands every piece (device pointer, bytes) to `piece`.
+template <typename F>
+int for_each_state_piece(const wick_rocm_lfm2* model, uint32_t seq_len, F&& piece) {
+    const wick_rocm_lfm2_config& c = model->cfg;
+    for (const LayerWeights& L : model->layers) {
+        if (L.n_kv) {
+            const size_t half = (size_t)seq_len * L.n_kv * (c.hidden_size / c.n_heads) * sizeof(float);
+            if (half == 0) continue;
+            if (int rc = piece(L.k_cache, half)) return rc;
+            if (int rc = piece(L.v_cache, half)) return rc;
+        } else if (L.conv_state) {
+            if (int rc = piece(L.conv_state, (size_t)(c.conv_kernel_size - 1) * c.hidden_size * sizeof(float))) return rc;
+        }
+    }
     return WICK_ROCM_OK;
 }
 
@@ -717,8 +761,31 @@ int wick_rocm_lfm2_forward(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t t
     std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);  // nothing else gets onto the context's stream (or into a capture) in between
     if (int rc = check_step(ctx, model, token, pos, 1)) return rc;
     if (int rc = set_step(ctx, model, token, pos)) return rc;
-    if (int rc = run_step(ctx, model, false)) return rc;
+    if (int rc = run_step(ctx, model, kStepLogits)) return rc;
     if (logits) return wick_rocm_download(ctx, logits, model->logits, (size_t)model->cfg.vocab_size * sizeof(float));
+    return wick_rocm_sync(ctx);
+}
+
+// Shared body of the two prompt entry points: exactly one of tokens / embeddings is given.
+static int prefill_locked(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, const uint32_t* tokens, const float* embeddings, uint32_t n, uint32_t start_pos,
+                          float* logits) {
+    const wick_rocm_lfm2_config& c = model->cfg;
+    if ((uint64_t)start_pos + n > c.max_seq_len) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: position beyond the context size");
+    if (int rc = ensure_prefill_buffers(ctx, model)) return rc;
+    uint32_t last = 0;
+    for (uint32_t done = 0; done < n; done += model->prefill_cap) {
+        last = n - done < model->prefill_cap ? n - done : model->prefill_cap;
+        if (tokens) {
+            if (int rc = wick_rocm_upload(ctx, model->pTokens, tokens + done, (size_t)last * sizeof(uint32_t))) return rc;
+        } else {  // frame j of the prompt is row j of the pass's input (wick/src/model/lfm2.rs:2452-2487)
+            if (int rc = wick_rocm_upload(ctx, model->pX, embeddings + (size_t)done * c.hidden_size, (size_t)last * c.hidden_size * sizeof(float))) return rc;
+        }
+        if (int rc = enqueue_prompt_pass(ctx, model, last, start_pos + done, tokens != nullptr)) return rc;
+    }
+    // output norm + tied LM head on the last token only (wick/src/model/lfm2.rs:2080-2109)
+    const float* h_last = model->pX + (size_t)(last - 1) * c.hidden_size;
+    if (int rc = gemv_normed(ctx, {model->embd}, {model->logits}, h_last, model->out_norm, c.rms_norm_eps)) return rc;
+    if (logits) return wick_rocm_download(ctx, logits, model->logits, (size_t)c.vocab_size * sizeof(float));
     return wick_rocm_sync(ctx);
 }
 
@@ -727,22 +794,18 @@ int wick_rocm_lfm2_forward_prefill(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, co
     if (!tokens || n == 0) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 prefill: empty prompt");
     std::lock_guard<std::mutex> lk(model->mu);
     std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);  // nothing else gets onto the context's stream (or into a capture) in between
-    const wick_rocm_lfm2_config& c = model->cfg;
     for (uint32_t j = 0; j < n; j++)
-        if (tokens[j] >= c.vocab_size) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: token_id out of range");
-    if ((uint64_t)start_pos + n > c.max_seq_len) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: position beyond the context size");
-    if (int rc = ensure_prefill_buffers(ctx, model)) return rc;
-    uint32_t last = 0;
-    for (uint32_t done = 0; done < n; done += model->prefill_cap) {
-        last = n - done < model->prefill_cap ? n - done : model->prefill_cap;
-        if (int rc = wick_rocm_upload(ctx, model->pTokens, tokens + done, (size_t)last * sizeof(uint32_t))) return rc;
-        if (int rc = enqueue_prompt_pass(ctx, model, last, start_pos + done)) return rc;
-    }
-    // output norm + tied LM head on the last token only (wick/src/model/lfm2.rs:2080-2109)
-    const float* h_last = model->pX + (size_t)(last - 1) * c.hidden_size;
-    if (int rc = gemv_normed(ctx, {model->embd}, {model->logits}, h_last, model->out_norm, c.rms_norm_eps)) return rc;
-    if (logits) return wick_rocm_download(ctx, logits, model->logits, (size_t)c.vocab_size * sizeof(float));
-    return wick_rocm_sync(ctx);
+        if (tokens[j] >= model->cfg.vocab_size) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: token_id out of range");
+    return prefill_locked(ctx, model, tokens, nullptr, n, start_pos, logits);
+}
+
+int wick_rocm_lfm2_forward_prefill_from_embeddings(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, const float* embeddings, uint32_t n, uint32_t start_pos,
+                                                   float* logits) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    if (!embeddings || n == 0) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 prefill: at least one frame is required");
+    std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);
+    return prefill_locked(ctx, model, nullptr, embeddings, n, start_pos, logits);
 }
 
 int wick_rocm_lfm2_forward_prefill_chunked(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, const uint32_t* tokens, uint32_t n, uint32_t start_pos,
@@ -776,8 +839,116 @@ int wick_rocm_lfm2_generate_greedy(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, ui
     if (int rc = check_step(ctx, model, token, pos, n)) return rc;
     if (int rc = set_step(ctx, model, token, pos)) return rc;
     for (uint32_t i = 0; i < n; i++)  // the pick of step i is written to the device-side token and position pos + i of the history
-        if (int rc = run_step(ctx, model, true)) return rc;
+        if (int rc = run_step(ctx, model, kStepGreedy)) return rc;
     return wick_rocm_download(ctx, out_tokens, model->d_history + pos, (size_t)n * sizeof(uint32_t));
+}
+
+// One step whose input is the token's embedding row (embedding == null) or the caller's hidden-size vector; ends per `mode`.
+static int step_locked(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t token, const float* embedding, uint32_t pos, StepMode mode, float* out) {
+    const wick_rocm_lfm2_config& c = model->cfg;
+    if (int rc = check_step(ctx, model, embedding ? 0u : token, pos, 1)) return rc;
+    if (embedding) {  // position only; the input vector goes where the lookup would have put the row
+        {
+            std::lock_guard<std::recursive_mutex> lk(ctx->mu);
+            const hipError_t e = launch_set_step(nullptr, 0, model->d_pos, pos, ctx->launch());
+            if (e != hipSuccess) return fail_hip(ctx, e, "set_step launch");
+        }
+        if (int rc = wick_rocm_upload(ctx, model->hidden, embedding, (size_t)c.hidden_size * sizeof(float))) return rc;
+    } else if (int rc = set_step(ctx, model, token, pos)) {
+        return rc;
+    }
+    if (int rc = run_step(ctx, model, mode)) return rc;
+    if (!out) return wick_rocm_sync(ctx);
+    return mode == kStepHidden ? wick_rocm_download(ctx, out, model->gated, (size_t)c.hidden_size * sizeof(float))
+                               : wick_rocm_download(ctx, out, model->logits, (size_t)c.vocab_size * sizeof(float));
+}
+
+int wick_rocm_lfm2_forward_from_embedding(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, const float* embedding, uint32_t pos, float* logits) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    if (!embedding) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: null embedding pointer");
+    std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);
+    return step_locked(ctx, model, 0, embedding, pos, kStepLogits, logits);
+}
+
+int wick_rocm_lfm2_forward_embedding(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t token, uint32_t pos, float* hidden) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);
+    return step_locked(ctx, model, token, nullptr, pos, kStepHidden, hidden);
+}
+
+int wick_rocm_lfm2_forward_hidden_from_embedding(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, const float* embedding, uint32_t pos, float* hidden) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    if (!embedding) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2: null embedding pointer");
+    std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole_step(ctx->mu);
+    return step_locked(ctx, model, 0, embedding, pos, kStepHidden, hidden);
+}
+
+// ---- state snapshots and the context shift -------------------------------------------------
+
+size_t wick_rocm_lfm2_layer_state_bytes(const wick_rocm_lfm2* model, uint32_t layer, uint32_t seq_len) {
+    if (!model || layer >= model->cfg.n_layers || seq_len > model->cfg.max_seq_len) return 0;
+    const wick_rocm_lfm2_config& c = model->cfg;
+    const LayerWeights& L = model->layers[layer];
+    if (L.n_kv) return 2 * (size_t)seq_len * L.n_kv * (c.hidden_size / c.n_heads) * sizeof(float);
+    return (size_t)(c.conv_kernel_size - 1) * c.hidden_size * sizeof(float);
+}
+
+size_t wick_rocm_lfm2_state_bytes(const wick_rocm_lfm2* model, uint32_t seq_len) {
+    if (!model) return 0;
+    size_t total = 0;
+    for (uint32_t i = 0; i < model->cfg.n_layers; i++) total += wick_rocm_lfm2_layer_state_bytes(model, i, seq_len);
+    return total;
+}
+
+int wick_rocm_lfm2_snapshot_state(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t seq_len, void* out, size_t nbytes) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole(ctx->mu);
+    if (seq_len > model->cfg.max_seq_len) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 snapshot: seq_len beyond the context size");
+    if (nbytes != wick_rocm_lfm2_state_bytes(model, seq_len) || (!out && nbytes))
+        return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 snapshot: the buffer must hold exactly wick_rocm_lfm2_state_bytes(model, seq_len) bytes");
+    uint8_t* at = static_cast<uint8_t*>(out);
+    return for_each_state_piece(model, seq_len, [&](const void* d, size_t n) {
+        const int rc = wick_rocm_download(ctx, at, d, n);
+        at += n;
+        return rc;
+    });
+}
+
+int wick_rocm_lfm2_restore_state(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t seq_len, const void* in, size_t nbytes) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole(ctx->mu);
+    if (seq_len > model->cfg.max_seq_len) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 restore: seq_len beyond the context size");
+    if (nbytes != wick_rocm_lfm2_state_bytes(model, seq_len) || (!in && nbytes))
+        return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 restore: the snapshot must hold exactly wick_rocm_lfm2_state_bytes(model, seq_len) bytes");
+    const uint8_t* at = static_cast<const uint8_t*>(in);
+    return for_each_state_piece(model, seq_len, [&](void* d, size_t n) {
+        const int rc = wick_rocm_upload(ctx, d, at, n);
+        at += n;
+        return rc;
+    });
+}
+
+int wick_rocm_lfm2_shift_kv(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t seq_len, uint32_t n_keep, uint32_t shift) {
+    if (!ctx || !model) return WICK_ROCM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lk(model->mu);
+    std::lock_guard<std::recursive_mutex> whole(ctx->mu);
+    const wick_rocm_lfm2_config& c = model->cfg;
+    if (shift == 0) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 shift_kv: shift must be > 0");
+    if (seq_len > c.max_seq_len || (uint64_t)n_keep + shift > seq_len)
+        return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2 shift_kv: shift range out of bounds (n_keep + shift > seq_len)");
+    if (seq_len - n_keep - shift == 0) return WICK_ROCM_OK;  // nothing behind the dropped rows: only the caller's seq_len changes
+    const uint32_t hd = c.hidden_size / c.n_heads;
+    if (!model->shift_stage && c.n_kv_heads)
+        if (int rc = alloc_t(ctx, model, 2 * (size_t)c.max_seq_len * c.n_kv_heads * hd, &model->shift_stage)) return rc;
+    for (const LayerWeights& L : model->layers)  // conv layers keep their rolling buffer (wick/src/kv_cache.rs:584-590)
+        if (L.n_kv)
+            if (int rc = wick_rocm_kv_shift(ctx, L.k_cache, L.v_cache, model->shift_stage, seq_len, n_keep, shift, L.n_kv, hd, model->theta_scale)) return rc;
+    return wick_rocm_sync(ctx);
 }
 
 const float* wick_rocm_lfm2_logits_device(const wick_rocm_lfm2* model) { return model ? model->logits : nullptr; }

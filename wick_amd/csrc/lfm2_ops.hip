@@ -225,6 +225,50 @@ __global__ __launch_bounds__(256) void qk_norm_rope_tokens64_kernel(QkNormRopeAr
     }
 }
 
+// ---- n_keep context shift -----------------------------------------------------------------
+// InferenceState::shift_kv_with_rope for one attention layer (wick/src/kv_cache.rs:601-700): cache rows
+// [n_keep, n_keep + shift) are dropped, the `retained` rows behind them move down by `shift`, and every key head that
+// moves is rotated by -shift positions (apply_rope_delta_to_head, wick/src/backend/cpu.rs:2174-2187: the pairs and the
+// f32 theta schedule of the forward rotation, started from the angle (float)(-shift); separate multiplies and adds).
+// Source and destination rows overlap, so this kernel writes the moved rows -- keys rotated, values as they are -- to
+// staging buffers ([retained][kv_dim] each) and plain device copies put them in place afterwards.  A workgroup takes
+// kShiftRows rows and computes the sines and cosines once for all of them.
+struct KvShiftArgs {
+    const float* k_cache;
+    const float* v_cache;
+    float* k_stage;
+    float* v_stage;
+    uint32_t n_keep, shift, retained, n_kv_heads, head_dim;
+    float theta_scale;
+};
+constexpr uint32_t kShiftRows = 8;
+
+__global__ __launch_bounds__(256) void kv_shift_stage_kernel(KvShiftArgs a) {
+    __shared__ float sn_tab[kRopeTableMax], cs_tab[kRopeTableMax];
+    const uint32_t hd = a.head_dim, half = hd >> 1, kv_dim = a.n_kv_heads * hd;
+    for (uint32_t i = threadIdx.x; i < half; i += 256) {
+        float theta = -(float)a.shift;
+        for (uint32_t j = 0; j < i; j++) theta = __fmul_rn(theta, a.theta_scale);
+        sincosf(theta, &sn_tab[i], &cs_tab[i]);
+    }
+    __syncthreads();
+    const uint32_t r0 = blockIdx.x * kShiftRows, r1 = r0 + kShiftRows < a.retained ? r0 + kShiftRows : a.retained;
+    for (uint32_t r = r0; r < r1; r++) {
+        const float* ks = a.k_cache + (size_t)(a.n_keep + a.shift + r) * kv_dim;
+        const float* vs = a.v_cache + (size_t)(a.n_keep + a.shift + r) * kv_dim;
+        float* kd = a.k_stage + (size_t)r * kv_dim;
+        float* vd = a.v_stage + (size_t)r * kv_dim;
+        for (uint32_t e = threadIdx.x; e < a.n_kv_heads * half; e += 256) {
+            const uint32_t at = (e / half) * hd + e % half;
+            const float sn = sn_tab[e % half], cs = cs_tab[e % half];
+            const float x0 = ks[at], x1 = ks[at + half];
+            kd[at] = __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn));
+            kd[at + half] = __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, cs));
+        }
+        for (uint32_t e = threadIdx.x; e < kv_dim; e += 256) vd[e] = vs[e];
+    }
+}
+
 // ---- decode attention -----------------------------------------------------------------
 // forward_attn_block's tail (wick/src/model/lfm2.rs:984-1006) = attn_scores -> softmax_inplace -> attn_values
 // (cpu.rs:1346-1355, 715-731, 1391-1401), one 256-thread block per query head over positions [0, seq_len).
@@ -1244,6 +1288,19 @@ hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const f
     if (n_tokens > 1 && head_dim == 64) return launch_kernel(L, kFamOther, qk_norm_rope_tokens64_kernel, dim3(n_tokens), dim3(256), a);
     if (n_tokens > 1 && head_dim / 2 <= kRopeTableMax) return launch_kernel(L, kFamOther, qk_norm_rope_tokens_kernel, dim3(n_tokens), dim3(256), a);
     return launch_kernel(L, kFamOther, qk_norm_rope_kernel, dim3(n_heads + n_kv_heads, n_tokens), dim3(64), a);
+}
+
+hipError_t launch_kv_shift(float* d_k_cache, float* d_v_cache, float* d_stage, uint32_t seq_len, uint32_t n_keep, uint32_t shift,
+                           uint32_t n_kv_heads, uint32_t head_dim, float theta_scale, const Launch& L) {
+    const uint32_t retained = seq_len - n_keep - shift;
+    if (retained == 0) return hipSuccess;  // everything behind n_keep is dropped: nothing moves
+    const size_t kv_dim = (size_t)n_kv_heads * head_dim, floats = (size_t)retained * kv_dim;
+    KvShiftArgs a{d_k_cache, d_v_cache, d_stage, d_stage + floats, n_keep, shift, retained, n_kv_heads, head_dim, theta_scale};
+    hipError_t e = launch_kernel(L, kFamOther, kv_shift_stage_kernel, dim3((retained + kShiftRows - 1) / kShiftRows), dim3(256), a);
+    if (e != hipSuccess) return e;
+    e = hipMemcpyAsync(d_k_cache + (size_t)n_keep * kv_dim, a.k_stage, floats * sizeof(float), hipMemcpyDeviceToDevice, L.stream);
+    if (e != hipSuccess) return e;
+    return hipMemcpyAsync(d_v_cache + (size_t)n_keep * kv_dim, a.v_stage, floats * sizeof(float), hipMemcpyDeviceToDevice, L.stream);
 }
 
 hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scores,

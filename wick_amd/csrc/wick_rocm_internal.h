@@ -161,6 +161,10 @@ hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const f
                                float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
                                uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L, uint32_t n_tokens = 1, uint32_t q_stride = 0,
                                uint32_t kv_stride = 0);
+// Drops cache rows [n_keep, n_keep + shift) of one attention layer and re-rotates the keys that move; d_stage holds
+// 2 * (seq_len - n_keep - shift) * n_kv_heads * head_dim floats.
+hipError_t launch_kv_shift(float* d_k_cache, float* d_v_cache, float* d_stage, uint32_t seq_len, uint32_t n_keep, uint32_t shift,
+                           uint32_t n_kv_heads, uint32_t head_dim, float theta_scale, const Launch& L);
 // A prompt of n tokens at once (token j at position pos + j): embedding rows [n][k], the short conv of every (token, channel), causal attention over caches that already hold the prompt's K / V rows (head_dim 32 / 64 / 128 / 256;
 // scratch: attention_prefill_scratch_floats).
 hipError_t launch_embed_rows(const uint8_t* d_w, int type, uint32_t m, uint32_t k, const uint32_t* d_tokens, uint32_t n, float* d_out,

@@ -212,7 +212,50 @@ public:
         return out;
     }
 
+    // supports_embedding_input() == true: steps and prompts fed with hidden-size vectors, and steps that stop after the output norm
+    std::vector<float> forward_from_embedding(const std::vector<float>& embedding, uint32_t pos) {
+        check_embedding(embedding.size(), 1);
+        std::vector<float> logits(cfg_.vocab_size);
+        ctx_.check(wick_rocm_lfm2_forward_from_embedding(ctx_.raw(), m_, embedding.data(), pos, logits.data()));
+        return logits;
+    }
+    std::vector<float> forward_embedding(uint32_t token, uint32_t pos) {
+        std::vector<float> hidden(cfg_.hidden_size);
+        ctx_.check(wick_rocm_lfm2_forward_embedding(ctx_.raw(), m_, token, pos, hidden.data()));
+        return hidden;
+    }
+    std::vector<float> forward_hidden_from_embedding(const std::vector<float>& embedding, uint32_t pos) {
+        check_embedding(embedding.size(), 1);
+        std::vector<float> hidden(cfg_.hidden_size);
+        ctx_.check(wick_rocm_lfm2_forward_hidden_from_embedding(ctx_.raw(), m_, embedding.data(), pos, hidden.data()));
+        return hidden;
+    }
+    std::vector<float> forward_prefill_from_embeddings(const std::vector<float>& embeddings, uint32_t n_tokens, uint32_t start_pos) {
+        check_embedding(embeddings.size(), n_tokens);
+        std::vector<float> logits(cfg_.vocab_size);
+        ctx_.check(wick_rocm_lfm2_forward_prefill_from_embeddings(ctx_.raw(), m_, embeddings.data(), n_tokens, start_pos, logits.data()));
+        return logits;
+    }
+
+    // snapshot_state / restore_state: the state after seq_len positions as bytes (per layer: keys then values, or the conv buffer)
+    std::vector<uint8_t> snapshot_state(uint32_t seq_len) {
+        std::vector<uint8_t> out(wick_rocm_lfm2_state_bytes(m_, seq_len));
+        ctx_.check(wick_rocm_lfm2_snapshot_state(ctx_.raw(), m_, seq_len, out.data(), out.size()));
+        return out;
+    }
+    void restore_state(const std::vector<uint8_t>& snapshot, uint32_t seq_len) {
+        ctx_.check(wick_rocm_lfm2_restore_state(ctx_.raw(), m_, seq_len, snapshot.data(), snapshot.size()));
+    }
+    // supports_kv_shift() == true: shift_kv on a state of seq_len positions; returns the new position count
+    uint32_t shift_kv(uint32_t seq_len, uint32_t n_keep, uint32_t shift) {
+        ctx_.check(wick_rocm_lfm2_shift_kv(ctx_.raw(), m_, seq_len, n_keep, shift));
+        return seq_len - shift;
+    }
+
 private:
+    void check_embedding(size_t len, size_t frames) const {
+        if (frames == 0 || len != frames * cfg_.hidden_size) throw std::invalid_argument("embedding length != frames * hidden_size");
+    }
     RocmContext& ctx_;
     wick_rocm_lfm2* m_ = nullptr;
     wick_rocm_lfm2_config cfg_{};

@@ -58,6 +58,19 @@ static int model_check(const char* path) {
         std::vector<float> logits;
         for (uint32_t pos = 0; pos < picks.size(); pos++) logits = model.forward(picks[pos], pos);
         std::printf("prefill: %zu %zu\n", a, argmax(logits));
+        // state snapshot: the step after a restore repeats the step after the snapshot
+        const std::vector<uint8_t> snap = model.snapshot_state(10);
+        const std::vector<float> first = model.forward(picks[0], 10);
+        model.restore_state(snap, 10);
+        if (model.forward(picks[0], 10) != first) { std::printf("restore_state does not bring the snapshot back\n"); return 1; }
+        // a token's hidden state fed back as an embedding-input step, a context shift, then a step at the shifted position
+        const std::vector<float> hidden = model.forward_embedding(picks[1], 11);
+        const std::vector<float> after = model.forward_from_embedding(hidden, 12);
+        if (hidden.size() != model.config().hidden_size || after.size() != model.config().vocab_size || !std::isfinite(after[0])) return 1;
+        if (model.shift_kv(13, 2, 5) != 8 || !std::isfinite(model.forward(picks[2], 8)[0])) { std::printf("shift_kv failed\n"); return 1; }
+        bool bad_len = false;
+        try { model.forward_prefill_from_embeddings(hidden, 2, 0); } catch (const std::invalid_argument&) { bad_len = true; }
+        if (!bad_len) { std::printf("embedding length not checked\n"); return 1; }
         bool threw = false;
         try { model.forward(model.config().vocab_size, 0); } catch (const wick::BackendError& e) { threw = e.status == WICK_ROCM_ERR_INVALID_ARG; }
         if (!threw) { std::printf("token out of range not reported\n"); return 1; }

@@ -60,6 +60,17 @@ _SIGNATURES = {
     "wick_rocm_lfm2_forward_greedy": (C.c_int, [_P, _P, _U32, _U32, C.POINTER(_U32)]),
     "wick_rocm_lfm2_generate_greedy": (C.c_int, [_P, _P, _U32, _U32, _U32, _P]),
     "wick_rocm_lfm2_logits_device": (_P, [_P]),
+    "wick_rocm_kv_shift_scratch_floats": (C.c_size_t, [_U32, _U32, _U32, _U32, _U32]),
+    "wick_rocm_kv_shift": (C.c_int, [_P, _P, _P, _P, _U32, _U32, _U32, _U32, _U32, _F]),
+    "wick_rocm_lfm2_forward_prefill_from_embeddings": (C.c_int, [_P, _P, _P, _U32, _U32, _P]),
+    "wick_rocm_lfm2_forward_from_embedding": (C.c_int, [_P, _P, _P, _U32, _P]),
+    "wick_rocm_lfm2_forward_embedding": (C.c_int, [_P, _P, _U32, _U32, _P]),
+    "wick_rocm_lfm2_forward_hidden_from_embedding": (C.c_int, [_P, _P, _P, _U32, _P]),
+    "wick_rocm_lfm2_layer_state_bytes": (C.c_size_t, [_P, _U32, _U32]),
+    "wick_rocm_lfm2_state_bytes": (C.c_size_t, [_P, _U32]),
+    "wick_rocm_lfm2_snapshot_state": (C.c_int, [_P, _P, _U32, _P, C.c_size_t]),
+    "wick_rocm_lfm2_restore_state": (C.c_int, [_P, _P, _U32, _P, C.c_size_t]),
+    "wick_rocm_lfm2_shift_kv": (C.c_int, [_P, _P, _U32, _U32, _U32]),
 }
 
 _bound = False
@@ -113,6 +124,15 @@ class Lfm2Ops:
         self.ctx._check(self._l.wick_rocm_qk_norm_rope_tokens(self.ctx._h, _ptr(q), q_stride, _ptr(k), _ptr(v), kv_stride, _ptr(q_norm), _ptr(k_norm),
                                                               _ptr(k_cache), _ptr(v_cache), pos0, n, max_seq, head_dim, n_heads, n_kv_heads, eps,
                                                               theta_scale))
+
+    def kv_shift_scratch_floats(self, seq_len: int, n_keep: int, shift: int, n_kv_heads: int, head_dim: int) -> int:
+        return int(self._l.wick_rocm_kv_shift_scratch_floats(seq_len, n_keep, shift, n_kv_heads, head_dim))
+
+    def encode_kv_shift(self, k_cache, v_cache, scratch, seq_len: int, n_keep: int, shift: int, n_kv_heads: int, head_dim: int,
+                        theta_scale: float) -> None:
+        """One layer's n_keep context shift: cache rows [n_keep, n_keep + shift) dropped, the keys behind them re-rotated."""
+        self.ctx._check(self._l.wick_rocm_kv_shift(self.ctx._h, _ptr(k_cache), _ptr(v_cache), _ptr(scratch), seq_len, n_keep, shift, n_kv_heads,
+                                                   head_dim, theta_scale))
 
     def encode_attention(self, q, k_cache, v_cache, out, scores, seq_len: int, max_seq: int, n_heads: int, n_kv_heads: int, head_dim: int,
                          d_pos=None) -> None:
@@ -247,6 +267,56 @@ class RocmLfm2Model:
                                                                        C.addressof(cancel) if cancel is not None else None, C.byref(consumed),
                                                                        logits.ctypes.data))
         return consumed.value, (logits if consumed.value else None)
+
+    def forward_prefill_from_embeddings(self, embeddings, start_pos: int) -> np.ndarray:
+        """Model::forward_prefill_from_embeddings: `embeddings` is [n][hidden_size]; logits of the last frame."""
+        e = np.ascontiguousarray(embeddings, dtype=np.float32).reshape(-1, self.config["hidden_size"])
+        logits = np.empty(self.config["vocab_size"], np.float32)
+        self.ctx._check(self._l.wick_rocm_lfm2_forward_prefill_from_embeddings(self.ctx._h, self._h, e.ctypes.data, e.shape[0], start_pos,
+                                                                               logits.ctypes.data))
+        return logits
+
+    def _embedding(self, embedding) -> np.ndarray:
+        e = np.ascontiguousarray(embedding, dtype=np.float32).ravel()
+        if e.size != self.config["hidden_size"]:
+            raise ValueError(f"embedding has {e.size} elements, hidden_size is {self.config['hidden_size']}")
+        return e
+
+    def forward_from_embedding(self, embedding, pos: int) -> np.ndarray:
+        """Model::forward_from_embedding: a step fed with a hidden-size vector instead of a token -> logits."""
+        e, logits = self._embedding(embedding), np.empty(self.config["vocab_size"], np.float32)
+        self.ctx._check(self._l.wick_rocm_lfm2_forward_from_embedding(self.ctx._h, self._h, e.ctypes.data, pos, logits.ctypes.data))
+        return logits
+
+    def forward_embedding(self, token: int, pos: int) -> np.ndarray:
+        """Model::forward_embedding: a token step that returns the hidden state after the output norm (no LM head)."""
+        hidden = np.empty(self.config["hidden_size"], np.float32)
+        self.ctx._check(self._l.wick_rocm_lfm2_forward_embedding(self.ctx._h, self._h, token, pos, hidden.ctypes.data))
+        return hidden
+
+    def forward_hidden_from_embedding(self, embedding, pos: int) -> np.ndarray:
+        e, hidden = self._embedding(embedding), np.empty(self.config["hidden_size"], np.float32)
+        self.ctx._check(self._l.wick_rocm_lfm2_forward_hidden_from_embedding(self.ctx._h, self._h, e.ctypes.data, pos, hidden.ctypes.data))
+        return hidden
+
+    def layer_state_bytes(self, layer: int, seq_len: int) -> int:
+        return int(self._l.wick_rocm_lfm2_layer_state_bytes(self._h, layer, seq_len))
+
+    def snapshot_state(self, seq_len: int) -> np.ndarray:
+        """Model::snapshot_state: the state after seq_len positions as bytes (layer by layer: keys then values, or the conv buffer)."""
+        out = np.empty(int(self._l.wick_rocm_lfm2_state_bytes(self._h, seq_len)), np.uint8)
+        self.ctx._check(self._l.wick_rocm_lfm2_snapshot_state(self.ctx._h, self._h, seq_len, out.ctypes.data, out.size))
+        return out
+
+    def restore_state(self, snapshot, seq_len: int) -> None:
+        """Model::restore_state: the inverse of snapshot_state(seq_len)."""
+        b = np.ascontiguousarray(snapshot, dtype=np.uint8)
+        self.ctx._check(self._l.wick_rocm_lfm2_restore_state(self.ctx._h, self._h, seq_len, b.ctypes.data, b.size))
+
+    def shift_kv(self, seq_len: int, n_keep: int, shift: int) -> int:
+        """Model::shift_kv on a state of seq_len positions; returns the new position count."""
+        self.ctx._check(self._l.wick_rocm_lfm2_shift_kv(self.ctx._h, self._h, seq_len, n_keep, shift))
+        return seq_len - shift
 
     def forward_greedy(self, token: int, pos: int) -> int:
         nxt = _U32()
