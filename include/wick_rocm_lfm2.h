@@ -175,6 +175,14 @@ int wick_rocm_ffn_gate_up_silu_quantize_q8(wick_rocm_ctx *ctx, const wick_rocm_w
  * cpu_argmax (wick/src/sampler.rs:7-19).  d_out[0] = pick; when given, *d_token = pick and *d_pos += 1. */
 int wick_rocm_argmax(wick_rocm_ctx *ctx, const float *d_logits, uint32_t n, uint32_t *d_out, uint32_t *d_token, uint32_t *d_pos);
 
+/* The tail of forward_greedy as one call (encode_rmsnorm + encode_gemv_output + argmax_f32, wick/src/model/metal_lfm2.rs:2180-2195):
+ * d_logits[w->m] = W rmsnorm(d_x) with the output norm's weights, then wick_rocm_argmax over them.  A Q6_K head (the tied
+ * embedding of shipped Q4_0 files) norms and quantizes its input inside the GEMV's launch and leaves the pick's first stage
+ * behind as one key per wave: two launches, where wick_rocm_gemv_rmsnorm_f32_multi + wick_rocm_argmax take three; logits and
+ * pick are bit-identical to that sequence.  d_x, d_norm_weight, d_logits 16-byte aligned. */
+int wick_rocm_lm_head_greedy_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const float *d_x, const float *d_norm_weight, float eps,
+                                 float *d_logits, uint32_t *d_out, uint32_t *d_token, uint32_t *d_pos);
+
 /* ---- the model --------------------------------------------------------------------------- */
 
 typedef struct wick_rocm_lfm2 wick_rocm_lfm2;

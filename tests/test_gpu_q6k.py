@@ -7,6 +7,8 @@ import pytest
 import wick_amd as W
 from conftest import assert_f32_parity
 from gpu_util import Problem, fetch_gemm
+from oracle import lfm2_oracle as L
+from wick_amd.lfm2 import Lfm2Ops
 
 pytestmark = pytest.mark.gpu
 
@@ -90,6 +92,66 @@ def test_q6k_batched(ctx, oracle, layout):
         y = fetch_gemm(d_y, m, n, stride, layout)
         for j in range(n):
             assert_f32_parity(y[:, j], oracle.gemv_q6k_q8(p.wb, p.s[j], p.q[j], m, k), f"q6k batched col {j}")
+
+
+@pytest.mark.parametrize("m,k", [(1, 256), (130, 512), (65, 768), (4099, 1024), (300, 2048), (31, 2560), (17, 8192), (65536, 1024)])
+def test_q6k_norm_and_quantizer_inside_the_gemv_launch(ctx, oracle, m, k):
+    """y = W rmsnorm(x), the LM head's form: every wave of the Q6_K GEMV norms and quantizes x itself.  Bit-identical to the norm +
+    quantizer launch followed by the pre-quantized GEMV (also with accumulate), and within the f32 bar of the oracle's GEMV on the
+    same quants."""
+    ops, eps = Lfm2Ops(ctx), 1e-5
+    with Problem(ctx, oracle, W.Q6_K, m, k, seed=2 * m + k) as p:
+        x = oracle.fill_normal(m + k, 1.7, k)
+        nw = (1 + 0.3 * oracle.fill_normal(k, 1.0, k)).astype(np.float32)
+        d_x, d_nw = p.to_device(x), p.to_device(nw)
+        d_q, d_s = p.alloc(k), p.alloc(k // 32 * 4)
+        ops.rmsnorm_quantize(d_x, d_nw, 1, k, eps, d_q, d_s)
+        y0 = oracle.fill_normal(5, 1.0, m)
+        d_y, d_z, d_ya, d_za = p.alloc(m * 4), p.alloc(m * 4), p.to_device(y0), p.to_device(y0)
+        ctx.gemv_with_preq(p.w, d_s, d_q, d_z)
+        ctx.encode_gemv_rmsnorm_fused([p.w], d_x, d_nw, eps, [d_y])
+        y, z = d_y.download(np.float32, m), d_z.download(np.float32, m)
+        assert np.array_equal(y.view(np.uint32), z.view(np.uint32))
+        ctx.gemv_with_preq(p.w, d_s, d_q, d_za, accumulate=True)
+        ctx.encode_gemv_rmsnorm_fused([p.w], d_x, d_nw, eps, [d_ya], accumulate=True)
+        assert np.array_equal(d_ya.download(np.float32, m).view(np.uint32), d_za.download(np.float32, m).view(np.uint32))
+        q, sc = d_q.download(np.int8, k), d_s.download(np.float32, k // 32)
+        assert_f32_parity(y, oracle.gemv_q6k_q8(p.wb, sc, q, m, k), f"q6k norm-fused gemv {m}x{k}")
+        # the quants themselves: the oracle's norm then quantizer (inv_rms may differ in its last bit: at most a quant step)
+        sr, qr = oracle.quantize_q8_0(L.rmsnorm(x, nw, eps))
+        assert np.abs(q.astype(np.int32) - qr.astype(np.int32)).max() <= 1 and np.allclose(sc, sr, rtol=1e-3, atol=0)  # scales: f16 values, at most one step apart
+
+
+@pytest.mark.parametrize("dtype,m,k", [(W.Q6_K, 5000, 1024), (W.Q6_K, 65536, 1024), (W.Q6_K, 300, 512), (W.Q6_K, 3, 256), (W.Q4_0, 5000, 1024), (W.Q8_0, 777, 256)])
+def test_lm_head_and_greedy_pick_in_two_launches(ctx, oracle, dtype, m, k):
+    """Output norm + LM head + greedy pick as one call: logits bit-identical to the norm-fused GEMV, the pick is cpu_argmax of them
+    (wick/src/sampler.rs:7-19) -- for a Q6_K head taken from the keys its waves leave behind."""
+    ops, eps = Lfm2Ops(ctx), 1e-5
+    with Problem(ctx, oracle, dtype, m, k, seed=m + k) as p:
+        x = oracle.fill_normal(3 * m + k, 1.3, k)
+        nw = (1 + 0.3 * oracle.fill_normal(k + 1, 1.0, k)).astype(np.float32)
+        d_x, d_nw = p.to_device(x), p.to_device(nw)
+        d_y, d_z, d_out = p.alloc(m * 4), p.alloc(m * 4), p.alloc(4)
+        d_tok, d_pos = p.to_device(np.array([0], np.uint32)), p.to_device(np.array([9], np.uint32))
+        ctx.encode_gemv_rmsnorm_fused([p.w], d_x, d_nw, eps, [d_z])
+        ops.lm_head_greedy(p.w, d_x, d_nw, eps, d_y, d_out, d_token=d_tok, d_pos=d_pos)
+        y, z = d_y.download(np.float32, m), d_z.download(np.float32, m)
+        assert np.array_equal(y.view(np.uint32), z.view(np.uint32))
+        pick = int(d_out.download(np.uint32, 1)[0])
+        assert pick == L.argmax(y) and int(d_tok.download(np.uint32, 1)[0]) == pick and int(d_pos.download(np.uint32, 1)[0]) == 10
+
+
+def test_lm_head_greedy_pick_takes_the_last_of_equal_logits(ctx, oracle):
+    """Every row of the head is the same row: all logits are equal and the pick is the last index, whichever wave holds it."""
+    ops, m, k = Lfm2Ops(ctx), 3001, 1024
+    row = oracle.synth_weight(W.Q6_K, 1, k, 12)
+    wb = np.tile(row, m)
+    with Problem(ctx, oracle, W.Q6_K, m, k, seed=1, weight_bytes=wb) as p:
+        d_x, d_nw = p.to_device(oracle.fill_normal(4, 1.0, k)), p.to_device(np.ones(k, np.float32))
+        d_y, d_out = p.alloc(m * 4), p.alloc(4)
+        ops.lm_head_greedy(p.w, d_x, d_nw, 1e-5, d_y, d_out)
+        y = d_y.download(np.float32, m)
+        assert (y == y[0]).all() and int(d_out.download(np.uint32, 1)[0]) == m - 1
 
 
 def test_q6k_rejects(ctx, oracle):

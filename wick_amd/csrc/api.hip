@@ -448,13 +448,15 @@ int gemv_xform_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, flo
         hipError_t e = launch_gemv_f32(ws[0]->type, b, k, x, accumulate, ctx->num_cus, ctx->launch(), xform, d_aux, eps);
         return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "fused gemv launch");
     }
-    if (int rc = ensure_scratch(ctx, k, k / 32u, k)) return rc;
     hipError_t e;
-    if (xform == kXformRmsNorm && ws[0]->type == kTypeQ6_K && aligned16(x) && aligned16(d_aux)) {  // norm and quantizer in one launch
-        e = launch_rmsnorm_quantize(x, d_aux, 1, k, k, eps, ctx->scratch_q, ctx->scratch_s, ctx->launch());
-        if (e != hipSuccess) return fail_hip(ctx, e, "rmsnorm_quantize launch");
-        return q6k_gemv_locked(ctx, ws, d_ys, count, ctx->scratch_q, ctx->scratch_s, accumulate);
+    if (xform == kXformRmsNorm && ws[0]->type == kTypeQ6_K && aligned16(x) && aligned16(d_aux)) {  // norm and quantizer inside the GEMV's launch
+        for (uint32_t i = 0; i < count; i++) {
+            e = launch_gemv_q6k_rmsnorm(static_cast<const uint8_t*>(ws[i]->d), ws[i]->m, k, x, d_aux, eps, d_ys[i], accumulate, ctx->num_cus, ctx->launch());
+            if (e != hipSuccess) return fail_hip(ctx, e, "Q6_K gemv launch");
+        }
+        return WICK_ROCM_OK;
     }
+    if (int rc = ensure_scratch(ctx, k, k / 32u, k)) return rc;
     if (xform == kXformRmsNorm) {
         e = launch_rmsnorm(x, d_aux, ctx->scratch_f, 1, k, k, k, eps, ctx->launch());
     } else {

@@ -21,6 +21,8 @@
 // consecutive 16-byte pieces (nontemporal, every cache line exactly once), parks it in a
 // wave-private LDS slot and each lane reads its runs back.  Blocks are only 2-byte aligned,
 // so runs are read as aligned dwords and funnel-shifted by 0 or 2 bytes.
+#include <type_traits>
+
 #include "wick_rocm_device.h"
 #include "wick_rocm_internal.h"
 
@@ -42,6 +44,12 @@ struct Q6kArgs {
     uint32_t rows_per_wave;
     uint32_t y_row_stride;  // y[row * y_row_stride]
     int accumulate;
+    // FUSED variant: the f32 activations and the RMSNorm weights in front of them (xq / xs unused)
+    const float* xf;        // [k]
+    const float* norm_w;    // [k]
+    float eps;
+    // when given, every wave also leaves the greedy-pick key of its best row here (partial[blockIdx.x])
+    unsigned long long* partial;
 };
 
 // NDW dwords starting at byte `off` (even) of the LDS slot.
@@ -56,8 +64,14 @@ __device__ __forceinline__ void read_run(const uint8_t* slot, uint32_t off, uint
     for (int i = 0; i < NDW; i++) out[i] = __builtin_amdgcn_alignbyte(t[i + 1], t[i], sh);
 }
 
-template <int LPR, bool DUMP>
+// FUSED: the wave norms and quantizes the f32 activation vector itself (rmsnorm_quantize_kernel's arithmetic, bit for bit:
+// its 256 threads are played by the wave's lanes four at a time, so that every f64 partial sum is taken over the same
+// elements in the same order; eight lanes per 32-element block in the quantizer) into LDS, under the latency of its first
+// weight span, and reads its half block's quants and scales back from there.  One launch less in front of the LM head;
+// every wave redoes the vector (k floats from the L2), which costs less than that launch.
+template <int LPR, bool DUMP, bool FUSED = false>
 __global__ __launch_bounds__(64) void gemv_q6k_kernel(Q6kArgs a) {
+    static_assert(!(DUMP && FUSED), "the parity hook runs on pre-quantized activations");
     constexpr int RPW = 64 / LPR;  // rows per pass
     constexpr int PIECES = (15 + RPW * LPR * kHalfBytes + 15) / 16;  // upper bound of 16-byte pieces per span
     constexpr int PPL = (PIECES + 63) / 64;                      // pieces per lane
@@ -94,14 +108,77 @@ __global__ __launch_bounds__(64) void gemv_q6k_kernel(Q6kArgs a) {
         }
     };
 
+    // FUSED: the activations and norm weights are requested before the weight span (they come from the L2 and the load
+    // counter retires in order), so that the norm and the quantizer run while the span is still on its way from HBM.
+    constexpr int XE = FUSED ? 2 * LPR : 1;        // k / 64 elements per lane in the order of the f64 sums
+    constexpr int XQ = FUSED ? (LPR + 1) / 2 : 1;  // k / 256 quads per lane for the quantizer
+    float xe[XE];
+    float4 xv4[XQ], wv4[XQ];
+    if constexpr (FUSED) {
+        const uint32_t quads = a.k >> 2;  // a multiple of 64
+#pragma unroll
+        for (int j = 0; j < XE; j++) {
+            const uint32_t e = 64u * j + lane;
+            xe[j] = a.xf[e < a.k ? e : lane];
+        }
+#pragma unroll
+        for (int j = 0; j < XQ; j++) {
+            const uint32_t quad = lane + 64u * j;
+            xv4[j] = reinterpret_cast<const float4*>(a.xf)[quad < quads ? quad : lane];
+            wv4[j] = reinterpret_cast<const float4*>(a.norm_w)[quad < quads ? quad : lane];
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
     issue(wave_row0);
+
+    __shared__ __align__(16) uint32_t fq[FUSED ? LPR * 32 : 4];  // k <= 128 LPR quants
+    __shared__ float fs[FUSED ? LPR * 4 : 1];
+    if constexpr (FUSED) {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        double part[4] = {0.0, 0.0, 0.0, 0.0};  // of the four threads (lane, lane + 64, ..) this lane stands for
+#pragma unroll
+        for (int b = 0; b < XE / 4; b++) {
+            if (256u * b < a.k) {  // uniform; k % 256 == 0
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const double x = (double)xe[4 * b + v];
+                    part[v] += x * x;
+                }
+            }
+        }
+        double total = 0.0;
+#pragma unroll
+        for (int v = 0; v < 4; v++) total += wave_sum_f64(part[v]);
+        const float inv_rms = (float)(1.0 / sqrt(total / (double)a.k + (double)a.eps));
+        const uint32_t quads = a.k >> 2;
+#pragma unroll
+        for (int j = 0; j < XQ; j++) {
+            const uint32_t quad = lane + 64u * j;
+            if (64u * j < quads) {  // uniform: whole rounds
+                const float4 v = xv4[j], w = wv4[j];
+                const float v0 = __fmul_rn(__fmul_rn(v.x, inv_rms), w.x), v1 = __fmul_rn(__fmul_rn(v.y, inv_rms), w.y);
+                const float v2 = __fmul_rn(__fmul_rn(v.z, inv_rms), w.z), v3 = __fmul_rn(__fmul_rn(v.w, inv_rms), w.w);
+                float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+                amax = group_max8(amax);
+                float id;
+                const float scale = q8_scale_and_inverse(amax, id);
+                fq[quad] = q8_pack4(v0, v1, v2, v3, id);
+                if ((quad & 7u) == 0) fs[quad >> 3] = scale;
+            }
+        }
+        // the same wave reads the vector back below; LDS operations of a wave execute in order
+    }
 
     // This lane's 128 activation quants (4 Q8_0 blocks), their scales and the eight 16-element sums.
     uint32_t xq[32];
     float xsc[4];
     int xsum[8];
     {
-        const uint4* src = reinterpret_cast<const uint4*>(a.xq + (size_t)blk * 256 + 128 * n);
+        const uint4* src = FUSED ? reinterpret_cast<const uint4*>(fq + blk * 64 + 32 * n)
+                                 : reinterpret_cast<const uint4*>(a.xq + (size_t)blk * 256 + 128 * n);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const uint4 v = src[i];
@@ -110,6 +187,7 @@ __global__ __launch_bounds__(64) void gemv_q6k_kernel(Q6kArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             if constexpr (DUMP) xsc[i] = 0.0f;  // no scales behind the parity hook
+            else if constexpr (FUSED) xsc[i] = hvalid ? fs[blk * 8 + 4 * n + i] : 0.0f;
             else xsc[i] = hvalid ? a.xs[blk * 8 + 4 * n + i] : 0.0f;
         }
 #pragma unroll
@@ -121,6 +199,7 @@ __global__ __launch_bounds__(64) void gemv_q6k_kernel(Q6kArgs a) {
         }
     }
 
+    unsigned long long best = 0ull;  // below every real key
     for (uint32_t row0 = wave_row0; row0 < wave_row1; row0 += RPW) {
         // span -> LDS (same wave writes and reads; LDS operations of a wave execute in order)
 #pragma unroll
@@ -165,35 +244,65 @@ __global__ __launch_bounds__(64) void gemv_q6k_kernel(Q6kArgs a) {
             const float tot = group_sum<LPR>(hvalid ? acc : 0.0f);
             if (sub == 0 && row < wave_row1) {
                 float* dst = a.y + (size_t)row * a.y_row_stride;
-                *dst = a.accumulate ? *dst + tot : tot;
+                const float out = a.accumulate ? *dst + tot : tot;
+                *dst = out;
+                if (a.partial) {
+                    const unsigned long long key = argmax_key(out, row);
+                    best = key > best ? key : best;
+                }
             }
+        }
+    }
+    if constexpr (!DUMP) {
+        if (a.partial) {  // uniform
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const unsigned long long o = __shfl_xor(best, off, 64);
+                best = o > best ? o : best;
+            }
+            if (lane == 0) a.partial[blockIdx.x] = best;
         }
     }
 }
 
-template <int LPR, bool DUMP>
-hipError_t launch_lpr(Q6kArgs& a, int num_cus, const Launch& L) {
+// The norm-fused variant runs fewer, longer waves: each redoes the norm once (4, 6, 8, 12, 16 per CU measured inside a decode
+// step: 8 best by 0.1 - 0.8 %).
+constexpr uint32_t kFusedWavesPerCu = 8;
+
+// Rows per wave and waves of a launch over m rows with LPR lanes per row.
+template <int LPR>
+uint32_t plan_lpr(uint32_t m, int num_cus, uint32_t& rows_per_wave, uint32_t waves_per_cu = 12u) {
     constexpr uint32_t RPW = 64 / LPR;
-    const uint32_t passes = (a.m + RPW - 1) / RPW;
-    const uint32_t max_waves = (uint32_t)num_cus * 12u;  // measured best on the 65536 x 1024 LM head (8..16 within 7 %)
+    const uint32_t passes = (m + RPW - 1) / RPW;
+    const uint32_t max_waves = (uint32_t)num_cus * waves_per_cu;  // 12: measured best on the 65536 x 1024 LM head (8..16 within 7 %)
     uint32_t ppw = (passes + max_waves - 1) / max_waves;
     if (ppw == 0) ppw = 1;
-    a.rows_per_wave = ppw * RPW;
-    const uint32_t waves = (a.m + a.rows_per_wave - 1) / a.rows_per_wave;
-    return launch_kernel(L, kFamGemv, gemv_q6k_kernel<LPR, DUMP>, dim3(waves), dim3(64), a);
+    rows_per_wave = ppw * RPW;
+    return (m + rows_per_wave - 1) / rows_per_wave;
 }
 
-template <bool DUMP>
+template <int LPR, bool DUMP, bool FUSED>
+hipError_t launch_lpr(Q6kArgs& a, int num_cus, const Launch& L) {
+    const uint32_t waves = plan_lpr<LPR>(a.m, num_cus, a.rows_per_wave, FUSED ? kFusedWavesPerCu : 12u);
+    return launch_kernel(L, kFamGemv, gemv_q6k_kernel<LPR, DUMP, FUSED>, dim3(waves), dim3(64), a);
+}
+
+template <typename F>
+auto with_lpr(uint32_t k, F&& f) {
+    const uint32_t halves = k >> 7;
+    if (halves <= 2) return f(std::integral_constant<int, 2>{});
+    if (halves <= 4) return f(std::integral_constant<int, 4>{});
+    if (halves <= 8) return f(std::integral_constant<int, 8>{});
+    if (halves <= 16) return f(std::integral_constant<int, 16>{});
+    if (halves <= 32) return f(std::integral_constant<int, 32>{});
+    return f(std::integral_constant<int, 64>{});
+}
+
+template <bool DUMP, bool FUSED = false>
 hipError_t dispatch(Q6kArgs& a, int num_cus, const Launch& L) {
     if (a.m == 0) return hipSuccess;
-    const uint32_t halves = a.k >> 7;
-    if (halves <= 2) return launch_lpr<2, DUMP>(a, num_cus, L);
-    if (halves <= 4) return launch_lpr<4, DUMP>(a, num_cus, L);
-    if (halves <= 8) return launch_lpr<8, DUMP>(a, num_cus, L);
-    if (halves <= 16) return launch_lpr<16, DUMP>(a, num_cus, L);
-    if (halves <= 32) return launch_lpr<32, DUMP>(a, num_cus, L);
-    if (halves <= 64) return launch_lpr<64, DUMP>(a, num_cus, L);
-    return hipErrorInvalidValue;  // k > 8192: callers reject it
+    if ((a.k >> 7) > 64) return hipErrorInvalidValue;  // k > 8192: callers reject it
+    return with_lpr(a.k, [&](auto lpr) { return launch_lpr<decltype(lpr)::value, DUMP, FUSED>(a, num_cus, L); });
 }
 
 }  // namespace
@@ -204,6 +313,20 @@ hipError_t launch_gemv_q6k(const uint8_t* d_w, uint32_t m, uint32_t k, const int
     a.w = d_w, a.xq = d_q, a.xs = d_scales, a.y = d_y, a.dots = nullptr;
     a.m = m, a.k = k, a.y_row_stride = y_row_stride, a.accumulate = accumulate;
     return dispatch<false>(a, num_cus, L);
+}
+
+uint32_t gemv_q6k_waves(uint32_t m, uint32_t k, int num_cus) {
+    if (m == 0 || (k >> 7) > 64) return 0;
+    uint32_t rpw = 0;
+    return with_lpr(k, [&](auto lpr) { return plan_lpr<decltype(lpr)::value>(m, num_cus, rpw, kFusedWavesPerCu); });
+}
+
+hipError_t launch_gemv_q6k_rmsnorm(const uint8_t* d_w, uint32_t m, uint32_t k, const float* d_x, const float* d_norm_weight, float eps, float* d_y,
+                                   int accumulate, int num_cus, const Launch& L, unsigned long long* d_partial) {
+    Q6kArgs a{};
+    a.w = d_w, a.y = d_y, a.xf = d_x, a.norm_w = d_norm_weight, a.eps = eps, a.partial = d_partial;
+    a.m = m, a.k = k, a.y_row_stride = 1, a.accumulate = accumulate;
+    return dispatch<false, true>(a, num_cus, L);
 }
 
 hipError_t launch_group_dots_q6k(const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, int32_t* d_out, int num_cus,

@@ -269,6 +269,42 @@ int wick_rocm_argmax(wick_rocm_ctx* ctx, const float* d_logits, uint32_t n, uint
 
 }  // extern "C"
 
+namespace {
+
+// Output norm + LM head + greedy pick (lock held).  A Q6_K head norms and quantizes its input itself and leaves one pick key
+// per wave, so the pick's first stage is not launched: two launches instead of four.  `history` / `emb_out`: the model's
+// extras of launch_argmax (may be null).
+int lm_head_greedy_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const float* d_x, const float* d_norm_weight, float eps, float* d_logits,
+                          unsigned long long* d_partial, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos, uint32_t* d_history,
+                          uint32_t history_len, float* d_emb_out) {
+    const uint8_t* wd = static_cast<const uint8_t*>(w->d);
+    const uint32_t waves = w->type == kTypeQ6_K ? gemv_q6k_waves(w->m, w->k, ctx->num_cus) : 0u;
+    if (waves != 0 && waves <= kArgmaxPartials && !misaligned(d_x, 16) && !misaligned(d_norm_weight, 16)) {
+        hipError_t e = launch_gemv_q6k_rmsnorm(wd, w->m, w->k, d_x, d_norm_weight, eps, d_logits, 0, ctx->num_cus, ctx->launch(), d_partial);
+        if (e != hipSuccess) return fail_hip(ctx, e, "Q6_K gemv launch");
+        e = launch_argmax_final(d_partial, waves, w->m, d_out, d_token, d_pos, d_history, history_len, ctx->launch(), wd, w->type, w->m, w->k, d_emb_out);
+        return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
+    }
+    if (int rc = wick_rocm_gemv_rmsnorm_f32_multi(ctx, &w, &d_logits, 1, d_x, d_norm_weight, eps, 0)) return rc;
+    hipError_t e = launch_argmax(d_logits, w->m, d_partial, d_out, d_token, d_pos, d_history, history_len, ctx->launch(), wd, w->type, w->m, w->k, d_emb_out);
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
+}
+
+}  // namespace
+
+extern "C" int wick_rocm_lm_head_greedy_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const float* d_x, const float* d_norm_weight, float eps,
+                                            float* d_logits, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos) {
+    WR_ENTER(ctx);
+    if (!w || !w->d) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "null weight handle");
+    if (!d_x || !d_norm_weight || !d_logits || !d_out) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lm_head_greedy: null device pointer");
+    if (misaligned(d_logits, 16)) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lm_head_greedy: logits must be 16-byte aligned");
+    if (!ctx->argmax_partial) {
+        if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "lm_head_greedy: first use inside a graph capture (call it once before capturing)");
+        WR_HIP(ctx, hipMalloc(reinterpret_cast<void**>(&ctx->argmax_partial), kArgmaxPartials * sizeof(unsigned long long)));
+    }
+    return lm_head_greedy_locked(ctx, w, d_x, d_norm_weight, eps, d_logits, ctx->argmax_partial, d_out, d_token, d_pos, nullptr, 0, nullptr);
+}
+
 // ---------------------------------------------------------------------------------------------
 // The model.
 
@@ -425,12 +461,10 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, StepMode mode) {
     }
     if (rc) return rc;
     if (mode == kStepHidden) return wick_rocm_rmsnorm(ctx, m->hidden, m->out_norm, m->gated, 1, hs, hs, hs, c.rms_norm_eps);  // m->gated is free here
-    if ((rc = gemv_normed(ctx, {m->embd}, {m->logits}, m->hidden, m->out_norm, c.rms_norm_eps))) return rc;
-    if (mode != kStepGreedy) return WICK_ROCM_OK;
+    if (mode != kStepGreedy) return gemv_normed(ctx, {m->embd}, {m->logits}, m->hidden, m->out_norm, c.rms_norm_eps);
     std::lock_guard<std::recursive_mutex> lk(ctx->mu);
-    hipError_t e = launch_argmax(m->logits, c.vocab_size, m->d_argmax_partial, m->d_pick, m->d_token, m->d_pos, m->d_history, c.max_seq_len,
-                                 ctx->launch(), static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m, c.hidden_size, m->hidden);
-    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "argmax launch");
+    return lm_head_greedy_locked(ctx, m->embd, m->hidden, m->out_norm, c.rms_norm_eps, m->logits, m->d_argmax_partial, m->d_pick, m->d_token, m->d_pos,
+                                 m->d_history, c.max_seq_len, m->hidden);
 }
 
 int step_graph(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, StepMode mode, wick_rocm_graph** out) {

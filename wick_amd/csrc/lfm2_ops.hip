@@ -1160,13 +1160,6 @@ __global__ __launch_bounds__(256) void silu_mul_quantize_kernel(const float* __r
 // equal maxima wins; bit-exact.  Two small launches (64 blocks, then one wave over their partial keys): a single
 // block would spend 20 us walking a 65536-entry vocabulary.  Optionally publishes the pick as the next step's
 // token and advances the device-side position.
-__device__ __forceinline__ unsigned long long argmax_key(float f, uint32_t index) {
-    if (f != f) f = -__builtin_inff();
-    int32_t b = (int32_t)__float_as_uint(f);
-    b ^= (int32_t)(((uint32_t)(b >> 31)) >> 1);                 // total_cmp's transform: signed order
-    const uint32_t ordered = (uint32_t)b ^ 0x80000000u;          // ... as unsigned order
-    return ((unsigned long long)ordered << 32) | index;          // equal values: the larger index wins
-}
 
 constexpr uint32_t kArgmaxBlocks = 64;
 
@@ -1210,7 +1203,8 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __rest
     }
 }
 
-// Stage 2: one wave merges the partial keys and publishes the pick.
+// Stage 2: one workgroup (one wave when there are at most 64 keys and nothing to look up) merges the partial keys and
+// publishes the pick.
 // An embedding to look the next step's input up in (w null: none): row `token` of w as k floats into `out`.
 struct EmbedArgs {
     const uint8_t* w;
@@ -1223,23 +1217,35 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(const unsigned long l
                                                            uint32_t* __restrict__ out, uint32_t* __restrict__ d_token, uint32_t* __restrict__ d_pos,
                                                            uint32_t* __restrict__ d_history, uint32_t history_len, EmbedArgs emb) {
     __shared__ uint32_t picked;
-    if (threadIdx.x < 64) {  // the first wave reduces the (at most 64) partial keys
-        unsigned long long best = threadIdx.x < blocks ? partial[threadIdx.x] : 0ull;
+    __shared__ unsigned long long red[4];
+    const uint32_t waves = blockDim.x >> 6;  // 1 (at most 64 partial keys) or 4
+    unsigned long long best = 0ull;
+    for (uint32_t i = threadIdx.x; i < blocks; i += blockDim.x) {
+        const unsigned long long k = partial[i];
+        best = k > best ? k : best;
+    }
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const unsigned long long o = __shfl_xor(best, off, 64);
-            best = o > best ? o : best;
-        }
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long o = __shfl_xor(best, off, 64);
+        best = o > best ? o : best;
+    }
+    if (waves > 1) {
+        if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = best;
+        __syncthreads();
         if (threadIdx.x == 0) {
-            const uint32_t pick = n ? (uint32_t)(best & 0xffffffffull) : 0u;
-            picked = pick;
-            out[0] = pick;
-            if (d_token) *d_token = pick;
-            if (d_pos) {
-                const uint32_t pos = *d_pos;
-                if (d_history && pos < history_len) d_history[pos] = pick;  // the pick made after the token at `pos`
-                *d_pos = pos + 1u;
-            }
+            const unsigned long long a = red[0] > red[1] ? red[0] : red[1], b = red[2] > red[3] ? red[2] : red[3];
+            best = a > b ? a : b;
+        }
+    }
+    if (threadIdx.x == 0) {
+        const uint32_t pick = n ? (uint32_t)(best & 0xffffffffull) : 0u;
+        picked = pick;
+        out[0] = pick;
+        if (d_token) *d_token = pick;
+        if (d_pos) {
+            const uint32_t pos = *d_pos;
+            if (d_history && pos < history_len) d_history[pos] = pick;  // the pick made after the token at `pos`
+            *d_pos = pos + 1u;
         }
     }
     if (!emb.w) return;
@@ -1465,8 +1471,15 @@ hipError_t launch_argmax(const float* d_x, uint32_t n, unsigned long long* d_par
     const uint32_t blocks = n >= 4096u ? kArgmaxBlocks : 1u;
     hipError_t e = launch_kernel(L, kFamOther, argmax_partial_kernel, dim3(blocks), dim3(256), d_x, n, d_partial);
     if (e != hipSuccess) return e;
+    return launch_argmax_final(d_partial, blocks, n, d_out, d_token, d_pos, d_history, history_len, L, d_embd, embd_type, embd_m, embd_k, d_embd_out);
+}
+
+hipError_t launch_argmax_final(const unsigned long long* d_partial, uint32_t n_partials, uint32_t n, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos,
+                               uint32_t* d_history, uint32_t history_len, const Launch& L, const uint8_t* d_embd, int embd_type, uint32_t embd_m,
+                               uint32_t embd_k, float* d_embd_out) {
     const EmbedArgs emb{d_embd_out ? d_embd : nullptr, d_embd_out, embd_type, embd_m, embd_k};
-    return launch_kernel(L, kFamOther, argmax_final_kernel, dim3(1), dim3(emb.w ? 256 : 64), d_partial, blocks, n, d_out, d_token, d_pos, d_history, history_len, emb);
+    return launch_kernel(L, kFamOther, argmax_final_kernel, dim3(1), dim3(emb.w || n_partials > 64u ? 256 : 64), d_partial, n_partials, n, d_out, d_token,
+                         d_pos, d_history, history_len, emb);
 }
 
 hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L, const uint8_t* d_embd, int embd_type,

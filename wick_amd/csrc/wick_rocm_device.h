@@ -231,6 +231,16 @@ __device__ __forceinline__ float wave_max_f32(float v) {
     return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
 
+// The greedy pick's ordering (cpu_argmax, wick/src/sampler.rs:7-19) as one unsigned key: NaN counts as -inf, values order
+// by f32::total_cmp, and of equal values the larger index wins; 0 is below every real key.
+__device__ __forceinline__ unsigned long long argmax_key(float f, uint32_t index) {
+    if (f != f) f = -__builtin_inff();
+    int32_t b = (int32_t)__float_as_uint(f);
+    b ^= (int32_t)(((uint32_t)(b >> 31)) >> 1);                 // total_cmp's transform: signed order
+    const uint32_t ordered = (uint32_t)b ^ 0x80000000u;          // ... as unsigned order
+    return ((unsigned long long)ordered << 32) | index;          // equal values: the larger index wins
+}
+
 __device__ __forceinline__ float bits_f(uint32_t u) { return __uint_as_float(u); }
 
 // ggml_expf (wick/src/backend/cpu.rs:604-652), operation for operation: bit-exact.

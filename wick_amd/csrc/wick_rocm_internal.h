@@ -113,6 +113,12 @@ hipError_t launch_gemv_shortconv_f32(int type, const uint8_t* d_w, uint32_t m, u
 // 16 bytes; y[row * y_row_stride].  launch_group_dots_q6k is its parity hook: out[i * (k/16) + g] = exact i32 dot of 16-weight group g.
 constexpr int kTypeQ6_K = 14;  // ggml id, wick/src/gguf.rs:36-51
 constexpr int kQ6KBlockBytes = 210;
+// y = W rmsnorm(x) with the norm and the Q8_0 quantizer inside the GEMV's launch (bit-identical to launch_rmsnorm_quantize +
+// launch_gemv_q6k); d_x / d_norm_weight 16-byte aligned.  d_partial non-null: gemv_q6k_waves(m, k, num_cus) greedy-pick keys, one
+// per wave, for launch_argmax_final.
+uint32_t gemv_q6k_waves(uint32_t m, uint32_t k, int num_cus);
+hipError_t launch_gemv_q6k_rmsnorm(const uint8_t* d_w, uint32_t m, uint32_t k, const float* d_x, const float* d_norm_weight, float eps, float* d_y,
+                                   int accumulate, int num_cus, const Launch& L, unsigned long long* d_partial = nullptr);
 hipError_t launch_gemv_q6k(const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, const float* d_scales, float* d_y,
                            uint32_t y_row_stride, int accumulate, int num_cus, const Launch& L);
 hipError_t launch_group_dots_q6k(const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, int32_t* d_out, int num_cus,
@@ -203,11 +209,15 @@ hipError_t launch_silu_mul_quantize(const float* d_gate, const float* d_up, uint
 hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const Launch& L);
 // d_history[pos] = pick (pos = *d_pos before it is advanced), when given.  d_partial: scratch of kArgmaxPartials keys, 8-byte aligned;
 // d_x 16-byte aligned.
-constexpr uint32_t kArgmaxPartials = 64;
+constexpr uint32_t kArgmaxPartials = 4096;  // 64 for the two-stage pick; up to one key per wave of a Q6_K LM head that leaves its own
 // d_embd_out non-null: the pick's row of the embedding (d_embd, type, m x k) is written there as the next step's input.
 hipError_t launch_argmax(const float* d_x, uint32_t n, unsigned long long* d_partial, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos,
                          uint32_t* d_history, uint32_t history_len, const Launch& L, const uint8_t* d_embd = nullptr, int embd_type = 0,
                          uint32_t embd_m = 0, uint32_t embd_k = 0, float* d_embd_out = nullptr);
+// The second stage on its own, over n_partials keys that a producer has left in d_partial (n = the number of candidates; 0: pick 0).
+hipError_t launch_argmax_final(const unsigned long long* d_partial, uint32_t n_partials, uint32_t n, uint32_t* d_out, uint32_t* d_token, uint32_t* d_pos,
+                               uint32_t* d_history, uint32_t history_len, const Launch& L, const uint8_t* d_embd = nullptr, int embd_type = 0,
+                               uint32_t embd_m = 0, uint32_t embd_k = 0, float* d_embd_out = nullptr);
 hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, uint32_t pos, const Launch& L, const uint8_t* d_embd = nullptr,
                            int embd_type = 0, uint32_t embd_m = 0, uint32_t embd_k = 0, float* d_embd_out = nullptr);
 hipError_t launch_advance_pos(uint32_t* d_pos, const Launch& L);

@@ -42,6 +42,7 @@ _SIGNATURES = {
     "wick_rocm_shortconv_step": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32]),
     "wick_rocm_silu_mul": (C.c_int, [_P, _P, _P, _U32]),
     "wick_rocm_argmax": (C.c_int, [_P, _P, _U32, _P, _P, _P]),
+    "wick_rocm_lm_head_greedy_f32": (C.c_int, [_P, _P, _P, _P, _F, _P, _P, _P, _P]),
     "wick_rocm_rmsnorm_quantize_q8_0": (C.c_int, [_P, _P, _P, _U32, _U32, _U32, _F, _P, _P]),
     "wick_rocm_silu_mul_quantize_q8_0": (C.c_int, [_P, _P, _P, _U32, _U32, _P, _P]),
     "wick_rocm_lfm2_load": (C.c_int, [_P, _P, _U32, C.POINTER(_P)]),
@@ -206,6 +207,11 @@ class Lfm2Ops:
 
     def argmax(self, logits, n: int, out, d_token=None, d_pos=None) -> None:
         self.ctx._check(self._l.wick_rocm_argmax(self.ctx._h, _ptr(logits), n, _ptr(out), _ptr(d_token), _ptr(d_pos)))
+
+    def lm_head_greedy(self, w, x, norm_weight, eps: float, logits, out, d_token=None, d_pos=None) -> None:
+        """Output norm + LM head + greedy pick: logits = W rmsnorm(x), out[0] = argmax (and the device-side token / position)."""
+        self.ctx._check(self._l.wick_rocm_lm_head_greedy_f32(self.ctx._h, w.handle, _ptr(x), _ptr(norm_weight), eps, _ptr(logits), _ptr(out),
+                                                             _ptr(d_token), _ptr(d_pos)))
 
 
 class RocmLfm2Model:
