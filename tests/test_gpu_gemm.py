@@ -105,7 +105,8 @@ def test_accumulate(ctx, oracle, dtype, n):
     ((64, 96), 5, 256, W.LAYOUT_TOKEN_MAJOR, False),             # below the MFMA hand-off: one call per weight
 ])
 def test_gemm_multi_equals_one_launch_per_weight(ctx, oracle, dtype, ms, n, k, layout, acc):
-    """Up to three weights over the same activations in one launch: bit-identical to one launch per weight."""
+    """Up to three weights over the same activations in one launch: bit-identical to one launch per weight (each taken unsplit:
+    a single weight's launch with few tiles may otherwise walk K in shares, which moves its sums by a few 1e-7)."""
     with Problem(ctx, oracle, dtype, ms[0], k, n, seed=sum(ms) + n) as p:
         ws = [p.w] + [ctx.upload_weight(oracle.synth_weight(dtype, m, k, 50 + i, 0.02), dtype, m, k) for i, m in enumerate(ms[1:])]
         tm = layout == W.LAYOUT_TOKEN_MAJOR
@@ -117,11 +118,20 @@ def test_gemm_multi_equals_one_launch_per_weight(ctx, oracle, dtype, ms, n, k, l
         ya = [d_a.ptr + elem(o) for o in offs]
         yb = [d_b.ptr + elem(o) for o in offs]
         ctx.gemm_preq_multi(ws, p.d_s, p.d_q, n, ya, stride, layout=layout, accumulate=acc)
-        for w, y in zip(ws, yb):
-            ctx.gemm_preq(w, p.d_s, p.d_q, n, y, y_stride=stride, layout=layout, accumulate=acc)
+        ctx.set_gemm_max_k_splits(1)
+        try:
+            for w, y in zip(ws, yb):
+                ctx.gemm_preq(w, p.d_s, p.d_q, n, y, y_stride=stride, layout=layout, accumulate=acc)
+        finally:
+            ctx.set_gemm_max_k_splits(0)
         a, b = d_a.download(np.float32, y0.size), d_b.download(np.float32, y0.size)
         assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
         assert not np.array_equal(a, y0)
+        d_c = p.to_device(y0)  # the same launches as the library routes them by default: equal to the f32 bar
+        for w, o in zip(ws, offs):
+            ctx.gemm_preq(w, p.d_s, p.d_q, n, d_c.ptr + elem(o), y_stride=stride, layout=layout, accumulate=acc)
+        c = d_c.download(np.float32, y0.size)
+        assert np.linalg.norm(c.astype(np.float64) - a) <= 1e-6 * np.linalg.norm(a)
         with pytest.raises(W.RocmError, match="share k and dtype"):
             other = ctx.upload_weight(oracle.synth_weight(dtype, 32, k + 128, 3, 0.02), dtype, 32, k + 128)
             ws.append(other)
@@ -176,6 +186,11 @@ def test_argument_errors(ctx, oracle):
     (W.Q4_0, 300, 70, 4608, "row", True),        # ragged rows and tokens, 8 shares, row-major output
     (W.Q8_0, 2048, 640, 6912, "token", False),   # 160 tiles: no split (would pass 256)
     (W.Q4_0, 1024, 2002, 4608, "token", False),  # 256 tiles: no split
+    (W.Q4_0, 256, 300, 1024, "row", False),      # 10 tiles (not a multiple of the 8 slots the tile map deals out), 4 shares of 2 stages
+    (W.Q8_0, 640, 200, 2048, "token", True),     # 20 tiles, 4 shares
+    (W.Q4_0, 384, 130, 1152, "token", False),    # 9 stages in 4 shares: 2, 2, 2, 3
+    (W.Q8_0, 200, 40, 4224, "row", True),        # 33 stages in 8 shares: 4 or 5 each
+    (W.Q4_0, 3072, 128, 1024, "token", False),   # the in projection of a short prompt: 48 tiles, 4 shares
 ])
 def test_gemm_split_over_k(ctx, oracle, dtype, m, n, k, layout, accumulate):
     """GEMM launches with few tiles and a long K walk K in shares (one workgroup per tile and share, a second launch adds the

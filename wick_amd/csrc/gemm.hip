@@ -577,9 +577,9 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     const uint32_t nb = a.k >> 5;
     // this workgroup's stages: [first, first + stages)
     const uint32_t all_stages = nb / KB;
-    const uint32_t per_split = (all_stages + ksplit - 1) / ksplit;
-    const uint32_t first = split * per_split;
-    const uint32_t stages = min(all_stages, first + per_split) - first;  // >= 1: the host splits only where every share is
+    // shares differ by at most one stage and none is empty (the host splits only where all_stages >= 2 * ksplit)
+    const uint32_t first = split * all_stages / ksplit;
+    const uint32_t stages = (split + 1u) * all_stages / ksplit - first;
 
     float acc[4][4];
 #pragma unroll
@@ -678,15 +678,16 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 }
 
 // How many ways a single-weight launch is split over K: only narrow launches that leave at least half of the CUs without
-// a tile, with K long enough (>= 16 stages) that the shorter walk pays for the second launch, every share >= 4 stages.
+// a tile, with K long enough (>= 8 stages) that the shorter walk pays for the second launch, every share >= 2 stages (a stage
+// of a launch with few tiles costs a whole memory round trip, 1.2 - 1.4 us: nothing else is there to hide it).
 uint32_t split_k_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits) {
     const uint32_t row_tiles = (m + BM - 1) / BM;
     const bool narrow = n <= BN_NARROW || row_tiles * ((n + BN - 1) / BN) <= 256;
     if (!narrow) return 1;
     const uint32_t tiles = row_tiles * ((n + BN_NARROW - 1) / BN_NARROW), stages = (k >> 5) / KB;
-    if (stages < 16) return 1;
+    if (stages < 8) return 1;
     uint32_t s_ = 1;
-    while (2 * s_ <= max_splits && tiles * 2 * s_ <= 256 && stages / (2 * s_) >= 4) s_ *= 2;
+    while (2 * s_ <= max_splits && tiles * 2 * s_ <= 256 && stages / (2 * s_) >= 2) s_ *= 2;
     return s_;
 }
 
@@ -708,7 +709,7 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0) {
     const uint32_t blocks = ((tiles + 7u) / 8u) * 8u;  // every XCD gets the same number of slots
     if (narrow) {
         if (!DUMP && a.ksplit > 1) {
-            const uint32_t split_blocks = ((tiles * a.ksplit + 7u) / 8u) * 8u;
+            const uint32_t split_blocks = blocks * a.ksplit;  // tile id = blockIdx.x / ksplit must run over all `blocks` slots of the tile map
             hipError_t e = type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(split_blocks), dim3(THREADS), a)
                                              : launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(split_blocks), dim3(THREADS), a);
             if (e != hipSuccess) return e;
