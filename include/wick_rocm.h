@@ -165,9 +165,19 @@ int wick_rocm_gemm_q8(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_
 /* The same for 1..3 weights of one dtype and k over the same quantized activations (Q / K / V, gate / up of a prompt
  * pass: the batched counterpart of encode_gemv_qkv / encode_gemv_gate_up, wick/src/model/metal_lfm2.rs:1043-1119) in
  * one launch, y_i written like wick_rocm_gemm_q8 writes it (shared stride, layout, accumulate flag); results are those
- * of one wick_rocm_gemm_q8 call per weight, bit for bit. */
+ * of one wick_rocm_gemm_q8 call per weight taken without the K split (wick_rocm_set_gemm_max_k_splits), bit for bit. */
 int wick_rocm_gemm_q8_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *ws, float *const *d_ys, uint32_t count,
                             const int8_t *d_quants, const float *d_scales, uint32_t n, uint32_t y_stride, int y_layout, int accumulate);
+
+/* A residual projection of a prompt pass together with the norm and quantizer behind it (encode_gemm_add + encode_rmsnorm_batch /
+ * encode_add_rmsnorm_batch + quantize_columns, wick/src/model/metal_lfm2.rs:998-1041, 1400-1460; CPU: wick/src/model/lfm2.rs:1380-1420):
+ * x[j][.] += W * (activation j) for n token rows x[j * x_stride ..] (w->m floats each), then d_out_quants / d_out_scales =
+ * Q8_0(rmsnorm(x[j]) * norm_weight) ([n][m] quants, [n][m / 32] scales).  The same bits as wick_rocm_gemm_q8 (token-major,
+ * accumulate) followed by wick_rocm_rmsnorm_quantize_q8_0; when the projection is split over K, the norm's kernel adds the shares
+ * up and the split's own reduce launch is not made.  The output may be the projection's own input buffers.  m % 32 == 0. */
+int wick_rocm_gemm_q8_residual_rmsnorm_quantize(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_t *d_quants, const float *d_scales,
+                                                uint32_t n, float *d_x, uint32_t x_stride, const float *d_norm_weight, float eps,
+                                                int8_t *d_out_quants, float *d_out_scales);
 
 /* The n at and above which wick_rocm_gemm_q8 / wick_rocm_matmul_f32 hand off from the
  * multi-token GEMV to the MFMA GEMM (default 16, the reference's GEMM_MIN_N,

@@ -223,3 +223,52 @@ def test_gemm_split_over_k(ctx, oracle, dtype, m, n, k, layout, accumulate):
     assert_f32_parity(outs[2], ref, "unsplit GEMM")
     assert np.linalg.norm(outs[0].astype(np.float64) - outs[2]) <= 1e-6 * np.linalg.norm(outs[2])
     w.free(), d_q.free(), d_s.free()
+
+
+@pytest.mark.parametrize("dtype,m,n,k,pad", [
+    (W.Q4_0, 1024, 512, 4608, 0),   # the down projection of a 512-token prompt: split, the norm's kernel adds the shares up
+    (W.Q8_0, 1024, 100, 1024, 8),   # an out projection of a short prompt: split in 4, padded rows
+    (W.Q4_0, 256, 300, 1024, 0),    # 10 tiles
+    (W.Q4_0, 1024, 2002, 4608, 0),  # 256 tiles: unsplit, the plain norm kernel
+    (W.Q8_0, 512, 7, 256, 4),       # below the MFMA hand-off: multi-token GEMV, then the norm
+])
+def test_residual_projection_with_norm_and_quantizer(ctx, oracle, dtype, m, n, k, pad):
+    """x += W a, then Q8_0(rmsnorm(x)): one call == wick_rocm_gemm_q8 (accumulate) + wick_rocm_rmsnorm_quantize_q8_0, bit for bit -- the
+    residual rows, the quants and the scales -- whether or not the projection is split over K; and x against the oracle."""
+    from wick_amd.lfm2 import Lfm2Ops
+    ops, eps, stride = Lfm2Ops(ctx), 1e-5, m + pad
+    wb = oracle.synth_weight(dtype, m, k, seed=31)
+    w = ctx.upload_weight(wb, dtype, m, k)
+    s, q = oracle.quantize_q8_0_batch(oracle.fill_normal(5, 1.0, n * k), n, k)
+    d_q, d_s = ctx.to_device(q), ctx.to_device(s)
+    x0 = oracle.fill_normal(6, 1.0, n * stride)
+    nw = (1 + 0.3 * oracle.fill_normal(7, 1.0, m)).astype(np.float32)
+    d_nw = ctx.to_device(nw)
+    res = []
+    for fused in (True, False):
+        d_x, d_oq, d_os = ctx.to_device(x0), ctx.alloc(n * m), ctx.alloc(n * (m // 32) * 4)
+        if fused:
+            ctx.gemm_preq_residual_rmsnorm_quantize(w, d_s, d_q, n, d_x, stride, d_nw, eps, d_oq, d_os)
+        else:
+            ctx.gemm_preq(w, d_s, d_q, n, d_x, y_stride=stride, layout=W.LAYOUT_TOKEN_MAJOR, accumulate=True)
+            ops.rmsnorm_quantize(d_x, d_nw, n, m, eps, d_oq, d_os, x_stride=stride)
+        res.append((d_x.download(np.float32, n * stride), d_oq.download(np.int8, n * m), d_os.download(np.float32, n * (m // 32))))
+        for b in (d_x, d_oq, d_os):
+            b.free()
+    for a, b in zip(*res):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    x = res[0][0].reshape(n, stride)
+    assert np.array_equal(x[:, m:], x0.reshape(n, stride)[:, m:])  # padding untouched
+    ref = oracle.gemm_q8(dtype, wb, s, q, m, n, k, f64=True).T + x0.reshape(n, stride)[:, :m]
+    assert_f32_parity(x[:, :m], ref, "residual projection")
+    # quantizing the input in place of the projection's own input buffers is what the prompt pass does
+    if m == k:
+        d_x, d_q2, d_s2 = ctx.to_device(x0), ctx.to_device(q), ctx.to_device(s)
+        ctx.gemm_preq_residual_rmsnorm_quantize(w, d_s2, d_q2, n, d_x, stride, d_nw, eps, d_q2, d_s2)
+        assert np.array_equal(d_q2.download(np.int8, n * m), res[0][1]) and np.array_equal(d_s2.download(np.float32, n * (m // 32)).view(np.uint32), res[0][2].view(np.uint32))
+        for b in (d_x, d_q2, d_s2):
+            b.free()
+    with pytest.raises(W.RocmError, match="multiple of 32"):
+        w2 = ctx.upload_weight(oracle.synth_weight(dtype, 48, 256, seed=1), dtype, 48, 256)
+        ctx.gemm_preq_residual_rmsnorm_quantize(w2, d_s, d_q, 1, d_nw, 48, d_nw, eps, d_q, d_s)
+    w.free(), w2.free(), d_q.free(), d_s.free(), d_nw.free()

@@ -60,8 +60,11 @@ int ensure_scratch(wick_rocm_ctx* ctx, size_t q_bytes, size_t s_floats, size_t f
 // Routing shared by wick_rocm_gemm_q8 and wick_rocm_matmul_f32 (lock already held).
 // may_split: the call may take the K-split launch pair, whose partial sums live in context scratch (never the entry point
 // that must not allocate, never during a capture that has not reserved the room).
+// deferred (may be null): when given and the launch is split, the shares are left in ctx->scratch_f for the caller's next
+// kernel to add up (*deferred = their number); otherwise *deferred = 0 and y is complete.
 int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q, const float* d_s, uint32_t n,
-                float* d_y, uint32_t y_stride, int y_layout, int accumulate, bool may_split = true) {
+                float* d_y, uint32_t y_stride, int y_layout, int accumulate, bool may_split = true, uint32_t* deferred = nullptr) {
+    if (deferred) *deferred = 0;
     if (!d_q || !d_s || !d_y) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "null device pointer");
     if (n == 0) return WICK_ROCM_OK;
     if (y_layout != WICK_ROCM_LAYOUT_TOKEN_MAJOR && y_layout != WICK_ROCM_LAYOUT_ROW_MAJOR)
@@ -88,8 +91,10 @@ int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q
             if (ctx->capturing && floats > ctx->scratch_f_cap) splits = 1;  // no room reserved: the unsplit launch, same result to the f32 bar
             else if (int rc = ensure_scratch(ctx, 0, 0, floats)) return rc;
         }
+        const bool defer = deferred && splits > 1;
         e = launch_gemm_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
-                             y_layout, accumulate, ctx->launch(), splits, splits > 1 ? ctx->scratch_f : nullptr);
+                             y_layout, accumulate, ctx->launch(), splits, splits > 1 ? ctx->scratch_f : nullptr, defer);
+        if (defer && e == hipSuccess) *deferred = splits;
     } else
         e = launch_gemv_tokens(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
                                y_layout, accumulate, ctx->num_cus, ctx->launch());
@@ -588,6 +593,29 @@ int wick_rocm_gemm_q8(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_
     WR_ENTER(ctx);
     if (int rc = check_weight(ctx, w)) return rc;
     return gemm_locked(ctx, w, d_quants, d_scales, n, d_y, y_stride, y_layout, accumulate);
+}
+
+int wick_rocm_gemm_q8_residual_rmsnorm_quantize(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_quants, const float* d_scales,
+                                                uint32_t n, float* d_x, uint32_t x_stride, const float* d_norm_weight, float eps,
+                                                int8_t* d_out_quants, float* d_out_scales) {
+    WR_ENTER(ctx);
+    if (int rc = check_weight(ctx, w)) return rc;
+    if (!d_x || !d_norm_weight || !d_out_quants || !d_out_scales) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemm + norm: null device pointer");
+    if (w->m % 32u != 0 || x_stride < w->m || x_stride % 4u != 0)
+        return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "gemm + norm: rows must be a multiple of 32, x_stride >= rows and a multiple of 4");
+    if (reinterpret_cast<uintptr_t>(d_x) % 16u != 0 || reinterpret_cast<uintptr_t>(d_norm_weight) % 16u != 0 ||
+        reinterpret_cast<uintptr_t>(d_out_quants) % 4u != 0)
+        return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "gemm + norm: x and the norm weights must be 16-byte aligned");
+    if (n == 0) return WICK_ROCM_OK;
+    uint32_t shares = 0;
+    if (int rc = gemm_locked(ctx, w, d_quants, d_scales, n, d_x, x_stride, WICK_ROCM_LAYOUT_TOKEN_MAJOR, 1, true,
+                             w->m <= kResidualNormMaxDim ? &shares : nullptr))
+        return rc;
+    // a split projection's shares are added up by the norm's kernel instead of a launch of their own
+    const hipError_t e = shares > 1 ? launch_residual_rmsnorm_quantize(d_x, ctx->scratch_f, shares, d_norm_weight, n, w->m, x_stride, eps, d_out_quants,
+                                                                       d_out_scales, ctx->launch())
+                                    : launch_rmsnorm_quantize(d_x, d_norm_weight, n, w->m, x_stride, eps, d_out_quants, d_out_scales, ctx->launch());
+    return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "rmsnorm_quantize launch");
 }
 
 int wick_rocm_gemm_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* ws, float* const* d_ys, uint32_t count, const int8_t* d_quants,

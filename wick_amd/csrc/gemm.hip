@@ -666,15 +666,22 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
 }
 
 // y (+)= partial[0] + partial[1] + ... in that order, element by element (token-major partials [split][n][m]).
-__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial, uint32_t splits, uint32_t n, uint32_t m,
+// (S a template parameter: all of an element's loads are in flight together instead of one round trip per share.)
+template <int S>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial, uint32_t n, uint32_t m,
                                                                  float* __restrict__ y, uint32_t y_stride, int y_row_major, int accumulate) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, total = (size_t)n * m;
     if (i >= total) return;
-    float sum = partial[i];
-    for (uint32_t s_ = 1; s_ < splits; s_++) sum += partial[(size_t)s_ * total + i];
     const uint32_t tok = (uint32_t)(i / m), row = (uint32_t)(i % m);
     float* dst = y_row_major ? y + (size_t)row * y_stride + tok : y + (size_t)tok * y_stride + row;
-    *dst = accumulate ? *dst + sum : sum;
+    float p[S];
+#pragma unroll
+    for (int s_ = 0; s_ < S; s_++) p[s_] = partial[(size_t)s_ * total + i];
+    const float old = accumulate ? *dst : 0.0f;
+    float sum = p[0];
+#pragma unroll
+    for (int s_ = 1; s_ < S; s_++) sum += p[s_];
+    *dst = accumulate ? old + sum : sum;
 }
 
 // How many ways a single-weight launch is split over K: only narrow launches that leave at least half of the CUs without
@@ -692,7 +699,7 @@ uint32_t split_k_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits)
 }
 
 template <bool DUMP>
-hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0) {
+hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0, bool defer_reduce = false) {
     if (a.m == 0 || a.n == 0) return hipSuccess;
     a.row_tiles = (a.m + BM - 1) / BM;
     a.tile_start[0] = a.tile_start[1] = UINT32_MAX;
@@ -712,10 +719,16 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0) {
             const uint32_t split_blocks = blocks * a.ksplit;  // tile id = blockIdx.x / ksplit must run over all `blocks` slots of the tile map
             hipError_t e = type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(split_blocks), dim3(THREADS), a)
                                              : launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(split_blocks), dim3(THREADS), a);
-            if (e != hipSuccess) return e;
+            if (e != hipSuccess || defer_reduce) return e;  // deferred: the caller's next kernel adds the shares up itself
             const size_t total = (size_t)a.n * a.m;
-            return launch_kernel(L, kFamGemm, gemm_splitk_reduce_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256),
-                                 static_cast<const float*>(a.partial), a.ksplit, a.n, a.m, a.y, a.y_stride, a.y_row_major, a.accumulate);
+            const auto reduce = [&](auto kernel) {
+                return launch_kernel(L, kFamGemm, kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), static_cast<const float*>(a.partial), a.n, a.m,
+                                     a.y, a.y_stride, a.y_row_major, a.accumulate);
+            };
+            if (a.ksplit == 2) return reduce(gemm_splitk_reduce_kernel<2>);
+            if (a.ksplit == 4) return reduce(gemm_splitk_reduce_kernel<4>);
+            if (a.ksplit == 8) return reduce(gemm_splitk_reduce_kernel<8>);
+            return hipErrorInvalidValue;  // split_k_factor makes 2, 4 or 8 shares
         }
         if (type == kTypeQ4_0) return launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
         return launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
@@ -732,7 +745,7 @@ uint32_t gemm_split_k(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits) {
 // splits > 1 (= gemm_split_k(m, n, k, ...)) with d_partial holding splits * n * m floats: the K-split launch pair.
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                             const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
-                            int accumulate, const Launch& L, uint32_t splits, float* d_partial) {
+                            int accumulate, const Launch& L, uint32_t splits, float* d_partial, bool defer_reduce) {
     GemmArgs a{};
     a.w = d_w, a.xq = d_q, a.xs = d_scales, a.y = d_y, a.dots = nullptr;
     a.m = m, a.n = n, a.k = k, a.y_stride = y_stride;
@@ -741,8 +754,10 @@ hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k
     if (splits > 1 && d_partial) {
         if (splits != split_k_factor(m, n, k, splits)) return hipErrorInvalidValue;  // the shape does not carry that split
         a.ksplit = splits, a.partial = d_partial;
+    } else if (defer_reduce) {
+        return hipErrorInvalidValue;  // nothing to defer on an unsplit launch
     }
-    return launch<false>(type, a, L);
+    return launch<false>(type, a, L, 0, defer_reduce);
 }
 
 // The same launch over up to three weights of one type and k that share the activations: outputs y[i] (same stride,

@@ -557,9 +557,16 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
     int rc = !lookup ? WICK_ROCM_OK
                      : locked([&] { return launch_embed_rows(static_cast<const uint8_t*>(m->embd->d), m->embd->type, m->embd->m, hs, m->pTokens, n, m->pX, ctx->launch()); },
                               "embed_rows launch");
+    // A residual projection and the norm + quantizer behind it go out as one call (a split projection's shares are then added
+    // up by the norm's kernel): the out projection with the FFN norm, the down projection with the NEXT layer's first norm.
+    auto project_and_norm = [&](const wick_rocm_weight* w, const int8_t* q, const float* s, const float* norm_weight) {
+        return wick_rocm_gemm_q8_residual_rmsnorm_quantize(ctx, w, q, s, n, m->pX, hs, norm_weight, c.rms_norm_eps, m->pQ, m->pS);
+    };
     for (uint32_t i = 0; rc == 0 && i < c.n_layers; i++) {
         const LayerWeights& L = m->layers[i];
-        if ((rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.attn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
+        const float* next_norm = i + 1 < c.n_layers ? m->layers[i + 1].attn_norm : nullptr;
+        // layer 0 norms its own input; every later layer's came with the previous layer's down projection
+        if (i == 0 && (rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.attn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
         bool quantized = false;
         if (L.n_kv == 0) {
             if ((rc = gemm(ctx, L.in_proj, m, n, m->pA, 3 * hs, 0))) break;
@@ -593,20 +600,20 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
         }
         // the out projection's input: already Q8_0 blocks when its producer wrote them itself
         if (!quantized && (rc = wick_rocm_quantize_q8_0(ctx, m->pG, n, hs, hs, m->pQ, m->pS))) break;
-        if ((rc = gemm(ctx, L.n_kv == 0 ? L.out_proj : L.o, m, n, m->pX, hs, 1))) break;  // hidden += out projection
-        if ((rc = wick_rocm_rmsnorm_quantize_q8_0(ctx, m->pX, L.ffn_norm, n, hs, hs, c.rms_norm_eps, m->pQ, m->pS))) break;
+        if ((rc = project_and_norm(L.n_kv == 0 ? L.out_proj : L.o, m->pQ, m->pS, L.ffn_norm))) break;  // hidden += out projection; FFN norm
         if (L.gate->type == kTypeQ4_0 && L.gate->k <= 1024 && wick_rocm_ffn_gate_up_silu_quantize_applies(L.gate, L.up, n)) {
             // gate, up, SiLU gate and the down projection's quantizer in one launch; its output cannot overwrite its own input.
             // (Where it pays, measured on one GPU against GEMM + gate kernel: Q4_0 with k = 1024 6-7 % faster; k = 2048 2-8 %
             // slower -- the epilogue's exp / divide work sits on the vector ALU that bounds the GEMM; Q8_0, whose kernel is
             // two registers over its budget, 11 % slower.)
             if ((rc = wick_rocm_ffn_gate_up_silu_quantize_q8(ctx, L.gate, L.up, m->pQ, m->pS, n, m->pQ2, m->pS2))) break;
-            rc = wick_rocm_gemm_q8(ctx, L.down, m->pQ2, m->pS2, n, m->pX, hs, WICK_ROCM_LAYOUT_TOKEN_MAJOR, 1);
+            rc = next_norm ? project_and_norm(L.down, m->pQ2, m->pS2, next_norm)
+                           : wick_rocm_gemm_q8(ctx, L.down, m->pQ2, m->pS2, n, m->pX, hs, WICK_ROCM_LAYOUT_TOKEN_MAJOR, 1);
             continue;
         }
         if ((rc = gemm_group(ctx, {L.gate, L.up}, {m->pGate, m->pUp}, m, n, inter))) break;
         if ((rc = wick_rocm_silu_mul_quantize_q8_0(ctx, m->pGate, m->pUp, n, inter, m->pQ, m->pS))) break;
-        rc = gemm(ctx, L.down, m, n, m->pX, hs, 1);
+        rc = next_norm ? project_and_norm(L.down, m->pQ, m->pS, next_norm) : gemm(ctx, L.down, m, n, m->pX, hs, 1);
     }
     return rc;
 }

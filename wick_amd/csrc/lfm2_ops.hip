@@ -1134,6 +1134,65 @@ __global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const float* __re
     }
 }
 
+// The K shares of a split projection added onto the residual rows, then rmsnorm_quantize_kernel of the updated rows, bit for bit
+// what gemm_splitk_reduce_kernel (accumulating) followed by rmsnorm_quantize_kernel leave: the shares are summed in ascending
+// order and then added to x; thread t covers the same elements t, t + 256, .. in the same order for the f64 sum of squares.  The
+// updated row is written back and kept in LDS for the quantizer's pass.  partial: [splits][rows][dim].
+template <int S>
+__global__ __launch_bounds__(256) void residual_rmsnorm_quantize_kernel(float* __restrict__ x, const float* __restrict__ partial, size_t share_stride,
+                                                                        const float* __restrict__ weight, int8_t* __restrict__ q,
+                                                                        float* __restrict__ scales, uint32_t dim, uint32_t x_stride, float eps) {
+    __shared__ double slots[16];
+    __shared__ __align__(16) float row[kResidualNormMaxDim];
+    float* xr = x + (size_t)blockIdx.x * x_stride;
+    const float* pr = partial + (size_t)blockIdx.x * dim;
+    double s = 0.0;
+    for (uint32_t i0 = threadIdx.x; i0 < dim; i0 += 4u * 256u) {  // four elements' loads (S + 1 each) in flight together
+        float xv[4], pv[4][S];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t i = i0 + 256u * j < dim ? i0 + 256u * j : i0;
+            xv[j] = xr[i];
+#pragma unroll
+            for (int p = 0; p < S; p++) pv[j][p] = pr[(size_t)p * share_stride + i];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t i = i0 + 256u * j;
+            if (i < dim) {
+                float sum = pv[j][0];
+#pragma unroll
+                for (int p = 1; p < S; p++) sum += pv[j][p];
+                const float h = xv[j] + sum;
+                xr[i] = h, row[i] = h;
+                const double v = (double)h;
+                s += v * v;
+            }
+        }
+    }
+    const double total = block_sum_f64(s, slots);  // its barriers also publish row[]
+    const float inv_rms = (float)(1.0 / sqrt(total / (double)dim + (double)eps));
+    const uint32_t quads = dim >> 2;
+    for (uint32_t quad0 = 0; quad0 < quads; quad0 += blockDim.x) {
+        const uint32_t quad = quad0 + threadIdx.x;
+        const bool live = quad < quads;
+        const uint32_t qd = live ? quad : 0;
+        const float4 v = reinterpret_cast<const float4*>(row)[qd];
+        const float4 w = reinterpret_cast<const float4*>(weight)[qd];
+        const float v0 = __fmul_rn(__fmul_rn(v.x, inv_rms), w.x), v1 = __fmul_rn(__fmul_rn(v.y, inv_rms), w.y);
+        const float v2 = __fmul_rn(__fmul_rn(v.z, inv_rms), w.z), v3 = __fmul_rn(__fmul_rn(v.w, inv_rms), w.w);
+        float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+        amax = group_max8(amax);
+        float id;
+        const float scale = q8_scale_and_inverse(amax, id);
+        const uint32_t packed = q8_pack4(v0, v1, v2, v3, id);
+        if (live) {
+            *reinterpret_cast<uint32_t*>(q + (size_t)blockIdx.x * dim + 4u * quad) = packed;
+            if ((quad & 7u) == 0) scales[(size_t)blockIdx.x * (dim >> 5) + (quad >> 3)] = scale;
+        }
+    }
+}
+
 // silu_mul_kernel followed by the quantizer, bit for bit: the gated values go straight into Q8_0 blocks.
 // gate / up: [n][dim] floats, contiguous, 16-byte aligned.
 __global__ __launch_bounds__(256) void silu_mul_quantize_kernel(const float* __restrict__ gate, const float* __restrict__ up, int8_t* __restrict__ q,
@@ -1452,6 +1511,19 @@ hipError_t launch_rmsnorm_quantize(const float* d_x, const float* d_weight, uint
                                    float* d_scales, const Launch& L) {
     if (rows == 0) return hipSuccess;
     return launch_kernel(L, kFamQuantize, rmsnorm_quantize_kernel, dim3(rows), dim3(256), d_x, d_weight, d_q, d_scales, dim, x_stride, eps);
+}
+
+hipError_t launch_residual_rmsnorm_quantize(float* d_x, const float* d_partial, uint32_t splits, const float* d_weight, uint32_t rows, uint32_t dim,
+                                            uint32_t x_stride, float eps, int8_t* d_q, float* d_scales, const Launch& L) {
+    if (rows == 0) return hipSuccess;
+    if (dim > kResidualNormMaxDim) return hipErrorInvalidValue;
+    const auto go = [&](auto kernel) {
+        return launch_kernel(L, kFamQuantize, kernel, dim3(rows), dim3(256), d_x, d_partial, (size_t)rows * dim, d_weight, d_q, d_scales, dim, x_stride, eps);
+    };
+    if (splits == 2) return go(residual_rmsnorm_quantize_kernel<2>);
+    if (splits == 4) return go(residual_rmsnorm_quantize_kernel<4>);
+    if (splits == 8) return go(residual_rmsnorm_quantize_kernel<8>);
+    return hipErrorInvalidValue;  // the K split makes 2, 4 or 8 shares
 }
 
 hipError_t launch_silu_mul_quantize(const float* d_gate, const float* d_up, uint32_t n, uint32_t dim, int8_t* d_q, float* d_scales, const Launch& L) {

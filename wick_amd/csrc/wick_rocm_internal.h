@@ -132,7 +132,9 @@ hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t
 // int8-MFMA GEMM.  Requires k % 128 == 0.
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                             const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
-                            int accumulate, const Launch& L, uint32_t splits = 1, float* d_partial = nullptr);
+                            int accumulate, const Launch& L, uint32_t splits = 1, float* d_partial = nullptr, bool defer_reduce = false);
+// defer_reduce (splits > 1 only): the shares stay in d_partial ([splits][n][m], token-major) and the caller's next kernel adds them
+// up in ascending order onto y itself (launch_residual_rmsnorm_quantize).
 // Ways (1, 2, 4 or 8, at most max_splits) the launch above may be split over K: > 1 only for launches of few tiles and long K.
 uint32_t gemm_split_k(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits);
 hipError_t launch_gemm_mfma_multi(int type, const uint8_t* const* d_w, const uint32_t* m, uint32_t count, uint32_t k, const int8_t* d_q,
@@ -205,6 +207,12 @@ hipError_t launch_shortconv_step(const float* d_proj, float* d_buffer, const flo
                                  uint32_t kernel_size, const Launch& L);
 hipError_t launch_rmsnorm_quantize(const float* d_x, const float* d_weight, uint32_t rows, uint32_t dim, uint32_t x_stride, float eps, int8_t* d_q,
                                    float* d_scales, const Launch& L);
+// The same with a residual update in front: x[r][i] += partial[0][r][i] + partial[1][r][i] + .. (the K shares of a split projection,
+// added in that order; the sum first, then onto x -- what the split's own reduce launch computes), then norm and quantizer
+// of the updated rows.  dim <= kResidualNormMaxDim.
+constexpr uint32_t kResidualNormMaxDim = 8192;
+hipError_t launch_residual_rmsnorm_quantize(float* d_x, const float* d_partial, uint32_t splits, const float* d_weight, uint32_t rows, uint32_t dim,
+                                            uint32_t x_stride, float eps, int8_t* d_q, float* d_scales, const Launch& L);
 hipError_t launch_silu_mul_quantize(const float* d_gate, const float* d_up, uint32_t n, uint32_t dim, int8_t* d_q, float* d_scales, const Launch& L);
 hipError_t launch_silu_mul(float* d_gate, const float* d_up, uint32_t n, const Launch& L);
 // d_history[pos] = pick (pos = *d_pos before it is advanced), when given.  d_partial: scratch of kArgmaxPartials keys, 8-byte aligned;

@@ -86,6 +86,7 @@ _SIGNATURES = {
     "wick_rocm_gemv_q8_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, _P, C.c_int]),
     "wick_rocm_gemm_q8": (C.c_int, [_P, _P, _P, _P, C.c_uint32, _P, C.c_uint32, C.c_int, C.c_int]),
     "wick_rocm_gemm_q8_multi": (C.c_int, [_P, _P, _P, C.c_uint32, _P, _P, C.c_uint32, C.c_uint32, C.c_int, C.c_int]),
+    "wick_rocm_gemm_q8_residual_rmsnorm_quantize": (C.c_int, [_P, _P, _P, _P, C.c_uint32, _P, C.c_uint32, _P, C.c_float, _P, _P]),
     "wick_rocm_matmul_f32": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_uint32, C.c_uint32, _P, C.c_size_t, C.c_uint32, C.c_int]),
     "wick_rocm_matmul_f32_noalloc": (C.c_int, [_P, _P, _P, C.c_size_t, C.c_uint32, C.c_uint32, _P, C.c_size_t, C.c_uint32, C.c_int]),
     "wick_rocm_gemv_f32_multi": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_uint32, _P, C.c_size_t, C.c_int]),
@@ -292,6 +293,13 @@ class RocmContext:
         wa = (_P * c)(*[w.handle for w in ws])
         ya = (_P * c)(*[_ptr(y) for y in ys])
         self._check(self._lib.wick_rocm_gemm_q8_multi(self._h, wa, ya, c, _ptr(quants), _ptr(scales), n, y_stride, layout, int(accumulate)))
+
+    def gemm_preq_residual_rmsnorm_quantize(self, w: RocmWeight, scales, quants, n: int, x, x_stride: int, norm_weight, eps: float,
+                                            out_quants, out_scales) -> None:
+        """x[j] += W (activation j), then (out_quants, out_scales) = Q8_0(rmsnorm(x[j]) * norm_weight): a prompt pass's residual
+        projection with the norm and quantizer behind it."""
+        self._check(self._lib.wick_rocm_gemm_q8_residual_rmsnorm_quantize(self._h, w.handle, _ptr(quants), _ptr(scales), n, _ptr(x), x_stride,
+                                                                          _ptr(norm_weight), eps, _ptr(out_quants), _ptr(out_scales)))
 
     def block_dots_i32(self, w: RocmWeight, quants, n: int, out) -> None:
         self._check(self._lib.wick_rocm_block_dots_i32(self._h, w.handle, _ptr(quants), n, _ptr(out)))
