@@ -1107,9 +1107,17 @@ __global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const float* __re
     __shared__ double slots[16];
     const float* xr = x + (size_t)blockIdx.x * x_stride;
     double s = 0.0;
-    for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
-        const double v = (double)xr[i];
-        s += v * v;
+    for (uint32_t i0 = threadIdx.x; i0 < dim; i0 += 4u * 256u) {  // four loads in flight; elements t, t + 256, .. in order, as rmsnorm_kernel sums them
+        float xv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) xv[j] = xr[i0 + 256u * j < dim ? i0 + 256u * j : i0];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (i0 + 256u * j < dim) {
+                const double v = (double)xv[j];
+                s += v * v;
+            }
+        }
     }
     const double total = block_sum_f64(s, slots);
     const float inv_rms = (float)(1.0 / sqrt(total / (double)dim + (double)eps));
@@ -1272,6 +1280,24 @@ struct EmbedArgs {
     uint32_t m, k;
 };
 
+// Row `row` of the embedding into emb.out by the calling workgroup, four elements per thread at a time: their loads are all issued
+// before the first store (the stores could alias the loads as far as the compiler knows, which would chain the round trips).
+__device__ __forceinline__ void embed_row_batched(const EmbedArgs& emb, uint32_t row) {
+    for (uint32_t e0 = threadIdx.x; e0 < emb.k; e0 += 4u * blockDim.x) {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t e = e0 + j * blockDim.x;
+            v[j] = dequant_element(emb.w, emb.type, row, emb.k, e < emb.k ? e : e0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t e = e0 + j * blockDim.x;
+            if (e < emb.k) emb.out[e] = v[j];
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void argmax_final_kernel(const unsigned long long* __restrict__ partial, uint32_t blocks, uint32_t n,
                                                            uint32_t* __restrict__ out, uint32_t* __restrict__ d_token, uint32_t* __restrict__ d_pos,
                                                            uint32_t* __restrict__ d_history, uint32_t history_len, EmbedArgs emb) {
@@ -1279,9 +1305,15 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(const unsigned long l
     __shared__ unsigned long long red[4];
     const uint32_t waves = blockDim.x >> 6;  // 1 (at most 64 partial keys) or 4
     unsigned long long best = 0ull;
-    for (uint32_t i = threadIdx.x; i < blocks; i += blockDim.x) {
-        const unsigned long long k = partial[i];
-        best = k > best ? k : best;
+    for (uint32_t i0 = threadIdx.x; i0 < blocks; i0 += 8u * blockDim.x) {  // eight keys per thread in flight (one round trip for <= 2048 keys)
+        unsigned long long k[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t i = i0 + j * blockDim.x;
+            k[j] = partial[i < blocks ? i : i0];  // clamped: a repeated key cannot change the maximum
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) best = k[j] > best ? k[j] : best;
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -1310,8 +1342,7 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(const unsigned long l
     if (!emb.w) return;
     __syncthreads();
     const uint32_t pick = picked;  // the pick is the next step's token: its embedding row is that step's input
-    if (pick < emb.m)
-        for (uint32_t e = threadIdx.x; e < emb.k; e += blockDim.x) emb.out[e] = dequant_element(emb.w, emb.type, pick, emb.k, e);
+    if (pick < emb.m) embed_row_batched(emb, pick);
 }
 
 // Sets the device-side token / position of the next step (either may be null) and, when an embedding is given, looks
@@ -1321,8 +1352,7 @@ __global__ __launch_bounds__(256) void set_step_kernel(uint32_t* d_token, uint32
         if (d_token) *d_token = token;
         if (d_pos) *d_pos = pos;
     }
-    if (emb.w && token < emb.m)
-        for (uint32_t e = threadIdx.x; e < emb.k; e += blockDim.x) emb.out[e] = dequant_element(emb.w, emb.type, token, emb.k, e);
+    if (emb.w && token < emb.m) embed_row_batched(emb, token);
 }
 
 __global__ void advance_pos_kernel(uint32_t* d_pos) {
