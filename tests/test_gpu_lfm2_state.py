@@ -231,3 +231,52 @@ def test_prefill_from_embeddings(ctx, oracle, tmp_path, name, n):
     with pytest.raises(W.RocmError, match="beyond the context"):
         model.forward_prefill_from_embeddings(frames, 64 - n + 1)
     model.free()
+
+
+def test_two_threads_share_one_context(ctx, oracle, tmp_path):
+    """The context serialises its callers (the reference's infer_lock, wick/src/model/metal_lfm2.rs:254-267): a model stepping in one
+    thread and another thread issuing matmuls and a second model's steps on the same context leave every result as it is when each runs
+    alone -- nothing of one caller ends up in the other's captured step or scratch."""
+    import threading
+    model, ref, cfg = load(ctx, oracle, tmp_path, **CLEAR["q4_0+q6k"])
+    other, _, _ = load(ctx, oracle, tmp_path, **CLEAR["q8_0"])
+    tokens = np.random.default_rng(2).integers(0, cfg["vocab_size"], 24)
+    m, k, n = 300, 1024, 40
+    wb = oracle.synth_weight(W.Q4_0, m, k, seed=9)
+    w = ctx.upload_weight(wb, W.Q4_0, m, k)
+    x = oracle.fill_normal(3, 1.0, n * k)
+    d_x, d_y = ctx.to_device(x), ctx.alloc(n * m * 4)
+
+    def steps(mod):
+        mod.reset()
+        return [mod.forward(int(t), p) for p, t in enumerate(tokens)]
+
+    def matmuls(reps):
+        out = []
+        for _ in range(reps):
+            ctx.encode_gemm(w, d_x, 0, d_y, 0, n, k, m)
+            out.append(d_y.download(np.float32, n * m))
+        return out
+
+    alone_a, alone_b, alone_mm = steps(model), steps(other), matmuls(1)[0]
+    got, errors = {}, []
+
+    def run(name, fn, *args):
+        try:
+            got[name] = fn(*args)
+        except Exception as e:  # noqa: BLE001 - reported below
+            errors.append((name, e))
+
+    threads = [threading.Thread(target=run, args=("a", steps, model)), threading.Thread(target=run, args=("b", steps, other)),
+               threading.Thread(target=run, args=("mm", matmuls, 30))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for name, alone in (("a", alone_a), ("b", alone_b)):
+        for x1, x2 in zip(alone, got[name]):
+            assert np.array_equal(bits(x1), bits(x2)), name
+    for y in got["mm"]:
+        assert np.array_equal(bits(y), bits(alone_mm))
+    model.free(), other.free(), w.free(), d_x.free(), d_y.free()
