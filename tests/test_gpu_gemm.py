@@ -184,8 +184,10 @@ def test_argument_errors(ctx, oracle):
     (W.Q4_0, 1024, 512, 4608, "token", True),    # the down projection of a 512-token prompt: 64 tiles, 4 shares
     (W.Q8_0, 1024, 100, 2048, "token", False),   # 16 tiles, 4 shares of 4 stages
     (W.Q4_0, 300, 70, 4608, "row", True),        # ragged rows and tokens, 8 shares, row-major output
-    (W.Q8_0, 2048, 640, 6912, "token", False),   # 160 tiles: no split (would pass 256)
-    (W.Q4_0, 1024, 2002, 4608, "token", False),  # 256 tiles: no split
+    (W.Q8_0, 2048, 640, 6912, "token", False),   # 160 narrow tiles (80 wide): 4 shares on the wide tile
+    (W.Q4_0, 1024, 2002, 4608, "token", False),  # 256 narrow tiles = 128 wide ones with a long K: 4 shares on the wide tile
+    (W.Q8_0, 2048, 700, 4224, "row", True),      # 96 wide tiles, 33 stages: 4 shares of 8 or 9 on the wide tile, ragged tokens
+    (W.Q8_0, 1024, 2002, 2048, "token", False),  # 16 stages: too short for the wide split, too many tiles for the narrow one
     (W.Q4_0, 256, 300, 1024, "row", False),      # 10 tiles (not a multiple of the 8 slots the tile map deals out), 4 shares of 2 stages
     (W.Q8_0, 640, 200, 2048, "token", True),     # 20 tiles, 4 shares
     (W.Q4_0, 384, 130, 1152, "token", False),    # 9 stages in 4 shares: 2, 2, 2, 3

@@ -378,7 +378,10 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
     __shared__ Smem sm;
     uint32_t row_tile, tok_tile;
     bool valid_tile;
-    tile_of_block(blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
+    // K split (plain single-weight launches only): workgroup (tile, share) walks the stages [first, first + stages) of its tile
+    const uint32_t ksplit = DUMP || GATED || a.ksplit < 2 ? 1u : a.ksplit;
+    const uint32_t split = ksplit > 1 ? blockIdx.x % ksplit : 0u;
+    tile_of_block(ksplit > 1 ? blockIdx.x / ksplit : blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
     if (!valid_tile) return;  // whole workgroup leaves together
     if constexpr (!GATED) select_weight(a, row_tile);
     const uint32_t row0 = row_tile * (GATED ? BM / 2 : BM);  // GATED: 64 output rows per tile, see load_stage
@@ -391,7 +394,9 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
     const uint32_t wrow0 = (wave >> 2) * 64;  // wave's rows within the tile
     const uint32_t wtok0 = (wave & 3u) * 32;  // wave's tokens within the tile
     const uint32_t nb = a.k >> 5;
-    const uint32_t stages = nb / KB;
+    const uint32_t all_stages = nb / KB;
+    const uint32_t first = split * all_stages / ksplit;  // shares differ by at most one stage, none is empty
+    const uint32_t stages = (split + 1u) * all_stages / ksplit - first;
 
     float acc[TT][RT][4];
 #pragma unroll
@@ -405,8 +410,8 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
     asm volatile("" : "+v"(cbias));  // keep it in registers (left alone, the compiler rebuilds it before every MFMA)
 
     StageRegs<TYPE> regs;
-    dma_activations(a, sm.st[0], tok0, 0);
-    load_stage<TYPE, BN, GATED>(a, row0, tok0, 0, regs);
+    dma_activations(a, sm.st[0], tok0, first * KB);
+    load_stage<TYPE, BN, GATED>(a, row0, tok0, first * KB, regs);
     store_stage<TYPE, BN>(sm.st[0], regs);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
     __syncthreads();
@@ -416,8 +421,8 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
         if (st + 1 < stages) {
             // the other LDS stage was last read in stage st-1 and every wave has passed the
             // barrier that ended it, so it can be refilled from here on
-            dma_activations(a, sm.st[(st + 1) & 1u], tok0, (st + 1) * KB);
-            load_stage<TYPE, BN, GATED>(a, row0, tok0, (st + 1) * KB, regs);
+            dma_activations(a, sm.st[(st + 1) & 1u], tok0, (first + st + 1) * KB);
+            load_stage<TYPE, BN, GATED>(a, row0, tok0, (first + st + 1) * KB, regs);
         }
 
         // 8 MFMA tiles per block, software-pipelined by hand: four result buffers, the matrix
@@ -443,7 +448,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
 #pragma unroll 1
         for (int b = 0; b < KB; b++) {
             next_block(la, (uint32_t)b, b + 1 < KB);  // last iteration: harmless re-read of its own block
-            const uint32_t row = row0 + wrow0 + l16, tok = tok0 + wtok0 + 4 * kq, blk = st * KB + b;
+            const uint32_t row = row0 + wrow0 + l16, tok = tok0 + wtok0 + 4 * kq, blk = (first + st) * KB + b;
             v4i d[4];
             lds_wait<6>(mt);  // the six reads issued after the matrices may still be in flight
 #pragma unroll
@@ -510,8 +515,12 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
                 for (int r = 0; r < 4; r++) {
                     const uint32_t tok = tok0 + wtok0 + 16 * tt + 4 * kq + r;
                     if (row < a.m && tok < a.n) {
-                        float* dst = a.y_row_major ? a.y + (size_t)row * a.y_stride + tok : a.y + (size_t)tok * a.y_stride + row;
-                        *dst = a.accumulate ? *dst + acc[tt][rt][r] : acc[tt][rt][r];
+                        if (ksplit > 1) {  // this share's sums; the reduce launch (or the caller's next kernel) adds the shares up
+                            a.partial[((size_t)split * a.n + tok) * a.m + row] = acc[tt][rt][r];
+                        } else {
+                            float* dst = a.y_row_major ? a.y + (size_t)row * a.y_stride + tok : a.y + (size_t)tok * a.y_stride + row;
+                            *dst = a.accumulate ? *dst + acc[tt][rt][r] : acc[tt][rt][r];
+                        }
                     }
                 }
             }
@@ -687,7 +696,20 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 // How many ways a single-weight launch is split over K: only narrow launches that leave at least half of the CUs without
 // a tile, with K long enough (>= 8 stages) that the shorter walk pays for the second launch, every share >= 2 stages (a stage
 // of a launch with few tiles costs a whole memory round trip, 1.2 - 1.4 us: nothing else is there to hide it).
+// The same on the wide tile: a long-K launch of 64 .. 256 wide tiles (the down projection of a long prompt: 1024 x 2002 x 4608 is
+// 128 of them) fills the chip's 512 workgroup slots with (tile, share) pairs of the wide kernel, whose block loop is the faster one,
+// instead of one narrow tile per CU.  Shares of >= 8 stages.
+uint32_t wide_split_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits) {
+    const uint32_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN), stages = (k >> 5) / KB;
+    if (n <= BN_NARROW || tiles < 64 || tiles > 256 || stages < 32) return 1;
+    uint32_t s_ = 1;
+    while (2 * s_ <= max_splits && tiles * 2 * s_ <= 512 && stages / (2 * s_) >= 8) s_ *= 2;
+    return s_;
+}
+
 uint32_t split_k_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits) {
+    const uint32_t ws = wide_split_factor(m, n, k, max_splits);
+    if (ws > 1) return ws;
     const uint32_t row_tiles = (m + BM - 1) / BM;
     const bool narrow = n <= BN_NARROW || row_tiles * ((n + BN - 1) / BN) <= 256;
     if (!narrow) return 1;
@@ -696,6 +718,19 @@ uint32_t split_k_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits)
     uint32_t s_ = 1;
     while (2 * s_ <= max_splits && tiles * 2 * s_ <= 256 && stages / (2 * s_) >= 2) s_ *= 2;
     return s_;
+}
+
+// The second launch of a split GEMM: y (+)= the shares in ascending order.
+hipError_t launch_reduce(const GemmArgs& a, const Launch& L) {
+    const size_t total = (size_t)a.n * a.m;
+    const auto reduce = [&](auto kernel) {
+        return launch_kernel(L, kFamGemm, kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), static_cast<const float*>(a.partial), a.n, a.m, a.y,
+                             a.y_stride, a.y_row_major, a.accumulate);
+    };
+    if (a.ksplit == 2) return reduce(gemm_splitk_reduce_kernel<2>);
+    if (a.ksplit == 4) return reduce(gemm_splitk_reduce_kernel<4>);
+    if (a.ksplit == 8) return reduce(gemm_splitk_reduce_kernel<8>);
+    return hipErrorInvalidValue;  // split_k_factor makes 2, 4 or 8 shares
 }
 
 template <bool DUMP>
@@ -709,7 +744,8 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0, boo
     }
     // The narrow tile also serves small problems that would leave more than half of the
     // 512 resident workgroup slots (2 per CU) empty with the wide tile: twice the tiles.
-    const bool narrow = a.n <= BN_NARROW || a.row_tiles * ((a.n + BN - 1) / BN) <= 256;
+    const bool wide_split = !DUMP && more == 0 && a.ksplit > 1 && wide_split_factor(a.m, a.n, a.k, a.ksplit) == a.ksplit;
+    const bool narrow = !wide_split && (a.n <= BN_NARROW || a.row_tiles * ((a.n + BN - 1) / BN) <= 256);
     a.tok_tiles = narrow ? (a.n + BN_NARROW - 1) / BN_NARROW : (a.n + BN - 1) / BN;
     if ((uint64_t)a.row_tiles * a.tok_tiles > 0x7fffff00ull) return hipErrorInvalidValue;  // beyond a launch's grid
     const uint32_t tiles = a.row_tiles * a.tok_tiles;
@@ -720,19 +756,18 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0, boo
             hipError_t e = type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(split_blocks), dim3(THREADS), a)
                                              : launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(split_blocks), dim3(THREADS), a);
             if (e != hipSuccess || defer_reduce) return e;  // deferred: the caller's next kernel adds the shares up itself
-            const size_t total = (size_t)a.n * a.m;
-            const auto reduce = [&](auto kernel) {
-                return launch_kernel(L, kFamGemm, kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), static_cast<const float*>(a.partial), a.n, a.m,
-                                     a.y, a.y_stride, a.y_row_major, a.accumulate);
-            };
-            if (a.ksplit == 2) return reduce(gemm_splitk_reduce_kernel<2>);
-            if (a.ksplit == 4) return reduce(gemm_splitk_reduce_kernel<4>);
-            if (a.ksplit == 8) return reduce(gemm_splitk_reduce_kernel<8>);
-            return hipErrorInvalidValue;  // split_k_factor makes 2, 4 or 8 shares
+            return launch_reduce(a, L);
         }
         if (type == kTypeQ4_0) return launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
         return launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
     }
+    if (wide_split) {
+        hipError_t e = type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, DUMP>, dim3(blocks * a.ksplit), dim3(THREADS), a)
+                                         : launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, DUMP>, dim3(blocks * a.ksplit), dim3(THREADS), a);
+        if (e != hipSuccess || defer_reduce) return e;
+        return launch_reduce(a, L);
+    }
+    a.ksplit = 1;  // an unsplit launch of the wide kernel
     if (type == kTypeQ4_0)
         return launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
     return launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
