@@ -1521,8 +1521,11 @@ hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, co
     if (d_q8 && !(aligned && attention_prefill_quantize_applies(d_q, d_k_cache, d_v_cache, n, q_stride, head_dim))) return hipErrorInvalidValue;
     if (head_dim == 64 && aligned && n >= 16) {
         const uint32_t qblocks = (n + 63u) / 64u;
-        if (qblocks == 1)
-            return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<1>, dim3(n_heads, 1), dim3(512), a, pos0, n, q_stride, out_stride, d_q8,
+        // (long, short) pairs balance the causal work once there are more query blocks than CUs; below that one block per
+        // workgroup (longest first) spreads wider: 17.7 -> 14.9, 25.8 -> 23.5, 43.5 -> 41.7 us at 256 / 512 / 1024 tokens of 16
+        // heads, but 82 -> 94 us at 2002.  The same arithmetic per query either way.
+        if (n_heads * qblocks <= 256u)
+            return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<1>, dim3(n_heads, qblocks), dim3(512), a, pos0, n, q_stride, out_stride, d_q8,
                                  d_q8_scales);
         return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride,
                              out_stride, d_q8, d_q8_scales);
