@@ -84,7 +84,8 @@ int wick_rocm_attention_decode(wick_rocm_ctx *ctx, const float *d_q, const float
  * seq_len = pos0 + j + 1.  d_q: [n][q_stride] floats (a token's n_heads * head_dim query values first), d_out:
  * [n][out_stride].  head_dim 32 / 64 / 128 / 256; head_dim 64 with 16-byte aligned rows and n >= 16 runs on the matrix
  * cores with every f32 operand split into two f16 halves and three exact-product MFMAs per product (f32 accuracy: measured
- * rel-L2 2e-7 against an f64 evaluation; sums in another order than the reference's loops).  That path needs |q| / sqrt(head_dim),
+ * rel-L2 2e-7 against an f64 evaluation; sums in another order than the reference's loops, softmax weights from the hardware's exp2
+ * instead of ggml_expf: an ulp or two apart).  That path needs |q| / sqrt(head_dim),
  * |k| and |v| below the f16 range (65504) -- the range the reference's own GPU path assumes when it keeps its KV caches in f16
  * (encode_cast_f32_to_f16, wick/src/model/metal_lfm2.rs:4178-4193). */
 int wick_rocm_attention_prefill(wick_rocm_ctx *ctx, const float *d_q, uint32_t q_stride, const float *d_k_cache, const float *d_v_cache,

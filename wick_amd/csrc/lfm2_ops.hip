@@ -726,6 +726,11 @@ __device__ __forceinline__ float groups_sum(float v) {
     return __uint_as_float(q[0]) + __uint_as_float(q[1]);
 }
 
+// exp(x) for x <= 0 (-inf included) on the hardware's exp2 (v_exp_f32, about one ulp): two instructions where the polynomial of
+// ggml_expf takes about thirty, and the softmax of a tile is nine of them per lane.  The weights differ from ggml_expf's in the
+// last bit or two; the streaming softmax of this kernel differs from the reference's two-pass one at that level anyway.
+__device__ __forceinline__ float exp_nonpos_hw(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
 template <int HALVES>
 __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride,
                                                                                 int8_t* q_out, float* s_out) {
@@ -872,7 +877,7 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
             tmax = groups_max(tmax);
             const float m_new = fmaxf(m_run, tmax);
             const float m_sub = m_new == -__builtin_inff() ? 0.0f : m_new;
-            const float alpha = ggml_expf_nonpos(m_run - m_sub);
+            const float alpha = exp_nonpos_hw(m_run - m_sub);
             m_run = m_new;
             float psum = 0.0f;
             h8 ph, pl;
@@ -880,7 +885,7 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
             for (int u = 0; u < 2; u++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const float pw = ggml_expf_nonpos(sc[u][r] - m_sub);
+                    const float pw = exp_nonpos_hw(sc[u][r] - m_sub);
                     psum += pw;
                     _Float16 hi, lo;
                     split_f16(pw * kPScale, hi, lo);
@@ -919,7 +924,7 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
         if (ksp == 1) return;
         const float m_b = xch[0], l_b = xch[64];
         const float m_all = fmaxf(m_run, m_b);
-        const float fa = ggml_expf_nonpos(m_run - m_all), fb = ggml_expf_nonpos(m_b - m_all);
+        const float fa = exp_nonpos_hw(m_run - m_all), fb = exp_nonpos_hw(m_b - m_all);
         l_run = l_run * fa + l_b * fb;
 #pragma unroll
         for (int c = 0; c < 4; c++)
