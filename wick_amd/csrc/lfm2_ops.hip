@@ -1029,10 +1029,14 @@ __global__ __launch_bounds__(256) void shortconv_seq_kernel(const float* __restr
 // shortconv_seq_kernel followed by the Q8_0 quantizer, bit for bit: a thread takes four consecutive channels of one
 // token (16-byte loads), eight threads one 32-channel block, and the gated convolution goes straight into Q8_0 blocks
 // for the out projection -- the f32 result never touches memory.  hidden % 32 == 0, 16-byte aligned buffers.
+// KS: the kernel size when known at compile time (3, the reference's default: the taps unroll and all of a thread's loads are
+// issued together), 0: read from kernel_size.
+template <int KS>
 __global__ __launch_bounds__(256) void shortconv_seq_quantize_kernel(const float* __restrict__ proj, const float* __restrict__ buffer,
                                                                      const float* __restrict__ conv_w, int8_t* __restrict__ q,
-                                                                     float* __restrict__ scales, uint32_t hidden, uint32_t kernel_size,
+                                                                     float* __restrict__ scales, uint32_t hidden, uint32_t kernel_size_arg,
                                                                      uint64_t total_quads) {
+    const uint32_t kernel_size = KS ? (uint32_t)KS : kernel_size_arg;
     const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const bool live = t < total_quads;
     const uint64_t tt = live ? t : 0;
@@ -1041,17 +1045,16 @@ __global__ __launch_bounds__(256) void shortconv_seq_quantize_kernel(const float
     const uint32_t d_conv = kernel_size - 1;
     const float* w = conv_w + (size_t)c0 * kernel_size;
     float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
     for (uint32_t k = 0; k < d_conv; k++) {
         const int src = (int)j - (int)d_conv + (int)k;  // token of this tap, < 0: before the prompt
-        float tap[4];
-        if (src < 0) {
-            const float4 s4 = *reinterpret_cast<const float4*>(buffer + (size_t)(src + (int)d_conv) * hidden + c0);
-            tap[0] = s4.x, tap[1] = s4.y, tap[2] = s4.z, tap[3] = s4.w;
-        } else {
-            const float* p = proj + (size_t)src * 3 * hidden;
-            const float4 b = *reinterpret_cast<const float4*>(p + c0), x = *reinterpret_cast<const float4*>(p + 2 * hidden + c0);
-            tap[0] = __fmul_rn(b.x, x.x), tap[1] = __fmul_rn(b.y, x.y), tap[2] = __fmul_rn(b.z, x.z), tap[3] = __fmul_rn(b.w, x.w);
-        }
+        // Both candidates are loaded (clamped addresses) and one is selected: no branch between the loads, so the taps' loads
+        // and the token's own go out together.
+        const float4 s4 = *reinterpret_cast<const float4*>(buffer + (size_t)(src < 0 ? src + (int)d_conv : 0) * hidden + c0);
+        const float* p = proj + (size_t)(src < 0 ? 0 : src) * 3 * hidden;
+        const float4 b = *reinterpret_cast<const float4*>(p + c0), x = *reinterpret_cast<const float4*>(p + 2 * hidden + c0);
+        float tap[4] = {__fmul_rn(b.x, x.x), __fmul_rn(b.y, x.y), __fmul_rn(b.z, x.z), __fmul_rn(b.w, x.w)};
+        if (src < 0) tap[0] = s4.x, tap[1] = s4.y, tap[2] = s4.z, tap[3] = s4.w;
 #pragma unroll
         for (int i = 0; i < 4; i++) sum[i] = __fadd_rn(sum[i], __fmul_rn(tap[i], w[(size_t)i * kernel_size + k]));
     }
@@ -1499,8 +1502,11 @@ hipError_t launch_shortconv_seq_quantize(const float* d_proj, float* d_buffer, c
     if (n == 0) return hipSuccess;
     if (!shortconv_seq_quantize_applies(d_proj, d_buffer, hidden)) return hipErrorInvalidValue;
     const uint64_t total = (uint64_t)n * (hidden >> 2);
-    hipError_t e = launch_kernel(L, kFamQuantize, shortconv_seq_quantize_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), d_proj,
-                                 static_cast<const float*>(d_buffer), d_conv_w, d_q, d_scales, hidden, kernel_size, total);
+    const auto go = [&](auto kernel) {
+        return launch_kernel(L, kFamQuantize, kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), d_proj, static_cast<const float*>(d_buffer),
+                             d_conv_w, d_q, d_scales, hidden, kernel_size, total);
+    };
+    hipError_t e = kernel_size == 3 ? go(shortconv_seq_quantize_kernel<3>) : go(shortconv_seq_quantize_kernel<0>);
     if (e != hipSuccess || kernel_size < 2) return e;
     return launch_kernel(L, kFamOther, shortconv_state_kernel, dim3((hidden + 255u) / 256u), dim3(256), d_proj, d_buffer, hidden, kernel_size, n);
 }
