@@ -266,29 +266,6 @@ __device__ __forceinline__ float ggml_expf(float x) {
     return __fmul_rn(__fadd_rn(s2, __fmul_rn(s2, j)), s1);
 }
 
-// ggml_expf for x <= 0 (-inf included) without branches: the same operations on the same values, the three result
-// ranges picked by selects, so the bits are ggml_expf's.  For softmax weights exp(score - max), where a divergent
-// branch per element costs more than the few extra operations.
-__device__ __forceinline__ float ggml_expf_nonpos(float x) {
-    const float R = bits_f(0x4B400000u), LOG2E = bits_f(0x3FB8AA3Bu);
-    const float LN2_HI = bits_f(0x3F317200u), LN2_LO = bits_f(0x35BFBE8Eu);
-    const float C1 = bits_f(0x3F7FFFF6u), C2 = bits_f(0x3EFFFEDBu), C3 = bits_f(0x3E2AAF33u);
-    const float C4 = bits_f(0x3D2B9F17u), C5 = bits_f(0x3C072010u);
-    const float z = __fadd_rn(R, __fmul_rn(x, LOG2E));
-    const float n = __fsub_rn(z, R);  // <= 0
-    const float b = __fsub_rn(__fsub_rn(x, __fmul_rn(n, LN2_HI)), __fmul_rn(n, LN2_LO));
-    const uint32_t e = __float_as_uint(z) << 23;
-    const float k = bits_f(e + 0x3F800000u);
-    const float u = __fmul_rn(b, b);
-    const float inner = __fadd_rn(__fadd_rn(C2, __fmul_rn(C3, b)), __fmul_rn(__fadd_rn(C4, __fmul_rn(C5, b)), u));
-    const float j = __fadd_rn(__fmul_rn(C1, b), __fmul_rn(inner, u));
-    const float abs_n = fabsf(n);
-    const float near = __fadd_rn(k, __fmul_rn(j, k));
-    const float s2 = bits_f(e - 0x82000000u);
-    const float tail = __fmul_rn(__fadd_rn(s2, __fmul_rn(s2, j)), bits_f(0x01000000u));
-    return abs_n <= 126.0f ? near : (abs_n > 192.0f ? 0.0f : tail);
-}
-
 // silu_mul_inplace's element (wick/src/backend/cpu.rs:668-673): g / (1 + expf(-g)) * u, bit-exact.
 __device__ __forceinline__ float silu_mul(float g, float u) { return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, ggml_expf(-g))), u); }
 
