@@ -373,6 +373,47 @@ def test_lfm2_350m_shaped_model(ctx, oracle, tmp_path):
     model.free()
 
 
+def test_lfm2_1p2b_wide_layers(ctx, oracle, tmp_path):
+    """Three layers (gated conv, attention, gated conv) of the LFM2-1.2B's widths -- hidden 2048, FFN 6912, 32 / 8 heads of 64 --
+    over a 4096-entry vocabulary: what the 350M shape does not reach as a composition (the conv fused into its out projection
+    at the widest hidden size that kernel takes, the gated gate / up kernel at k = 2048, the down projection's 108 block pairs
+    per row, 32-head attention, the prompt pass's K split at k = 6912).  Four decode steps, a 200-token prompt, a step after it;
+    held to the oracle's own spread under a two-ulp jitter of its f32 sums, like the 350M-shaped model."""
+    model, ref, cfg = load(ctx, oracle, tmp_path, context=512, n_layers=3, hidden=2048, inter=6912, n_heads=32, kv_heads=(0, 8, 0), vocab=4096,
+                           sigma=0.02, seed=12)
+    steps = [5, 77, 1000, 4095]
+
+    def decode(r):
+        st = r.new_state()
+        return [r.forward(t, p, st) for p, t in enumerate(steps)]
+
+    want, spread = _oracle_spread(cfg, ref.t, decode, seeds=(1, 2, 3))
+    allowed = np.maximum.accumulate(spread)
+    for pos, tok in enumerate(steps):
+        got = model.forward(tok, pos)
+        err = rel_l2(got, want[pos])
+        assert np.isfinite(got).all()
+        assert err <= max(LOGITS_REL_L2, 2.0 * allowed[pos]), f"pos {pos}: rel-L2 {err:.2e}, the oracle's own spread is {allowed[pos]:.2e}"
+        assert cosine(got, want[pos]) >= LOOSE_COSINE
+    assert spread.max() <= LOOSE_REL_L2, "the jittered oracle itself leaves the loose bar: pick another model seed"
+    tokens = np.random.default_rng(12).integers(0, cfg["vocab_size"], 200)
+
+    def prompt(r):
+        st = r.new_state()
+        for j, t in enumerate(tokens[:-1]):
+            r.hidden_after_layers(int(t), j, st)
+        return [r.forward(int(tokens[-1]), 199, st), r.forward(123, 200, st)]
+
+    want, spread = _oracle_spread(cfg, ref.t, prompt, seeds=(4,))
+    model.reset()
+    got = [model.forward_prefill(tokens, 0), model.forward(123, 200)]
+    for what, g, w, sp in zip(("prompt of 200", "step after the prompt"), got, want, np.maximum.accumulate(spread)):
+        assert np.isfinite(g).all()
+        assert rel_l2(g, w) <= max(LOGITS_REL_L2, 3.0 * sp), f"{what}: rel-L2 {rel_l2(g, w):.2e}, the oracle's own spread is {sp:.2e}"
+        assert cosine(g, w) >= LOOSE_COSINE
+    model.free()
+
+
 def test_cpp_host_mirror_runs_the_model(ctx, oracle, tmp_path):
     """The C++ mirror's RocmLfm2Model (statically linked selftest binary) and this binding drive the same library:
     same greedy tokens from the same GGUF file, and they are the oracle's."""
