@@ -150,19 +150,22 @@ struct StageRegs {
 // tokens reading one chunk then spread over all banks.  16 instructions per stage, two
 // per wave.
 __device__ __forceinline__ uint32_t xt_swizzle(uint32_t token_in_tile) { return (token_in_tile >> 1) & 7u; }
+// A thread's global read positions of the stage to fetch next.  Set up once per tile; every fetch moves them one stage
+// (128 K-elements) on, one 64-bit add each, instead of rebuilding row / token / block addresses per stage.
 template <int NTOK>
-__device__ __forceinline__ void dma_activations(const GemmArgs& a, StageT<NTOK>& s, uint32_t tok0, uint32_t kb0) {
+struct StagePtrs {
+    const int8_t* x[NTOK / 8 / (THREADS / 64)];  // this lane's 16-byte activation chunks (direct-to-LDS copies)
+    const uint8_t* wd;                            // threads 0 .. 2 BM - 1: a weight block pair; the next NTOK threads: a token's four scales
+};
+template <int NTOK>
+__device__ __forceinline__ void dma_activations(StagePtrs<NTOK>& p, StageT<NTOK>& s) {
     constexpr int PER_WAVE = NTOK / 8 / (THREADS / 64);  // instructions per wave and stage
-    const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 #pragma unroll
     for (int j = 0; j < PER_WAVE; j++) {
-        const uint32_t t = 8u * (PER_WAVE * wave + j) + (lane >> 3);  // token within the tile
-        const uint32_t chunk = (lane & 7u) ^ xt_swizzle(t);
-        const uint32_t tok = min(tok0 + t, a.n - 1);
-        const int8_t* src = a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + 16u * chunk;
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)p.x[j],
                                          (void __attribute__((address_space(3)))*)&s.xt[8u * (PER_WAVE * wave + j)][0], 16, 0, 0);
+        p.x[j] += KB * 32;
     }
 }
 
@@ -174,11 +177,19 @@ __device__ __forceinline__ void dma_activations(const GemmArgs& a, StageT<NTOK>&
 // that every wave (64 operand rows = four 16-row MFMA tiles) holds {gate rows A, gate rows B, up rows A, up rows B} of
 // the same 32 output rows: the SiLU gate and a whole Q8_0 block of its result then sit in one wave's registers.
 template <int TYPE, int NTOK, bool GATED = false>
-__device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uint32_t tok0, uint32_t kb0,
-                                           StageRegs<TYPE>& r) {
+__device__ __forceinline__ void init_stage_ptrs(const GemmArgs& a, uint32_t row0, uint32_t tok0, uint32_t kb0, StagePtrs<NTOK>& p) {
     using PT = PairTraits<TYPE>;
-    const uint32_t t = threadIdx.x;
+    constexpr int PER_WAVE = NTOK / 8 / (THREADS / 64);
+    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
     const uint32_t nb = a.k >> 5;
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; j++) {
+        const uint32_t tt = 8u * (PER_WAVE * wave + j) + (lane >> 3);  // token within the tile
+        const uint32_t chunk = (lane & 7u) ^ xt_swizzle(tt);
+        const uint32_t tok = min(tok0 + tt, a.n - 1);
+        p.x[j] = a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + 16u * chunk;
+    }
+    p.wd = nullptr;
     if (t < 2 * BM) {
         const uint32_t lr = t >> 1;  // operand row of the tile
         uint32_t row = row0 + lr;
@@ -188,11 +199,23 @@ __device__ __forceinline__ void load_stage(const GemmArgs& a, uint32_t row0, uin
             w = (lr >> 5) & 1u ? a.w_up : a.w;
         }
         row = min(row, a.m - 1);
-        const uint8_t* p = w + ((size_t)row * nb + kb0 + 2 * (t & 1u)) * (PT::BYTES / 2);
-        load_pair<PT::DWORDS>(p, r.w);
+        p.wd = w + ((size_t)row * nb + kb0 + 2 * (t & 1u)) * (PT::BYTES / 2);
     } else if (t < 2 * BM + NTOK && a.xs) {  // xs is null only for the parity hook, which never scales
         const uint32_t tok = min(tok0 + (t - 2 * BM), a.n - 1);
-        r.dx = *reinterpret_cast<const float4*>(a.xs + (size_t)tok * nb + kb0);
+        p.wd = reinterpret_cast<const uint8_t*>(a.xs + (size_t)tok * nb + kb0);
+    }
+}
+
+template <int TYPE, int NTOK>
+__device__ __forceinline__ void load_stage(StagePtrs<NTOK>& p, StageRegs<TYPE>& r) {
+    using PT = PairTraits<TYPE>;
+    const uint32_t t = threadIdx.x;
+    if (t < 2 * BM) {
+        load_pair<PT::DWORDS>(p.wd, r.w);
+        p.wd += KB * (PT::BYTES / 2);
+    } else if (p.wd) {
+        r.dx = *reinterpret_cast<const float4*>(p.wd);
+        p.wd += KB * sizeof(float);
     } else {
         r.dx = make_float4(0.f, 0.f, 0.f, 0.f);
     }
@@ -410,19 +433,34 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
     asm volatile("" : "+v"(cbias));  // keep it in registers (left alone, the compiler rebuilds it before every MFMA)
 
     StageRegs<TYPE> regs;
-    dma_activations(a, sm.st[0], tok0, first * KB);
-    load_stage<TYPE, BN, GATED>(a, row0, tok0, first * KB, regs);
+    StagePtrs<BN> ptrs;
+    init_stage_ptrs<TYPE, BN, GATED>(a, row0, tok0, first * KB, ptrs);
+    dma_activations(ptrs, sm.st[0]);
+    load_stage<TYPE, BN>(ptrs, regs);
     store_stage<TYPE, BN>(sm.st[0], regs);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
     __syncthreads();
 
+    // This lane's LDS read addresses: block 0 of buffer 0 here, moved from block to block by next_block and from one buffer to
+    // the other at the end of every stage (four additions instead of rebuilding them).
+    LaneAddr la;
+    {
+        const Stage& s = sm.st[0];
+        // this lane's token row; K-chunk 2*block + (kq >> 1) sits at position chunk ^ swizzle
+        la.xsh = xt_swizzle(wtok0 + l16) >> 1;
+        la.xbase = lds_addr(&s.xt[wtok0 + l16][0]) + ((((kq >> 1) ^ xt_swizzle(wtok0 + l16)) & 1u) << 4) + 8 * (kq & 1u);
+        la.xt = la.xbase + (la.xsh << 5);
+        la.wt = lds_addr(&s.wt[kq >> 1][0][wrow0 + l16]) + 8 * (kq & 1u);
+        la.dws = lds_addr(&s.dws[0][wrow0 + l16]);
+        la.dxf = lds_addr(&s.dxf[0][wtok0 + 4 * kq]);
+    }
+
     for (uint32_t st = 0; st < stages; st++) {
-        const Stage& s = sm.st[st & 1u];
         if (st + 1 < stages) {
             // the other LDS stage was last read in stage st-1 and every wave has passed the
             // barrier that ended it, so it can be refilled from here on
-            dma_activations(a, sm.st[(st + 1) & 1u], tok0, (first + st + 1) * KB);
-            load_stage<TYPE, BN, GATED>(a, row0, tok0, (first + st + 1) * KB, regs);
+            dma_activations(ptrs, sm.st[(st + 1) & 1u]);
+            load_stage<TYPE, BN>(ptrs, regs);
         }
 
         // 8 MFMA tiles per block, software-pipelined by hand: four result buffers, the matrix
@@ -431,14 +469,6 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
         // issued, so LDS latency stays out of the wave's dependency chain.  The scheduling
         // barriers pin that order; the block loop stays rolled.
         // Tile order: t = 4 * token tile + row tile.
-        LaneAddr la;  // block 0 of this stage's buffer
-        // this lane's token row; K-chunk 2*block + (kq >> 1) sits at position chunk ^ swizzle
-        la.xsh = xt_swizzle(wtok0 + l16) >> 1;
-        la.xbase = lds_addr(&s.xt[wtok0 + l16][0]) + ((((kq >> 1) ^ xt_swizzle(wtok0 + l16)) & 1u) << 4) + 8 * (kq & 1u);
-        la.xt = la.xbase + (la.xsh << 5);
-        la.wt = lds_addr(&s.wt[kq >> 1][0][wrow0 + l16]) + 8 * (kq & 1u);
-        la.dws = lds_addr(&s.dws[0][wrow0 + l16]);
-        la.dxf = lds_addr(&s.dxf[0][wtok0 + 4 * kq]);
         Mats mt;
         Scales sc;
         load_mats(la, mt);              // 6 reads
@@ -474,6 +504,14 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
             load_row_scales(la, sc);
         }
         lds_wait<0>(sc);  // nothing of this stage's buffer is read past this point
+        {   // block 0 of the other buffer (the block loop left wt / dws / dxf at block KB - 1)
+            const uint32_t other = (st & 1u) ? 0u - (uint32_t)sizeof(Stage) : (uint32_t)sizeof(Stage);
+            la.xbase += other;
+            la.xt = la.xbase + (la.xsh << 5);
+            la.wt += other - (KB - 1) * kOffWt;
+            la.dws += other - (KB - 1) * kOffDws;
+            la.dxf += other - (KB - 1) * kOffDxf;
+        }
 
         // The other buffer was last read in stage st-1; every wave has passed the barrier
         // that ended that stage, so it is free to be refilled now.
@@ -600,26 +638,31 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     asm volatile("" : "+v"(cbias));
 
     StageRegs<TYPE> regs;
-    dma_activations(a, sm.st[0], tok0, first * KB);
-    load_stage<TYPE, BN_NARROW>(a, row0, tok0, first * KB, regs);
+    StagePtrs<BN_NARROW> ptrs;
+    init_stage_ptrs<TYPE, BN_NARROW>(a, row0, tok0, first * KB, ptrs);
+    dma_activations(ptrs, sm.st[0]);
+    load_stage<TYPE, BN_NARROW>(ptrs, regs);
     store_stage<TYPE, BN_NARROW>(sm.st[0], regs);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
     __syncthreads();
 
-    for (uint32_t st = 0; st < stages; st++) {
-        const StageT<BN_NARROW>& s = sm.st[st & 1u];
-        if (st + 1 < stages) {
-            dma_activations(a, sm.st[(st + 1) & 1u], tok0, (first + st + 1) * KB);
-            load_stage<TYPE, BN_NARROW>(a, row0, tok0, (first + st + 1) * KB, regs);
-        }
-
-        LaneAddr la;  // block 0 of this stage's buffer
+    LaneAddr la;  // block 0 of buffer 0; moved on as in the wide kernel
+    {
+        const StageT<BN_NARROW>& s = sm.st[0];
         la.xsh = xt_swizzle(l16) >> 1;
         la.xbase = lds_addr(&s.xt[l16][0]) + ((((kq >> 1) ^ xt_swizzle(l16)) & 1u) << 4) + 8 * (kq & 1u);
         la.xt = la.xbase + (la.xsh << 5);
         la.wt = lds_addr(&s.wt[kq >> 1][0][wrow0 + l16]) + 8 * (kq & 1u);
         la.dws = lds_addr(&s.dws[0][wrow0 + l16]);
         la.dxf = lds_addr(&s.dxf[0][4 * kq]);
+    }
+
+    for (uint32_t st = 0; st < stages; st++) {
+        if (st + 1 < stages) {
+            dma_activations(ptrs, sm.st[(st + 1) & 1u]);
+            load_stage<TYPE, BN_NARROW>(ptrs, regs);
+        }
+
         NarrowMats mt;
         NarrowScales sc;
         load_mats(la, mt);    // 5 reads
@@ -649,6 +692,14 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
             load_scales(la, sc);
         }
         lds_wait<0>(sc);  // nothing of this stage's buffer is read past this point
+        {
+            const uint32_t other = (st & 1u) ? 0u - (uint32_t)sizeof(StageT<BN_NARROW>) : (uint32_t)sizeof(StageT<BN_NARROW>);
+            la.xbase += other;
+            la.xt = la.xbase + (la.xsh << 5);
+            la.wt += other - (KB - 1) * kOffWt;
+            la.dws += other - (KB - 1) * kOffDws;
+            la.dxf += other - (KB - 1) * kOffDxfNarrow;
+        }
 
         if (st + 1 < stages) store_stage<TYPE, BN_NARROW>(sm.st[(st + 1) & 1u], regs);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS copies of the next stage have landed
