@@ -170,6 +170,35 @@ def test_qk_norm_rope_and_append(ctx, ops, oracle, n_heads, n_kv, hd, pos):
         b.free()
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,max_seq", [(16, 8, 64, 4096), (4, 2, 64, 100), (8, 2, 128, 512), (3, 1, 96, 70)])
+def test_attention_over_one_position_returns_the_value_row(ctx, ops, oracle, n_heads, n_kv, hd, max_seq):
+    """The closed form the reference's own test leans on (wick/tests/single_token_attn.rs:33-43): with one cached position
+    softmax([score]) = [1] for every head, so the attention's output is the value row, repeated for the query heads of a
+    group -- bit for bit here, since ggml_expf(0) = 1 and v * 1 / 1 = v.  Through both decode paths (plain attention over a
+    cache that holds the row, and the block that appends the row itself) and the prompt kernel with one token."""
+    kv_dim = n_kv * hd
+    q, v = oracle.fill_normal(1, 3.0, n_heads * hd), oracle.fill_normal(2, 1.0, kv_dim)
+    kc = oracle.fill_normal(3, 1.0, max_seq * kv_dim)
+    vc = np.full(max_seq * kv_dim, np.nan, np.float32)  # nothing past the first row may be looked at
+    vc[:kv_dim] = v
+    want = np.concatenate([v[(h // (n_heads // n_kv)) * hd:(h // (n_heads // n_kv) + 1) * hd] for h in range(n_heads)])
+    d_q, d_kc, d_vc = ctx.to_device(q), ctx.to_device(kc), ctx.to_device(vc)
+    d_out, d_sc = ctx.alloc(n_heads * hd * 4), ctx.alloc(attention_block_scratch_bytes(max_seq, n_heads, hd))
+    ops.encode_attention(d_q, d_kc, d_vc, d_out, d_sc, 1, max_seq, n_heads, n_kv, hd)
+    assert np.array_equal(bits(d_out.download(np.float32, n_heads * hd)), bits(want))
+    if hd != 96:  # the prompt kernels take head dims 32 / 64 / 128 / 256 (a model with another one attends token by token)
+        ops.encode_attention_prefill(d_q, n_heads * hd, d_kc, d_vc, d_out, n_heads * hd, 0, 1, max_seq, n_heads, n_kv, hd)
+        assert np.array_equal(bits(d_out.download(np.float32, n_heads * hd)), bits(want))
+    # the block: norms and rotates q and k, appends k and v at position 0, attends over that one row
+    d_k, d_v = ctx.to_device(oracle.fill_normal(4, 1.0, kv_dim)), ctx.to_device(v)
+    d_qn, d_kn = ctx.to_device(1 + 0.2 * oracle.fill_normal(5, 1.0, hd)), ctx.to_device(1 + 0.2 * oracle.fill_normal(6, 1.0, hd))
+    d_vc2 = ctx.to_device(np.full(max_seq * kv_dim, np.nan, np.float32))
+    ops.encode_attention_block(d_q, d_k, d_v, d_qn, d_kn, d_kc, d_vc2, d_out, d_sc, 0, max_seq, hd, n_heads, n_kv, 1e-5, rope_theta_scale(hd, 1_000_000.0))
+    assert np.array_equal(bits(d_out.download(np.float32, n_heads * hd)), bits(want))
+    for b in (d_q, d_kc, d_vc, d_out, d_sc, d_k, d_v, d_qn, d_kn, d_vc2):
+        b.free()
+
+
 @pytest.mark.parametrize("n_heads,n_kv,hd,pos0,n,pad", [(16, 8, 64, 0, 40, 0), (4, 2, 64, 4000, 96, 8), (3, 1, 128, 7, 5, 0), (2, 2, 256, 100, 3, 4),
                                                         (5, 5, 32, 0, 1, 0)])
 def test_qk_norm_rope_of_a_prompt(ctx, ops, oracle, n_heads, n_kv, hd, pos0, n, pad):
