@@ -111,7 +111,8 @@ int wick_rocm_copy(wick_rocm_ctx *ctx, void *d_dst, const void *d_src, size_t nb
  * Stands in for MetalWeight {mmap_offset, dtype, m, k} (wick/src/model/metal_lfm2.rs:28-36,
  * 409-421).  A discrete GPU cannot wrap the GGUF mmap in place, so the block
  * bytes are copied once, verbatim, into HBM.  `nbytes` must equal
- * m * (k/32) * block_bytes(ggml_type), for Q6_K m * (k/256) * 210.  The handle stays valid until
+ * m * (k/32) * block_bytes(ggml_type), for Q6_K m * (k/256) * 210.  Q4_0 / Q8_0 weights with k % 128 == 0 also get
+ * the prefill GEMM's own layout of the same values (see wick_rocm_set_gemm_packing).  The handle stays valid until
  * wick_rocm_weight_free or context destruction. */
 int wick_rocm_weight_upload(wick_rocm_ctx *ctx, const void *host_blocks, size_t nbytes, int ggml_type,
                             uint32_t m, uint32_t k, wick_rocm_weight **out);
@@ -178,6 +179,17 @@ int wick_rocm_gemm_q8_multi(wick_rocm_ctx *ctx, const wick_rocm_weight *const *w
 int wick_rocm_gemm_q8_residual_rmsnorm_quantize(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const int8_t *d_quants, const float *d_scales,
                                                 uint32_t n, float *d_x, uint32_t x_stride, const float *d_norm_weight, float eps,
                                                 int8_t *d_out_quants, float *d_out_scales);
+
+/* wick_rocm_weight_upload keeps the raw blocks (what the decode GEMVs stream, as the reference's MetalWeight does,
+ * wick/src/model/metal_lfm2.rs:28-36) and, for Q4_0 / Q8_0 weights with k % 128 == 0, also makes the prefill GEMM's own copy on
+ * the device: the same int8 values and scales laid out in the order the GEMM's workgroups read them (32-row granules, one
+ * contiguous 5 KB slab per granule and 128 K-elements; 1.25 bytes per weight), so that a stage of weights reaches the matrix
+ * cores' operand buffer with plain coalesced copies and no unpacking in the main loop.  Results do not depend on it (same
+ * integers, same scales).  enabled = 0 switches the copy off for weights uploaded from then on: they take the multi-token GEMV
+ * route for any n (slower prompts, 1.25 bytes per weight less memory).  wick_rocm_weight_device_bytes: what a weight holds on
+ * the device, both copies.  No counterpart in the reference (its GPU GEMM reads the raw blocks). */
+int wick_rocm_set_gemm_packing(wick_rocm_ctx *ctx, int enabled);
+size_t wick_rocm_weight_device_bytes(const wick_rocm_weight *w);
 
 /* The n at and above which wick_rocm_gemm_q8 / wick_rocm_matmul_f32 hand off from the
  * multi-token GEMV to the MFMA GEMM (default 16, the reference's GEMM_MIN_N,

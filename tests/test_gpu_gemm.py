@@ -96,6 +96,48 @@ def test_accumulate(ctx, oracle, dtype, n):
         assert_f32_parity(fetch_gemm(d_y, m, n, m, W.LAYOUT_TOKEN_MAJOR), ref, "gemm accumulate")
 
 
+def test_weights_without_the_gemm_copy_take_the_gemv_route(ctx, oracle):
+    """wick_rocm_set_gemm_packing(0): weights uploaded from then on hold the raw blocks only (no second layout for the
+    matrix-core kernel) and run as multi-token GEMVs for any n -- same block dots bit for bit, f32 results to the bar."""
+    m, n, k = 200, 70, 512
+    for dtype, raw_per_block in ((W.Q4_0, 18), (W.Q8_0, 34)):
+        wb = oracle.synth_weight(dtype, m, k, 5, 0.02)
+        s, q = oracle.quantize_q8_0_batch(oracle.fill_normal(6, 1.0, n * k), n, k)
+        packed = ctx.upload_weight(wb, dtype, m, k)
+        ctx.set_gemm_packing(False)
+        try:
+            plain = ctx.upload_weight(wb, dtype, m, k)
+        finally:
+            ctx.set_gemm_packing(True)
+        raw = m * (k // 32) * raw_per_block
+        assert plain.device_bytes == raw
+        # whole pairs of 32-row granules, 5 KB per granule and 128 K-elements
+        assert packed.device_bytes == raw + 2 * ((m + 63) // 64) * (k // 128) * 5120
+        d_q, d_s = ctx.to_device(q), ctx.to_device(s)
+        ref = oracle.gemm_q8(dtype, wb, s, q, m, n, k)
+        outs, dots = [], []
+        for w in (packed, plain):
+            d_y, d_d = ctx.alloc(n * m * 4), ctx.alloc(n * m * (k // 32) * 4)
+            ctx.gemm_preq(w, d_s, d_q, n, d_y, y_stride=m, layout=W.LAYOUT_TOKEN_MAJOR)
+            ctx.block_dots_i32(w, d_q, n, d_d)
+            outs.append(fetch_gemm(d_y, m, n, m, W.LAYOUT_TOKEN_MAJOR))
+            dots.append(d_d.download(np.int32, n * m * (k // 32)))
+            d_y.free(), d_d.free()
+        assert_f32_parity(outs[0], ref, "packed weight")
+        assert_f32_parity(outs[1], ref, "raw-only weight")
+        assert np.array_equal(dots[0], dots[1])
+        assert np.array_equal(dots[0].reshape(n, m, k // 32), oracle.block_dots_i32(dtype, wb, q, m, n, k))
+        # a launch over several weights falls back to one call per weight when one of them has no copy
+        d_a, d_b = ctx.alloc(n * 2 * m * 4), ctx.alloc(n * 2 * m * 4)
+        ctx.gemm_preq_multi([packed, plain], d_s, d_q, n, [d_a.ptr, d_a.ptr + m * 4], 2 * m)
+        ctx.gemm_preq(packed, d_s, d_q, n, d_b.ptr, y_stride=2 * m, layout=W.LAYOUT_TOKEN_MAJOR)
+        ctx.gemm_preq(plain, d_s, d_q, n, d_b.ptr + m * 4, y_stride=2 * m, layout=W.LAYOUT_TOKEN_MAJOR)
+        assert np.array_equal(d_a.download(np.uint32, n * 2 * m), d_b.download(np.uint32, n * 2 * m))
+        for b in (d_q, d_s, d_a, d_b):
+            b.free()
+        packed.free(), plain.free()
+
+
 @pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
 @pytest.mark.parametrize("ms,n,k,layout,acc", [
     ((256, 128, 128), 200, 512, W.LAYOUT_TOKEN_MAJOR, False),   # Q / K / V into one [n][q|k|v] row

@@ -81,7 +81,7 @@ int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q
         }
         return WICK_ROCM_OK;
     }
-    const bool mfma_ok = (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_q) % 16u == 0) &&
+    const bool mfma_ok = w->d_gemm && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_q) % 16u == 0) &&
                          (reinterpret_cast<uintptr_t>(d_s) % 16u == 0);
     hipError_t e;
     if (n >= ctx->gemm_min_n && mfma_ok) {
@@ -92,7 +92,7 @@ int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q
             else if (int rc = ensure_scratch(ctx, 0, 0, floats)) return rc;
         }
         const bool defer = deferred && splits > 1;
-        e = launch_gemm_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_q, d_s, n, d_y, y_stride,
+        e = launch_gemm_mfma(w->type, static_cast<const uint8_t*>(w->d_gemm), w->m, w->k, d_q, d_s, n, d_y, y_stride,
                              y_layout, accumulate, ctx->launch(), splits, splits > 1 ? ctx->scratch_f : nullptr, defer);
         if (defer && e == hipSuccess) *deferred = splits;
     } else
@@ -261,6 +261,14 @@ int wick_rocm_set_gemm_max_k_splits(wick_rocm_ctx* ctx, uint32_t max_splits) {
     return WICK_ROCM_OK;
 }
 
+int wick_rocm_set_gemm_packing(wick_rocm_ctx* ctx, int enabled) {
+    WR_ENTER(ctx);
+    ctx->gemm_packing = enabled != 0;
+    return WICK_ROCM_OK;
+}
+
+size_t wick_rocm_weight_device_bytes(const wick_rocm_weight* w) { return w ? w->nbytes + w->gemm_bytes : 0; }
+
 int wick_rocm_set_gemm_min_n(wick_rocm_ctx* ctx, uint32_t min_n) {
     WR_ENTER(ctx);
     ctx->gemm_min_n = min_n == 0 ? kGemmMinN : min_n;
@@ -299,9 +307,18 @@ int wick_rocm_weight_upload(wick_rocm_ctx* ctx, const void* host_blocks, size_t 
     // (+64: the Q6_K kernel reads its last 16-byte piece whole)
     hipError_t e = hipMalloc(&w->d, nbytes + 64);
     if (e == hipSuccess) e = hipMemcpyAsync(w->d, host_blocks, nbytes, hipMemcpyHostToDevice, ctx->stream);
+    // The prefill GEMM reads its own layout of the weight (see gemm.hip): made here, once, on the device.  Weights the GEMM does
+    // not take (Q6_K, k % 128 != 0) or uploaded with packing switched off keep the raw blocks only and run as GEMVs for any n.
+    if (e == hipSuccess && ctx->gemm_packing && ggml_type != kTypeQ6_K && k % 128u == 0) {
+        w->gemm_bytes = gemm_packed_bytes(m, k);
+        e = hipMalloc(&w->d_gemm, w->gemm_bytes);
+        if (e == hipSuccess)
+            e = launch_gemm_pack(ggml_type, static_cast<const uint8_t*>(w->d), m, k, static_cast<uint8_t*>(w->d_gemm), ctx->launch());
+    }
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
         if (w->d) (void)hipFree(w->d);
+        if (w->d_gemm) (void)hipFree(w->d_gemm);
         delete w;
         return fail_hip(ctx, e, "weight_upload");
     }
@@ -330,6 +347,7 @@ int wick_rocm_weight_free(wick_rocm_ctx* ctx, wick_rocm_weight* w) {
     if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "weight_free during graph capture");
     WR_HIP(ctx, hipStreamSynchronize(ctx->stream));
     if (w->d) WR_HIP(ctx, hipFree(w->d));
+    if (w->d_gemm) WR_HIP(ctx, hipFree(w->d_gemm));
     delete w;
     return WICK_ROCM_OK;
 }
@@ -627,7 +645,9 @@ int wick_rocm_gemm_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* w
         if (ws[i]->type != ws[0]->type || ws[i]->k != ws[0]->k) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "gemm_q8_multi: weights must share k and dtype");
     }
     const wick_rocm_weight* w0 = ws[0];
-    const bool one_launch = count > 1 && w0->type != kTypeQ6_K && n >= ctx->gemm_min_n && w0->k % 128u == 0 && d_quants && d_scales &&
+    bool packed = true;
+    for (uint32_t i = 0; i < count; i++) packed = packed && ws[i]->d_gemm != nullptr;
+    const bool one_launch = count > 1 && packed && w0->type != kTypeQ6_K && n >= ctx->gemm_min_n && w0->k % 128u == 0 && d_quants && d_scales &&
                             reinterpret_cast<uintptr_t>(d_quants) % 16u == 0 && reinterpret_cast<uintptr_t>(d_scales) % 16u == 0;
     if (!one_launch) {  // shapes without a batched launch: one call per weight, same results
         for (uint32_t i = 0; i < count; i++)
@@ -642,7 +662,7 @@ int wick_rocm_gemm_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* w
         if (!d_ys[i]) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "null device pointer");
         if (y_layout == WICK_ROCM_LAYOUT_TOKEN_MAJOR ? y_stride < ws[i]->m : y_stride < n)
             return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "y_stride smaller than the output extent");
-        wp[i] = static_cast<const uint8_t*>(ws[i]->d), ms[i] = ws[i]->m;
+        wp[i] = static_cast<const uint8_t*>(ws[i]->d_gemm), ms[i] = ws[i]->m;
     }
     hipError_t e = launch_gemm_mfma_multi(w0->type, wp, ms, count, w0->k, d_quants, d_scales, n, d_ys, y_stride, y_layout, accumulate, ctx->launch());
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "gemm launch");
@@ -716,8 +736,8 @@ int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, cons
         }
         return WICK_ROCM_OK;
     }
-    const bool mfma = n >= ctx->gemm_min_n && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
-    hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->launch())
+    const bool mfma = w->d_gemm && n >= ctx->gemm_min_n && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
+    hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d_gemm), w->m, w->k, d_quants, n, d_out, ctx->launch())
                         : launch_block_dots_gemv(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->num_cus, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "block_dots launch");
     return WICK_ROCM_OK;

@@ -1,12 +1,11 @@
-// Batched prefill GEMM: raw GGUF Q4_0 / Q8_0 weight blocks x Q8_0-quantized
-// activations -> f32, on the gfx950 int8 matrix cores.
+// Batched prefill GEMM: Q4_0 / Q8_0 weights x Q8_0-quantized activations -> f32, on the gfx950 int8 matrix cores.
 //
 // Arithmetic: gemm_q4_0_q8_0_neon / gemm_q8_0_q8_0_neon
 // (wick/src/backend/simd.rs:696-925, 937-1019):
 //   C[i,j] = sum_b f32(isum_{i,j,b}) * (f32(f16 d_w[i,b]) * xs[j,b]),  isum exact i32
 // with one scale pair per 32-element block, so i32 accumulation cannot run across
-// blocks: every v_mfma_i32_32x32x32_i8 covers exactly one block (K = 32) and its
-// 32x32 i32 result is scaled into f32 accumulators on the vector ALU.
+// blocks: every MFMA covers exactly one block (K = 32) and its i32 result is scaled
+// into f32 accumulators on the vector ALU.
 //
 // Workgroup = 512 threads = 8 waves, tile = 128 weight rows x 128 tokens, each wave
 // owns 64 rows x 32 tokens = 4 x 2 tiles of v_mfma_i32_16x16x32_i8.  The small MFMA
@@ -16,22 +15,24 @@
 // instruction runs at half the 32x32x32 rate, 1.9 vs 3.8 POP/s measured): a wave can issue
 // a vector-ALU instruction only every ~4.7 cycles while a SIMD retires one every ~2.2, and
 // the kernel is bound by the two scaling FMAs per result.
-// One stage = 4 blocks (128 elements of K):
-//   * weights: threads 0-255 read one 36/68-byte block pair each with dword-aligned wide
-//     loads, unpack nibbles to int8 and write 16-byte operand rows to LDS;
-//   * activations: copied global -> LDS directly (global_load_lds_dwordx4, asynchronous,
-//     no registers); token scales through registers.
-// LDS holds two stages (77 KB, two workgroups per CU).  The global loads of stage s+1 are
-// issued before stage s is computed and written to the other LDS buffer after it, so there
-// is one barrier per stage and the load latency hides behind the stage's ALU work.
+// One stage = 4 blocks (128 elements of K).  Both operands are copied global -> LDS directly
+// (global_load_lds_dwordx4: asynchronous, no registers, 1 KB per wave instruction):
+//   * weights from the GEMM's own copy of the matrix, made from the raw GGUF blocks when the
+//     weight is uploaded (gemm_pack_kernel, layout at StageT): int8 operand rows and
+//     {scale, -bias * scale} pairs already in the order a stage of LDS holds them, so the main
+//     loop neither unpacks nibbles nor converts scales nor stores to LDS;
+//   * activations from the token-major Q8_0 quants; token scales through registers (they are
+//     stored block-major).
+// LDS holds two stages (76 KB, two workgroups per CU).  The copies of stage s+1 are issued
+// before stage s is computed, so there is one barrier per stage and the load latency hides
+// behind the stage's ALU work.
 //
-// LDS operand layout: [block][khalf][row][16 bytes] (weights: [khalf][block][row]).  An
-// MFMA lane supplies 8 consecutive K-bytes of operand row lane % 16, K-quarter lane / 16,
-// so 32 consecutive lanes read 256 consecutive bytes (the two 8-byte halves of 16 rows):
-// conflict-free.  For Q4_0 the low nibbles of a block ARE its first 16 elements and the
-// high nibbles its last 16 (wick/src/quant.rs:82-88), so the two halves fall out of one
-// and / shift each.  (The K order inside an MFMA is irrelevant as long as both operands
-// use the same one.)
+// LDS operand layout: weights [granule of 32 rows][khalf][block][row][16 bytes], activations
+// [token][8 x 16 bytes, swizzled].  An MFMA lane supplies 8 consecutive K-bytes of operand row
+// lane % 16, K-quarter lane / 16, so 32 consecutive lanes read 256 consecutive bytes (the two
+// 8-byte halves of 16 rows): conflict-free.  For Q4_0 the low nibbles of a block ARE its first
+// 16 elements and the high nibbles its last 16 (wick/src/quant.rs:82-88): the two khalf planes.
+// (The K order inside an MFMA is irrelevant as long as both operands use the same one.)
 //
 // Roles: tokens are the MFMA "A" (M) operand, weight rows the "B" (N) operand, so in the
 // 16x16 result a lane holds ONE weight row (n = lane % 16) and 4 consecutive tokens
@@ -109,16 +110,28 @@ __device__ __forceinline__ void select_weight(GemmArgs& a, uint32_t& row_tile) {
     }
 }
 
-// One stage of operands.  Row counts are padded (one 16-byte operand row per
-// plane, two float2 per scale row) so that the stage WRITES, where neighbouring
-// lanes hit different planes of the same row, spread over the LDS banks; reads
-// walk consecutive rows of one plane.
+// The weights a GEMM launch reads are not the raw GGUF blocks but a copy laid out for this kernel, made once when the
+// weight is uploaded (gemm_pack_kernel): rows in granules of 32, and per (granule, stage of 4 blocks) one 5120-byte slab
+//   [khalf 2][block 4][row 32][16 bytes]   int8 operand rows (Q4_0: 16 * (nibble - 8)), 4096 bytes
+//   [block 4][row 32] {dw, -12582912 * dw}  scale pairs (dw x 1/16 for Q4_0), 1024 bytes
+// laid out [pair of granules][stage][granule of the pair]: the 64 rows x 128 K-elements a wave works on are 10 KB in one piece.  A slab is exactly what a stage of LDS holds for those 32 rows, so the weights go
+// global -> LDS directly like the activations: five 1 KB copies per granule, no staging registers, no unpack and no LDS
+// stores in the main loop, fully coalesced.  A tile is four granules (a gated tile: two of the gate weight and the same
+// two of the up weight).  1.25 bytes per weight instead of 0.5625 (Q4_0) / 1.0625 (Q8_0).
+constexpr int GR = 32;                              // rows per granule
+constexpr int kSlabWt = 2 * KB * GR * 16;           // 4096
+constexpr int kSlabDws = KB * GR * 8;               // 1024
+constexpr int kSlab = kSlabWt + kSlabDws;           // 5120
+constexpr int kSlabChunks = kSlab / 1024;           // 5 direct-to-LDS copies of 1 KB
+constexpr int kTileChunks = (BM / GR) * kSlabChunks;  // 20 per tile and stage
+
+// One stage of operands.
 template <int NTOK>  // tokens per workgroup tile: BN, or BN_NARROW for the narrow kernel
 struct StageT {
-    uint4 wt[2][KB][BM + 2];    // [khalf][block][row]  int8 weights (Q4_0: x16)
-    uint4 xt[NTOK][2 * KB];     // [token][16-byte K-chunk, swizzled] int8 activations, see dma_activations
-    float2 dws[KB][BM + 2];     // {dw, -12582912*dw} per block and row (dw x 1/16 for Q4_0)
-    float dxf[KB][NTOK];        // token scales
+    uint4 wt[BM / GR][2][KB][GR];  // [granule][khalf][block][row]  int8 weights: the slabs' first 4 KB
+    uint4 xt[NTOK][2 * KB];        // [token][16-byte K-chunk, swizzled] int8 activations, see dma_activations
+    float2 dws[BM / GR][KB][GR];   // {dw, -12582912*dw} per granule, block and row: the slabs' last 1 KB
+    float dxf[KB][NTOK];           // token scales
 };
 using Stage = StageT<BN>;
 
@@ -132,11 +145,37 @@ using Smem = SmemT<BN>;
 __device__ __forceinline__ uint32_t q4_lo_x16(uint32_t q) { return ((q << 4) & 0xf0f0f0f0u) ^ 0x80808080u; }
 __device__ __forceinline__ uint32_t q4_hi_x16(uint32_t q) { return (q & 0xf0f0f0f0u) ^ 0x80808080u; }
 
-template <int TYPE>
 struct StageRegs {
-    uint32_t w[PairTraits<TYPE>::DWORDS];
     float4 dx;
 };
+
+// Raw blocks -> slabs.  One workgroup per (granule, stage): thread (row = t % 32, block = t / 32).  Rows past the end of
+// the matrix become zero rows with zero scales.  For Q4_0 the low nibbles of a block ARE its first 16 elements and the high
+// nibbles its last 16 (wick/src/quant.rs:82-88): the two khalf planes.
+template <int TYPE>
+__global__ __launch_bounds__(GR * KB) void gemm_pack_kernel(const uint8_t* __restrict__ raw, uint32_t m, uint32_t nb, uint8_t* __restrict__ packed) {
+    constexpr int BB = TYPE == 2 ? 18 : 34;
+    const uint32_t stages = nb / KB, granule = blockIdx.x / stages, stage = blockIdx.x % stages;
+    const uint32_t within = threadIdx.x % GR, b = threadIdx.x / GR, row = granule * GR + within;
+    uint32_t lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
+    float dw = 0.0f;
+    if (row < m) {
+        const uint16_t* blk = reinterpret_cast<const uint16_t*>(raw + ((size_t)row * nb + stage * KB + b) * BB);  // blocks are 2-byte aligned
+        dw = f16_bits_to_f32(blk[0]) * (TYPE == 2 ? 0.0625f : 1.0f);
+        uint32_t q[8];
+#pragma unroll
+        for (int i = 0; i < (BB - 2) / 4; i++) q[i] = (uint32_t)blk[1 + 2 * i] | ((uint32_t)blk[2 + 2 * i] << 16);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            lo[i] = TYPE == 2 ? q4_lo_x16(q[i]) : q[i];
+            hi[i] = TYPE == 2 ? q4_hi_x16(q[i]) : q[4 + i];
+        }
+    }
+    uint8_t* slab = packed + (((size_t)(granule >> 1) * stages + stage) * 2 + (granule & 1u)) * kSlab;
+    reinterpret_cast<uint4*>(slab)[(0 * KB + b) * GR + within] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    reinterpret_cast<uint4*>(slab)[(1 * KB + b) * GR + within] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    reinterpret_cast<float2*>(slab + kSlabWt)[b * GR + within] = make_float2(dw, -kBias * dw);
+}
 
 // Activation tiles go global -> LDS directly (global_load_lds_dwordx4): no staging
 // registers, no unpack, no ds_write, and the copy runs asynchronously under the stage's
@@ -155,11 +194,18 @@ __device__ __forceinline__ uint32_t xt_swizzle(uint32_t token_in_tile) { return 
 template <int NTOK>
 struct StagePtrs {
     const int8_t* x[NTOK / 8 / (THREADS / 64)];  // this lane's 16-byte activation chunks (direct-to-LDS copies)
-    const uint8_t* wd;                            // threads 0 .. 2 BM - 1: a weight block pair; the next NTOK threads: a token's four scales
+    const uint8_t* wc[3];                         // this lane's 16 bytes of the wave's weight chunks wave, wave + 8, wave + 16 (of 20)
+    const uint8_t* dx;                            // threads 2 BM .. 2 BM + NTOK - 1: a token's four scales
 };
+// Where chunk c (0 .. 19) of a tile's stage lands: granule c / 5, its weights' kilobyte c % 5 or (the fifth) its scale pairs.
 template <int NTOK>
-__device__ __forceinline__ void dma_activations(StagePtrs<NTOK>& p, StageT<NTOK>& s) {
-    constexpr int PER_WAVE = NTOK / 8 / (THREADS / 64);  // instructions per wave and stage
+__device__ __forceinline__ void* chunk_dst(StageT<NTOK>& s, uint32_t c) {
+    const uint32_t g = c / kSlabChunks, part = c % kSlabChunks;
+    return part < 4 ? static_cast<void*>(reinterpret_cast<uint8_t*>(&s.wt[g][0][0][0]) + 1024u * part) : static_cast<void*>(&s.dws[g][0][0]);
+}
+template <int NTOK>
+__device__ __forceinline__ void dma_stage(StagePtrs<NTOK>& p, StageT<NTOK>& s) {
+    constexpr int PER_WAVE = NTOK / 8 / (THREADS / 64);  // activation instructions per wave and stage
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 #pragma unroll
     for (int j = 0; j < PER_WAVE; j++) {
@@ -167,21 +213,23 @@ __device__ __forceinline__ void dma_activations(StagePtrs<NTOK>& p, StageT<NTOK>
                                          (void __attribute__((address_space(3)))*)&s.xt[8u * (PER_WAVE * wave + j)][0], 16, 0, 0);
         p.x[j] += KB * 32;
     }
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const uint32_t c = wave + 8u * j;
+        if (c < (uint32_t)kTileChunks) {  // uniform per wave
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)p.wc[j],
+                                             (void __attribute__((address_space(3)))*)chunk_dst(s, c), 16, 0, 0);
+            p.wc[j] += 2 * kSlab;
+        }
+    }
 }
 
-// Thread -> work of one stage:
-//   weights      256 pairs   = 128 rows x 2 pairs             : threads 0..255, row = t >> 1, pair = t & 1
-//   activations  direct-to-LDS, see dma_activations
-//   token scales one float4 (4 blocks) per token               : threads 256..256+NTOK-1, token = t - 256
-// GATED: the tile's 128 operand rows are 64 output rows of the gate weight and the same 64 of the up weight, laid out so
-// that every wave (64 operand rows = four 16-row MFMA tiles) holds {gate rows A, gate rows B, up rows A, up rows B} of
-// the same 32 output rows: the SiLU gate and a whole Q8_0 block of its result then sit in one wave's registers.
-template <int TYPE, int NTOK, bool GATED = false>
-__device__ __forceinline__ void init_stage_ptrs(const GemmArgs& a, uint32_t row0, uint32_t tok0, uint32_t kb0, StagePtrs<NTOK>& p) {
-    using PT = PairTraits<TYPE>;
+template <int NTOK, bool GATED = false>
+__device__ __forceinline__ void init_stage_ptrs(const GemmArgs& a, uint32_t row_tile, uint32_t tok0, uint32_t kb0, StagePtrs<NTOK>& p) {
     constexpr int PER_WAVE = NTOK / 8 / (THREADS / 64);
-    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
-    const uint32_t nb = a.k >> 5;
+    const uint32_t t = threadIdx.x, lane = t & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(t >> 6));
+    const uint32_t nb = a.k >> 5, stages = nb / KB;
 #pragma unroll
     for (int j = 0; j < PER_WAVE; j++) {
         const uint32_t tt = 8u * (PER_WAVE * wave + j) + (lane >> 3);  // token within the tile
@@ -189,63 +237,38 @@ __device__ __forceinline__ void init_stage_ptrs(const GemmArgs& a, uint32_t row0
         const uint32_t tok = min(tok0 + tt, a.n - 1);
         p.x[j] = a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + 16u * chunk;
     }
-    p.wd = nullptr;
-    if (t < 2 * BM) {
-        const uint32_t lr = t >> 1;  // operand row of the tile
-        uint32_t row = row0 + lr;
-        const uint8_t* w = a.w;
-        if constexpr (GATED) {
-            row = row0 + 32u * (lr >> 6) + 16u * ((lr >> 4) & 1u) + (lr & 15u);
-            w = (lr >> 5) & 1u ? a.w_up : a.w;
-        }
-        row = min(row, a.m - 1);
-        p.wd = w + ((size_t)row * nb + kb0 + 2 * (t & 1u)) * (PT::BYTES / 2);
-    } else if (t < 2 * BM + NTOK && a.xs) {  // xs is null only for the parity hook, which never scales
+    const uint32_t granules = (a.m + GR - 1) / GR;
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const uint32_t c = min(wave + 8u * j, (uint32_t)kTileChunks - 1u), g = c / kSlabChunks, part = c % kSlabChunks;
+        // the tile's granule g: rows 32 g .. of a plain tile; of a gated tile (64 output rows) gate, up, gate, up of its two
+        uint32_t granule = GATED ? 2u * row_tile + (g >> 1) : (BM / GR) * row_tile + g;
+        const uint8_t* w = GATED && (g & 1u) ? a.w_up : a.w;
+        granule = min(granule, granules - 1u);  // past the end of the matrix: any rows, their results are not stored
+        p.wc[j] = w + (((size_t)(granule >> 1) * stages + kb0 / KB) * 2 + (granule & 1u)) * kSlab + 1024u * part + 16u * lane;
+    }
+    p.dx = nullptr;
+    if (t >= 2 * BM && t < 2 * BM + NTOK && a.xs) {  // xs is null only for the parity hook, which never scales
         const uint32_t tok = min(tok0 + (t - 2 * BM), a.n - 1);
-        p.wd = reinterpret_cast<const uint8_t*>(a.xs + (size_t)tok * nb + kb0);
+        p.dx = reinterpret_cast<const uint8_t*>(a.xs + (size_t)tok * nb + kb0);
     }
 }
 
-template <int TYPE, int NTOK>
-__device__ __forceinline__ void load_stage(StagePtrs<NTOK>& p, StageRegs<TYPE>& r) {
-    using PT = PairTraits<TYPE>;
-    const uint32_t t = threadIdx.x;
-    if (t < 2 * BM) {
-        load_pair<PT::DWORDS>(p.wd, r.w);
-        p.wd += KB * (PT::BYTES / 2);
-    } else if (p.wd) {
-        r.dx = *reinterpret_cast<const float4*>(p.wd);
-        p.wd += KB * sizeof(float);
+// Thread -> rest of a stage: one float4 (4 blocks) of token scales per token, threads 2 BM .. 2 BM + NTOK - 1, through registers
+// (they are stored block-major).
+template <int NTOK>
+__device__ __forceinline__ void load_stage(StagePtrs<NTOK>& p, StageRegs& r) {
+    if (p.dx) {
+        r.dx = *reinterpret_cast<const float4*>(p.dx);
+        p.dx += KB * sizeof(float);
     } else {
         r.dx = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 }
 
-template <int TYPE, int NTOK>
-__device__ __forceinline__ void store_stage(StageT<NTOK>& s, const StageRegs<TYPE>& r) {
-    using PT = PairTraits<TYPE>;
+template <int NTOK>
+__device__ __forceinline__ void store_stage(StageT<NTOK>& s, const StageRegs& r) {
     const uint32_t t = threadIdx.x;
-    if (t < 2 * BM) {
-        const uint32_t row = t >> 1;
-        const uint32_t b0 = 2 * (t & 1u);
-        uint32_t d0, d1, q0[PT::NQ], q1[PT::NQ];
-        split_pair<TYPE>(r.w, d0, d1, q0, q1);
-        const float scale = (TYPE == 2) ? 0.0625f : 1.0f;
-        const float dw0 = f16_bits_to_f32(d0) * scale, dw1 = f16_bits_to_f32(d1) * scale;
-        s.dws[b0][row] = make_float2(dw0, -kBias * dw0);
-        s.dws[b0 + 1][row] = make_float2(dw1, -kBias * dw1);
-        if constexpr (TYPE == 2) {
-            s.wt[0][b0][row] = make_uint4(q4_lo_x16(q0[0]), q4_lo_x16(q0[1]), q4_lo_x16(q0[2]), q4_lo_x16(q0[3]));
-            s.wt[1][b0][row] = make_uint4(q4_hi_x16(q0[0]), q4_hi_x16(q0[1]), q4_hi_x16(q0[2]), q4_hi_x16(q0[3]));
-            s.wt[0][b0 + 1][row] = make_uint4(q4_lo_x16(q1[0]), q4_lo_x16(q1[1]), q4_lo_x16(q1[2]), q4_lo_x16(q1[3]));
-            s.wt[1][b0 + 1][row] = make_uint4(q4_hi_x16(q1[0]), q4_hi_x16(q1[1]), q4_hi_x16(q1[2]), q4_hi_x16(q1[3]));
-        } else {
-            s.wt[0][b0][row] = make_uint4(q0[0], q0[1], q0[2], q0[3]);
-            s.wt[1][b0][row] = make_uint4(q0[4], q0[5], q0[6], q0[7]);
-            s.wt[0][b0 + 1][row] = make_uint4(q1[0], q1[1], q1[2], q1[3]);
-            s.wt[1][b0 + 1][row] = make_uint4(q1[4], q1[5], q1[6], q1[7]);
-        }
-    }
     if (t >= 2 * BM && t < 2 * BM + NTOK) {
         const uint32_t u = t - 2 * BM;
         s.dxf[0][u] = r.dx.x;
@@ -282,8 +305,8 @@ struct LaneAddr {
     uint32_t xt, wt, dws, dxf;
     uint32_t xbase, xsh;
 };
-constexpr int kOffWt = sizeof(uint4) * (BM + 2);      // one block of wt (within a khalf plane)
-constexpr int kOffDws = sizeof(float2) * (BM + 2);    // one block of dws
+constexpr int kOffWt = sizeof(uint4) * GR;            // one block of wt (within a granule's khalf plane)
+constexpr int kOffDws = sizeof(float2) * GR;          // one block of dws (within a granule)
 constexpr int kOffDxf = sizeof(float) * BN;           // one block of dxf
 __device__ __forceinline__ void next_block(LaneAddr& la, uint32_t block, bool advance) {
     la.xt = la.xbase + (((advance ? block + 1 : block) ^ la.xsh) << 5);
@@ -306,16 +329,16 @@ __device__ __forceinline__ void lds_read8(uint32_t addr, float2& dst) {
 __device__ __forceinline__ void load_mats(const LaneAddr& la, Mats& m) {  // TT + RT = 6 reads
     lds_read8<0 * 16 * 128>(la.xt, m.av[0]);  // 16 tokens further: same swizzle
     lds_read8<1 * 16 * 128>(la.xt, m.av[1]);
-    lds_read8<0 * 256>(la.wt, m.bv[0]);
-    lds_read8<1 * 256>(la.wt, m.bv[1]);
-    lds_read8<2 * 256>(la.wt, m.bv[2]);
-    lds_read8<3 * 256>(la.wt, m.bv[3]);
+    lds_read8<0>(la.wt, m.bv[0]);  // row tiles 0, 1: the two halves of the wave's first granule; 2, 3: of its second
+    lds_read8<256>(la.wt, m.bv[1]);
+    lds_read8<kSlabWt>(la.wt, m.bv[2]);
+    lds_read8<kSlabWt + 256>(la.wt, m.bv[3]);
 }
 __device__ __forceinline__ void load_row_scales(const LaneAddr& la, Scales& s) {  // RT = 4 reads
-    lds_read8<0 * 128>(la.dws, s.dw[0]);
-    lds_read8<1 * 128>(la.dws, s.dw[1]);
-    lds_read8<2 * 128>(la.dws, s.dw[2]);
-    lds_read8<3 * 128>(la.dws, s.dw[3]);
+    lds_read8<0>(la.dws, s.dw[0]);
+    lds_read8<128>(la.dws, s.dw[1]);
+    lds_read8<kSlabDws>(la.dws, s.dw[2]);
+    lds_read8<kSlabDws + 128>(la.dws, s.dw[3]);
 }
 template <int T>
 __device__ __forceinline__ void load_tok_scales(const LaneAddr& la, Scales& s) {  // 1 read
@@ -432,12 +455,12 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
     v4i cbias = {(int)kBiasBits, (int)kBiasBits, (int)kBiasBits, (int)kBiasBits};
     asm volatile("" : "+v"(cbias));  // keep it in registers (left alone, the compiler rebuilds it before every MFMA)
 
-    StageRegs<TYPE> regs;
+    StageRegs regs;
     StagePtrs<BN> ptrs;
-    init_stage_ptrs<TYPE, BN, GATED>(a, row0, tok0, first * KB, ptrs);
-    dma_activations(ptrs, sm.st[0]);
-    load_stage<TYPE, BN>(ptrs, regs);
-    store_stage<TYPE, BN>(sm.st[0], regs);
+    init_stage_ptrs<BN, GATED>(a, row_tile, tok0, first * KB, ptrs);
+    dma_stage(ptrs, sm.st[0]);
+    load_stage(ptrs, regs);
+    store_stage(sm.st[0], regs);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
     __syncthreads();
 
@@ -450,8 +473,8 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
         la.xsh = xt_swizzle(wtok0 + l16) >> 1;
         la.xbase = lds_addr(&s.xt[wtok0 + l16][0]) + ((((kq >> 1) ^ xt_swizzle(wtok0 + l16)) & 1u) << 4) + 8 * (kq & 1u);
         la.xt = la.xbase + (la.xsh << 5);
-        la.wt = lds_addr(&s.wt[kq >> 1][0][wrow0 + l16]) + 8 * (kq & 1u);
-        la.dws = lds_addr(&s.dws[0][wrow0 + l16]);
+        la.wt = lds_addr(&s.wt[wrow0 / GR][kq >> 1][0][l16]) + 8 * (kq & 1u);  // the wave's 64 rows are two granules
+        la.dws = lds_addr(&s.dws[wrow0 / GR][0][l16]);
         la.dxf = lds_addr(&s.dxf[0][wtok0 + 4 * kq]);
     }
 
@@ -459,8 +482,8 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
         if (st + 1 < stages) {
             // the other LDS stage was last read in stage st-1 and every wave has passed the
             // barrier that ended it, so it can be refilled from here on
-            dma_activations(ptrs, sm.st[(st + 1) & 1u]);
-            load_stage<TYPE, BN>(ptrs, regs);
+            dma_stage(ptrs, sm.st[(st + 1) & 1u]);
+            load_stage(ptrs, regs);
         }
 
         // 8 MFMA tiles per block, software-pipelined by hand: four result buffers, the matrix
@@ -515,7 +538,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
 
         // The other buffer was last read in stage st-1; every wave has passed the barrier
         // that ended that stage, so it is free to be refilled now.
-        if (st + 1 < stages) store_stage<TYPE, BN>(sm.st[(st + 1) & 1u], regs);
+        if (st + 1 < stages) store_stage(sm.st[(st + 1) & 1u], regs);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS copies of the next stage have landed
         __syncthreads();
     }
@@ -637,12 +660,12 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     v4i cbias = {(int)kBiasBits, (int)kBiasBits, (int)kBiasBits, (int)kBiasBits};
     asm volatile("" : "+v"(cbias));
 
-    StageRegs<TYPE> regs;
+    StageRegs regs;
     StagePtrs<BN_NARROW> ptrs;
-    init_stage_ptrs<TYPE, BN_NARROW>(a, row0, tok0, first * KB, ptrs);
-    dma_activations(ptrs, sm.st[0]);
-    load_stage<TYPE, BN_NARROW>(ptrs, regs);
-    store_stage<TYPE, BN_NARROW>(sm.st[0], regs);
+    init_stage_ptrs<BN_NARROW>(a, row_tile, tok0, first * KB, ptrs);
+    dma_stage(ptrs, sm.st[0]);
+    load_stage(ptrs, regs);
+    store_stage(sm.st[0], regs);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
     __syncthreads();
 
@@ -652,15 +675,15 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
         la.xsh = xt_swizzle(l16) >> 1;
         la.xbase = lds_addr(&s.xt[l16][0]) + ((((kq >> 1) ^ xt_swizzle(l16)) & 1u) << 4) + 8 * (kq & 1u);
         la.xt = la.xbase + (la.xsh << 5);
-        la.wt = lds_addr(&s.wt[kq >> 1][0][wrow0 + l16]) + 8 * (kq & 1u);
-        la.dws = lds_addr(&s.dws[0][wrow0 + l16]);
+        la.wt = lds_addr(&s.wt[wrow0 / GR][kq >> 1][0][(wrow0 % GR) + l16]) + 8 * (kq & 1u);  // the wave's 16 rows: half a granule
+        la.dws = lds_addr(&s.dws[wrow0 / GR][0][(wrow0 % GR) + l16]);
         la.dxf = lds_addr(&s.dxf[0][4 * kq]);
     }
 
     for (uint32_t st = 0; st < stages; st++) {
         if (st + 1 < stages) {
-            dma_activations(ptrs, sm.st[(st + 1) & 1u]);
-            load_stage<TYPE, BN_NARROW>(ptrs, regs);
+            dma_stage(ptrs, sm.st[(st + 1) & 1u]);
+            load_stage(ptrs, regs);
         }
 
         NarrowMats mt;
@@ -701,7 +724,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
             la.dxf += other - (KB - 1) * kOffDxfNarrow;
         }
 
-        if (st + 1 < stages) store_stage<TYPE, BN_NARROW>(sm.st[(st + 1) & 1u], regs);
+        if (st + 1 < stages) store_stage(sm.st[(st + 1) & 1u], regs);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS copies of the next stage have landed
         __syncthreads();
     }
@@ -827,6 +850,19 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0, boo
 }  // namespace
 
 uint32_t gemm_split_k(uint32_t m, uint32_t n, uint32_t k, uint32_t max_splits) { return split_k_factor(m, n, k, max_splits); }
+
+// The GEMM's own copy of a weight (slabs, see StageT): its size, and the kernel that makes it from the raw blocks.
+size_t gemm_packed_bytes(uint32_t m, uint32_t k) { return (size_t)((m + 2 * GR - 1) / (2 * GR)) * 2 * ((k >> 5) / KB) * kSlab; }
+
+hipError_t launch_gemm_pack(int type, const uint8_t* d_raw, uint32_t m, uint32_t k, uint8_t* d_packed, const Launch& L) {
+    const uint32_t nb = k >> 5;
+    if (m == 0 || nb == 0 || nb % KB != 0) return hipErrorInvalidValue;
+    const uint64_t blocks = (uint64_t)((m + 2 * GR - 1) / (2 * GR)) * 2 * (nb / KB);  // whole pairs: a last odd granule gets a zero partner
+    if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+    if (type == kTypeQ4_0) return launch_kernel(L, kFamOther, gemm_pack_kernel<2>, dim3((uint32_t)blocks), dim3(GR * KB), d_raw, m, nb, d_packed);
+    if (type == kTypeQ8_0) return launch_kernel(L, kFamOther, gemm_pack_kernel<8>, dim3((uint32_t)blocks), dim3(GR * KB), d_raw, m, nb, d_packed);
+    return hipErrorInvalidValue;
+}
 
 // splits > 1 (= gemm_split_k(m, n, k, ...)) with d_partial holding splits * n * m floats: the K-split launch pair.
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,

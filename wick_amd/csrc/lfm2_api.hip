@@ -144,7 +144,7 @@ int wick_rocm_attention_prefill_quantize_q8_0(wick_rocm_ctx* ctx, const float* d
 }
 
 int wick_rocm_ffn_gate_up_silu_quantize_applies(const wick_rocm_weight* w_gate, const wick_rocm_weight* w_up, uint32_t n) {
-    if (!w_gate || !w_up || !w_gate->d || !w_up->d) return 0;
+    if (!w_gate || !w_up || !w_gate->d_gemm || !w_up->d_gemm) return 0;
     if (w_gate->type != w_up->type || (w_gate->type != kTypeQ4_0 && w_gate->type != kTypeQ8_0)) return 0;
     if (w_gate->m != w_up->m || w_gate->k != w_up->k) return 0;
     return gemm_gated_applies(w_gate->m, n, w_gate->k) ? 1 : 0;
@@ -159,7 +159,7 @@ int wick_rocm_ffn_gate_up_silu_quantize_q8(wick_rocm_ctx* ctx, const wick_rocm_w
         return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE,
                     "ffn_gate_up_silu_quantize: needs two Q4_0 or two Q8_0 weights of one shape, m % 32 == 0, k % 128 == 0, n > 64, more than 256 "
                     "tiles and 16-byte aligned activations (use gemm_q8_multi + silu_mul_quantize_q8_0)");
-    hipError_t e = launch_gemm_mfma_gated(w_gate->type, static_cast<const uint8_t*>(w_gate->d), static_cast<const uint8_t*>(w_up->d), w_gate->m, w_gate->k,
+    hipError_t e = launch_gemm_mfma_gated(w_gate->type, static_cast<const uint8_t*>(w_gate->d_gemm), static_cast<const uint8_t*>(w_up->d_gemm), w_gate->m, w_gate->k,
                                           d_quants, d_scales, n, d_out_quants, d_out_scales, ctx->launch());
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "ffn_gate_up_silu_quantize launch");
 }
@@ -391,7 +391,7 @@ int upload_weight(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, const wick_gguf* g, con
                   wick_rocm_weight** out) {
     if (int rc = wick_rocm_weight_from_gguf(ctx, g, name.c_str(), out)) return rc;
     m->weights.push_back(*out);
-    m->bytes += (*out)->nbytes;
+    m->bytes += (*out)->nbytes + (*out)->gemm_bytes;
     if ((*out)->m != rows || (*out)->k != cols)
         return ctx_fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "lfm2_load: " + name + " has an unexpected shape");
     return WICK_ROCM_OK;

@@ -34,6 +34,7 @@ struct wick_rocm_ctx {
     bool capture_used_scratch = false;
     unsigned char* noalloc_scratch = nullptr;  // this device's address of the static scratch array of wick_rocm_matmul_f32_noalloc
     uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
+    bool gemm_packing = true;         // weight_upload also makes the GEMM's own copy of a Q4_0 / Q8_0 weight
     uint32_t gemm_max_splits = kGemmMaxSplits;  // K split of GEMM launches with few tiles (1: off)
     KernelTimer timer;
     int64_t gemv_direct_max_bytes = -1;
@@ -43,8 +44,10 @@ struct wick_rocm_ctx {
 };
 
 struct wick_rocm_weight {
-    void* d = nullptr;
+    void* d = nullptr;       // the raw blocks, as uploaded: what the decode GEMVs stream
     size_t nbytes = 0;
+    void* d_gemm = nullptr;  // the prefill GEMM's own copy (gemm_packed_bytes, see gemm.hip); null: the weight takes the GEMV route for any n
+    size_t gemm_bytes = 0;
     int type = 0;
     uint32_t m = 0, k = 0;
 };

@@ -129,7 +129,10 @@ hipError_t launch_gemv_tokens(int type, const uint8_t* d_w, uint32_t m, uint32_t
                               const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
                               int accumulate, int num_cus, const Launch& L);
 
-// int8-MFMA GEMM.  Requires k % 128 == 0.
+// int8-MFMA GEMM.  Requires k % 128 == 0.  d_w / d_w_gate / d_w_up of the GEMM launchers are the weights' PACKED copies
+// (gemm_packed_bytes bytes, made by launch_gemm_pack from the raw blocks when the weight is uploaded), not the raw blocks.
+size_t gemm_packed_bytes(uint32_t m, uint32_t k);
+hipError_t launch_gemm_pack(int type, const uint8_t* d_raw, uint32_t m, uint32_t k, uint8_t* d_packed, const Launch& L);
 hipError_t launch_gemm_mfma(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q,
                             const float* d_scales, uint32_t n, float* d_y, uint32_t y_stride, int y_layout,
                             int accumulate, const Launch& L, uint32_t splits = 1, float* d_partial = nullptr, bool defer_reduce = false);

@@ -73,6 +73,8 @@ _SIGNATURES = {
     "wick_rocm_sync": (C.c_int, [_P]),
     "wick_rocm_copy": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_set_gemm_min_n": (C.c_int, [_P, C.c_uint32]),
+    "wick_rocm_set_gemm_packing": (C.c_int, [_P, C.c_int]),
+    "wick_rocm_weight_device_bytes": (C.c_size_t, [_P]),
     "wick_rocm_set_gemm_max_k_splits": (C.c_int, [_P, C.c_uint32]),
     "wick_rocm_set_gemv_policy": (C.c_int, [_P, C.c_int64]),
     "wick_rocm_probe_rate": (C.c_int, [_P, C.c_int, C.c_uint32, C.POINTER(C.c_double)]),
@@ -169,6 +171,11 @@ class RocmWeight:
     def __init__(self, ctx: "RocmContext", handle: int, dtype: int, m: int, k: int, nbytes: int):
         self.ctx, self.handle, self.dtype, self.m, self.k, self.nbytes = ctx, handle, dtype, m, k, nbytes
 
+    @property
+    def device_bytes(self) -> int:
+        """Bytes this weight holds on the device: the raw blocks plus, where it was made, the prefill GEMM's own copy."""
+        return int(self.ctx._lib.wick_rocm_weight_device_bytes(self.handle))
+
     def free(self) -> None:
         if self.handle:
             self.ctx._check(self.ctx._lib.wick_rocm_weight_free(self.ctx._h, self.handle))
@@ -236,6 +243,10 @@ class RocmContext:
     def set_gemv_policy(self, direct_max_bytes: int = -1) -> None:
         """Weight-fetch threshold of the n = 1 GEMV (negative = default); results do not depend on it."""
         self._check(self._lib.wick_rocm_set_gemv_policy(self._h, direct_max_bytes))
+
+    def set_gemm_packing(self, enabled: bool) -> None:
+        """Whether upload_weight also makes the prefill GEMM's own copy of a Q4_0 / Q8_0 weight (default: yes)."""
+        self._check(self._lib.wick_rocm_set_gemm_packing(self._h, 1 if enabled else 0))
 
     def set_gemm_min_n(self, min_n: int) -> None:
         self._check(self._lib.wick_rocm_set_gemm_min_n(self._h, min_n))
