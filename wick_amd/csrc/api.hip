@@ -312,8 +312,13 @@ int wick_rocm_weight_upload(wick_rocm_ctx* ctx, const void* host_blocks, size_t 
     if (e == hipSuccess && ctx->gemm_packing && ggml_type != kTypeQ6_K && k % 128u == 0) {
         w->gemm_bytes = gemm_packed_bytes(m, k);
         e = hipMalloc(&w->d_gemm, w->gemm_bytes);
-        if (e == hipSuccess)
+        if (e == hipErrorOutOfMemory) {  // no room for the second layout: the weight works without it (GEMV route for any n)
+            (void)hipGetLastError();
+            w->d_gemm = nullptr, w->gemm_bytes = 0;
+            e = hipSuccess;
+        } else if (e == hipSuccess) {
             e = launch_gemm_pack(ggml_type, static_cast<const uint8_t*>(w->d), m, k, static_cast<uint8_t*>(w->d_gemm), ctx->launch());
+        }
     }
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
