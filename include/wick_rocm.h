@@ -186,7 +186,8 @@ int wick_rocm_gemm_q8_residual_rmsnorm_quantize(wick_rocm_ctx *ctx, const wick_r
  * contiguous 5 KB slab per granule and 128 K-elements; 1.25 bytes per weight), so that a stage of weights reaches the matrix
  * cores' operand buffer with plain coalesced copies and no unpacking in the main loop.  Results do not depend on it (same
  * integers, same scales).  enabled = 0 switches the copy off for weights uploaded from then on: they take the multi-token GEMV
- * route for any n (slower prompts, 1.25 bytes per weight less memory).  wick_rocm_weight_device_bytes: what a weight holds on
+ * route for any n (slower prompts, 1.25 bytes per weight less memory); so does a weight for whose copy the device had no memory
+ * left at upload.  wick_rocm_weight_device_bytes: what a weight holds on
  * the device, both copies.  No counterpart in the reference (its GPU GEMM reads the raw blocks). */
 int wick_rocm_set_gemm_packing(wick_rocm_ctx *ctx, int enabled);
 size_t wick_rocm_weight_device_bytes(const wick_rocm_weight *w);
