@@ -221,6 +221,36 @@ def test_prefill_matches_the_oracle(ctx, oracle, tmp_path, name, n):
     model.free()
 
 
+def test_model_without_the_gemm_copies(ctx, oracle, tmp_path):
+    """A model loaded with wick_rocm_set_gemm_packing(0) keeps the raw blocks only: its prompt pass runs the projections as
+    multi-token GEMVs (and the unfused gate / up + SiLU path) and still meets the oracle; it holds less device memory."""
+    kw = CLEAR["q4_0+q6k"]
+    packed, ref, cfg = load(ctx, oracle, tmp_path, context=256, **kw)
+    ctx.set_gemm_packing(False)
+    try:
+        plain, _, _ = load(ctx, oracle, tmp_path, context=256, **kw)
+    finally:
+        ctx.set_gemm_packing(True)
+    assert plain.gpu_memory_bytes() < packed.gpu_memory_bytes()
+    for n in (24, 150):
+        tokens = np.random.default_rng(70 + n).integers(0, cfg["vocab_size"], n)
+        state = ref.new_state()
+        want = oracle_prompt(ref, tokens, state)
+        for model in (packed, plain):
+            model.reset()
+            got = model.forward_prefill(tokens, 0)
+            check_step(got, want, ref.min_margin, f"prompt of {n}")
+            assert cosine(got, want) >= 0.9999
+            check_step(model.forward(3, n), ref.forward(3, n, ref_copy(ref, state)), ref.min_margin, "step after the prompt")
+    packed.free(), plain.free()
+
+
+def ref_copy(ref, state):
+    """A copy of an oracle state (the same position is stepped from twice above)."""
+    import copy
+    return copy.deepcopy(state)
+
+
 def test_prefill_in_pieces_and_against_single_steps(ctx, oracle, tmp_path):
     model, ref, cfg = load(ctx, oracle, tmp_path, **CLEAR["q4_0+q6k"])
     tokens = np.random.default_rng(3).integers(0, cfg["vocab_size"], 30)
