@@ -97,6 +97,8 @@ public:
         return v;
     }
     void sync() { check(wick_rocm_sync(ctx_)); }
+    // whether upload_weight / weight_from_gguf also make the prefill GEMM's own layout of a Q4_0 / Q8_0 weight (default: yes)
+    void set_gemm_packing(bool enabled) { check(wick_rocm_set_gemm_packing(ctx_, enabled ? 1 : 0)); }
 
     RocmWeight upload_weight(const void* blocks, size_t nbytes, DType dtype, uint32_t m, uint32_t k) {
         RocmWeight w;
