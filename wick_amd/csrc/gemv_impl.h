@@ -575,12 +575,15 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
     const uint32_t waves = set_wave_ends(a);
     const dim3 grid = FUSEQ ? dim3((waves + kFusedWaves - 1) / kFusedWaves, 1) : dim3(waves, (a.n + NT - 1) / NT);
     const dim3 block(FUSEQ ? 64 * kFusedWaves : 64);
-    // Several tokens re-read the weights: only single-token launches stream them.
     const uint64_t bytes = (uint64_t)total_rows * (a.k >> 5) * (TYPE == 2 ? 18u : 34u) * (a.gated ? 2u : 1u);
     constexpr int kSmall = TYPE == 2 ? kDirectNT : kDirect;
     const uint64_t direct_max = L.gemv_direct_max_bytes >= 0 ? (uint64_t)L.gemv_direct_max_bytes : (TYPE == 2 ? kDirectMaxBytesQ4 : kDirectMaxBytesQ8);
-    const int mode = NT > 1 ? kDirect : (bytes < direct_max ? kSmall : kSpan);
     const bool multi = a.batch.count > 1;
+    // Several token groups re-read the weights (they should stay cached): only launches of ONE group -- a single token, or up
+    // to NT tokens of one Q8_0 weight -- stream them with whole-line nontemporal span loads (Q8_0 65536 x 2048 over four tokens:
+    // 34.7 -> 29.5 us; a Q4_0 lane's 36 bytes are three loads either way and the span form is 3 % slower there).
+    const bool one_group = NT == 1 || (TYPE == 8 && a.n <= (uint32_t)NT && !multi);
+    const int mode = !one_group ? kDirect : (bytes < direct_max ? (NT > 1 ? kDirect : kSmall) : kSpan);
     // hot scalars first (preloaded into SGPRs), then the whole argument block
     auto go = [&](auto kernel) {
         return launch_kernel(L, kFamGemv, kernel, grid, block, FUSEQ ? static_cast<const void*>(a.xf) : static_cast<const void*>(a.xq),
@@ -591,6 +594,7 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
             if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan, kXformNone, false, true>);
             return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall, kXformNone, false, true>);
         } else {
+            if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan, kXformNone, false, true>);
             return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kDirect, kXformNone, false, true>);
         }
     } else if constexpr (NT == 1 && FUSEQ) {
@@ -632,6 +636,7 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
         return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall>);
     } else {
         if (multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kDirect>);
+        if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan>);
         return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kDirect>);
     }
 }
