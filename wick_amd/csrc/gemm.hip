@@ -594,7 +594,9 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
 // row tile x four token tiles), so no matrix or scaling work is spent on token columns that
 // do not exist beyond the 64, and the weights -- the only large operand -- are streamed
 // exactly once.  Same staging, LDS layouts and arithmetic as the wide kernel; 60 KB of LDS,
-// two workgroups per CU.
+// two workgroups per CU.  TTN (1 .. 4): how many of the four token tiles the launch has tokens
+// for -- a launch of n <= 16 / 32 / 48 tokens reads and multiplies only those (these launches
+// are bound by their block loop, so the unused tiles were a third to three quarters of their time).
 struct NarrowMats {
     long av[4], bv;
 };
@@ -603,19 +605,22 @@ struct NarrowScales {
     v4f dx[4];
 };
 constexpr int kOffDxfNarrow = sizeof(float) * BN_NARROW;
-__device__ __forceinline__ void load_mats(const LaneAddr& la, NarrowMats& m) {  // 5 reads
+// TTN: the token tiles (of 16) the launch has tokens for; the others are neither read nor multiplied.
+template <int TTN>
+__device__ __forceinline__ void load_mats(const LaneAddr& la, NarrowMats& m) {  // TTN + 1 reads
     lds_read8<0 * 16 * 128>(la.xt, m.av[0]);
-    lds_read8<1 * 16 * 128>(la.xt, m.av[1]);
-    lds_read8<2 * 16 * 128>(la.xt, m.av[2]);
-    lds_read8<3 * 16 * 128>(la.xt, m.av[3]);
+    if constexpr (TTN > 1) lds_read8<1 * 16 * 128>(la.xt, m.av[1]);
+    if constexpr (TTN > 2) lds_read8<2 * 16 * 128>(la.xt, m.av[2]);
+    if constexpr (TTN > 3) lds_read8<3 * 16 * 128>(la.xt, m.av[3]);
     lds_read8<0>(la.wt, m.bv);
 }
-__device__ __forceinline__ void load_scales(const LaneAddr& la, NarrowScales& s) {  // 5 reads
+template <int TTN>
+__device__ __forceinline__ void load_scales(const LaneAddr& la, NarrowScales& s) {  // TTN + 1 reads
     lds_read8<0>(la.dws, s.dw);
     lds_read16<0 * 64>(la.dxf, s.dx[0]);
-    lds_read16<1 * 64>(la.dxf, s.dx[1]);
-    lds_read16<2 * 64>(la.dxf, s.dx[2]);
-    lds_read16<3 * 64>(la.dxf, s.dx[3]);
+    if constexpr (TTN > 1) lds_read16<1 * 64>(la.dxf, s.dx[1]);
+    if constexpr (TTN > 2) lds_read16<2 * 64>(la.dxf, s.dx[2]);
+    if constexpr (TTN > 3) lds_read16<3 * 64>(la.dxf, s.dx[3]);
 }
 template <int N>
 __device__ __forceinline__ void lds_wait(NarrowMats& m) {
@@ -626,7 +631,7 @@ __device__ __forceinline__ void lds_wait(NarrowScales& s) {
     asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(s.dw), "+v"(s.dx[0]), "+v"(s.dx[1]), "+v"(s.dx[2]), "+v"(s.dx[3]) : "n"(N) : "memory");
 }
 
-template <int TYPE, bool DUMP>
+template <int TYPE, bool DUMP, int TTN = 4>
 __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     __shared__ SmemT<BN_NARROW> sm;
     uint32_t row_tile, tok_tile;
@@ -686,10 +691,10 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
             load_stage(ptrs, regs);
         }
 
-        NarrowMats mt;
-        NarrowScales sc;
-        load_mats(la, mt);    // 5 reads
-        load_scales(la, sc);  // 5 reads
+        NarrowMats mt{};
+        NarrowScales sc{};
+        load_mats<TTN>(la, mt);    // TTN + 1 reads
+        load_scales<TTN>(la, sc);  // TTN + 1 reads
 #pragma unroll 1
         for (int b = 0; b < KB; b++) {
             // addresses of block b+1 (last iteration: harmless re-read of its own block)
@@ -699,20 +704,20 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
             la.dws += adv ? kOffDws : 0;
             la.dxf += adv ? kOffDxfNarrow : 0;
             const uint32_t row = row0 + wrow0 + l16, tok = tok0 + 4 * kq, blk = (first + st) * KB + b;
-            v4i d[4];
-            lds_wait<5>(mt);  // the five scale reads issued after the matrices may still be in flight
+            v4i d[TTN];
+            lds_wait<TTN + 1>(mt);  // the scale reads issued after the matrices may still be in flight
 #pragma unroll
-            for (int tt = 0; tt < 4; tt++) d[tt] = __builtin_amdgcn_mfma_i32_16x16x32_i8(mt.av[tt], mt.bv, cbias, 0, 0, 0);
-            load_mats(la, mt);  // in place: the MFMAs that read block b's operands have been issued
-            lds_wait<5>(sc);
+            for (int tt = 0; tt < TTN; tt++) d[tt] = __builtin_amdgcn_mfma_i32_16x16x32_i8(mt.av[tt], mt.bv, cbias, 0, 0, 0);
+            load_mats<TTN>(la, mt);  // in place: the MFMAs that read block b's operands have been issued
+            lds_wait<TTN + 1>(sc);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int tt = 0; tt < 4; tt++) {
+            for (int tt = 0; tt < TTN; tt++) {
                 if constexpr (DUMP) dump_tile<TYPE>(a, d[tt], row, tok + 16 * tt, nb, blk);
                 else scale_tile(d[tt], sc.dw, sc.dx[tt], acc[tt]);
             }
             __builtin_amdgcn_sched_barrier(0);
-            load_scales(la, sc);
+            load_scales<TTN>(la, sc);
         }
         lds_wait<0>(sc);  // nothing of this stage's buffer is read past this point
         {
@@ -732,7 +737,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     if constexpr (!DUMP) {
         const uint32_t row = row0 + wrow0 + l16;
 #pragma unroll
-        for (int tt = 0; tt < 4; tt++)
+        for (int tt = 0; tt < TTN; tt++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const uint32_t tok = tok0 + 16 * tt + 4 * kq + r;
@@ -825,15 +830,25 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0, boo
     const uint32_t tiles = a.row_tiles * a.tok_tiles;
     const uint32_t blocks = ((tiles + 7u) / 8u) * 8u;  // every XCD gets the same number of slots
     if (narrow) {
+        // a launch of at most 16 / 32 / 48 tokens computes one / two / three of the tile's four 16-token MFMA tiles (the parity
+        // hook: all four).  These launches are bound by their block loop, not by memory: 65536 x 16 x 2048 40 -> 34 us.
+        const auto narrow_launch = [&](uint32_t grid) {
+            if constexpr (!DUMP) {
+                if (a.n <= 16) return launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, false, 1>, dim3(grid), dim3(THREADS), a);
+                if (a.n <= 32) return launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, false, 2>, dim3(grid), dim3(THREADS), a);
+                if (a.n <= 48) return launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, false, 3>, dim3(grid), dim3(THREADS), a);
+            }
+            // (the product kernels do not depend on the weight type any more: the copy they read is the same for both)
+            return type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(grid), dim3(THREADS), a)
+                                     : launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(grid), dim3(THREADS), a);
+        };
         if (!DUMP && a.ksplit > 1) {
-            const uint32_t split_blocks = blocks * a.ksplit;  // tile id = blockIdx.x / ksplit must run over all `blocks` slots of the tile map
-            hipError_t e = type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(split_blocks), dim3(THREADS), a)
-                                             : launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(split_blocks), dim3(THREADS), a);
+            // tile id = blockIdx.x / ksplit must run over all `blocks` slots of the tile map
+            hipError_t e = narrow_launch(blocks * a.ksplit);
             if (e != hipSuccess || defer_reduce) return e;  // deferred: the caller's next kernel adds the shares up itself
             return launch_reduce(a, L);
         }
-        if (type == kTypeQ4_0) return launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
-        return launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
+        return narrow_launch(blocks);
     }
     if (wide_split) {
         hipError_t e = type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, DUMP>, dim3(blocks * a.ksplit), dim3(THREADS), a)
