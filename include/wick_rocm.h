@@ -22,7 +22,9 @@
  *     GPU models' `infer_lock` (wick/src/model/metal_lfm2.rs:254-267).
  *   - Weight bytes keep the GGUF block layout verbatim (wick/src/quant.rs:13-34):
  *     row-major, m rows of k/32 blocks; Q4_0 block = {f16 d; u8 qs[16]} (18 B),
- *     Q8_0 block = {f16 d; i8 qs[32]} (34 B).  Nothing is repacked.
+ *     Q8_0 block = {f16 d; i8 qs[32]} (34 B).  That is what is uploaded and what the decode
+ *     GEMVs read; the prefill GEMM reads a second layout of the same values that the library
+ *     derives on the device at upload (wick_rocm_set_gemm_packing).
  *   - Q6_K weights (wick/src/quant.rs:54-70: {u8 ql[128]; u8 qh[64]; i8 scales[16];
  *     f16 d}, 210 B per 256 weights, k % 256 == 0, k <= 8192) take the decode path
  *     only: the integer Q6_K x Q8_0 GEMV of wick/src/backend/simd.rs:547-640
