@@ -96,6 +96,30 @@ def test_accumulate(ctx, oracle, dtype, n):
         assert_f32_parity(fetch_gemm(d_y, m, n, m, W.LAYOUT_TOKEN_MAJOR), ref, "gemm accumulate")
 
 
+def test_weight_free_releases_both_copies(ctx, oracle):
+    """Uploading and freeing a weight over and over leaves the device's free memory where it was: the raw blocks and the
+    GEMM's copy both go (read through hipMemGetInfo of the HIP runtime the library itself is linked against)."""
+    import ctypes
+
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+
+    def free_bytes():
+        ctx.sync()
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    m, k = 16384, 2048  # 36 MB of Q8_0 blocks + 42 MB of slabs
+    wb = np.tile(oracle.synth_weight(W.Q8_0, 256, k, 9, 0.02), m // 256)
+    ctx.upload_weight(wb, W.Q8_0, m, k).free()  # the runtime's own pools settle on the first round
+    before = free_bytes()
+    for _ in range(12):
+        w = ctx.upload_weight(wb, W.Q8_0, m, k)
+        assert w.device_bytes > 2 * 36_000_000
+        w.free()
+    assert abs(before - free_bytes()) <= 8 << 20
+
+
 def test_weights_without_the_gemm_copy_take_the_gemv_route(ctx, oracle):
     """wick_rocm_set_gemm_packing(0): weights uploaded from then on hold the raw blocks only (no second layout for the
     matrix-core kernel) and run as multi-token GEMVs for any n -- same block dots bit for bit, f32 results to the bar."""
