@@ -602,7 +602,7 @@ def bench_lm_head_sweep(ctx, W, O, dtype=8, m=65536, k=2048, ns=(1, 4, 16, 64)):
         w.free()
     d_q.free(), d_s.free(), d_y.free()
     crossover = next((r["n"] for r in rows if "mfma" in r and r["mfma"]["us"] < r["gemv"]["us"]), None)
-    return {"dtype": dtype, "m": m, "k": k, "rows": rows, "first_n_where_mfma_wins": crossover, "library_hand_off_n": W.GEMM_MIN_N}
+    return {"dtype": dtype, "m": m, "k": k, "rows": rows, "first_n_where_mfma_wins": crossover, "library_hand_off_n": W.GEMM_MIN_N_LARGE if m * (k // 32) * 34 >= (16 << 20) else W.GEMM_MIN_N}
 
 
 def bench_probe(ctx, iters=20000):

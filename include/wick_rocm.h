@@ -195,9 +195,11 @@ int wick_rocm_set_gemm_packing(wick_rocm_ctx *ctx, int enabled);
 size_t wick_rocm_weight_device_bytes(const wick_rocm_weight *w);
 
 /* The n at and above which wick_rocm_gemm_q8 / wick_rocm_matmul_f32 hand off from the
- * multi-token GEMV to the MFMA GEMM (default 16, the reference's GEMM_MIN_N,
- * wick/src/model/metal_lfm2.rs:18-21); 0 restores the default.  A tuning knob, like
- * the reference's WICK_Q4_FAST / WICK_SPLITS switches (wick/src/backend/cpu.rs:23-27). */
+ * multi-token GEMV to the MFMA GEMM: the counterpart of the reference's GEMM_MIN_N = 16
+ * (wick/src/model/metal_lfm2.rs:18-21).  Default (min_n = 0): where the two routes cross on
+ * this GPU, per weight -- 9, and 5 for weights of 16 MB and more (an LM head).  Results agree
+ * to the f32 bar on either side.  A tuning knob, like the reference's WICK_Q4_FAST /
+ * WICK_SPLITS switches (wick/src/backend/cpu.rs:23-27). */
 int wick_rocm_set_gemm_min_n(wick_rocm_ctx *ctx, uint32_t min_n);
 
 /* A GEMM launch that would leave at least half of the CUs without a tile while walking a long K (few tokens x few rows x

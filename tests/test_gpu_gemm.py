@@ -1,5 +1,5 @@
 """Batched prefill GEMM on the GPU against the oracle, both output layouts, both
-kernel paths (multi-token GEMV below GEMM_MIN_N or when k % 256 != 0; int8 MFMA
+kernel paths (multi-token GEMV below the hand-off n or when k % 128 != 0; int8 MFMA
 otherwise).  Block dots BIT-EXACT, f32 within rel-L2 1e-5 / max-abs 1e-4 x RMS."""
 import numpy as np
 import pytest

@@ -8,6 +8,7 @@ mirror of the reference's call sites used by the tests and the benchmark.
 from . import build as build  # noqa: F401
 from .rocm import (  # noqa: F401
     GEMM_MIN_N,
+    GEMM_MIN_N_LARGE,
     LAYOUT_ROW_MAJOR,
     LAYOUT_TOKEN_MAJOR,
     Q4_0,

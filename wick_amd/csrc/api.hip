@@ -84,7 +84,7 @@ int gemm_locked(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const int8_t* d_q
     const bool mfma_ok = w->d_gemm && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_q) % 16u == 0) &&
                          (reinterpret_cast<uintptr_t>(d_s) % 16u == 0);
     hipError_t e;
-    if (n >= ctx->gemm_min_n && mfma_ok) {
+    if (n >= ctx->min_n_for(w->nbytes) && mfma_ok) {
         uint32_t splits = may_split && ctx->gemm_max_splits > 1 ? gemm_split_k(w->m, n, w->k, ctx->gemm_max_splits) : 1u;
         if (splits > 1) {
             const size_t floats = (size_t)splits * n * w->m;
@@ -271,7 +271,7 @@ size_t wick_rocm_weight_device_bytes(const wick_rocm_weight* w) { return w ? w->
 
 int wick_rocm_set_gemm_min_n(wick_rocm_ctx* ctx, uint32_t min_n) {
     WR_ENTER(ctx);
-    ctx->gemm_min_n = min_n == 0 ? kGemmMinN : min_n;
+    ctx->gemm_min_n = min_n;  // 0: back to the per-weight default
     return WICK_ROCM_OK;
 }
 
@@ -652,7 +652,9 @@ int wick_rocm_gemm_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* w
     const wick_rocm_weight* w0 = ws[0];
     bool packed = true;
     for (uint32_t i = 0; i < count; i++) packed = packed && ws[i]->d_gemm != nullptr;
-    const bool one_launch = count > 1 && packed && w0->type != kTypeQ6_K && n >= ctx->gemm_min_n && w0->k % 128u == 0 && d_quants && d_scales &&
+    size_t bytes = 0;  // the launch streams all of them
+    for (uint32_t i = 0; i < count; i++) bytes += ws[i]->nbytes;
+    const bool one_launch = count > 1 && packed && w0->type != kTypeQ6_K && n >= ctx->min_n_for(bytes) && w0->k % 128u == 0 && d_quants && d_scales &&
                             reinterpret_cast<uintptr_t>(d_quants) % 16u == 0 && reinterpret_cast<uintptr_t>(d_scales) % 16u == 0;
     if (!one_launch) {  // shapes without a batched launch: one call per weight, same results
         for (uint32_t i = 0; i < count; i++)
@@ -741,7 +743,7 @@ int wick_rocm_block_dots_i32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, cons
         }
         return WICK_ROCM_OK;
     }
-    const bool mfma = w->d_gemm && n >= ctx->gemm_min_n && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
+    const bool mfma = w->d_gemm && n >= ctx->min_n_for(w->nbytes) && (w->k % 128u == 0) && (reinterpret_cast<uintptr_t>(d_quants) % 16u == 0);
     hipError_t e = mfma ? launch_block_dots_mfma(w->type, static_cast<const uint8_t*>(w->d_gemm), w->m, w->k, d_quants, n, d_out, ctx->launch())
                         : launch_block_dots_gemv(w->type, static_cast<const uint8_t*>(w->d), w->m, w->k, d_quants, n, d_out, ctx->num_cus, ctx->launch());
     if (e != hipSuccess) return fail_hip(ctx, e, "block_dots launch");

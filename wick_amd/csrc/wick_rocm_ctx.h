@@ -33,7 +33,10 @@ struct wick_rocm_ctx {
     uint64_t scratch_gen = 0;
     bool capture_used_scratch = false;
     unsigned char* noalloc_scratch = nullptr;  // this device's address of the static scratch array of wick_rocm_matmul_f32_noalloc
-    uint32_t gemm_min_n = kGemmMinN;  // hand-off from the multi-token GEMV to the MFMA GEMM
+    uint32_t gemm_min_n = 0;  // hand-off from the multi-token GEMV to the MFMA GEMM; 0: the per-weight default (min_n_for)
+    uint32_t min_n_for(size_t weight_bytes) const {
+        return gemm_min_n ? gemm_min_n : (weight_bytes >= kGemmLargeWeightBytes ? kGemmMinNLarge : kGemmMinN);
+    }
     bool gemm_packing = true;         // weight_upload also makes the GEMM's own copy of a Q4_0 / Q8_0 weight
     uint32_t gemm_max_splits = kGemmMaxSplits;  // K split of GEMM launches with few tiles (1: off)
     KernelTimer timer;

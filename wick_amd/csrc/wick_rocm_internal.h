@@ -233,8 +233,15 @@ hipError_t launch_set_step(uint32_t* d_token, uint32_t token, uint32_t* d_pos, u
                            int embd_type = 0, uint32_t embd_m = 0, uint32_t embd_k = 0, float* d_embd_out = nullptr);
 hipError_t launch_advance_pos(uint32_t* d_pos, const Launch& L);
 
-// n at and above which gemm_q8 uses the MFMA kernel (when k % 128 == 0).
-constexpr uint32_t kGemmMinN = 16;  // cf. GEMM_MIN_N, wick/src/model/metal_lfm2.rs:18-21
+// n at and above which gemm_q8 uses the MFMA kernel (when k % 128 == 0): the counterpart of GEMM_MIN_N = 16
+// (wick/src/model/metal_lfm2.rs:18-21), set where the two routes cross on this GPU.  The multi-token GEMV streams the weight
+// once per group of four tokens; the narrow MFMA kernel streams it once and computes 16 token columns at a time.  A 1024 x 1024
+// projection inside a prompt pass: up to two groups (n <= 8) the GEMV wins, from n = 9 the MFMA kernel (passes of 12 / 15 tokens
+// 0.98 / 1.07 -> 0.89 ms).  A weight whose stream is what a launch costs (16 MB and more: an LM head): one group 29 us, two 58 us,
+// the MFMA kernel 34 us for any n <= 16, so it takes over from n = 5.
+constexpr uint32_t kGemmMinN = 9;
+constexpr uint32_t kGemmMinNLarge = 5;
+constexpr size_t kGemmLargeWeightBytes = 16u << 20;
 constexpr uint32_t kGemmMaxSplits = 8;  // most K shares of a GEMM launch with few tiles
 
 }  // namespace wick_rocm

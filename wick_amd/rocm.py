@@ -29,7 +29,8 @@ Q6_K = 14  # decode GEMV only; 210-byte blocks of 256 weights (wick/src/quant.rs
 BLOCK_BYTES = {Q4_0: 18, Q8_0: 34}
 LAYOUT_TOKEN_MAJOR = 0
 LAYOUT_ROW_MAJOR = 1
-GEMM_MIN_N = 16  # hand-off from the multi-token GEMV to the MFMA GEMM
+GEMM_MIN_N = 9  # default hand-off from the multi-token GEMV to the MFMA GEMM ...
+GEMM_MIN_N_LARGE = 5  # ... and for weights of 16 MB and more (the reference's GEMM_MIN_N for its Metal path is 16)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libwick_rocm.so")
