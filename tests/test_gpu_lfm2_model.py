@@ -204,9 +204,10 @@ def oracle_prompt(ref, tokens, state, start=0):
     return logits
 
 
-@pytest.mark.parametrize("name,n", [("q4_0+q6k", 5), ("q4_0+q6k", 24), ("q8_0", 17), ("kernel4", 33), ("kernel4", 2), ("mixed-qkv", 16), ("3-layer-q4embd", 40)])
+@pytest.mark.parametrize("name,n", [("q4_0+q6k", 1), ("q8_0", 3), ("q4_0+q6k", 5), ("q4_0+q6k", 11), ("q4_0+q6k", 24), ("q8_0", 17), ("kernel4", 33), ("kernel4", 2), ("mixed-qkv", 16), ("3-layer-q4embd", 40)])
 def test_prefill_matches_the_oracle(ctx, oracle, tmp_path, name, n):
-    """Short prompts (n <= 8) run the projections as multi-token GEMVs, longer ones on the int8-MFMA GEMM."""
+    """One or two tokens run as single steps, up to eight with the projections as multi-token GEMVs, longer prompts on the
+    int8-MFMA GEMM."""
     kw = CLEAR[name]
     model, ref, cfg = load(ctx, oracle, tmp_path, **kw)
     tokens = np.random.default_rng(7 + n).integers(0, cfg["vocab_size"], n)

@@ -206,7 +206,7 @@ def test_embedding_input_steps(ctx, oracle, tmp_path, name):
     model.free()
 
 
-@pytest.mark.parametrize("name,n", [("q4_0+q6k", 24), ("q8_0", 5)])
+@pytest.mark.parametrize("name,n", [("q4_0+q6k", 24), ("q8_0", 5), ("q4_0+q6k", 2), ("q8_0", 1)])
 def test_prefill_from_embeddings(ctx, oracle, tmp_path, name, n):
     """forward_prefill_from_embeddings (wick/src/model/lfm2.rs:2452-2487): the tokens' own rows give the token prompt bit for bit;
     arbitrary frames follow the oracle's frame-by-frame forward_from_embedding (the trait's default, wick/src/model/mod.rs:241-268)."""
