@@ -188,12 +188,43 @@ def bench_c1(ctx, W, O, steps, warmup, with_concurrent=True):
     b = gemv_bytes(dtype, m, k)
     res = {"m": m, "k": k, "dtype": dtype, "bytes_per_launch": b, "weight_copies": copies, "launches_per_step": copies, "ms_per_step": ms_step,
            "per_launch_in_graph": stats(each, copies), "GBps": b * copies / ms_step / 1e6}
+    res["kernel_span"] = bench_c1_span(ctx, W, ws, d_q, d_s, d_y, m, steps=min(steps, 20), warmup=warmup)
     if with_concurrent:
         res["concurrent"] = bench_c1_concurrent(ctx, W, ws, d_q, d_s, b, m)
     for w in ws:
         w.free()
     d_q.free(), d_s.free(), d_y.free()
     return res
+
+
+def bench_c1_span(ctx, W, ws, d_q, d_s, d_y, m, steps, warmup):
+    """Execution span of the GEMV launches INSIDE a graph replay: the same chain of launches through the product kernel with its
+    timing hook (two reads of the 100 MHz wall clock per wave, libwick_rocm_bench.so); span of a launch = first wave's first
+    instruction -> last wave's last store acknowledged.  A kernel tracer cannot give this figure (it splits a replay into single
+    dispatches and inflates each); per-dispatch events cannot either (graph nodes carry none)."""
+    from wick_amd import benchlib as B
+
+    spans = [ctx.alloc(m * 16) for _ in ws]
+    ctx.graph_begin()
+    waves = [B.gemv_q8_span(ctx, w, d_s, d_q, d_y, sp, m) for w, sp in zip(ws, spans)]
+    g = ctx.graph_end()
+    ms_step, _ = time_graph_steps(ctx, [g], steps, warmup)
+    per_launch, gaps = [], []
+    for _ in range(3):  # three more replays, each read back
+        ctx.graph_launch(g)
+        ctx.sync()
+        rec = [sp.download(np.uint64, 2 * nw).reshape(nw, 2) for sp, nw in zip(spans, waves)]
+        per_launch += [B.span_us(r) for r in rec]
+        starts, ends = [int(r[:, 0].min()) for r in rec], [int(r[:, 1].max()) for r in rec]
+        gaps += [(starts[i + 1] - ends[i]) / 100.0 for i in range(len(rec) - 1)]
+    ctx.graph_destroy(g)
+    for sp in spans:
+        sp.free()
+    a, gp = np.asarray(per_launch), np.asarray(gaps)
+    return {"launches_per_step": len(ws), "waves_per_launch": waves[0], "span_us_mean": float(a.mean()), "span_us_median": float(np.median(a)),
+            "span_us_min": float(a.min()), "span_us_p90": float(np.percentile(a, 90)), "samples": int(a.size),
+            "gap_to_next_launch_us_mean": float(gp.mean()), "gap_to_next_launch_us_median": float(np.median(gp)),
+            "step_ms_with_hook": ms_step, "sum_of_spans_ms": float(a.mean()) * len(ws) / 1e3, "clock": "100 MHz wall clock (s_memrealtime), 10 ns steps"}
 
 
 def bench_c1_concurrent(ctx, W, ws, d_q, d_s, b, m, streams=4, passes=8, reps=12):
@@ -573,9 +604,10 @@ def bench_gate_up_fused(ctx, W, O, dtype, m, k, n, wg=None, wu=None, reps=5):
     return out
 
 
-def bench_lm_head_sweep(ctx, W, O, dtype=8, m=65536, k=2048, ns=(1, 4, 16, 64)):
+def bench_lm_head_sweep(ctx, W, O, dtype=8, m=65536, k=2048, ns=(1, 4, 5, 6, 8, 12, 16, 64)):
     """Tied LM head: where the bandwidth-bound multi-token GEMV hands off to the MFMA GEMM.
-    Each n is timed through both kernels (hand-off forced), HBM-cold over three weight copies."""
+    Each n is timed through both kernels (hand-off forced), HBM-cold over three weight copies: the configuration's n = 1, 4, 16, 64
+    and the n between 4 and 16 where the routes cross, so that the crossing and the library's own hand-off come from the same data."""
     wb = O.synth_weight(dtype, m, k, seed=999)
     ws = [ctx.upload_weight(wb, dtype, m, k) for _ in range(3)]
     nmax = max(ns)
@@ -607,14 +639,16 @@ def bench_lm_head_sweep(ctx, W, O, dtype=8, m=65536, k=2048, ns=(1, 4, 16, 64)):
 
 def bench_probe(ctx, iters=20000):
     """Register-only ceilings of this GPU for the GEMM's two bounds (no memory traffic)."""
+    from wick_amd import benchlib as B
+
     out = {}
     for shape, name, unit in [(0, "mfma_i32_32x32x32_i8", "TOP/s"), (1, "mfma_i32_16x16x32_i8", "TOP/s"), (2, "v_fma_f32", "TFLOP/s"),
                               (3, "block_loop_8xmfma16_plus_64_scaling_fma", "TOP/s"), (4, "block_loop_2xmfma32_plus_64_scaling_fma", "TOP/s")]:
-        ctx.probe_rate(shape, iters)
+        B.probe_rate(ctx, shape, iters)
         ctx.sync()
         e0, e1 = ctx.event(), ctx.event()
         ctx.record(e0)
-        ops = ctx.probe_rate(shape, iters)
+        ops = B.probe_rate(ctx, shape, iters)
         ctx.record(e1)
         ms = ctx.elapsed_ms(e0, e1)
         ctx.event_destroy(e0), ctx.event_destroy(e1)
@@ -624,13 +658,15 @@ def bench_probe(ctx, iters=20000):
 
 def bench_copy(ctx, nbytes=256 << 20, reps=10):
     """Device-to-device copy of a known size: calibration of the FETCH_SIZE / WRITE_SIZE counters."""
+    from wick_amd import benchlib as B
+
     a, b = ctx.alloc(nbytes), ctx.alloc(nbytes)
-    ctx.copy(b, a, nbytes)
+    B.copy(ctx, b, a, nbytes)
     ctx.sync()
     e0, e1 = ctx.event(), ctx.event()
     ctx.record(e0)
     for _ in range(reps):
-        ctx.copy(b, a, nbytes)
+        B.copy(ctx, b, a, nbytes)
     ctx.record(e1)
     ms = ctx.elapsed_ms(e0, e1) / reps
     a.free(), b.free()
@@ -783,6 +819,34 @@ def main():
     avg_launch_us = c1["ms_per_step"] * 1e3 / c1["launches_per_step"]
     achieved = c1["bytes_per_launch"] / avg_launch_us / 1e3  # GB/s
     c1_profile = "gemv_q4_0_6912x2048_hbm_cold.txt"
+    span = c1["kernel_span"]
+    conc = c1.pop("concurrent", None)
+    roofline = {
+        "bound": "hbm",
+        "kernel": "gemv_pairs_kernel<Q4_0> (pre-quantized activation, span loads)",
+        "achieved": achieved,
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS,
+        "bytes_per_launch": c1["bytes_per_launch"],
+        "avg_launch_us": avg_launch_us,
+        "avg_launch_definition": "timed region / launches in it: kernel execution + the gap to the next dependent launch, an upper bound of the "
+                                 "kernel's own duration",
+        "per_launch": c1["per_launch_in_graph"],
+        "frac_best_step": c1["bytes_per_launch"] / c1["per_launch_in_graph"]["min_us"] / 1e3 / HBM_PEAK_GBS,
+        # the kernel's own execution inside the same chain (first wave's first instruction -> last wave's last store), from the
+        # timing hook: kernel_span_us x launches <= ms_per_step, the rest is the gap between dependent launches
+        "kernel_span_us": span["span_us_mean"],
+        "kernel_span_GBps": c1["bytes_per_launch"] / span["span_us_mean"] / 1e3,
+        "kernel_span_frac": c1["bytes_per_launch"] / span["span_us_mean"] / 1e3 / HBM_PEAK_GBS,
+        "gap_between_dependent_launches_us": span["gap_to_next_launch_us_mean"],
+        # HBM bytes per launch from the copy-calibrated FETCH_SIZE / WRITE_SIZE passes recorded in the profile summary
+        "traffic": profile_figure(c1_profile, "traffic_bytes_per_launch"),
+        "traffic_source": "profiles/" + c1_profile,
+    }
+    if conc:  # the same launches as independent work on four streams
+        roofline["independent_streams_us_per_launch"] = conc["per_launch"]["median_us"]
+        roofline["independent_streams_frac"] = conc["frac_of_hbm_peak_median"]
     out = {
         "metric": "Q4_0 GEMV GB/s (% HBM peak) + prefill int8 GEMM TOPS (% MFMA peak)",
         "value": c1["GBps"],
@@ -803,49 +867,38 @@ def main():
             "device": ctx.device_name,
             "value_definition": "algorithmic GEMV bytes per step (38 x (weights + Q8_0 activation + f32 output) = 38 x 7 992 448 B) / step time",
         },
-        "roofline": {
-            "bound": "hbm",
-            "kernel": "gemv_pairs_kernel<Q4_0> (pre-quantized activation, span loads)",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            "bytes_per_launch": c1["bytes_per_launch"],
-            "avg_launch_us": avg_launch_us,
-            "avg_launch_definition": "timed region / launches in it: kernel execution + the gap to the next dependent launch, an upper bound of the "
-                                     "kernel's own duration (the kernel trace of `bench.py --leg c1` in the profile gives the duration alone)",
-            "per_launch": c1["per_launch_in_graph"],
-            "frac_best_step": c1["bytes_per_launch"] / c1["per_launch_in_graph"]["min_us"] / 1e3 / HBM_PEAK_GBS,
-            # HBM bytes per launch from the copy-calibrated FETCH_SIZE / WRITE_SIZE passes recorded in the profile summary
-            "traffic": profile_figure(c1_profile, "traffic_bytes_per_launch"),
-            "traffic_source": "profiles/" + c1_profile,
-        },
         "gemv_6912x2048": c1,
     }
-    if "concurrent" in c1:
-        out["gemv_concurrent"] = c1.pop("concurrent")
+    if conc:
+        out["gemv_concurrent"] = conc
 
     gemm_profile = "gemm_q4_0_6912x2002x2048.txt"
     g = bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048, samples=100)
-    g["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma_kernel<Q4_0>", "achieved": g["gemm_kernel_TOPS"], "peak": INT8_PEAK_TOPS,
+    g["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma_kernel<Q4_0>", "workload": "prefill GEMM Q4_0 m=6912, n=2002, k=2048 (2 m n k int8 ops per launch)",
+                     "achieved": g["gemm_kernel_TOPS"], "peak": INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": g["gemm_kernel_TOPS"] / INT8_PEAK_TOPS, "frac_median": g["gemm_kernel_TOPS_median"] / INT8_PEAK_TOPS,
                      "frac_best": g["gemm_kernel_TOPS_best"] / INT8_PEAK_TOPS, "avg_launch_us": g["gemm_kernel_ms"] * 1e3,
                      "traffic": profile_figure(gemm_profile, "traffic_bytes_per_launch"), "traffic_source": "profiles/" + gemm_profile}
     out["gemm"] = g
+    roofline["gemm"] = g["roofline"]  # the matrix-core half of the metric, inside the object the record keeps
 
     if not args.skip_extra:
         out["measured_ceilings"] = bench_probe(ctx)
         g["roofline"]["frac_of_measured_block_loop_ceiling"] = g["gemm_kernel_TOPS"] / out["measured_ceilings"]["block_loop_2xmfma32_plus_64_scaling_fma"]["value"]
+        roofline["lm_head_first_n_where_mfma_wins"] = None  # filled below from the sweep
         dec = bench_decode(ctx, W, O, W.Q4_0, 50, args.warmup, synth_decode_weights(O, W.Q4_0))
         out["decode_step"] = dec
         dq = bench_decode(ctx, W, O, W.Q8_0, 25, args.warmup, synth_decode_weights(O, W.Q8_0), with_unfused=False)
         out["decode_step_q8_0"] = dq
         out["prefill_sites"] = bench_prefill_sites(ctx, W, O)
         out["lm_head_sweep"] = bench_lm_head_sweep(ctx, W, O)
+        roofline["lm_head_first_n_where_mfma_wins"] = out["lm_head_sweep"]["first_n_where_mfma_wins"]
+        roofline["lm_head_library_hand_off_n"] = out["lm_head_sweep"]["library_hand_off_n"]
         # shipped LFM2 Q4_0 files keep the tied embedding / LM head in Q6_K (wick/src/model/metal_lfm2.rs:175-180)
         out["lm_head_q6_k_65536x1024"] = bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024)
         out["lfm2_decode_step"] = bench_lfm2_step(ctx, W, O)
     ctx.close()
+    out["roofline"] = roofline  # (last, with cpu_baseline: the end of the line is what a truncated log still shows)
     if not args.skip_cpu:
         out["cpu_baseline"] = cpu_baseline(O, W)
     print(json.dumps(out))

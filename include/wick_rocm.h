@@ -95,20 +95,6 @@ int wick_rocm_buffer_free(wick_rocm_ctx *ctx, void *d_ptr);
 int wick_rocm_upload(wick_rocm_ctx *ctx, void *d_dst, const void *src, size_t nbytes);   /* H2D, ordered on the stream */
 int wick_rocm_download(wick_rocm_ctx *ctx, void *dst, const void *d_src, size_t nbytes); /* D2H, waits for the stream */
 int wick_rocm_sync(wick_rocm_ctx *ctx);
-/* Measurement aid with no counterpart in the reference: enqueues a register-only kernel that
- * does nothing but issue one instruction (shape 0 = v_mfma_i32_32x32x32_i8, 1 =
- * v_mfma_i32_16x16x32_i8, 2 = v_fma_f32) `iters` x 4 times per wave on every SIMD, and returns
- * the number of operations it performs (int8 ops / flops).  Shapes 3 and 4 run the GEMM's whole block
- * loop from registers instead: per iteration and wave one 32-element block of a 64 x 32 tile = 8
- * v_mfma_i32_16x16x32_i8 (3) or 2 v_mfma_i32_32x32x32_i8 (4) plus the two scaling FMAs of each of the
- * 32 results per lane, at the GEMM's occupancy (131072 int8 ops per wave and iteration).  Timed by the
- * caller (events or kernel timing, family 3), they give this GPU's own ceilings for the prefill GEMM. */
-int wick_rocm_probe_rate(wick_rocm_ctx *ctx, int shape, uint32_t iters, double *ops);
-
-/* Device-to-device copy enqueued on the context's stream (the counterpart of a Metal
- * blit between the reference's scratch buffers). */
-int wick_rocm_copy(wick_rocm_ctx *ctx, void *d_dst, const void *d_src, size_t nbytes);
-
 /* ---- weights ----------------------------------------------------------------
  * Stands in for MetalWeight {mmap_offset, dtype, m, k} (wick/src/model/metal_lfm2.rs:28-36,
  * 409-421).  A discrete GPU cannot wrap the GGUF mmap in place, so the block
@@ -227,15 +213,21 @@ int wick_rocm_matmul_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const fl
                          uint32_t x_stride, float *d_y, size_t y_off_bytes, uint32_t y_stride, int accumulate);
 /* wick_rocm_matmul_f32 for callers that cannot allocate.  It has no counterpart in the reference; it exists for callers
  * that must not reach hipMalloc / hipFree: code running under HIP graph capture, tight serving loops, harnesses that
- * forbid allocation.  Same arguments, same kernels and bit-identical results, but the Q8_0-quantized activations go
- * into a fixed array in device memory that is part of the library's image (4.5 MiB per GPU, held until the process
- * ends) instead of context scratch that grows on demand.  Limits and rules:
+ * forbid allocation.  Same arguments and same kernels, but the Q8_0-quantized activations go into a fixed array in device
+ * memory that is part of the library's image (4.5 MiB per GPU, held until the process ends) instead of context scratch that
+ * grows on demand.  Results are bit-identical to wick_rocm_matmul_f32 wherever that call does not split its launch over K
+ * (wick_rocm_set_gemm_max_k_splits: always with max_splits = 1; with the default only prompts of few tokens over a long K
+ * split) and within the f32 bar of it otherwise: this entry point never splits, the shares would need scratch of their own.
+ * Limits and rules:
  *   - n * k <= 4194304 elements (e.g. 2048 tokens x 2048, 512 x 8192); larger calls return WICK_ROCM_ERR_BAD_SHAPE;
  *   - no hipMalloc, hipFree or other allocating call is made, on any path; with per-dispatch kernel timing on
  *     (which creates events) the call returns WICK_ROCM_ERR_STATE instead;
  *   - every call on one GPU uses that GPU's one array, from any context: calls that overlap in time on one GPU race
- *     (calls on one context's stream are ordered and safe); the array keeps the last call's contents, and nothing in
- *     it needs clearing, because the quantizer rewrites every byte the matmul reads. */
+ *     (calls on one context's stream are ordered and safe).  The library refuses the overlap it can see: while one context's
+ *     calls (or replays of graphs that captured them) may still be running, a call from ANOTHER context of the same GPU
+ *     returns WICK_ROCM_ERR_STATE until the first context has synchronised (wick_rocm_sync, wick_rocm_download);
+ *   - the array keeps the last call's contents, and nothing in it needs clearing, because the quantizer rewrites every
+ *     byte the matmul reads. */
 int wick_rocm_matmul_f32_noalloc(wick_rocm_ctx *ctx, const wick_rocm_weight *w, const float *d_x, size_t x_off_bytes, uint32_t n,
                                  uint32_t x_stride, float *d_y, size_t y_off_bytes, uint32_t y_stride, int accumulate);
 /* encode_gemv_qkv / encode_gemv_gate_up (wick/src/model/metal_lfm2.rs:1043-1119):
@@ -274,7 +266,8 @@ int wick_rocm_ffn_gate_up_f32(wick_rocm_ctx *ctx, const wick_rocm_weight *w_gate
 
 /* Pre-sizes the context's scratch for up to max_n columns of up to max_k elements (max_k: the largest row length
  * or row count of any weight used; call before capturing a graph).  Used by wick_rocm_matmul_f32 (n > 1 or a shape
- * the fused kernels do not take) and by the unfused fallbacks of the calls above. */
+ * the fused kernels do not take) and by the unfused fallbacks of the calls above.  With max_n >= 5 it also holds the room
+ * the K shares of a split GEMM launch can take (32 MiB), so that no later batched call regrows the scratch. */
 int wick_rocm_reserve_scratch(wick_rocm_ctx *ctx, uint32_t max_n, uint32_t max_k);
 
 /* ---- parity hook ----------------------------------------------------------

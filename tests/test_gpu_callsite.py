@@ -157,17 +157,34 @@ def test_cpp_host_mirror_selftest():
     assert out.returncode == 0 and "selftest OK" in out.stdout, out.stdout + out.stderr
 
 
-def test_rate_probes(ctx):
-    """The register-only instruction-rate probes launch, report their operation counts and
-    reject bad arguments (they are measurement aids; nothing is checked about their speed)."""
+def test_bench_library_aids(ctx, oracle):
+    """bench.py's measurement aids (libwick_rocm_bench.so, not part of the backend): the register-only rate probes launch,
+    report their operation counts and reject bad arguments; the GEMV with the timing hook computes what the product call
+    computes and leaves one (start, end) wall-clock record per wave."""
+    from wick_amd import benchlib as B
+
     for shape, per_iter in [(0, 4 * 65536.0), (1, 4 * 16384.0), (2, 4 * 4 * 64 * 2.0), (3, 131072.0), (4, 131072.0)]:
-        ops = ctx.probe_rate(shape, 10)
+        ops = B.probe_rate(ctx, shape, 10)
         assert ops > 0 and ops % (per_iter * 10) == 0
     ctx.sync()
     with pytest.raises(W.RocmError):
-        ctx.probe_rate(5, 10)
+        B.probe_rate(ctx, 5, 10)
     with pytest.raises(W.RocmError):
-        ctx.probe_rate(0, 0)
+        B.probe_rate(ctx, 0, 0)
+    for dtype, m, k in [(W.Q4_0, 6912, 2048), (W.Q8_0, 1024, 1024), (W.Q4_0, 300, 512)]:
+        wb = oracle.synth_weight(dtype, m, k, seed=77)
+        w = ctx.upload_weight(wb, dtype, m, k)
+        s, q = oracle.quantize_q8_0(oracle.fill_normal(9, 1.0, k))
+        d_q, d_s, d_y, d_y2, d_span = ctx.to_device(q), ctx.to_device(s), ctx.alloc(m * 4), ctx.alloc(m * 4), ctx.alloc(m * 16)
+        ctx.gemv_with_preq(w, d_s, d_q, d_y)
+        waves = B.gemv_q8_span(ctx, w, d_s, d_q, d_y2, d_span, m)
+        assert 0 < waves <= m
+        assert np.array_equal(d_y.download(np.float32, m).view(np.uint32), d_y2.download(np.float32, m).view(np.uint32))
+        rec = d_span.download(np.uint64, 2 * waves).reshape(waves, 2)
+        assert np.all(rec[:, 1] >= rec[:, 0]) and 0 < B.span_us(rec) < 1000.0
+        for b in (d_q, d_s, d_y, d_y2, d_span):
+            b.free()
+        w.free()
 
 
 # ---- projections with the preceding norm / gate folded into their launch -----------------------------------

@@ -48,6 +48,54 @@ def test_no_alloc_matches_matmul_f32_twice_in_a_row(ctx, oracle):
     _both(ctx, oracle, W.Q6_K, 96, 512, 2, 512, 96, seed=5)                            # Q6_K: one GEMV per token
 
 
+def test_no_alloc_against_a_split_launch_at_default_settings(ctx, oracle):
+    """With the library's default K split the two entry points take different launches on a shape that splits (few tokens over a
+    long K): not the same low-order bits, both inside the f32 bar against the oracle and against each other."""
+    m, k, n = 2048, 6912, 20
+    wb = oracle.synth_weight(W.Q8_0, m, k, seed=31)
+    w = ctx.upload_weight(wb, W.Q8_0, m, k)
+    x = oracle.fill_normal(32, 1.0, n * k)
+    d_x, d_a, d_b = ctx.to_device(x), ctx.alloc(n * m * 4), ctx.alloc(n * m * 4)
+    ctx.set_gemm_max_k_splits(0)  # the default
+    ctx.encode_gemm(w, d_x, 0, d_a, 0, n, k, m)
+    ctx.encode_gemm_noalloc(w, d_x, 0, d_b, 0, n, k, m)
+    a, b = d_a.download(np.float32, n * m).reshape(n, m).T, d_b.download(np.float32, n * m).reshape(n, m).T
+    s, q = oracle.quantize_q8_0_batch(x, n, k)
+    ref = oracle.gemm_q8(W.Q8_0, wb, s, q, m, n, k, f64=True)
+    assert_f32_parity(a, ref, "matmul_f32 (split launch)")
+    assert_f32_parity(b, ref, "no-alloc matmul (unsplit launch)")
+    assert_f32_parity(b, a, "no-alloc vs split")
+    w.free(), d_x.free(), d_a.free(), d_b.free()
+
+
+def test_no_alloc_refuses_a_second_context_until_the_first_has_synchronised(ctx, oracle):
+    """One static array per GPU, shared by every context: the overlap the host can see is refused instead of raced."""
+    m, k, n = 64, 256, 4
+    wb = oracle.synth_weight(W.Q4_0, m, k, seed=41)
+    x = oracle.fill_normal(42, 1.0, n * k)
+    s, q = oracle.quantize_q8_0_batch(x, n, k)
+    ref = oracle.gemm_q8(W.Q4_0, wb, s, q, m, n, k)
+    other = W.RocmContext(0)
+    try:
+        wa, wo = ctx.upload_weight(wb, W.Q4_0, m, k), other.upload_weight(wb, W.Q4_0, m, k)
+        xa, ya, xo, yo = ctx.to_device(x), ctx.alloc(n * m * 4), other.to_device(x), other.alloc(n * m * 4)
+        ctx.sync()
+        ctx.encode_gemm_noalloc(wa, xa, 0, ya, 0, n, k, m)  # enqueued, not synchronised: the array is ctx's
+        with pytest.raises(W.RocmError, match="another context") as e:
+            other.encode_gemm_noalloc(wo, xo, 0, yo, 0, n, k, m)
+        assert e.value.status == -6
+        ctx.sync()
+        other.encode_gemm_noalloc(wo, xo, 0, yo, 0, n, k, m)  # free again
+        with pytest.raises(W.RocmError, match="another context"):
+            ctx.encode_gemm_noalloc(wa, xa, 0, ya, 0, n, k, m)
+        assert_f32_parity(yo.download(np.float32, n * m).reshape(n, m).T, ref, "second context")  # the download synchronises
+        ctx.encode_gemm_noalloc(wa, xa, 0, ya, 0, n, k, m)
+        assert_f32_parity(ya.download(np.float32, n * m).reshape(n, m).T, ref, "first context again")
+        wa.free(), xa.free(), ya.free(), wo.free(), xo.free(), yo.free()
+    finally:
+        other.close()
+
+
 def test_no_alloc_inside_a_graph_capture(ctx, oracle):
     """What it is for: a capture in which nothing may allocate.  No wick_rocm_reserve_scratch beforehand."""
     m, k, n = 256, 2080, 20  # 2080: a shape wick_rocm_matmul_f32 would need context scratch for

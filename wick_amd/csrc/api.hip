@@ -24,6 +24,32 @@ static __device__ __align__(256) unsigned char scratch[kNoallocScratchBytes];
 
 namespace {
 
+// Every context on a GPU shares that GPU's one array, and nothing orders the streams of two contexts.  The host therefore
+// keeps, per device, the context whose calls (or graph replays of them) may still be using the array: a call from another
+// context is refused until the owner has synchronised (wick_rocm_sync, a download, destruction), which is when its work on
+// the array is known to have finished.
+constexpr int kNoallocMaxDevices = 64;
+std::mutex g_noalloc_mu;
+wick_rocm_ctx* g_noalloc_owner[kNoallocMaxDevices] = {};
+
+int noalloc_claim(wick_rocm_ctx* ctx) {
+    if (ctx->device < 0 || ctx->device >= kNoallocMaxDevices) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "matmul_f32_noalloc: device index out of range");
+    std::lock_guard<std::mutex> lk(g_noalloc_mu);
+    wick_rocm_ctx*& owner = g_noalloc_owner[ctx->device];
+    if (owner && owner != ctx)
+        return fail(ctx, WICK_ROCM_ERR_STATE, "matmul_f32_noalloc: another context's work on this GPU's static scratch may still be in flight; "
+                                              "wick_rocm_sync that context first");
+    owner = ctx;
+    return WICK_ROCM_OK;
+}
+
+// The context's stream has drained (or the context goes away): whatever it enqueued on the array has finished.
+void noalloc_release(wick_rocm_ctx* ctx) {
+    if (ctx->device < 0 || ctx->device >= kNoallocMaxDevices) return;
+    std::lock_guard<std::mutex> lk(g_noalloc_mu);
+    if (g_noalloc_owner[ctx->device] == ctx) g_noalloc_owner[ctx->device] = nullptr;
+}
+
 int check_weight(wick_rocm_ctx* ctx, const wick_rocm_weight* w) {
     if (!w || !w->d) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "null weight handle");
     return WICK_ROCM_OK;
@@ -160,11 +186,11 @@ void wick_rocm_ctx_destroy(wick_rocm_ctx* ctx) {
             (void)hipStreamSynchronize(ctx->stream);
             (void)hipStreamDestroy(ctx->stream);
         }
+        noalloc_release(ctx);
         if (ctx->scratch_q) (void)hipFree(ctx->scratch_q);
         if (ctx->scratch_s) (void)hipFree(ctx->scratch_s);
         if (ctx->scratch_f) (void)hipFree(ctx->scratch_f);
         if (ctx->argmax_partial) (void)hipFree(ctx->argmax_partial);
-        if (ctx->probe_sink) (void)hipFree(ctx->probe_sink);
         for (auto* v : {&ctx->timer.recs, &ctx->timer.spares})
             for (KernelTimer::Rec& r : *v) {
                 (void)hipEventDestroy(r.start);
@@ -227,25 +253,7 @@ int wick_rocm_download(wick_rocm_ctx* ctx, void* dst, const void* d_src, size_t 
     if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "download during graph capture");
     WR_HIP(ctx, hipMemcpyAsync(dst, d_src, nbytes, hipMemcpyDeviceToHost, ctx->stream));
     WR_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    return WICK_ROCM_OK;
-}
-
-int wick_rocm_copy(wick_rocm_ctx* ctx, void* d_dst, const void* d_src, size_t nbytes) {
-    WR_ENTER(ctx);
-    if (nbytes == 0) return WICK_ROCM_OK;
-    if (!d_dst || !d_src) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "copy: null pointer");
-    WR_HIP(ctx, hipMemcpyAsync(d_dst, d_src, nbytes, hipMemcpyDeviceToDevice, ctx->stream));
-    return WICK_ROCM_OK;
-}
-
-int wick_rocm_probe_rate(wick_rocm_ctx* ctx, int shape, uint32_t iters, double* ops) {
-    WR_ENTER(ctx);
-    if (!ops || shape < 0 || shape > 4 || iters == 0) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "probe_rate: shape must be 0..4, iters > 0");
-    if (!ctx->probe_sink) {
-        if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "probe_rate: first call must be outside graph capture");
-        WR_HIP(ctx, hipMalloc(&ctx->probe_sink, 64));
-    }
-    WR_HIP(ctx, launch_probe(shape, iters, ctx->num_cus, reinterpret_cast<int*>(ctx->probe_sink), ops, ctx->launch()));
+    noalloc_release(ctx);
     return WICK_ROCM_OK;
 }
 
@@ -279,6 +287,7 @@ int wick_rocm_sync(wick_rocm_ctx* ctx) {
     WR_ENTER(ctx);
     if (ctx->capturing) return fail(ctx, WICK_ROCM_ERR_STATE, "sync during graph capture");
     WR_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    noalloc_release(ctx);
     return WICK_ROCM_OK;
 }
 
@@ -678,8 +687,11 @@ int wick_rocm_gemm_q8_multi(wick_rocm_ctx* ctx, const wick_rocm_weight* const* w
 int wick_rocm_reserve_scratch(wick_rocm_ctx* ctx, uint32_t max_n, uint32_t max_k) {
     WR_ENTER(ctx);
     if (max_k % 32u != 0) return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "reserve_scratch: max_k % 32 != 0");
-    // f32 scratch: one transformed activation vector + one projection output of the unfused fallbacks
-    return ensure_scratch(ctx, (size_t)max_n * max_k, (size_t)max_n * (max_k / 32u), 2 * (size_t)max_k);
+    // f32 scratch: one transformed activation vector + one projection output of the unfused fallbacks and, for batched calls
+    // that may take the MFMA GEMM, the K shares of a split launch ([shares][n][m] <= 512 tiles of 128 x 128 sums, whatever the shape)
+    const size_t split_floats = max_n >= kGemmMinNLarge && ctx->gemm_max_splits > 1 ? kGemmSplitScratchFloats : 0;
+    const size_t f_floats = 2 * (size_t)max_k > split_floats ? 2 * (size_t)max_k : split_floats;
+    return ensure_scratch(ctx, (size_t)max_n * max_k, (size_t)max_n * (max_k / 32u), f_floats);
 }
 
 int wick_rocm_matmul_f32(wick_rocm_ctx* ctx, const wick_rocm_weight* w, const float* d_x, size_t x_off_bytes, uint32_t n,
@@ -717,6 +729,8 @@ int wick_rocm_matmul_f32_noalloc(wick_rocm_ctx* ctx, const wick_rocm_weight* w, 
     if ((uint64_t)n * w->k > kNoallocMaxElems)
         return fail(ctx, WICK_ROCM_ERR_BAD_SHAPE, "matmul_f32_noalloc: n * k exceeds the static scratch (4194304 elements); use wick_rocm_matmul_f32");
     if (ctx->timer.enabled) return fail(ctx, WICK_ROCM_ERR_STATE, "matmul_f32_noalloc: per-dispatch kernel timing creates events; switch it off");
+    if (int rc = noalloc_claim(ctx)) return rc;
+    if (ctx->capturing) ctx->capture_used_noalloc = true;  // every replay of the graph will use the array again
     const float* x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(d_x) + x_off_bytes);
     float* y = reinterpret_cast<float*>(reinterpret_cast<char*>(d_y) + y_off_bytes);
     // this device's copy of the static array, never the array's name: quants first, scales behind them
@@ -770,6 +784,7 @@ int wick_rocm_graph_begin(wick_rocm_ctx* ctx) {
     WR_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     ctx->capturing = true;
     ctx->capture_used_scratch = false;
+    ctx->capture_used_noalloc = false;
     return WICK_ROCM_OK;
 }
 
@@ -798,6 +813,7 @@ int wick_rocm_graph_end(wick_rocm_ctx* ctx, wick_rocm_graph** out) {
     }
     g->uses_scratch = ctx->capture_used_scratch;
     g->scratch_gen = ctx->scratch_gen;
+    g->uses_noalloc = ctx->capture_used_noalloc;
     *out = g;
     return WICK_ROCM_OK;
 }
@@ -809,6 +825,8 @@ int wick_rocm_graph_launch(wick_rocm_ctx* ctx, wick_rocm_graph* g) {
     if (graph_is_stale(ctx, g))
         return fail(ctx, WICK_ROCM_ERR_STATE, "graph_launch: the context's scratch was regrown after this graph was captured (it holds freed addresses); "
                                               "capture it again, and size the scratch with wick_rocm_reserve_scratch before capturing");
+    if (g->uses_noalloc)
+        if (int rc = noalloc_claim(ctx)) return rc;
     WR_HIP(ctx, hipGraphLaunch(g->exec, ctx->stream));
     return WICK_ROCM_OK;
 }

@@ -1,8 +1,14 @@
-// Register-only probes that measure this GPU's own ceilings for the two instructions the
-// prefill GEMM is priced against (no memory traffic: operands never leave registers).
-// They exist so that "fraction of peak" can be stated against a measured denominator as
-// well as the datasheet one; nothing on the matmul path calls them.
-#include "wick_rocm_internal.h"
+// Measurement aids of the benchmark, built into a library of their own (libwick_rocm_bench.so): nothing here is part of
+// the backend's C ABI and libwick_rocm.{so,a} does not contain it.
+//   * Register-only probes that measure this GPU's own ceilings for the two instructions the prefill GEMM is priced
+//     against (no memory traffic: operands never leave registers), so that "fraction of peak" can be stated against a
+//     measured denominator as well as the datasheet one.
+//   * A device-to-device copy of known size (calibration of the memory-traffic counters).
+//   * The decode GEMV with the timing hook (gemv_impl.h, SPAN): the product kernel plus two wall-clock reads per wave, for
+//     the execution span of launches inside a graph replay.
+// Every entry point takes the hipStream_t to enqueue on (wick_rocm_ctx_stream of the backend's context).
+#include "gemv_impl.h"
+#include "wick_rocm_bench.h"
 
 namespace wick_rocm {
 
@@ -110,11 +116,14 @@ __global__ __launch_bounds__(kMixThreads) void probe_mix_kernel(int* sink, uint3
     if (s == 123.456f) sink[0] = 1;  // keeps the loop alive, practically never stores
 }
 
-}  // namespace
+static __device__ int probe_sink[16];  // the probes may (practically never do) store here
 
-// Enqueues one probe launch that fills the chip (8 workgroups of 4 waves per CU) and returns
-// the number of operations it performs (int8 ops for the MFMA shapes, flops for the FMA one).
-hipError_t launch_probe(int shape, uint32_t iters, int num_cus, int* d_sink, double* ops, const Launch& L) {
+// One probe launch that fills the chip (8 workgroups of 4 waves per CU); *ops = the operations it performs (int8 ops for the
+// MFMA shapes, flops for the FMA one).
+hipError_t launch_probe(int shape, uint32_t iters, int num_cus, double* ops, const Launch& L) {
+    int* d_sink = nullptr;
+    hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&d_sink), HIP_SYMBOL(probe_sink));
+    if (e != hipSuccess) return e;
     if (shape >= 3) {  // the block loop: 2 * 64 * 32 * 32 int8 ops per wave and iteration
         const dim3 grid((uint32_t)num_cus * 2u), block(kMixThreads);
         *ops = (double)grid.x * (kMixThreads / 64) * 131072.0 * iters;
@@ -130,4 +139,39 @@ hipError_t launch_probe(int shape, uint32_t iters, int num_cus, int* d_sink, dou
     return launch_kernel(L, kFamOther, probe_kernel<2>, grid, block, d_sink, iters);
 }
 
+}  // namespace
+
 }  // namespace wick_rocm
+
+using namespace wick_rocm;
+
+extern "C" {
+
+int wick_bench_probe_rate(void* stream, int shape, uint32_t iters, int num_cus, double* ops) {
+    if (!ops || shape < 0 || shape > 4 || iters == 0 || num_cus <= 0) return -1;
+    return launch_probe(shape, iters, num_cus, ops, Launch{static_cast<hipStream_t>(stream), nullptr}) == hipSuccess ? 0 : -4;
+}
+
+int wick_bench_copy(void* stream, void* d_dst, const void* d_src, size_t nbytes) {
+    if (!d_dst || !d_src) return -1;
+    return hipMemcpyAsync(d_dst, d_src, nbytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)) == hipSuccess ? 0 : -4;
+}
+
+int wick_bench_gemv_q8_span(void* stream, int ggml_type, const void* d_w, uint32_t m, uint32_t k, const int8_t* d_quants, const float* d_scales,
+                            float* d_y, int num_cus, unsigned long long* d_span, uint32_t span_capacity_waves, uint32_t* waves) {
+    if (!d_w || !d_quants || !d_scales || !d_y || !d_span || !waves || m == 0 || k == 0 || k % 64u != 0 || num_cus <= 0) return -1;
+    if (ggml_type != kTypeQ4_0 && ggml_type != kTypeQ8_0) return -2;
+    // the launch writes one record per wave: refuse a buffer that cannot hold the most waves any split of the rows makes
+    if (span_capacity_waves < m) return -1;
+    GemvArgs a{};
+    a.batch.w[0] = static_cast<const uint8_t*>(d_w), a.batch.y[0] = d_y, a.batch.row_end[0] = m, a.batch.count = 1;
+    a.xq = d_quants, a.xs = d_scales;
+    a.k = k, a.n = 1;
+    a.dots = reinterpret_cast<int32_t*>(d_span);
+    const Launch L{static_cast<hipStream_t>(stream), nullptr};
+    const hipError_t e = ggml_type == kTypeQ4_0 ? dispatch<2, 1, false, false, true>(a, num_cus, L) : dispatch<8, 1, false, false, true>(a, num_cus, L);
+    *waves = a.total_waves;
+    return e == hipSuccess ? 0 : -4;
+}
+
+}  // extern "C"

@@ -109,7 +109,12 @@ enum { kDirect = 0, kDirectNT = 1, kSpan = 2 };
 // launch and the round trip through memory in between.
 // DUMP: the parity hook.  The same loads, LDS hand-over, unpack and v_dot4 as the product kernel; the exact i32 dot of
 // every (token, row, block) is written out where the product kernel would scale and sum it.
-template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI, int MODE, int XF = kXformNone, bool GATED = false, bool DUMP = false>
+// SPAN: the timing hook.  The product instruction stream plus two reads of the 100 MHz wall clock per wave: the wave's first
+// instruction and, after its last store has been acknowledged, its last.  Both go to a.dots (as [wave][2] 64-bit words); the
+// host takes first start -> last end as the launch's execution span (the counterpart of the reference's per-dispatch GPU
+// timestamps, wick/src/model/metal_lfm2.rs:3367-4116, for launches inside a graph replay, which carry no events).
+template <int TYPE, int LPR, int NCHUNK, int U, int NT, bool FUSEQ, bool MULTI, int MODE, int XF = kXformNone, bool GATED = false, bool DUMP = false,
+          bool SPAN = false>
 __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kernel(const void* p_x, const uint8_t* p_w0, float* p_y0,
                                                                                   uint32_t p_k, uint32_t p_rows0,
                                                                                   uint32_t p_rows_per_wave, uint32_t p_total_waves,
@@ -117,6 +122,9 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
     static_assert(XF == kXformNone || FUSEQ, "activation transforms belong to the fused-quantizer variant");
     static_assert(!GATED || (FUSEQ && !MULTI && NT == 1 && U % 2 == 0), "the gated variant pairs lane slots");
     static_assert(!DUMP || (!MULTI && !GATED && XF == kXformNone), "the parity hook runs the plain single-weight variants");
+    static_assert(!SPAN || (!DUMP && !FUSEQ && !MULTI && NT == 1), "the timing hook runs the plain single-token variants");
+    unsigned long long span_t0 = 0;
+    if constexpr (SPAN) span_t0 = __builtin_amdgcn_s_memrealtime();
     constexpr int UR = GATED ? U / 2 : U;  // distinct rows per lane and pass
     using PT = PairTraits<TYPE>;
     constexpr int RPW = 64 / LPR;  // rows per wave pass
@@ -476,6 +484,14 @@ __global__ __launch_bounds__(FUSEQ ? 64 * kFusedWaves : 64) void gemv_pairs_kern
             }
         }
     }
+    if constexpr (SPAN) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the wave's stores have been acknowledged
+        const unsigned long long t1 = __builtin_amdgcn_s_memrealtime();
+        if (lane == 0) {
+            unsigned long long* o = reinterpret_cast<unsigned long long*>(a.dots) + 2 * (size_t)gwave;
+            o[0] = span_t0, o[1] = t1;
+        }
+    }
 }
 
 // Any k % 32 == 0, any byte alignment: one wave per row, lanes stride over single
@@ -563,7 +579,7 @@ inline uint32_t set_wave_ends(GemvArgs& a) {
 //     matrices, 6.4 TB/s kernel-time on a 142 MB Q8_0 matrix.
 constexpr uint64_t kDirectMaxBytesQ4 = 3ull << 20;
 constexpr uint64_t kDirectMaxBytesQ8 = 512ull << 10;
-template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ, int U, bool DUMP>
+template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ, int U, bool DUMP, bool SPAN = false>
 hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
     const uint32_t pass_rows = (64 / LPR) * (a.gated ? U / 2 : U);
     // Enough waves to give every CU ~16, and every wave at least one full pass.
@@ -629,6 +645,10 @@ hipError_t launch_pairs_u(GemvArgs& a, uint32_t total_rows, int num_cus, const L
         if (a.xform == kXformRmsNorm) return with_xform(std::integral_constant<int, kXformRmsNorm>{});
         if (a.xform == kXformSiluMul) return with_xform(std::integral_constant<int, kXformSiluMul>{});
         return with_xform(std::integral_constant<int, kXformNone>{});
+    } else if constexpr (SPAN) {  // the timing hook: single weight, the fetch mode of the product launch
+        if (multi) return hipErrorInvalidValue;
+        if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan, kXformNone, false, false, true>);
+        return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSmall, kXformNone, false, false, true>);
     } else if constexpr (NT == 1) {
         if (mode == kSpan && multi) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, true, kSpan>);
         if (mode == kSpan) return go(gemv_pairs_kernel<TYPE, LPR, NCHUNK, U, NT, FUSEQ, false, kSpan>);
@@ -654,11 +674,11 @@ inline int gemv_u_override() {
     return v;
 }
 
-template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ, bool DUMP>
+template <int TYPE, int LPR, int NCHUNK, int NT, bool FUSEQ, bool DUMP, bool SPAN = false>
 hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, const Launch& L) {
     constexpr int UMAX = (NT > 1 || NCHUNK > 1) ? (TYPE == 2 && NT == 1 ? 2 : 1) : (TYPE == 2 ? 4 : 2);
     if (a.gated) {  // one gate row and one up row per lane and pass
-        if constexpr (FUSEQ && NT == 1 && NCHUNK == 1) return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 2, DUMP>(a, total_rows, num_cus, L);
+        if constexpr (FUSEQ && NT == 1 && NCHUNK == 1) return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 2, DUMP, SPAN>(a, total_rows, num_cus, L);
         else return hipErrorInvalidValue;
     }
     int u = UMAX;
@@ -666,14 +686,14 @@ hipError_t launch_pairs(GemvArgs& a, uint32_t total_rows, int num_cus, const Lau
     while (u > 1 && total_rows / ((64 / LPR) * u) < want_waves) u >>= 1;
     if (gemv_u_override() > 0) u = gemv_u_override() < UMAX ? gemv_u_override() : UMAX;
     if constexpr (UMAX >= 4)
-        if (u >= 4) return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 4, DUMP>(a, total_rows, num_cus, L);
+        if (u >= 4) return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 4, DUMP, SPAN>(a, total_rows, num_cus, L);
     if constexpr (UMAX >= 2)
-        if (u >= 2) return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 2, DUMP>(a, total_rows, num_cus, L);
-    return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 1, DUMP>(a, total_rows, num_cus, L);
+        if (u >= 2) return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 2, DUMP, SPAN>(a, total_rows, num_cus, L);
+    return launch_pairs_u<TYPE, LPR, NCHUNK, NT, FUSEQ, 1, DUMP, SPAN>(a, total_rows, num_cus, L);
 }
 
 // FUSEQ callers have checked that the pair kernel applies (pairs_kernel_applies).
-template <int TYPE, int NT, bool FUSEQ = false, bool DUMP = false>
+template <int TYPE, int NT, bool FUSEQ = false, bool DUMP = false, bool SPAN = false>
 hipError_t dispatch(GemvArgs& a, int num_cus, const Launch& L) {
     const uint32_t total_rows = a.batch.row_end[a.batch.count - 1];
     if (total_rows == 0 || a.n == 0) return hipSuccess;
@@ -682,14 +702,14 @@ hipError_t dispatch(GemvArgs& a, int num_cus, const Launch& L) {
     bool aligned = (nb % 2u) == 0 && (FUSEQ || (reinterpret_cast<uintptr_t>(a.xq) % 16u) == 0);
     for (uint32_t i = 0; i < a.batch.count; i++) aligned = aligned && (reinterpret_cast<uintptr_t>(a.batch.w[i]) % 4u) == 0;
     if (aligned && ppr <= 128) {
-        if (ppr <= 4) return launch_pairs<TYPE, 4, 1, NT, FUSEQ, DUMP>(a, total_rows, num_cus, L);
-        if (ppr <= 8) return launch_pairs<TYPE, 8, 1, NT, FUSEQ, DUMP>(a, total_rows, num_cus, L);
-        if (ppr <= 16) return launch_pairs<TYPE, 16, 1, NT, FUSEQ, DUMP>(a, total_rows, num_cus, L);
-        if (ppr <= 32) return launch_pairs<TYPE, 32, 1, NT, FUSEQ, DUMP>(a, total_rows, num_cus, L);
-        if (ppr <= 64) return launch_pairs<TYPE, 64, 1, NT, FUSEQ, DUMP>(a, total_rows, num_cus, L);
-        return launch_pairs<TYPE, 64, 2, NT, FUSEQ, DUMP>(a, total_rows, num_cus, L);
+        if (ppr <= 4) return launch_pairs<TYPE, 4, 1, NT, FUSEQ, DUMP, SPAN>(a, total_rows, num_cus, L);
+        if (ppr <= 8) return launch_pairs<TYPE, 8, 1, NT, FUSEQ, DUMP, SPAN>(a, total_rows, num_cus, L);
+        if (ppr <= 16) return launch_pairs<TYPE, 16, 1, NT, FUSEQ, DUMP, SPAN>(a, total_rows, num_cus, L);
+        if (ppr <= 32) return launch_pairs<TYPE, 32, 1, NT, FUSEQ, DUMP, SPAN>(a, total_rows, num_cus, L);
+        if (ppr <= 64) return launch_pairs<TYPE, 64, 1, NT, FUSEQ, DUMP, SPAN>(a, total_rows, num_cus, L);
+        return launch_pairs<TYPE, 64, 2, NT, FUSEQ, DUMP, SPAN>(a, total_rows, num_cus, L);
     }
-    if (FUSEQ) return hipErrorInvalidValue;  // unreachable: see pairs_kernel_applies
+    if (FUSEQ || SPAN) return hipErrorInvalidValue;  // FUSEQ: unreachable, see pairs_kernel_applies; the timing hook: pair kernel only
     a.rows_per_wave = 1;
     dim3 grid(set_wave_ends(a), (a.n + NT - 1) / NT);
     return launch_kernel(L, kFamGemv, gemv_generic_kernel<TYPE, NT, DUMP>, dim3(grid), dim3(64), a);

@@ -520,6 +520,9 @@ int ensure_prefill_buffers(wick_rocm_ctx* ctx, wick_rocm_lfm2* m) {
         (rc = alloc_t(ctx, m, attention_prefill_scratch_floats((uint32_t)P, c.n_heads, (uint32_t)hd), &m->pAttn)) ||
         (rc = alloc_t(ctx, m, P, &m->pTokens)))
         return rc;
+    // room for the K shares of a split projection, once: no prompt then regrows the context's scratch (a regrow waits for the
+    // stream and makes every captured step graph stale)
+    if ((rc = wick_rocm_reserve_scratch(ctx, (uint32_t)P, 0))) return rc;
     m->prefill_cap = (uint32_t)P;
     return WICK_ROCM_OK;
 }
@@ -736,7 +739,16 @@ int wick_rocm_lfm2_load(wick_rocm_ctx* ctx, const wick_gguf* g, uint32_t context
                        wick_rocm_shortconv_fusable(L.out_proj, L.gate, L.up, c.conv_kernel_size) != 0;
     }
     if ((rc = upload_f32(ctx, m, g, "token_embd_norm.weight", hs, &m->out_norm))) return bail(rc);
-    if ((rc = upload_weight(ctx, m, g, "token_embd.weight", c.vocab_size, hs, &m->embd))) return bail(rc);
+    {
+        // The tied embedding serves row lookups and the LM head over ONE token (a prompt pass takes the last token's logits only,
+        // wick/src/model/lfm2.rs:2190-2212): it never runs as a batched GEMM, so it keeps its raw blocks only.
+        std::lock_guard<std::recursive_mutex> lk(ctx->mu);
+        const bool packing = ctx->gemm_packing;
+        ctx->gemm_packing = false;
+        rc = upload_weight(ctx, m, g, "token_embd.weight", c.vocab_size, hs, &m->embd);
+        ctx->gemm_packing = packing;
+        if (rc) return bail(rc);
+    }
 
     const uint32_t kv_max = (c.n_kv_heads ? c.n_kv_heads : 1) * hd;
     if ((rc = alloc_t(ctx, m, hs, &m->hidden)) || (rc = alloc_t(ctx, m, 3 * (size_t)hs, &m->proj)) ||

@@ -32,6 +32,7 @@ struct wick_rocm_ctx {
     // scratch remembers the generation it was captured under and refuses to launch under another one.
     uint64_t scratch_gen = 0;
     bool capture_used_scratch = false;
+    bool capture_used_noalloc = false;  // the capture in progress holds a wick_rocm_matmul_f32_noalloc call
     unsigned char* noalloc_scratch = nullptr;  // this device's address of the static scratch array of wick_rocm_matmul_f32_noalloc
     uint32_t gemm_min_n = 0;  // hand-off from the multi-token GEMV to the MFMA GEMM; 0: the per-weight default (min_n_for)
     uint32_t min_n_for(size_t weight_bytes) const {
@@ -42,7 +43,6 @@ struct wick_rocm_ctx {
     KernelTimer timer;
     int64_t gemv_direct_max_bytes = -1;
     unsigned long long* argmax_partial = nullptr;  // kArgmaxPartials keys for wick_rocm_argmax
-    void* probe_sink = nullptr;  // 64 bytes the rate probes may (never do) write to
     Launch launch() { return Launch{stream, &timer, gemv_direct_max_bytes}; }
 };
 
@@ -60,6 +60,7 @@ struct wick_rocm_graph {
     hipGraphExec_t exec = nullptr;
     bool uses_scratch = false;  // some captured launch reads or writes the context's scratch
     uint64_t scratch_gen = 0;   // ... as it was laid out then
+    bool uses_noalloc = false;  // some captured launch uses the GPU's static scratch array (wick_rocm_matmul_f32_noalloc)
 };
 
 // True when the graph refers to scratch memory that has been freed and reallocated since its capture.

@@ -148,12 +148,8 @@ bool gemm_gated_applies(uint32_t m, uint32_t n, uint32_t k);
 hipError_t launch_gemm_mfma_gated(int type, const uint8_t* d_w_gate, const uint8_t* d_w_up, uint32_t m, uint32_t k, const int8_t* d_q,
                                   const float* d_scales, uint32_t n, int8_t* d_out_q, float* d_out_scales, const Launch& L);
 
-// Per-block i32 dots, out[(j*m + i)*nb + b], through the GEMM's loads / LDS layout / MFMA (k % 128 == 0).
-// Register-only instruction-rate probes (probe.hip): shape 0 = v_mfma_i32_32x32x32_i8, 1 = v_mfma_i32_16x16x32_i8,
-// 2 = v_fma_f32.
-hipError_t launch_probe(int shape, uint32_t iters, int num_cus, int* d_sink, double* ops, const Launch& L);
-
-// The same through the decode GEMV's own kernels (gemv_dump.hip): every fetch mode, token count and the fused
+// Per-block i32 dots, out[(j*m + i)*nb + b], through the GEMM's loads / LDS layout / MFMA (k % 128 == 0): launch_block_dots_mfma
+// below.  The same through the decode GEMV's own kernels (gemv_dump.hip): every fetch mode, token count and the fused
 // in-kernel quantizer, exactly as a product launch of that shape would run them.
 hipError_t launch_block_dots_gemv(int type, const uint8_t* d_w, uint32_t m, uint32_t k, const int8_t* d_q, uint32_t n, int32_t* d_out,
                                   int num_cus, const Launch& L);
@@ -243,5 +239,8 @@ constexpr uint32_t kGemmMinN = 9;
 constexpr uint32_t kGemmMinNLarge = 5;
 constexpr size_t kGemmLargeWeightBytes = 16u << 20;
 constexpr uint32_t kGemmMaxSplits = 8;  // most K shares of a GEMM launch with few tiles
+// Most floats the shares of a split launch can take: (tile, share) pairs fill at most the chip's 512 workgroup slots, a tile is
+// at most 128 x 128 sums, and shares x n x m <= pairs x tile.
+constexpr size_t kGemmSplitScratchFloats = 512u * 128u * 128u;
 
 }  // namespace wick_rocm

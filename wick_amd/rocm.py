@@ -72,13 +72,11 @@ _SIGNATURES = {
     "wick_rocm_upload": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_download": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_sync": (C.c_int, [_P]),
-    "wick_rocm_copy": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_set_gemm_min_n": (C.c_int, [_P, C.c_uint32]),
     "wick_rocm_set_gemm_packing": (C.c_int, [_P, C.c_int]),
     "wick_rocm_weight_device_bytes": (C.c_size_t, [_P]),
     "wick_rocm_set_gemm_max_k_splits": (C.c_int, [_P, C.c_uint32]),
     "wick_rocm_set_gemv_policy": (C.c_int, [_P, C.c_int64]),
-    "wick_rocm_probe_rate": (C.c_int, [_P, C.c_int, C.c_uint32, C.POINTER(C.c_double)]),
     "wick_rocm_weight_upload": (C.c_int, [_P, _P, C.c_size_t, C.c_int, C.c_uint32, C.c_uint32, C.POINTER(_P)]),
     "wick_rocm_weight_from_gguf": (C.c_int, [_P, _P, C.c_char_p, C.POINTER(_P)]),
     "wick_rocm_weight_free": (C.c_int, [_P, _P]),
@@ -177,6 +175,11 @@ class RocmWeight:
         """Bytes this weight holds on the device: the raw blocks plus, where it was made, the prefill GEMM's own copy."""
         return int(self.ctx._lib.wick_rocm_weight_device_bytes(self.handle))
 
+    @property
+    def device_ptr(self) -> int:
+        """Device address of the raw blocks (what the decode GEMVs stream)."""
+        return int(self.ctx._lib.wick_rocm_weight_device_ptr(self.handle))
+
     def free(self) -> None:
         if self.handle:
             self.ctx._check(self.ctx._lib.wick_rocm_weight_free(self.ctx._h, self.handle))
@@ -231,15 +234,6 @@ class RocmContext:
 
     def sync(self) -> None:
         self._check(self._lib.wick_rocm_sync(self._h))
-
-    def copy(self, dst, src, nbytes: int) -> None:
-        self._check(self._lib.wick_rocm_copy(self._h, _ptr(dst), _ptr(src), nbytes))
-
-    def probe_rate(self, shape: int, iters: int) -> float:
-        """Enqueues a register-only instruction-rate probe; returns the operations it performs."""
-        ops = C.c_double()
-        self._check(self._lib.wick_rocm_probe_rate(self._h, shape, iters, C.byref(ops)))
-        return ops.value
 
     def set_gemv_policy(self, direct_max_bytes: int = -1) -> None:
         """Weight-fetch threshold of the n = 1 GEMV (negative = default); results do not depend on it."""
