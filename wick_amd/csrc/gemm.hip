@@ -186,16 +186,21 @@ __global__ __launch_bounds__(GR * KB) void gemm_pack_kernel(const uint8_t* __res
 // [token][8 positions] rows of 128 bytes, which an MFMA operand read (16 tokens, same
 // chunk) would hit with an 8-way bank conflict.  So position p of token t holds K-chunk
 // p ^ ((t >> 1) & 7): the lane picks its GLOBAL chunk accordingly, and 16 consecutive
-// tokens reading one chunk then spread over all banks.  16 instructions per stage, two
-// per wave.
+// tokens reading one chunk then spread over all banks.  16 instructions per stage, four
+// per loader wave (dma_stage).
 __device__ __forceinline__ uint32_t xt_swizzle(uint32_t token_in_tile) { return (token_in_tile >> 1) & 7u; }
 // A thread's global read positions of the stage to fetch next.  Set up once per tile; every fetch moves them one stage
 // (128 K-elements) on, one 64-bit add each, instead of rebuilding row / token / block addresses per stage.
+// Only the first kLoaderWaves waves of a workgroup issue the stage's global -> LDS copies (and fetch the token scales): the
+// address unit takes a copy instruction every 16 cycles, so 36 of them per stage and workgroup queue up, and a wave waiting in
+// that queue issues nothing else.  The later waves of a workgroup are the ones that lag in the block loop (the SIMD favours the
+// older wave), so they get no copies to issue at all and the earlier ones, which would otherwise idle at the stage barrier, all.
+constexpr int kLoaderWaves = 4;
 template <int NTOK>
 struct StagePtrs {
-    const int8_t* x[NTOK / 8 / (THREADS / 64)];  // this lane's 16-byte activation chunks (direct-to-LDS copies)
-    const uint8_t* wc[3];                         // this lane's 16 bytes of the wave's weight chunks wave, wave + 8, wave + 16 (of 20)
-    const uint8_t* dx;                            // threads 2 BM .. 2 BM + NTOK - 1: a token's four scales
+    const int8_t* x[NTOK / 8 / kLoaderWaves];  // this lane's 16-byte activation chunks (direct-to-LDS copies)
+    const uint8_t* wc;                          // this lane's 16 bytes of the first kilobyte of granule `wave`'s slab
+    const uint8_t* dx;                          // threads 0 .. NTOK - 1: a token's four scales
 };
 // Where chunk c (0 .. 19) of a tile's stage lands: granule c / 5, its weights' kilobyte c % 5 or (the fifth) its scale pairs.
 template <int NTOK>
@@ -205,8 +210,10 @@ __device__ __forceinline__ void* chunk_dst(StageT<NTOK>& s, uint32_t c) {
 }
 template <int NTOK>
 __device__ __forceinline__ void dma_stage(StagePtrs<NTOK>& p, StageT<NTOK>& s) {
-    constexpr int PER_WAVE = NTOK / 8 / (THREADS / 64);  // activation instructions per wave and stage
+    constexpr int PER_WAVE = NTOK / 8 / kLoaderWaves;  // activation instructions per loader wave and stage
+    static_assert(BM / GR == kLoaderWaves, "one granule's slab per loader wave");
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (wave >= (uint32_t)kLoaderWaves) return;  // uniform per wave
 #pragma unroll
     for (int j = 0; j < PER_WAVE; j++) {
         __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)p.x[j],
@@ -214,21 +221,17 @@ __device__ __forceinline__ void dma_stage(StagePtrs<NTOK>& p, StageT<NTOK>& s) {
         p.x[j] += KB * 32;
     }
 #pragma unroll
-    for (int j = 0; j < 3; j++) {
-        const uint32_t c = wave + 8u * j;
-        if (c < (uint32_t)kTileChunks) {  // uniform per wave
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)p.wc[j],
-                                             (void __attribute__((address_space(3)))*)chunk_dst(s, c), 16, 0, 0);
-            p.wc[j] += 2 * kSlab;
-        }
-    }
+    for (int part = 0; part < kSlabChunks; part++)
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(p.wc + 1024 * part),
+                                         (void __attribute__((address_space(3)))*)chunk_dst(s, kSlabChunks * wave + part), 16, 0, 0);
+    p.wc += 2 * kSlab;
 }
 
 template <int NTOK, bool GATED = false>
 __device__ __forceinline__ void init_stage_ptrs(const GemmArgs& a, uint32_t row_tile, uint32_t tok0, uint32_t kb0, StagePtrs<NTOK>& p) {
-    constexpr int PER_WAVE = NTOK / 8 / (THREADS / 64);
+    constexpr int PER_WAVE = NTOK / 8 / kLoaderWaves;
     const uint32_t t = threadIdx.x, lane = t & 63u;
-    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(t >> 6));
+    const uint32_t wave = min((uint32_t)__builtin_amdgcn_readfirstlane((int)(t >> 6)), (uint32_t)kLoaderWaves - 1u);  // (later waves: unused values)
     const uint32_t nb = a.k >> 5, stages = nb / KB;
 #pragma unroll
     for (int j = 0; j < PER_WAVE; j++) {
@@ -238,23 +241,22 @@ __device__ __forceinline__ void init_stage_ptrs(const GemmArgs& a, uint32_t row_
         p.x[j] = a.xq + (size_t)tok * a.k + (size_t)kb0 * 32 + 16u * chunk;
     }
     const uint32_t granules = (a.m + GR - 1) / GR;
-#pragma unroll
-    for (int j = 0; j < 3; j++) {
-        const uint32_t c = min(wave + 8u * j, (uint32_t)kTileChunks - 1u), g = c / kSlabChunks, part = c % kSlabChunks;
+    {
+        const uint32_t g = wave;
         // the tile's granule g: rows 32 g .. of a plain tile; of a gated tile (64 output rows) gate, up, gate, up of its two
         uint32_t granule = GATED ? 2u * row_tile + (g >> 1) : (BM / GR) * row_tile + g;
         const uint8_t* w = GATED && (g & 1u) ? a.w_up : a.w;
         granule = min(granule, granules - 1u);  // past the end of the matrix: any rows, their results are not stored
-        p.wc[j] = w + (((size_t)(granule >> 1) * stages + kb0 / KB) * 2 + (granule & 1u)) * kSlab + 1024u * part + 16u * lane;
+        p.wc = w + (((size_t)(granule >> 1) * stages + kb0 / KB) * 2 + (granule & 1u)) * kSlab + 16u * lane;
     }
     p.dx = nullptr;
-    if (t >= 2 * BM && t < 2 * BM + NTOK && a.xs) {  // xs is null only for the parity hook, which never scales
-        const uint32_t tok = min(tok0 + (t - 2 * BM), a.n - 1);
+    if (t < NTOK && a.xs) {  // xs is null only for the parity hook, which never scales
+        const uint32_t tok = min(tok0 + t, a.n - 1);
         p.dx = reinterpret_cast<const uint8_t*>(a.xs + (size_t)tok * nb + kb0);
     }
 }
 
-// Thread -> rest of a stage: one float4 (4 blocks) of token scales per token, threads 2 BM .. 2 BM + NTOK - 1, through registers
+// Thread -> rest of a stage: one float4 (4 blocks) of token scales per token, threads 0 .. NTOK - 1 (loader waves), through registers
 // (they are stored block-major).
 template <int NTOK>
 __device__ __forceinline__ void load_stage(StagePtrs<NTOK>& p, StageRegs& r) {
@@ -269,8 +271,8 @@ __device__ __forceinline__ void load_stage(StagePtrs<NTOK>& p, StageRegs& r) {
 template <int NTOK>
 __device__ __forceinline__ void store_stage(StageT<NTOK>& s, const StageRegs& r) {
     const uint32_t t = threadIdx.x;
-    if (t >= 2 * BM && t < 2 * BM + NTOK) {
-        const uint32_t u = t - 2 * BM;
+    if (t < NTOK) {
+        const uint32_t u = t;
         s.dxf[0][u] = r.dx.x;
         s.dxf[1][u] = r.dx.y;
         s.dxf[2][u] = r.dx.z;
