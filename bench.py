@@ -418,17 +418,17 @@ def trace_lfm2_prefill(ctx, W, O, n=2002, context=4096):
     return {"prompt_tokens": n, "passes": 2, "argmax": int(np.argmax(logits))}
 
 
-def bench_lfm2_step(ctx, W, O, tokens=64, context=4096, body=2, embd=14, dims=None, label="LFM2-350M-shaped", kernel_times=True):
+def bench_lfm2_step(ctx, W, O, tokens=64, context=4096, body=2, embd=14, dims=None, label="LFM2-350M-shaped", kernel_times=True, kv_f16=False):
     """Whole decode steps of the model handle (embedding, 16 layers with their norms / conv / attention / gates, tied
     LM head, greedy pick), replayed as one graph per token with token and position resident on the device."""
     from wick_amd import gguf as G
     from wick_amd.lfm2 import RocmLfm2Model
 
     with G.GgufFile.from_bytes(lfm2_350m_image(O, body=body, embd=embd, **(dims or {}))) as g:
-        model = RocmLfm2Model(ctx, g, context)
+        model = RocmLfm2Model(ctx, g, context, kv_f16=kv_f16)
     model.generate_greedy(1, 0, 8)  # captures the graph, warms up
     names = {2: "Q4_0", 8: "Q8_0", 14: "Q6_K"}
-    out = {"model": f"{label}, {names[body]} body + {names[embd]} tied embedding, random init", "context": context,
+    out = {"model": f"{label}, {names[body]} body + {names[embd]} tied embedding, random init", "context": context, "kv_cache": "f16" if kv_f16 else "f32",
            "gpu_memory_MB": model.gpu_memory_bytes() / 1e6, "runs": []}
     for start in (0, 1024, context - tokens):  # attention cost grows with the position
         model.reset()
@@ -772,7 +772,7 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="only the headline GEMV, the GEMM (+ CPU baseline)")
     ap.add_argument("--prompt-tokens", type=int, default=2002, help="lfm2_prefill_trace: tokens of the traced prompt pass")
     ap.add_argument("--graph-only", action="store_true", help="decode legs: graph replays only, no eager launches (for kernel tracers)")
-    ap.add_argument("--leg", default="all", help="all | c1 | gemm | decode | decode_q8 | gemv | prefill_sites | lm_head | lm_head_q6k | upload | lfm2_step | lfm2_step_q8 | lfm2_step_1p2b | lfm2_step_trace | lfm2_prefill_trace | copy | probe | cpu")
+    ap.add_argument("--leg", default="all", help="all | c1 | gemm | decode | decode_q8 | gemv | prefill_sites | lm_head | lm_head_q6k | upload | lfm2_step | lfm2_step_q8 | lfm2_step_kv16 | lfm2_step_1p2b | lfm2_step_trace | lfm2_prefill_trace | copy | probe | cpu")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -800,6 +800,7 @@ def main():
             "lm_head_q6k": lambda: bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024),
             "lfm2_step": lambda: bench_lfm2_step(ctx, W, O),
             "lfm2_step_q8": lambda: bench_lfm2_step(ctx, W, O, body=8, embd=8),
+            "lfm2_step_kv16": lambda: bench_lfm2_step(ctx, W, O, kv_f16=True),  # KV caches of f16 rows
             # the per-layer shapes of an LFM2-1.2B: hidden 2048, FFN 6912, 32 heads / 8 KV heads
             "lfm2_step_1p2b": lambda: bench_lfm2_step(ctx, W, O, dims=dict(HS=2048, IS=6912, KV=512), label="LFM2-1.2B-shaped"),
             "lfm2_step_trace": lambda: trace_lfm2_step(ctx, W, O),

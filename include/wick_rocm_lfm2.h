@@ -200,6 +200,16 @@ typedef struct wick_rocm_lfm2_config {
  * KV caches for min(context_size, lfm2.context_length) positions, conv state and scratch.  The GGUF handle is not
  * referenced after the call returns. */
 int wick_rocm_lfm2_load(wick_rocm_ctx *ctx, const struct wick_gguf *gguf, uint32_t context_size, wick_rocm_lfm2 **out);
+/* The same with the element type of the KV caches chosen by the caller.  WICK_ROCM_KV_F32 (what wick_rocm_lfm2_load takes):
+ * f32 rows, the CPU model's caches (wick/src/kv_cache.rs) -- what the oracle of this backend computes on.  WICK_ROCM_KV_F16:
+ * f16 rows, the reference's GPU models' caches (K after QK-norm and RoPE and V are cast to half on their way in and the
+ * attention kernels read half, wick/src/model/metal_lfm2.rs:4117-4247, 2906-3364): half the cache memory and half the
+ * attention's cache traffic; every cached value is rounded once, to nearest even, when it is appended (or moved by
+ * wick_rocm_lfm2_shift_kv), all arithmetic stays f32.  Snapshots then hold f16 rows (wick_rocm_lfm2_layer_state_bytes says
+ * how many bytes). */
+enum { WICK_ROCM_KV_F32 = 0, WICK_ROCM_KV_F16 = 1 };
+int wick_rocm_lfm2_load_kv(wick_rocm_ctx *ctx, const struct wick_gguf *gguf, uint32_t context_size, int kv_dtype, wick_rocm_lfm2 **out);
+int wick_rocm_lfm2_kv_dtype(const wick_rocm_lfm2 *model);
 int wick_rocm_lfm2_free(wick_rocm_ctx *ctx, wick_rocm_lfm2 *model);
 int wick_rocm_lfm2_get_config(const wick_rocm_lfm2 *model, wick_rocm_lfm2_config *out);
 /* kv_heads_per_layer (0 = gated-conv layer). */
@@ -255,7 +265,8 @@ int wick_rocm_lfm2_forward_hidden_from_embedding(wick_rocm_ctx *ctx, wick_rocm_l
 
 /* Model::snapshot_state / restore_state (wick/src/model/mod.rs:301-315; snapshot_state_locked / restore_state_locked,
  * wick/src/model/metal_lfm2.rs:2535-2634): the model's state after seq_len positions as host bytes, layer by layer in model
- * order -- an attention layer contributes its key rows [0, seq_len) then its value rows [0, seq_len) (f32, [seq_len][kv_dim];
+ * order -- an attention layer contributes its key rows [0, seq_len) then its value rows [0, seq_len) (f32, or f16 for a model
+ * loaded with WICK_ROCM_KV_F16, [seq_len][kv_dim];
  * LayerSnapshot::Attention's k_data, v_data), a gated-conv layer its rolling buffer ((conv_kernel_size - 1) * hidden_size f32;
  * LayerSnapshot::Conv's buffer).  wick_rocm_lfm2_layer_state_bytes gives one layer's share (an attention layer's is split
  * evenly between keys and values), wick_rocm_lfm2_state_bytes the total; `nbytes` must equal it.  The position count itself

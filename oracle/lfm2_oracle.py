@@ -166,13 +166,23 @@ def quantizer_margin(x) -> float:
     return min(tie, float(edge.min()) * 1e3)
 
 
+def _f16_round(x) -> np.ndarray:
+    """f32 -> nearest-even f16 -> f32 (what a cache of f16 rows keeps of a value)."""
+    with np.errstate(over="ignore"):
+        return np.asarray(x, np.float32).astype(np.float16).astype(np.float32)
+
+
 class Lfm2Oracle:
     """`cfg`: n_layers, hidden_size, intermediate_size, n_heads, vocab_size, rope_theta, rms_norm_eps,
     conv_kernel_size, kv_heads_per_layer (0 = gated-conv layer).  `tensors`: GGUF name -> (ggml_type, dims, array),
     quantized weights as raw block bytes (dims [k, m]), norms / conv kernels as float32."""
 
-    def __init__(self, cfg: dict, tensors: dict, jitter_seed=None):
+    def __init__(self, cfg: dict, tensors: dict, jitter_seed=None, kv_f16=False):
         self.cfg, self.t = cfg, tensors
+        # KV caches of f16 rows, the reference's GPU models' caches (wick/src/model/metal_lfm2.rs:4117-4247: K after QK-norm and
+        # RoPE and V are cast to half on their way in, the attention reads half): every cached value is rounded to nearest even
+        # f16 when it is appended or moved by a context shift; the arithmetic on the widened values is the f32 one below.
+        self.kv_f16 = kv_f16
         self.min_margin = float("inf")  # smallest quantizer_margin over every GEMV input so far
         # Sensitivity probe: with a seed, every GEMV output is moved by up to 2^-22 of its value (about two ulp), which is
         # what another order of the f32 block sums does to it -- the order is not part of the contract (rel-L2 1e-5 is).
@@ -228,6 +238,8 @@ class Lfm2Oracle:
                     k[h * hd:(h + 1) * hd] = rmsnorm(k[h * hd:(h + 1) * hd], kn, eps)
                 q, k = rope(q, k, pos, c["n_heads"], n_kv, hd, c["rope_theta"])
                 ls = state["layers"][i]
+                if self.kv_f16:
+                    k, v = _f16_round(k), _f16_round(v)
                 ls["k"].append(k), ls["v"].append(v)
                 attn = attention(q, np.concatenate(ls["k"]), np.concatenate(ls["v"]), c["n_heads"], n_kv, hd, len(ls["k"]))
                 out = self._gemv(f"blk.{i}.attn_output.weight", attn)
@@ -259,6 +271,8 @@ class Lfm2Oracle:
                 continue
             assert len(ls["k"]) == seq
             k, v = shift_kv(np.concatenate(ls["k"]), np.concatenate(ls["v"]), seq, n_keep, shift, n_kv, hd, c["rope_theta"])
+            if self.kv_f16:  # the re-rotated keys go back into f16 rows (kept rows and values are f16 values already)
+                k = _f16_round(k)
             kvd = n_kv * hd
             ls["k"] = [k[t * kvd:(t + 1) * kvd].copy() for t in range(seq - shift)]
             ls["v"] = [v[t * kvd:(t + 1) * kvd].copy() for t in range(seq - shift)]

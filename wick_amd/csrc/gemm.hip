@@ -123,7 +123,6 @@ constexpr int kSlabWt = 2 * KB * GR * 16;           // 4096
 constexpr int kSlabDws = KB * GR * 8;               // 1024
 constexpr int kSlab = kSlabWt + kSlabDws;           // 5120
 constexpr int kSlabChunks = kSlab / 1024;           // 5 direct-to-LDS copies of 1 KB
-constexpr int kTileChunks = (BM / GR) * kSlabChunks;  // 20 per tile and stage
 
 // One stage of operands.
 template <int NTOK>  // tokens per workgroup tile: BN, or BN_NARROW for the narrow kernel

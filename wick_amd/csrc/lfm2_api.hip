@@ -189,9 +189,13 @@ size_t wick_rocm_attention_block_scratch_bytes(uint32_t max_seq, uint32_t n_head
     return attention_scratch_floats(max_seq, n_heads, head_dim) * sizeof(float);
 }
 
-int wick_rocm_attention_block(wick_rocm_ctx* ctx, float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
-                              float* d_k_cache, float* d_v_cache, float* d_out, void* d_scratch, uint32_t pos, const uint32_t* d_pos,
-                              uint32_t max_seq, uint32_t head_dim, uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale) {
+}  // extern "C"
+
+// The attention block over caches of either element type (the model handle's route; the public entry point below is the
+// f32-cache form).
+static int attention_block_kv(wick_rocm_ctx* ctx, float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
+                              void* d_k_cache, void* d_v_cache, float* d_out, void* d_scratch, uint32_t pos, const uint32_t* d_pos,
+                              uint32_t max_seq, uint32_t head_dim, uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale, bool kv_f16) {
     WR_ENTER(ctx);
     if (!d_q || !d_k || !d_v || !d_q_norm || !d_k_norm || !d_k_cache || !d_v_cache || !d_out || !d_scratch)
         return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "attention_block: null device pointer");
@@ -205,15 +209,24 @@ int wick_rocm_attention_block(wick_rocm_ctx* ctx, float* d_q, float* d_k, const 
     hipError_t e;
     if (attention_layer_applies(head_dim)) {
         e = launch_attention_layer(d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, d_out, partials, pos, d_pos, max_seq, n_heads,
-                                   n_kv_heads, head_dim, eps, theta_scale, scale, ctx->launch());
+                                   n_kv_heads, head_dim, eps, theta_scale, scale, ctx->launch(), kv_f16);
     } else {
         e = launch_qk_norm_rope(d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, pos, d_pos, max_seq, head_dim, n_heads, n_kv_heads, eps,
-                                theta_scale, ctx->launch());
+                                theta_scale, ctx->launch(), 1, 0, 0, kv_f16);
         if (e == hipSuccess)
             e = launch_attention_decode(d_q, d_k_cache, d_v_cache, d_out, partials, pos + 1u, d_pos, max_seq, n_heads, n_kv_heads, head_dim, scale,
-                                        ctx->launch());
+                                        ctx->launch(), kv_f16);
     }
     return e == hipSuccess ? WICK_ROCM_OK : fail_hip(ctx, e, "attention_block launch");
+}
+
+extern "C" {
+
+int wick_rocm_attention_block(wick_rocm_ctx* ctx, float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
+                              float* d_k_cache, float* d_v_cache, float* d_out, void* d_scratch, uint32_t pos, const uint32_t* d_pos,
+                              uint32_t max_seq, uint32_t head_dim, uint32_t n_heads, uint32_t n_kv_heads, float eps, float theta_scale) {
+    return attention_block_kv(ctx, d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, d_out, d_scratch, pos, d_pos, max_seq, head_dim, n_heads,
+                              n_kv_heads, eps, theta_scale, false);
 }
 
 int wick_rocm_shortconv_step(wick_rocm_ctx* ctx, const float* d_proj, float* d_buffer, const float* d_conv_weight, float* d_out, uint32_t hidden,
@@ -316,7 +329,8 @@ struct LayerWeights {
     wick_rocm_weight *q = nullptr, *k = nullptr, *v = nullptr, *o = nullptr;  // attention
     wick_rocm_weight *gate = nullptr, *up = nullptr, *down = nullptr;
     float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr, *conv_w = nullptr;
-    float *k_cache = nullptr, *v_cache = nullptr, *conv_state = nullptr;
+    void *k_cache = nullptr, *v_cache = nullptr;  // [max_seq][kv_dim] of the model's cache element type
+    float* conv_state = nullptr;
     bool conv_fused = false;  // gated-conv layer whose convolution rides in its out projection and gate / up launches
 };
 
@@ -341,7 +355,9 @@ struct wick_rocm_lfm2 {
     float *pX = nullptr, *pA = nullptr, *pG = nullptr, *pGate = nullptr, *pUp = nullptr, *pS = nullptr, *pS2 = nullptr, *pAttn = nullptr;
     int8_t *pQ = nullptr, *pQ2 = nullptr;
     uint32_t* pTokens = nullptr;
-    float* shift_stage = nullptr;  // staging rows of a context shift, allocated by the first one
+    void* shift_stage = nullptr;   // staging rows of a context shift, allocated by the first one
+    bool kv_f16 = false;           // the KV caches hold f16 rows (wick_rocm_lfm2_load_kv); f32 otherwise
+    size_t kv_elem() const { return kv_f16 ? 2 : 4; }
     wick_rocm_graph* g_step[3] = {nullptr, nullptr, nullptr};  // one captured step per StepMode
     bool use_graph = true;
     std::mutex mu;
@@ -445,8 +461,8 @@ int enqueue_step(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, StepMode mode) {
             }
         } else {
             if ((rc = gemv_normed(ctx, {L.q, L.k, L.v}, {m->q, m->k, m->v}, m->hidden, L.attn_norm, c.rms_norm_eps))) break;
-            if ((rc = wick_rocm_attention_block(ctx, m->q, m->k, m->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, m->attn, m->scores, 0, m->d_pos,
-                                                c.max_seq_len, hd, c.n_heads, L.n_kv, c.rms_norm_eps, m->theta_scale)))
+            if ((rc = attention_block_kv(ctx, m->q, m->k, m->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, m->attn, m->scores, 0, m->d_pos,
+                                         c.max_seq_len, hd, c.n_heads, L.n_kv, c.rms_norm_eps, m->theta_scale, m->kv_f16)))
                 break;
             if ((rc = gemv_residual(ctx, L.o, m->hidden, m->attn))) break;
         }
@@ -586,19 +602,21 @@ int enqueue_prompt_pass(wick_rocm_ctx* ctx, wick_rocm_lfm2* m, uint32_t n, uint3
             if ((rc = gemm_group(ctx, {L.q, L.k, L.v}, {q, k, v}, m, n, S))) break;
             if ((rc = locked([&] {
                      return launch_qk_norm_rope(q, k, v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, pos0, nullptr, c.max_seq_len, hd, c.n_heads, L.n_kv,
-                                                c.rms_norm_eps, m->theta_scale, ctx->launch(), n, S, S);
+                                                c.rms_norm_eps, m->theta_scale, ctx->launch(), n, S, S, m->kv_f16);
                  }, "qk_norm_rope launch")))
                 break;
             if (attention_layer_applies(hd)) {
                 quantized = attention_prefill_quantize_applies(q, L.k_cache, L.v_cache, n, S, hd);
                 rc = locked([&] {
                     return launch_attention_prefill(q, L.k_cache, L.v_cache, m->pG, m->pAttn, pos0, nullptr, n, S, hs, c.max_seq_len, c.n_heads, L.n_kv, hd,
-                                                    scale, ctx->launch(), quantized ? m->pQ : nullptr, quantized ? m->pS : nullptr);
+                                                    scale, ctx->launch(), quantized ? m->pQ : nullptr, quantized ? m->pS : nullptr, m->kv_f16);
                 }, "attention_prefill launch");
             } else {  // head dims without a batched kernel: the decode kernel, token by token
                 for (uint32_t j = 0; rc == 0 && j < n; j++)
-                    rc = wick_rocm_attention_decode(ctx, q + (size_t)j * S, L.k_cache, L.v_cache, m->pG + (size_t)j * hs, m->scores, pos0 + j + 1, nullptr,
-                                                    c.max_seq_len, c.n_heads, L.n_kv, hd);
+                    rc = locked([&] {
+                        return launch_attention_decode(q + (size_t)j * S, L.k_cache, L.v_cache, m->pG + (size_t)j * hs, m->scores, pos0 + j + 1, nullptr,
+                                                       c.max_seq_len, c.n_heads, L.n_kv, hd, scale, ctx->launch(), m->kv_f16);
+                    }, "attention_decode launch");
             }
             if (rc) break;
         }
@@ -641,7 +659,7 @@ int for_each_state_piece(const wick_rocm_lfm2* model, uint32_t seq_len, F&& piec
     const wick_rocm_lfm2_config& c = model->cfg;
     for (const LayerWeights& L : model->layers) {
         if (L.n_kv) {
-            const size_t half = (size_t)seq_len * L.n_kv * (c.hidden_size / c.n_heads) * sizeof(float);
+            const size_t half = (size_t)seq_len * L.n_kv * (c.hidden_size / c.n_heads) * model->kv_elem();
             if (half == 0) continue;
             if (int rc = piece(L.k_cache, half)) return rc;
             if (int rc = piece(L.v_cache, half)) return rc;
@@ -657,9 +675,17 @@ int for_each_state_piece(const wick_rocm_lfm2* model, uint32_t seq_len, F&& piec
 extern "C" {
 
 int wick_rocm_lfm2_load(wick_rocm_ctx* ctx, const wick_gguf* g, uint32_t context_size, wick_rocm_lfm2** out) {
+    return wick_rocm_lfm2_load_kv(ctx, g, context_size, WICK_ROCM_KV_F32, out);
+}
+
+int wick_rocm_lfm2_kv_dtype(const wick_rocm_lfm2* model) { return model && model->kv_f16 ? WICK_ROCM_KV_F16 : WICK_ROCM_KV_F32; }
+
+int wick_rocm_lfm2_load_kv(wick_rocm_ctx* ctx, const wick_gguf* g, uint32_t context_size, int kv_dtype, wick_rocm_lfm2** out) {
     if (!ctx) return WICK_ROCM_ERR_INVALID_ARG;
     if (!g || !out) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2_load: null argument");
     *out = nullptr;
+    if (kv_dtype != WICK_ROCM_KV_F32 && kv_dtype != WICK_ROCM_KV_F16)
+        return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2_load: kv_dtype must be WICK_ROCM_KV_F32 or WICK_ROCM_KV_F16");
     if (context_size == 0) return ctx_fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "lfm2_load: context_size must be > 0");
 
     // metadata, wick/src/model/lfm2.rs:104-136
@@ -695,6 +721,7 @@ int wick_rocm_lfm2_load(wick_rocm_ctx* ctx, const wick_gguf* g, uint32_t context
 
     std::unique_ptr<wick_rocm_lfm2> holder(new wick_rocm_lfm2);
     wick_rocm_lfm2* m = holder.get();
+    m->kv_f16 = kv_dtype == WICK_ROCM_KV_F16;
     auto bail = [&](int rc) {
         release(ctx, holder.release());
         return rc;
@@ -724,8 +751,8 @@ int wick_rocm_lfm2_load(wick_rocm_ctx* ctx, const wick_gguf* g, uint32_t context
             if ((rc = upload_weight(ctx, m, g, p + "attn_k.weight", kv_dim, hs, &L.k))) return bail(rc);
             if ((rc = upload_weight(ctx, m, g, p + "attn_v.weight", kv_dim, hs, &L.v))) return bail(rc);
             if ((rc = upload_weight(ctx, m, g, p + "attn_output.weight", hs, hs, &L.o))) return bail(rc);
-            if ((rc = alloc_t(ctx, m, (size_t)c.max_seq_len * kv_dim, &L.k_cache))) return bail(rc);
-            if ((rc = alloc_t(ctx, m, (size_t)c.max_seq_len * kv_dim, &L.v_cache))) return bail(rc);
+            if ((rc = alloc(ctx, m, (size_t)c.max_seq_len * kv_dim * m->kv_elem(), &L.k_cache))) return bail(rc);
+            if ((rc = alloc(ctx, m, (size_t)c.max_seq_len * kv_dim * m->kv_elem(), &L.v_cache))) return bail(rc);
         } else {
             if ((rc = upload_f32(ctx, m, g, p + "shortconv.conv.weight", (uint64_t)hs * c.conv_kernel_size, &L.conv_w))) return bail(rc);
             if ((rc = upload_weight(ctx, m, g, p + "shortconv.in_proj.weight", 3 * hs, hs, &L.in_proj))) return bail(rc);
@@ -963,7 +990,7 @@ size_t wick_rocm_lfm2_layer_state_bytes(const wick_rocm_lfm2* model, uint32_t la
     if (!model || layer >= model->cfg.n_layers || seq_len > model->cfg.max_seq_len) return 0;
     const wick_rocm_lfm2_config& c = model->cfg;
     const LayerWeights& L = model->layers[layer];
-    if (L.n_kv) return 2 * (size_t)seq_len * L.n_kv * (c.hidden_size / c.n_heads) * sizeof(float);
+    if (L.n_kv) return 2 * (size_t)seq_len * L.n_kv * (c.hidden_size / c.n_heads) * model->kv_elem();
     return (size_t)(c.conv_kernel_size - 1) * c.hidden_size * sizeof(float);
 }
 
@@ -1015,10 +1042,13 @@ int wick_rocm_lfm2_shift_kv(wick_rocm_ctx* ctx, wick_rocm_lfm2* model, uint32_t 
     if (seq_len - n_keep - shift == 0) return WICK_ROCM_OK;  // nothing behind the dropped rows: only the caller's seq_len changes
     const uint32_t hd = c.hidden_size / c.n_heads;
     if (!model->shift_stage && c.n_kv_heads)
-        if (int rc = alloc_t(ctx, model, 2 * (size_t)c.max_seq_len * c.n_kv_heads * hd, &model->shift_stage)) return rc;
+        if (int rc = alloc(ctx, model, 2 * (size_t)c.max_seq_len * c.n_kv_heads * hd * model->kv_elem(), &model->shift_stage)) return rc;
     for (const LayerWeights& L : model->layers)  // conv layers keep their rolling buffer (wick/src/kv_cache.rs:584-590)
-        if (L.n_kv)
-            if (int rc = wick_rocm_kv_shift(ctx, L.k_cache, L.v_cache, model->shift_stage, seq_len, n_keep, shift, L.n_kv, hd, model->theta_scale)) return rc;
+        if (L.n_kv) {
+            const hipError_t e = launch_kv_shift(L.k_cache, L.v_cache, model->shift_stage, seq_len, n_keep, shift, L.n_kv, hd, model->theta_scale,
+                                                 ctx->launch(), model->kv_f16);
+            if (e != hipSuccess) return fail_hip(ctx, e, "kv_shift launch");
+        }
     return wick_rocm_sync(ctx);
 }
 

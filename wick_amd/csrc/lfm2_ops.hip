@@ -19,6 +19,29 @@ namespace wick_rocm {
 
 namespace {
 
+// The KV caches hold f32 rows, like the reference's CPU model (wick/src/kv_cache.rs), or f16 rows, like its GPU models
+// (wick/src/model/metal_lfm2.rs:4117-4247: K after QK-norm and RoPE and V are cast to half on their way into the caches and
+// the attention kernels read half).  Every kernel that touches a cache is a template over the element type KV: a value is
+// rounded once, to nearest even, when it is appended (or moved by a context shift) and widened exactly when it is read; all
+// arithmetic stays f32.
+typedef _Float16 kv_h4 __attribute__((ext_vector_type(4)));
+template <typename KV>
+__device__ __forceinline__ float4 kv_load4(const KV* p) {
+    if constexpr (std::is_same<KV, float>::value) {
+        return *reinterpret_cast<const float4*>(p);
+    } else {
+        const kv_h4 v = *reinterpret_cast<const kv_h4*>(p);
+        return make_float4((float)v[0], (float)v[1], (float)v[2], (float)v[3]);
+    }
+}
+template <typename KV>
+__device__ __forceinline__ float kv_load(const KV* p) { return (float)*p; }
+template <typename KV>
+__device__ __forceinline__ void kv_store(KV* p, float v) { *p = (KV)v; }
+// launch_kernel over the cache element type: F(float{}) or F(_Float16{}).
+template <typename F>
+inline hipError_t with_kv_type(bool kv_f16, F&& f) { return kv_f16 ? f(_Float16{}) : f(float{}); }
+
 // Sum over a block of up to 16 waves; every thread gets the total.  `slots` holds 16 doubles.
 __device__ __forceinline__ double block_sum_f64(double v, double* slots) {
     v = wave_sum_f64(v);
@@ -103,8 +126,8 @@ struct QkNormRopeArgs {
     const float* v;         // [n_kv_heads * head_dim]
     const float* q_norm;    // [head_dim]
     const float* k_norm;    // [head_dim]
-    float* k_cache;         // [max_seq][kv_dim]
-    float* v_cache;
+    void* k_cache;          // [max_seq][kv_dim] of the cache's element type
+    void* v_cache;
     const uint32_t* d_pos;  // may be null
     uint32_t pos, max_seq, head_dim, n_heads, n_kv_heads;
     float eps, theta_scale;
@@ -121,8 +144,9 @@ __device__ __forceinline__ void rope_sincos(uint32_t pos, uint32_t i, float thet
 
 // RMSNorm + RoPE of one head by the calling wave: dst[] (and dst2[], when given) receive the result; src may equal dst.
 // sn_tab / cs_tab: the position's sines and cosines per pair when the caller has them already (else computed here).
+template <typename D1, typename D2>
 __device__ __forceinline__ void norm_rope_head(const float* src, const float* w, uint32_t hd, uint32_t pos, float eps, float theta_scale,
-                                               float* dst, float* dst2, const float* sn_tab = nullptr, const float* cs_tab = nullptr) {
+                                               D1* dst, D2* dst2, const float* sn_tab = nullptr, const float* cs_tab = nullptr) {
     const uint32_t lane = threadIdx.x & 63u, half = hd >> 1;
     double s = 0.0;
     for (uint32_t i = lane; i < hd; i += 64) {
@@ -138,11 +162,12 @@ __device__ __forceinline__ void norm_rope_head(const float* src, const float* w,
         const float x1 = __fmul_rn(__fmul_rn(src[i + half], inv_rms), w[i + half]);
         const float r0 = __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn));
         const float r1 = __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, cs));
-        dst[i] = r0, dst[i + half] = r1;
-        if (dst2) dst2[i] = r0, dst2[i + half] = r1;
+        kv_store(dst + i, r0), kv_store(dst + i + half, r1);
+        if (dst2) kv_store(dst2 + i, r0), kv_store(dst2 + i + half, r1);
     }
 }
 
+template <typename KV>
 __device__ __forceinline__ void qk_norm_rope_one_head(const QkNormRopeArgs& a, uint32_t tok, uint32_t pos, uint32_t hh, const float* sn_tab,
                                                       const float* cs_tab) {
     const bool is_q = hh < a.n_heads;
@@ -151,35 +176,38 @@ __device__ __forceinline__ void qk_norm_rope_one_head(const QkNormRopeArgs& a, u
     float* head = (is_q ? a.q + (size_t)tok * a.q_stride : a.k + (size_t)tok * a.kv_stride) + (size_t)h * hd;
     const bool store = !is_q && pos < a.max_seq;  // the host checks a by-value pos; a device-side pos past the cache is dropped
     norm_rope_head(head, is_q ? a.q_norm : a.k_norm, hd, pos, a.eps, a.theta_scale, head,
-                   store ? a.k_cache + (size_t)pos * kv_dim + (size_t)h * hd : nullptr, sn_tab, cs_tab);
+                   store ? static_cast<KV*>(a.k_cache) + (size_t)pos * kv_dim + (size_t)h * hd : static_cast<KV*>(nullptr), sn_tab, cs_tab);
     if (store) {
         const float* vh = a.v + (size_t)tok * a.kv_stride + (size_t)h * hd;
-        float* vc = a.v_cache + (size_t)pos * kv_dim + (size_t)h * hd;
-        for (uint32_t i = threadIdx.x & 63u; i < hd; i += 64) vc[i] = vh[i];
+        KV* vc = static_cast<KV*>(a.v_cache) + (size_t)pos * kv_dim + (size_t)h * hd;
+        for (uint32_t i = threadIdx.x & 63u; i < hd; i += 64) kv_store(vc + i, vh[i]);
     }
 }
 
+template <typename KV>
 __global__ __launch_bounds__(64) void qk_norm_rope_kernel(QkNormRopeArgs a) {
     const uint32_t tok = blockIdx.y;
     const uint32_t pos = (a.d_pos ? *a.d_pos : a.pos) + tok;
-    qk_norm_rope_one_head(a, tok, pos, blockIdx.x, nullptr, nullptr);
+    qk_norm_rope_one_head<KV>(a, tok, pos, blockIdx.x, nullptr, nullptr);
 }
 
 // The same for the tokens of a prompt: one workgroup per token works out the position's sines and cosines once (every
 // head of the token uses the same ones) and its four waves share the heads.  Same operations per element: bit-identical.
 constexpr uint32_t kRopeTableMax = 128;  // pairs = head_dim / 2
+template <typename KV>
 __global__ __launch_bounds__(256) void qk_norm_rope_tokens_kernel(QkNormRopeArgs a) {
     __shared__ float sn_tab[kRopeTableMax], cs_tab[kRopeTableMax];
     const uint32_t tok = blockIdx.x;
     const uint32_t pos = (a.d_pos ? *a.d_pos : a.pos) + tok;
     for (uint32_t i = threadIdx.x; i < (a.head_dim >> 1); i += 256) rope_sincos(pos, i, a.theta_scale, sn_tab[i], cs_tab[i]);
     __syncthreads();
-    for (uint32_t hh = threadIdx.x >> 6; hh < a.n_heads + a.n_kv_heads; hh += 4) qk_norm_rope_one_head(a, tok, pos, hh, sn_tab, cs_tab);
+    for (uint32_t hh = threadIdx.x >> 6; hh < a.n_heads + a.n_kv_heads; hh += 4) qk_norm_rope_one_head<KV>(a, tok, pos, hh, sn_tab, cs_tab);
 }
 
 // head_dim 64: a lane owns one element of a head, so a wave keeps up to six heads in flight -- all their loads first,
 // then the arithmetic, then the stores: one memory round trip per wave instead of one per head.  The rotation partner
 // (element i +- 32) comes through a lane exchange of the normalised value.  Same operations per element: bit-identical.
+template <typename KV>
 __global__ __launch_bounds__(256) void qk_norm_rope_tokens64_kernel(QkNormRopeArgs a) {
     constexpr uint32_t HD = 64, HB = 6;
     __shared__ float sn_tab[HD / 2], cs_tab[HD / 2];
@@ -218,8 +246,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_tokens64_kernel(QkNormRopeAr
             head[t][lane] = r;
             if (!is_q && store) {
                 const size_t at = (size_t)pos * kv_dim + (size_t)(hh - a.n_heads) * HD + lane;
-                a.k_cache[at] = r;
-                a.v_cache[at] = vv[t];
+                kv_store(static_cast<KV*>(a.k_cache) + at, r);
+                kv_store(static_cast<KV*>(a.v_cache) + at, vv[t]);
             }
         }
     }
@@ -234,15 +262,16 @@ __global__ __launch_bounds__(256) void qk_norm_rope_tokens64_kernel(QkNormRopeAr
 // staging buffers ([retained][kv_dim] each) and plain device copies put them in place afterwards.  A workgroup takes
 // kShiftRows rows and computes the sines and cosines once for all of them.
 struct KvShiftArgs {
-    const float* k_cache;
-    const float* v_cache;
-    float* k_stage;
-    float* v_stage;
+    const void* k_cache;  // caches and staging buffers of the cache's element type
+    const void* v_cache;
+    void* k_stage;
+    void* v_stage;
     uint32_t n_keep, shift, retained, n_kv_heads, head_dim;
     float theta_scale;
 };
 constexpr uint32_t kShiftRows = 8;
 
+template <typename KV>
 __global__ __launch_bounds__(256) void kv_shift_stage_kernel(KvShiftArgs a) {
     __shared__ float sn_tab[kRopeTableMax], cs_tab[kRopeTableMax];
     const uint32_t hd = a.head_dim, half = hd >> 1, kv_dim = a.n_kv_heads * hd;
@@ -254,16 +283,16 @@ __global__ __launch_bounds__(256) void kv_shift_stage_kernel(KvShiftArgs a) {
     __syncthreads();
     const uint32_t r0 = blockIdx.x * kShiftRows, r1 = r0 + kShiftRows < a.retained ? r0 + kShiftRows : a.retained;
     for (uint32_t r = r0; r < r1; r++) {
-        const float* ks = a.k_cache + (size_t)(a.n_keep + a.shift + r) * kv_dim;
-        const float* vs = a.v_cache + (size_t)(a.n_keep + a.shift + r) * kv_dim;
-        float* kd = a.k_stage + (size_t)r * kv_dim;
-        float* vd = a.v_stage + (size_t)r * kv_dim;
+        const KV* ks = static_cast<const KV*>(a.k_cache) + (size_t)(a.n_keep + a.shift + r) * kv_dim;
+        const KV* vs = static_cast<const KV*>(a.v_cache) + (size_t)(a.n_keep + a.shift + r) * kv_dim;
+        KV* kd = static_cast<KV*>(a.k_stage) + (size_t)r * kv_dim;
+        KV* vd = static_cast<KV*>(a.v_stage) + (size_t)r * kv_dim;
         for (uint32_t e = threadIdx.x; e < a.n_kv_heads * half; e += 256) {
             const uint32_t at = (e / half) * hd + e % half;
             const float sn = sn_tab[e % half], cs = cs_tab[e % half];
-            const float x0 = ks[at], x1 = ks[at + half];
-            kd[at] = __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn));
-            kd[at + half] = __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, cs));
+            const float x0 = kv_load(ks + at), x1 = kv_load(ks + at + half);
+            kv_store(kd + at, __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn)));
+            kv_store(kd + at + half, __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, cs)));
         }
         for (uint32_t e = threadIdx.x; e < kv_dim; e += 256) vd[e] = vs[e];
     }
@@ -279,8 +308,8 @@ __global__ __launch_bounds__(256) void kv_shift_stage_kernel(KvShiftArgs a) {
 // `scores` is scratch [n_heads][max_seq].
 struct AttentionArgs {
     const float* q;
-    const float* k_cache;
-    const float* v_cache;
+    const void* k_cache;  // of the cache's element type
+    const void* v_cache;
     float* out;     // [n_heads * head_dim]
     float* scores;  // [n_heads][max_seq]
     const uint32_t* d_pos;  // seq_len = *d_pos + 1 when non-null
@@ -288,6 +317,7 @@ struct AttentionArgs {
     float scale;
 };
 
+template <typename KV>
 __global__ __launch_bounds__(256) void attention_decode_kernel(AttentionArgs a) {
     __shared__ double slots[16];
     __shared__ float red[256];
@@ -296,8 +326,8 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttentionArgs a) 
     uint32_t seq = a.d_pos ? *a.d_pos + 1u : a.seq_len;
     if (seq > a.max_seq) seq = a.max_seq;
     const uint32_t kvh = h / (a.n_heads / a.n_kv_heads);
-    const float* kbase = a.k_cache + (size_t)kvh * hd;
-    const float* vbase = a.v_cache + (size_t)kvh * hd;
+    const KV* kbase = static_cast<const KV*>(a.k_cache) + (size_t)kvh * hd;
+    const KV* vbase = static_cast<const KV*>(a.v_cache) + (size_t)kvh * hd;
     float* sc = a.scores + (size_t)h * a.max_seq;
     const uint32_t tid = threadIdx.x;
 
@@ -306,10 +336,10 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttentionArgs a) 
 
     float mx = -__builtin_inff();
     for (uint32_t t = tid; t < seq; t += 256) {
-        const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)t * kv_dim);
+        const KV* kr = kbase + (size_t)t * kv_dim;
         float dot = 0.0f;
         for (uint32_t d = 0; d < hd; d += 4) {
-            const float4 kv = kr[d >> 2];
+            const float4 kv = kv_load4(kr + d);
             dot = __fadd_rn(dot, __fmul_rn(qs[d], kv.x));
             dot = __fadd_rn(dot, __fmul_rn(qs[d + 1], kv.y));
             dot = __fadd_rn(dot, __fmul_rn(qs[d + 2], kv.z));
@@ -342,7 +372,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttentionArgs a) 
     const uint32_t d = tid % lanes, part = tid / lanes;
     float acc = 0.0f;
     if (part < parts) {
-        for (uint32_t t = part; t < seq; t += parts) acc = __fadd_rn(acc, __fmul_rn(__fmul_rn(sc[t], inv), vbase[(size_t)t * kv_dim + d]));
+        for (uint32_t t = part; t < seq; t += parts) acc = __fadd_rn(acc, __fmul_rn(__fmul_rn(sc[t], inv), kv_load(vbase + (size_t)t * kv_dim + d)));
     }
     __syncthreads();
     red[tid] = acc;
@@ -365,7 +395,7 @@ constexpr uint32_t kAttnMaxSplits = 64;   // workgroups per head; contexts beyon
 
 // The chunks of workgroup (h, split): scores against q (HD floats, 16-byte aligned, global or LDS), streaming softmax,
 // weighted values; leaves {max, sum, acc[HD]} in the partial record of (h, split).  All 256 threads call it.
-template <int HD>
+template <int HD, typename KV>
 __device__ __forceinline__ void attention_chunks(const AttentionArgs& a, uint32_t splits, uint32_t h, uint32_t split, uint32_t seq, const float* q) {
     constexpr uint32_t LR = HD / 4;                  // lanes per cache row
     constexpr uint32_t RPP = 256 / LR;               // rows per pass of the block
@@ -379,8 +409,8 @@ __device__ __forceinline__ void attention_chunks(const AttentionArgs& a, uint32_
     __shared__ float red[256];
     const uint32_t kv_dim = a.n_kv_heads * HD;
     const uint32_t kvh = h / (a.n_heads / a.n_kv_heads);
-    const float* kbase = a.k_cache + (size_t)kvh * HD;
-    const float* vbase = a.v_cache + (size_t)kvh * HD;
+    const KV* kbase = static_cast<const KV*>(a.k_cache) + (size_t)kvh * HD;
+    const KV* vbase = static_cast<const KV*>(a.v_cache) + (size_t)kvh * HD;
     const uint32_t tid = threadIdx.x, quad = tid % LR, prow = tid / LR, d = tid % HD, g = tid / HD;
     const float4 q4 = reinterpret_cast<const float4*>(q)[quad];
     const uint32_t last = seq - 1u;
@@ -397,7 +427,7 @@ __device__ __forceinline__ void attention_chunks(const AttentionArgs& a, uint32_
 #pragma unroll
             for (uint32_t j = 0; j < KB; j++) {
                 const uint32_t row = t0 + prow + (i + j) * RPP;
-                kv[j] = reinterpret_cast<const float4*>(kbase + (size_t)(row < last ? row : last) * kv_dim)[quad];
+                kv[j] = kv_load4(kbase + (size_t)(row < last ? row : last) * kv_dim + 4u * quad);
             }
 #pragma unroll
             for (uint32_t j = 0; j < KB; j++) {
@@ -427,7 +457,7 @@ __device__ __forceinline__ void attention_chunks(const AttentionArgs& a, uint32_
 #pragma unroll
             for (uint32_t j = 0; j < VB; j++) {
                 const uint32_t row = t0 + g + (i + j) * VG;
-                vv[j] = vbase[(size_t)(row < last ? row : last) * kv_dim + d];
+                vv[j] = kv_load(vbase + (size_t)(row < last ? row : last) * kv_dim + d);
             }
 #pragma unroll
             for (uint32_t j = 0; j < VB; j++) acc += sc[g + (i + j) * VG] * vv[j];
@@ -499,12 +529,12 @@ __device__ __forceinline__ uint32_t attention_seq(const AttentionArgs& a) {
     return seq > a.max_seq ? a.max_seq : seq;
 }
 
-template <int HD>
+template <int HD, typename KV>
 __global__ __launch_bounds__(256) void attention_split_kernel(AttentionArgs a, uint32_t splits) {
     const uint32_t h = blockIdx.x / splits, split = blockIdx.x % splits;
     const uint32_t seq = attention_seq(a);
     if (split * kAttnChunk >= seq) return;  // the combine step derives the number of partials from seq as well
-    attention_chunks<HD>(a, splits, h, split, seq, a.q + (size_t)h * HD);
+    attention_chunks<HD, KV>(a, splits, h, split, seq, a.q + (size_t)h * HD);
 }
 
 template <int HD>
@@ -528,12 +558,12 @@ struct AttentionLayerArgs {
     const float* v;       // [n_kv_heads * HD]
     const float* q_norm;
     const float* k_norm;
-    float* k_cache;       // the same caches, writable
-    float* v_cache;
+    void* k_cache;        // the same caches, writable
+    void* v_cache;
     float eps, theta_scale;
 };
 
-template <int HD>
+template <int HD, typename KV>
 __global__ __launch_bounds__(256) void attention_layer_kernel(AttentionLayerArgs f, uint32_t splits) {
     __shared__ __align__(16) float qh[HD];
     const AttentionArgs& a = f.at;
@@ -541,19 +571,19 @@ __global__ __launch_bounds__(256) void attention_layer_kernel(AttentionLayerArgs
     const uint32_t seq = attention_seq(a);
     if (seq == 0 || split * kAttnChunk >= seq) return;
     const uint32_t pos = seq - 1u, kv_dim = a.n_kv_heads * HD, kvh = h / (a.n_heads / a.n_kv_heads);
-    if (tid < 64) norm_rope_head(f.q_raw + (size_t)h * HD, f.q_norm, HD, pos, f.eps, f.theta_scale, qh, nullptr);
+    if (tid < 64) norm_rope_head(f.q_raw + (size_t)h * HD, f.q_norm, HD, pos, f.eps, f.theta_scale, qh, static_cast<float*>(nullptr));
     if ((pos / kAttnChunk) % splits == split) {  // this workgroup's chunks include the new position
         if (tid >= 64 && tid < 128)
-            norm_rope_head(f.k_raw + (size_t)kvh * HD, f.k_norm, HD, pos, f.eps, f.theta_scale, f.k_cache + (size_t)pos * kv_dim + (size_t)kvh * HD,
-                           nullptr);
+            norm_rope_head(f.k_raw + (size_t)kvh * HD, f.k_norm, HD, pos, f.eps, f.theta_scale,
+                           static_cast<KV*>(f.k_cache) + (size_t)pos * kv_dim + (size_t)kvh * HD, static_cast<float*>(nullptr));
         if (tid >= 128) {
             const float* vh = f.v + (size_t)kvh * HD;
-            float* vc = f.v_cache + (size_t)pos * kv_dim + (size_t)kvh * HD;
-            for (uint32_t i = tid - 128; i < HD; i += 128) vc[i] = vh[i];
+            KV* vc = static_cast<KV*>(f.v_cache) + (size_t)pos * kv_dim + (size_t)kvh * HD;
+            for (uint32_t i = tid - 128; i < HD; i += 128) kv_store(vc + i, vh[i]);
         }
     }
     __syncthreads();  // qh[] and this workgroup's cache rows are complete
-    attention_chunks<HD>(a, splits, h, split, seq, qh);
+    attention_chunks<HD, KV>(a, splits, h, split, seq, qh);
 }
 
 // Causal attention for the n tokens of a prompt whose K / V rows are already in the caches (pass B of the reference's
@@ -563,7 +593,7 @@ __global__ __launch_bounds__(256) void attention_layer_kernel(AttentionLayerArgs
 // Per chunk: scores of the 8 queries (rows past a query's own position masked), streaming softmax with each wave
 // owning two queries (64 positions = one wave: shuffles only), then the weighted value sums for all eight from one set
 // of value loads.  q: [n][q_stride] floats, out: [n][out_stride].
-template <int HD>
+template <int HD, typename KV>
 __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride) {
     constexpr uint32_t QB = 8;
     constexpr uint32_t LR = HD / 4, RPP = 256 / LR, KROWS = kAttnChunk / RPP, KB = KROWS < 4 ? KROWS : 4;
@@ -577,8 +607,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
     const uint32_t nq = n - j0 < QB ? n - j0 : QB;  // queries of this workgroup
     const uint32_t base = a.d_pos ? *a.d_pos : pos0;
     const uint32_t kv_dim = a.n_kv_heads * HD, kvh = h / (a.n_heads / a.n_kv_heads);
-    const float* kbase = a.k_cache + (size_t)kvh * HD;
-    const float* vbase = a.v_cache + (size_t)kvh * HD;
+    const KV* kbase = static_cast<const KV*>(a.k_cache) + (size_t)kvh * HD;
+    const KV* vbase = static_cast<const KV*>(a.v_cache) + (size_t)kvh * HD;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, quad = tid % LR, prow = tid / LR, d = tid % HD, g = tid / HD;
     uint32_t seq_max = base + j0 + nq;  // positions the last query sees
     if (seq_max > a.max_seq) seq_max = a.max_seq;
@@ -600,7 +630,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
 #pragma unroll
             for (uint32_t jj = 0; jj < KB; jj++) {
                 const uint32_t row = t0 + prow + (i + jj) * RPP;
-                kv[jj] = reinterpret_cast<const float4*>(kbase + (size_t)(row < last ? row : last) * kv_dim)[quad];
+                kv[jj] = kv_load4(kbase + (size_t)(row < last ? row : last) * kv_dim + 4u * quad);
             }
 #pragma unroll
             for (uint32_t jj = 0; jj < KB; jj++) {
@@ -639,7 +669,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionArgs a,
 #pragma unroll
             for (uint32_t jj = 0; jj < VB; jj++) {
                 const uint32_t row = t0 + g * VROWS + i + jj;
-                vv[jj] = vbase[(size_t)(row < last ? row : last) * kv_dim + d];
+                vv[jj] = kv_load(vbase + (size_t)(row < last ? row : last) * kv_dim + d);
             }
 #pragma unroll
             for (uint32_t q = 0; q < QB; q++) {
@@ -731,9 +761,12 @@ __device__ __forceinline__ float groups_sum(float v) {
 // last bit or two; the streaming softmax of this kernel differs from the reference's two-pass one at that level anyway.
 __device__ __forceinline__ float exp_nonpos_hw(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 
-template <int HALVES>
+// KV = _Float16 (f16 caches): K and V are their own high halves and have no low halves, so the K_lo Q_hi and V_lo P_hi
+// products, their operand reads and the low planes' LDS writes drop out (8 of the 12 MFMAs per wave and tile remain).
+template <int HALVES, typename KV>
 __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(AttentionArgs a, uint32_t pos0, uint32_t n, uint32_t q_stride, uint32_t out_stride,
                                                                                 int8_t* q_out, float* s_out) {
+    constexpr bool LO = std::is_same<KV, float>::value;  // the caches' values have low halves
     constexpr int HD = 64, KT = 64, NT = 512 * HALVES;
     constexpr int LDH = 72;  // f16 per K row: 64 + 8 (144 bytes: 16-byte aligned rows, conflict-free 16-byte operand reads)
     constexpr int LDV = 68;  // f16 per V^T row: 64 + 4 (136 bytes: 8-byte aligned rows; 64 rows' 8-byte writes cover all banks twice)
@@ -751,8 +784,8 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
     const uint32_t j0 = qb * 64u;
     const uint32_t base = a.d_pos ? *a.d_pos : pos0;
     const uint32_t kv_dim = a.n_kv_heads * HD, kvh = h / (a.n_heads / a.n_kv_heads);
-    const float* kbase = a.k_cache + (size_t)kvh * HD;
-    const float* vbase = a.v_cache + (size_t)kvh * HD;
+    const KV* kbase = static_cast<const KV*>(a.k_cache) + (size_t)kvh * HD;
+    const KV* vbase = static_cast<const KV*>(a.v_cache) + (size_t)kvh * HD;
     const uint32_t jq = j0 + 16u * wave + l16;
     const uint32_t jl = jq < n ? jq : n - 1u;
     const uint32_t pq = base + jl;
@@ -788,8 +821,8 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
 #pragma unroll
         for (int i = 0; i < NR; i++) {
             const uint32_t key = min(t0 + r0 + i * RPP, wg_last);
-            kk[i] = reinterpret_cast<const float4*>(kbase + (size_t)key * kv_dim)[c4];
-            vv[i] = reinterpret_cast<const float4*>(vbase + (size_t)key * kv_dim)[c4];
+            kk[i] = kv_load4(kbase + (size_t)key * kv_dim + 4u * c4);
+            vv[i] = kv_load4(vbase + (size_t)key * kv_dim + 4u * c4);
         }
     };
     // A thread holds one key x four dims of K and of V.  K rows go to LDS as they are; V is transposed on the way: the four
@@ -812,7 +845,7 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
                 vp[j] = (uint32_t)__builtin_bit_cast(uint16_t, hi) | ((uint32_t)__builtin_bit_cast(uint16_t, lo) << 16);
             }
             *reinterpret_cast<h4*>(&kbuf[buf][0][key][4 * c4]) = khi;
-            *reinterpret_cast<h4*>(&kbuf[buf][1][key][4 * c4]) = klo;
+            if constexpr (LO) *reinterpret_cast<h4*>(&kbuf[buf][1][key][4 * c4]) = klo;
             // transpose M[g][j] (g = lane group = key, j = register = dim) in 2 x 2 blocks, then the blocks themselves
             auto s01 = __builtin_amdgcn_permlane16_swap(vp[0], vp[1], false, false);
             auto s23 = __builtin_amdgcn_permlane16_swap(vp[2], vp[3], false, false);
@@ -824,7 +857,7 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
             vlo.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u), vlo.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
             const uint32_t key4 = key & ~3u;
             *reinterpret_cast<uint2*>(&vbuf[buf][0][4 * c4 + g][key4]) = vhi;
-            *reinterpret_cast<uint2*>(&vbuf[buf][1][4 * c4 + g][key4]) = vlo;
+            if constexpr (LO) *reinterpret_cast<uint2*>(&vbuf[buf][1][4 * c4 + g][key4]) = vlo;
         }
     };
     fetch_tile(0);
@@ -843,12 +876,14 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
 #pragma unroll
                 for (int u = 0; u < 2; u++) {
                     kh[s][u] = *reinterpret_cast<const h8*>(&kbuf[cur][0][32u * ksp + 16 * u + l16][32 * s + 8 * g]);
-                    kl[s][u] = *reinterpret_cast<const h8*>(&kbuf[cur][1][32u * ksp + 16 * u + l16][32 * s + 8 * g]);
+                    if constexpr (LO) kl[s][u] = *reinterpret_cast<const h8*>(&kbuf[cur][1][32u * ksp + 16 * u + l16][32 * s + 8 * g]);
                 }
 #pragma unroll
             for (int s = 0; s < 2; s++) {
+                if constexpr (LO) {
 #pragma unroll
-                for (int u = 0; u < 2; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kl[s][u], qh[s], sc[u], 0, 0, 0);
+                    for (int u = 0; u < 2; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kl[s][u], qh[s], sc[u], 0, 0, 0);
+                }
 #pragma unroll
                 for (int u = 0; u < 2; u++) sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh[s][u], ql[s], sc[u], 0, 0, 0);
 #pragma unroll
@@ -860,10 +895,12 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
             for (int c = 0; c < 4; c++) {
                 const h4 a0 = *reinterpret_cast<const h4*>(&vbuf[cur][0][16 * c + l16][32u * ksp + 4 * g]);
                 const h4 a1 = *reinterpret_cast<const h4*>(&vbuf[cur][0][16 * c + l16][32u * ksp + 16 + 4 * g]);
-                const h4 b0 = *reinterpret_cast<const h4*>(&vbuf[cur][1][16 * c + l16][32u * ksp + 4 * g]);
-                const h4 b1 = *reinterpret_cast<const h4*>(&vbuf[cur][1][16 * c + l16][32u * ksp + 16 + 4 * g]);
                 vh[c] = h8{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-                vl[c] = h8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+                if constexpr (LO) {
+                    const h4 b0 = *reinterpret_cast<const h4*>(&vbuf[cur][1][16 * c + l16][32u * ksp + 4 * g]);
+                    const h4 b1 = *reinterpret_cast<const h4*>(&vbuf[cur][1][16 * c + l16][32u * ksp + 16 + 4 * g]);
+                    vl[c] = h8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+                }
             }
             float tmax = -__builtin_inff();
             const bool masked_tile = key0 + 31u > base + min(j0 + 16u * wave, n - 1u);
@@ -894,8 +931,10 @@ __global__ __launch_bounds__(512 * HALVES) void attention_prefill_f16x3_kernel(A
             l_run = l_run * alpha + psum;
 #pragma unroll
             for (int c = 0; c < 4; c++) o[c] *= alpha;
+            if constexpr (LO) {
 #pragma unroll
-            for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vl[c], ph, o[c], 0, 0, 0);
+                for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vl[c], ph, o[c], 0, 0, 0);
+            }
 #pragma unroll
             for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vh[c], pl, o[c], 0, 0, 0);
 #pragma unroll
@@ -1381,39 +1420,47 @@ hipError_t launch_rmsnorm(const float* d_x, const float* d_weight, float* d_y, u
     return launch_kernel(L, kFamOther, rmsnorm_kernel, dim3(rows), dim3(256), d_x, d_weight, d_y, dim, x_stride, y_stride, eps);
 }
 
-hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm, float* d_k_cache,
-                               float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
+hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm, void* d_k_cache,
+                               void* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
                                uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L, uint32_t n_tokens, uint32_t q_stride,
-                               uint32_t kv_stride) {
+                               uint32_t kv_stride, bool kv_f16) {
     if (n_tokens == 0) return hipSuccess;
     QkNormRopeArgs a{d_q, d_k, d_v, d_q_norm, d_k_norm, d_k_cache, d_v_cache, d_pos, pos, max_seq, head_dim, n_heads, n_kv_heads, eps, theta_scale,
                      q_stride, kv_stride};
-    if (n_tokens > 1 && head_dim == 64) return launch_kernel(L, kFamOther, qk_norm_rope_tokens64_kernel, dim3(n_tokens), dim3(256), a);
-    if (n_tokens > 1 && head_dim / 2 <= kRopeTableMax) return launch_kernel(L, kFamOther, qk_norm_rope_tokens_kernel, dim3(n_tokens), dim3(256), a);
-    return launch_kernel(L, kFamOther, qk_norm_rope_kernel, dim3(n_heads + n_kv_heads, n_tokens), dim3(64), a);
+    return with_kv_type(kv_f16, [&](auto kv) {
+        using KV = decltype(kv);
+        if (n_tokens > 1 && head_dim == 64) return launch_kernel(L, kFamOther, qk_norm_rope_tokens64_kernel<KV>, dim3(n_tokens), dim3(256), a);
+        if (n_tokens > 1 && head_dim / 2 <= kRopeTableMax) return launch_kernel(L, kFamOther, qk_norm_rope_tokens_kernel<KV>, dim3(n_tokens), dim3(256), a);
+        return launch_kernel(L, kFamOther, qk_norm_rope_kernel<KV>, dim3(n_heads + n_kv_heads, n_tokens), dim3(64), a);
+    });
 }
 
-hipError_t launch_kv_shift(float* d_k_cache, float* d_v_cache, float* d_stage, uint32_t seq_len, uint32_t n_keep, uint32_t shift,
-                           uint32_t n_kv_heads, uint32_t head_dim, float theta_scale, const Launch& L) {
+hipError_t launch_kv_shift(void* d_k_cache, void* d_v_cache, void* d_stage, uint32_t seq_len, uint32_t n_keep, uint32_t shift,
+                           uint32_t n_kv_heads, uint32_t head_dim, float theta_scale, const Launch& L, bool kv_f16) {
     const uint32_t retained = seq_len - n_keep - shift;
     if (retained == 0) return hipSuccess;  // everything behind n_keep is dropped: nothing moves
-    const size_t kv_dim = (size_t)n_kv_heads * head_dim, floats = (size_t)retained * kv_dim;
-    KvShiftArgs a{d_k_cache, d_v_cache, d_stage, d_stage + floats, n_keep, shift, retained, n_kv_heads, head_dim, theta_scale};
-    hipError_t e = launch_kernel(L, kFamOther, kv_shift_stage_kernel, dim3((retained + kShiftRows - 1) / kShiftRows), dim3(256), a);
+    const size_t kv_dim = (size_t)n_kv_heads * head_dim, elems = (size_t)retained * kv_dim, esize = kv_f16 ? 2 : 4;
+    uint8_t* const stage = static_cast<uint8_t*>(d_stage);
+    KvShiftArgs a{d_k_cache, d_v_cache, stage, stage + elems * esize, n_keep, shift, retained, n_kv_heads, head_dim, theta_scale};
+    hipError_t e = with_kv_type(kv_f16, [&](auto kv) {
+        return launch_kernel(L, kFamOther, kv_shift_stage_kernel<decltype(kv)>, dim3((retained + kShiftRows - 1) / kShiftRows), dim3(256), a);
+    });
     if (e != hipSuccess) return e;
-    e = hipMemcpyAsync(d_k_cache + (size_t)n_keep * kv_dim, a.k_stage, floats * sizeof(float), hipMemcpyDeviceToDevice, L.stream);
+    e = hipMemcpyAsync(static_cast<uint8_t*>(d_k_cache) + (size_t)n_keep * kv_dim * esize, a.k_stage, elems * esize, hipMemcpyDeviceToDevice, L.stream);
     if (e != hipSuccess) return e;
-    return hipMemcpyAsync(d_v_cache + (size_t)n_keep * kv_dim, a.v_stage, floats * sizeof(float), hipMemcpyDeviceToDevice, L.stream);
+    return hipMemcpyAsync(static_cast<uint8_t*>(d_v_cache) + (size_t)n_keep * kv_dim * esize, a.v_stage, elems * esize, hipMemcpyDeviceToDevice, L.stream);
 }
 
-hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scores,
+hipError_t launch_attention_decode(const float* d_q, const void* d_k_cache, const void* d_v_cache, float* d_out, float* d_scores,
                                    uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
-                                   uint32_t head_dim, float scale, const Launch& L) {
+                                   uint32_t head_dim, float scale, const Launch& L, bool kv_f16) {
     AttentionArgs a{d_q, d_k_cache, d_v_cache, d_out, d_scores, d_pos, seq_len, max_seq, n_heads, n_kv_heads, head_dim, scale};
     const uint32_t splits = attention_splits(max_seq);
     auto split_path = [&](auto hd) -> hipError_t {
         constexpr int HD = decltype(hd)::value;
-        hipError_t e = launch_kernel(L, kFamOther, attention_split_kernel<HD>, dim3(n_heads * splits), dim3(256), a, splits);
+        hipError_t e = with_kv_type(kv_f16, [&](auto kv) {
+            return launch_kernel(L, kFamOther, attention_split_kernel<HD, decltype(kv)>, dim3(n_heads * splits), dim3(256), a, splits);
+        });
         if (e != hipSuccess) return e;
         return launch_kernel(L, kFamOther, attention_combine_kernel<HD>, dim3(n_heads), dim3(256), a, splits);
     };
@@ -1427,16 +1474,16 @@ hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, con
             default: break;
         }
     }
-    return launch_kernel(L, kFamOther, attention_decode_kernel, dim3(n_heads), dim3(256), a);
+    return with_kv_type(kv_f16, [&](auto kv) { return launch_kernel(L, kFamOther, attention_decode_kernel<decltype(kv)>, dim3(n_heads), dim3(256), a); });
 }
 
 // The fused attention block; false when head_dim has no fused variant (the caller then runs the three launches).
 bool attention_layer_applies(uint32_t head_dim) { return head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256; }
 
 hipError_t launch_attention_layer(const float* d_q, const float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
-                                  float* d_k_cache, float* d_v_cache, float* d_out, float* d_scratch, uint32_t pos,
+                                  void* d_k_cache, void* d_v_cache, float* d_out, float* d_scratch, uint32_t pos,
                                   const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float eps,
-                                  float theta_scale, float scale, const Launch& L) {
+                                  float theta_scale, float scale, const Launch& L, bool kv_f16) {
     AttentionLayerArgs f{};
     f.at = AttentionArgs{nullptr, d_k_cache, d_v_cache, d_out, d_scratch, d_pos, pos + 1u, max_seq, n_heads, n_kv_heads, head_dim, scale};
     f.q_raw = d_q, f.k_raw = d_k, f.v = d_v, f.q_norm = d_q_norm, f.k_norm = d_k_norm;
@@ -1445,7 +1492,7 @@ hipError_t launch_attention_layer(const float* d_q, const float* d_k, const floa
     const dim3 grid(n_heads * splits), block(256);
     auto run = [&](auto hd) -> hipError_t {
         constexpr int HD = decltype(hd)::value;
-        hipError_t e = launch_kernel(L, kFamOther, attention_layer_kernel<HD>, grid, block, f, splits);
+        hipError_t e = with_kv_type(kv_f16, [&](auto kv) { return launch_kernel(L, kFamOther, attention_layer_kernel<HD, decltype(kv)>, grid, block, f, splits); });
         if (e != hipSuccess) return e;
         return launch_kernel(L, kFamOther, attention_combine_kernel<HD>, dim3(n_heads), block, f.at, splits);
     };
@@ -1513,17 +1560,17 @@ hipError_t launch_shortconv_seq_quantize(const float* d_proj, float* d_buffer, c
 
 size_t attention_prefill_scratch_floats(uint32_t, uint32_t, uint32_t) { return 4; }  // the kernel keeps everything on chip
 
-bool attention_prefill_quantize_applies(const float* d_q, const float* d_k_cache, const float* d_v_cache, uint32_t n, uint32_t q_stride,
+bool attention_prefill_quantize_applies(const float* d_q, const void* d_k_cache, const void* d_v_cache, uint32_t n, uint32_t q_stride,
                                         uint32_t head_dim) {
     return head_dim == 64 && n >= 16 && q_stride % 4u == 0 && ((uintptr_t)d_q | (uintptr_t)d_k_cache | (uintptr_t)d_v_cache) % 16u == 0;
 }
 
 // d_q8 / d_q8_scales given (attention_prefill_quantize_applies): the result is written as Q8_0 blocks, rows of
 // n_heads * head_dim quants, bit-identical to quantizing the float result; d_out is not written then.
-hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scratch,
+hipError_t launch_attention_prefill(const float* d_q, const void* d_k_cache, const void* d_v_cache, float* d_out, float* d_scratch,
                                     uint32_t pos0, const uint32_t* d_pos, uint32_t n, uint32_t q_stride, uint32_t out_stride, uint32_t max_seq,
                                     uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L, int8_t* d_q8,
-                                    float* d_q8_scales) {
+                                    float* d_q8_scales, bool kv_f16) {
     if (n == 0) return hipSuccess;
     AttentionArgs a{d_q, d_k_cache, d_v_cache, d_out, d_scratch, d_pos, 0u, max_seq, n_heads, n_kv_heads, head_dim, scale};
     // the matrix-core kernel needs 16-byte aligned rows (q, caches, out) and whole tiles of head dims
@@ -1535,20 +1582,26 @@ hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, co
         // (long, short) pairs balance the causal work once there are more query blocks than CUs; below that one block per
         // workgroup (longest first) spreads wider: 17.7 -> 14.9, 25.8 -> 23.5, 43.5 -> 41.7 us at 256 / 512 / 1024 tokens of 16
         // heads, but 82 -> 94 us at 2002.  The same arithmetic per query either way.
-        if (n_heads * qblocks <= 256u)
-            return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<1>, dim3(n_heads, qblocks), dim3(512), a, pos0, n, q_stride, out_stride, d_q8,
-                                 d_q8_scales);
-        return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<2>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride,
-                             out_stride, d_q8, d_q8_scales);
+        return with_kv_type(kv_f16, [&](auto kv) {
+            using KV = decltype(kv);
+            if (n_heads * qblocks <= 256u)
+                return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<1, KV>, dim3(n_heads, qblocks), dim3(512), a, pos0, n, q_stride, out_stride,
+                                     d_q8, d_q8_scales);
+            return launch_kernel(L, kFamOther, attention_prefill_f16x3_kernel<2, KV>, dim3(n_heads, (qblocks + 1u) / 2u), dim3(1024), a, pos0, n, q_stride,
+                                 out_stride, d_q8, d_q8_scales);
+        });
     }
     const dim3 grid(n_heads, (n + 7u) / 8u), block(256);
-    switch (head_dim) {
-        case 32: return launch_kernel(L, kFamOther, attention_prefill_kernel<32>, grid, block, a, pos0, n, q_stride, out_stride);
-        case 64: return launch_kernel(L, kFamOther, attention_prefill_kernel<64>, grid, block, a, pos0, n, q_stride, out_stride);
-        case 128: return launch_kernel(L, kFamOther, attention_prefill_kernel<128>, grid, block, a, pos0, n, q_stride, out_stride);
-        case 256: return launch_kernel(L, kFamOther, attention_prefill_kernel<256>, grid, block, a, pos0, n, q_stride, out_stride);
-        default: return hipErrorInvalidValue;
-    }
+    return with_kv_type(kv_f16, [&](auto kv) {
+        using KV = decltype(kv);
+        switch (head_dim) {
+            case 32: return launch_kernel(L, kFamOther, attention_prefill_kernel<32, KV>, grid, block, a, pos0, n, q_stride, out_stride);
+            case 64: return launch_kernel(L, kFamOther, attention_prefill_kernel<64, KV>, grid, block, a, pos0, n, q_stride, out_stride);
+            case 128: return launch_kernel(L, kFamOther, attention_prefill_kernel<128, KV>, grid, block, a, pos0, n, q_stride, out_stride);
+            case 256: return launch_kernel(L, kFamOther, attention_prefill_kernel<256, KV>, grid, block, a, pos0, n, q_stride, out_stride);
+            default: return hipErrorInvalidValue;
+        }
+    });
 }
 
 hipError_t launch_rmsnorm_quantize(const float* d_x, const float* d_weight, uint32_t rows, uint32_t dim, uint32_t x_stride, float eps, int8_t* d_q,

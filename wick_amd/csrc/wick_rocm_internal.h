@@ -164,14 +164,16 @@ hipError_t launch_embed_row(const uint8_t* d_w, int type, uint32_t m, uint32_t k
                             const Launch& L);
 hipError_t launch_rmsnorm(const float* d_x, const float* d_weight, float* d_y, uint32_t rows, uint32_t dim, uint32_t x_stride,
                           uint32_t y_stride, float eps, const Launch& L);
-hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm, float* d_k_cache,
-                               float* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
+// The KV caches of the launchers below hold f32 rows, or f16 rows with kv_f16 (values rounded once when they are appended or
+// moved, widened exactly when they are read; all arithmetic f32).
+hipError_t launch_qk_norm_rope(float* d_q, float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm, void* d_k_cache,
+                               void* d_v_cache, uint32_t pos, const uint32_t* d_pos, uint32_t max_seq, uint32_t head_dim, uint32_t n_heads,
                                uint32_t n_kv_heads, float eps, float theta_scale, const Launch& L, uint32_t n_tokens = 1, uint32_t q_stride = 0,
-                               uint32_t kv_stride = 0);
+                               uint32_t kv_stride = 0, bool kv_f16 = false);
 // Drops cache rows [n_keep, n_keep + shift) of one attention layer and re-rotates the keys that move; d_stage holds
-// 2 * (seq_len - n_keep - shift) * n_kv_heads * head_dim floats.
-hipError_t launch_kv_shift(float* d_k_cache, float* d_v_cache, float* d_stage, uint32_t seq_len, uint32_t n_keep, uint32_t shift,
-                           uint32_t n_kv_heads, uint32_t head_dim, float theta_scale, const Launch& L);
+// 2 * (seq_len - n_keep - shift) * n_kv_heads * head_dim cache elements.
+hipError_t launch_kv_shift(void* d_k_cache, void* d_v_cache, void* d_stage, uint32_t seq_len, uint32_t n_keep, uint32_t shift,
+                           uint32_t n_kv_heads, uint32_t head_dim, float theta_scale, const Launch& L, bool kv_f16 = false);
 // A prompt of n tokens at once (token j at position pos + j): embedding rows [n][k], the short conv of every (token, channel), causal attention over caches that already hold the prompt's K / V rows (head_dim 32 / 64 / 128 / 256;
 // scratch: attention_prefill_scratch_floats).
 hipError_t launch_embed_rows(const uint8_t* d_w, int type, uint32_t m, uint32_t k, const uint32_t* d_tokens, uint32_t n, float* d_out,
@@ -179,12 +181,12 @@ hipError_t launch_embed_rows(const uint8_t* d_w, int type, uint32_t m, uint32_t 
 hipError_t launch_shortconv_seq(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
                                 uint32_t kernel_size, uint32_t n, const Launch& L);
 size_t attention_prefill_scratch_floats(uint32_t n, uint32_t n_heads, uint32_t head_dim);
-hipError_t launch_attention_prefill(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scratch,
+hipError_t launch_attention_prefill(const float* d_q, const void* d_k_cache, const void* d_v_cache, float* d_out, float* d_scratch,
                                     uint32_t pos0, const uint32_t* d_pos, uint32_t n, uint32_t q_stride, uint32_t out_stride, uint32_t max_seq,
                                     uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float scale, const Launch& L, int8_t* d_q8 = nullptr,
-                                    float* d_q8_scales = nullptr);
+                                    float* d_q8_scales = nullptr, bool kv_f16 = false);
 // The two producers of an out projection's input written directly as Q8_0 blocks (no float result in memory).
-bool attention_prefill_quantize_applies(const float* d_q, const float* d_k_cache, const float* d_v_cache, uint32_t n, uint32_t q_stride,
+bool attention_prefill_quantize_applies(const float* d_q, const void* d_k_cache, const void* d_v_cache, uint32_t n, uint32_t q_stride,
                                         uint32_t head_dim);
 bool shortconv_seq_quantize_applies(const float* d_proj, const float* d_buffer, uint32_t hidden);
 hipError_t launch_shortconv_seq_quantize(const float* d_proj, float* d_buffer, const float* d_conv_w, int8_t* d_q, float* d_scales, uint32_t hidden,
@@ -192,16 +194,16 @@ hipError_t launch_shortconv_seq_quantize(const float* d_proj, float* d_buffer, c
 // d_scores is scratch of attention_scratch_floats(max_seq, n_heads, head_dim) floats.
 uint32_t attention_splits(uint32_t max_seq);
 size_t attention_scratch_floats(uint32_t max_seq, uint32_t n_heads, uint32_t head_dim);
-hipError_t launch_attention_decode(const float* d_q, const float* d_k_cache, const float* d_v_cache, float* d_out, float* d_scores,
+hipError_t launch_attention_decode(const float* d_q, const void* d_k_cache, const void* d_v_cache, float* d_out, float* d_scores,
                                    uint32_t seq_len, const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads,
-                                   uint32_t head_dim, float scale, const Launch& L);
+                                   uint32_t head_dim, float scale, const Launch& L, bool kv_f16 = false);
 // QK-norm + RoPE + KV append folded into the sequence-split attention kernel, then the merge (head_dim 32 / 64 / 128 / 256).
 // d_scratch as for launch_attention_decode.
 bool attention_layer_applies(uint32_t head_dim);
 hipError_t launch_attention_layer(const float* d_q, const float* d_k, const float* d_v, const float* d_q_norm, const float* d_k_norm,
-                                  float* d_k_cache, float* d_v_cache, float* d_out, float* d_scratch, uint32_t pos,
+                                  void* d_k_cache, void* d_v_cache, float* d_out, float* d_scratch, uint32_t pos,
                                   const uint32_t* d_pos, uint32_t max_seq, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, float eps,
-                                  float theta_scale, float scale, const Launch& L);
+                                  float theta_scale, float scale, const Launch& L, bool kv_f16 = false);
 hipError_t launch_shortconv_step(const float* d_proj, float* d_buffer, const float* d_conv_w, float* d_out, uint32_t hidden,
                                  uint32_t kernel_size, const Launch& L);
 hipError_t launch_rmsnorm_quantize(const float* d_x, const float* d_weight, uint32_t rows, uint32_t dim, uint32_t x_stride, float eps, int8_t* d_q,

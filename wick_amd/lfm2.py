@@ -46,6 +46,8 @@ _SIGNATURES = {
     "wick_rocm_rmsnorm_quantize_q8_0": (C.c_int, [_P, _P, _P, _U32, _U32, _U32, _F, _P, _P]),
     "wick_rocm_silu_mul_quantize_q8_0": (C.c_int, [_P, _P, _P, _U32, _U32, _P, _P]),
     "wick_rocm_lfm2_load": (C.c_int, [_P, _P, _U32, C.POINTER(_P)]),
+    "wick_rocm_lfm2_load_kv": (C.c_int, [_P, _P, _U32, C.c_int, C.POINTER(_P)]),
+    "wick_rocm_lfm2_kv_dtype": (C.c_int, [_P]),
     "wick_rocm_lfm2_free": (C.c_int, [_P, _P]),
     "wick_rocm_lfm2_get_config": (C.c_int, [_P, C.POINTER(Lfm2Config)]),
     "wick_rocm_lfm2_layer_kv_heads": (C.c_int, [_P, _U32, C.POINTER(_U32)]),
@@ -214,14 +216,22 @@ class Lfm2Ops:
                                                              _ptr(d_token), _ptr(d_pos)))
 
 
+KV_F32, KV_F16 = 0, 1  # wick_rocm_lfm2_load_kv's kv_dtype
+
+
 class RocmLfm2Model:
     """load_model_* counterpart (wick/src/model/mod.rs:385-403): owns weights, KV caches, conv state and scratch on the GPU."""
 
-    def __init__(self, ctx: RocmContext, gguf, context_size: int):
+    def __init__(self, ctx: RocmContext, gguf, context_size: int, kv_f16: bool = False):
+        """kv_f16: KV caches of f16 rows like the reference's GPU models (default: f32 rows like its CPU model)."""
         self.ctx, self._l = ctx, _lib()
         h = _P()
-        ctx._check(self._l.wick_rocm_lfm2_load(ctx._h, gguf.handle, context_size, C.byref(h)))
+        if kv_f16:
+            ctx._check(self._l.wick_rocm_lfm2_load_kv(ctx._h, gguf.handle, context_size, KV_F16, C.byref(h)))
+        else:
+            ctx._check(self._l.wick_rocm_lfm2_load(ctx._h, gguf.handle, context_size, C.byref(h)))
         self._h = h.value
+        self.kv_f16 = self._l.wick_rocm_lfm2_kv_dtype(self._h) == KV_F16
         cfg = Lfm2Config()
         ctx._check(self._l.wick_rocm_lfm2_get_config(self._h, C.byref(cfg)))
         self.config = {n: getattr(cfg, n) for n, _ in Lfm2Config._fields_}
