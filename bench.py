@@ -209,19 +209,24 @@ def bench_c1_span(ctx, W, ws, d_q, d_s, d_y, m, steps, warmup):
     waves = [B.gemv_q8_span(ctx, w, d_s, d_q, d_y, sp, m) for w, sp in zip(ws, spans)]
     g = ctx.graph_end()
     ms_step, _ = time_graph_steps(ctx, [g], steps, warmup)
-    per_launch, gaps = [], []
+    per_launch, gaps, start_off, wave_dur = [], [], [], []
     for _ in range(3):  # three more replays, each read back
         ctx.graph_launch(g)
         ctx.sync()
         rec = [sp.download(np.uint64, 2 * nw).reshape(nw, 2) for sp, nw in zip(spans, waves)]
         per_launch += [B.span_us(r) for r in rec]
+        start_off += [(r[:, 0] - r[:, 0].min()).astype(np.float64) / 100.0 for r in rec]
+        wave_dur += [(r[:, 1] - r[:, 0]).astype(np.float64) / 100.0 for r in rec]
         starts, ends = [int(r[:, 0].min()) for r in rec], [int(r[:, 1].max()) for r in rec]
         gaps += [(starts[i + 1] - ends[i]) / 100.0 for i in range(len(rec) - 1)]
     ctx.graph_destroy(g)
     for sp in spans:
         sp.free()
     a, gp = np.asarray(per_launch), np.asarray(gaps)
-    return {"launches_per_step": len(ws), "waves_per_launch": waves[0], "span_us_mean": float(a.mean()), "span_us_median": float(np.median(a)),
+    so, wd = np.concatenate(start_off), np.concatenate(wave_dur)
+    inside = {"wave_start_after_first_wave_us": {f"p{q}": float(np.percentile(so, q)) for q in (50, 90, 99, 100)},
+              "wave_duration_us": {f"p{q}": float(np.percentile(wd, q)) for q in (1, 50, 90, 100)}}
+    return {"launches_per_step": len(ws), "waves_per_launch": waves[0], **inside, "span_us_mean": float(a.mean()), "span_us_median": float(np.median(a)),
             "span_us_min": float(a.min()), "span_us_p90": float(np.percentile(a, 90)), "samples": int(a.size),
             "gap_to_next_launch_us_mean": float(gp.mean()), "gap_to_next_launch_us_median": float(np.median(gp)),
             "step_ms_with_hook": ms_step, "sum_of_spans_ms": float(a.mean()) * len(ws) / 1e3, "clock": "100 MHz wall clock (s_memrealtime), 10 ns steps"}
