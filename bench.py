@@ -10,14 +10,21 @@ p10 / p90 over the timed steps are reported.
 
 Beside it, in the same JSON line:
   roofline         the GEMV kernel: algorithmic bytes per launch / average launch duration of the timed region
-                   (step time / 38; the kernel runs nowhere else in that region), against 8 TB/s
+                   (step time / 38; the kernel runs nowhere else in that region), against 8 TB/s.  Inside it:
+                   kernel_span_* = the launch clocked by the kernel itself inside the same graph (first wave's first
+                   instruction -> last wave's last store acknowledged) and gap_between_dependent_launches_us, both from the
+                   timing-hook instantiation in libwick_rocm_bench.so; independent_streams_* = gemv_concurrent's figure;
+                   gemm = the prefill GEMM's roofline object (bound "mfma"), so that both halves of the metric sit in one
+                   place; lm_head_* = where the hand-off sweep says the MFMA kernel starts to win and where the library
+                   hands off
   gemv_concurrent  the same launches as INDEPENDENT work on four streams: what the kernel sustains when the gap between
                    dependent launches is taken out of the picture
   gemm             the prefill GEMM the matrix-core target is quoted on (Q4_0, m=6912, n=2002, k=2048) with its own
                    roofline object (per-launch kernel timestamps, median / min over 100 launches)
   decode_step, decode_step_q8_0, prefill_sites, lm_head_sweep, lm_head_q6_k_65536x1024, lfm2_decode_step
                    the other configurations (LFM2-350M-shaped decode weight set, the nine LFM2-1.2B prefill call sites at
-                   n = 4096, the 65536 x 2048 head at n = 1 / 4 / 16 / 64, a whole model step)
+                   n = 4096, the 65536 x 2048 head at n = 1 / 4 / 5 / 6 / 8 / 12 / 16 / 64, a whole model step;
+                   `--leg lfm2_step_kv16` times the same model with f16 KV caches)
   cpu_baseline     the reference's x86 CPU path (f32 per-token GEMV; Q4_0 rows serial, Q8_0 rows over T threads) timed on
                    this host on bounded samples of the same workloads
 
