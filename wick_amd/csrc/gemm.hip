@@ -410,6 +410,64 @@ __device__ __forceinline__ void tile_of_block(uint32_t bid, uint32_t row_tiles, 
     tok_tile = sc * S + t2 % w;
 }
 
+// Results of a wave's MFMA tiles into the output (or into a K share's partial sums): element (tt, rt, r) of the wave tile is
+// (row + 16 rt, tok + 16 tt + r), `row` / `tok` being this lane's first row and token.  One instantiation per output layout
+// so that the inner index is an immediate offset of the store; CHECK = false for wave tiles that lie inside the matrix (no
+// predicates at all), ACC adds onto what is there.  The mode is uniform per launch, the bounds are uniform per wave: the
+// callers branch once, not per element.
+template <int NTT, int NRT, bool ROW_MAJOR, bool CHECK, bool ACC, typename F>
+__device__ __forceinline__ void store_results(float* __restrict__ base, size_t stride, uint32_t row, uint32_t tok, uint32_t m, uint32_t n,
+                                              F&& value) {
+    if constexpr (ROW_MAJOR) {
+#pragma unroll
+        for (int rt = 0; rt < NRT; rt++) {
+            float* q = base + (size_t)(row + 16 * rt) * stride + tok;
+#pragma unroll
+            for (int tt = 0; tt < NTT; tt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (CHECK && !(row + 16 * rt < m && tok + 16 * tt + r < n)) continue;
+                    const float v = value(tt, rt, r);
+                    q[16 * tt + r] = ACC ? q[16 * tt + r] + v : v;
+                }
+        }
+    } else {
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float* q = base + (size_t)(tok + 16 * tt + r) * stride + row;
+#pragma unroll
+                for (int rt = 0; rt < NRT; rt++) {
+                    if (CHECK && !(row + 16 * rt < m && tok + 16 * tt + r < n)) continue;
+                    const float v = value(tt, rt, r);
+                    q[16 * rt] = ACC ? q[16 * rt] + v : v;
+                }
+            }
+    }
+}
+// The launch's output mode picked once per wave: a K share's partial sums [share][n][m], or y in either layout, plain or accumulating.
+template <int NTT, int NRT, typename F>
+__device__ __forceinline__ void store_wave_tile(const GemmArgs& a, uint32_t ksplit, uint32_t split, uint32_t row, uint32_t tok, F&& value) {
+    // the wave tile's corner is the same for every lane: keep the test (and the branches on it) scalar
+    const uint32_t row_end = (uint32_t)__builtin_amdgcn_readfirstlane((int)(row - (row & 15u))) + 16u * NRT;
+    const uint32_t tok_end = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tok - (tok & 15u))) + 16u * NTT;
+    const bool inside = row_end <= a.m && tok_end <= a.n;
+    if (ksplit > 1) {  // this share's sums; the reduce launch (or the caller's next kernel) adds the shares up
+        float* base = a.partial + (size_t)split * a.n * a.m;
+        if (inside) store_results<NTT, NRT, false, false, false>(base, a.m, row, tok, a.m, a.n, value);
+        else store_results<NTT, NRT, false, true, false>(base, a.m, row, tok, a.m, a.n, value);
+    } else if (a.y_row_major) {
+        if (a.accumulate) store_results<NTT, NRT, true, true, true>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        else if (inside) store_results<NTT, NRT, true, false, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        else store_results<NTT, NRT, true, true, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+    } else {
+        if (a.accumulate) store_results<NTT, NRT, false, true, true>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        else if (inside) store_results<NTT, NRT, false, false, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        else store_results<NTT, NRT, false, true, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+    }
+}
+
 // Maximum over the 16 lanes of a DPP row (lanes that share lane / 16); every lane of the row ends with it.
 __device__ __forceinline__ float row_max16(float v) {
     v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false)));   // quad_perm [1,0,3,2]
@@ -568,24 +626,8 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
                 }
             }
     } else if constexpr (!DUMP) {
-#pragma unroll
-        for (int tt = 0; tt < TT; tt++)
-#pragma unroll
-            for (int rt = 0; rt < RT; rt++) {
-                const uint32_t row = row0 + wrow0 + 16 * rt + l16;
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const uint32_t tok = tok0 + wtok0 + 16 * tt + 4 * kq + r;
-                    if (row < a.m && tok < a.n) {
-                        if (ksplit > 1) {  // this share's sums; the reduce launch (or the caller's next kernel) adds the shares up
-                            a.partial[((size_t)split * a.n + tok) * a.m + row] = acc[tt][rt][r];
-                        } else {
-                            float* dst = a.y_row_major ? a.y + (size_t)row * a.y_stride + tok : a.y + (size_t)tok * a.y_stride + row;
-                            *dst = a.accumulate ? *dst + acc[tt][rt][r] : acc[tt][rt][r];
-                        }
-                    }
-                }
-            }
+        store_wave_tile<TT, RT>(a, ksplit, split, row0 + wrow0 + l16, tok0 + wtok0 + 4 * kq,
+                                [&](int tt, int rt, int r) { return acc[tt][rt][r]; });
     }
 }
 
@@ -736,21 +778,7 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     }
 
     if constexpr (!DUMP) {
-        const uint32_t row = row0 + wrow0 + l16;
-#pragma unroll
-        for (int tt = 0; tt < TTN; tt++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const uint32_t tok = tok0 + 16 * tt + 4 * kq + r;
-                if (row < a.m && tok < a.n) {
-                    if (ksplit > 1) {
-                        a.partial[((size_t)split * a.n + tok) * a.m + row] = acc[tt][r];
-                    } else {
-                        float* dst = a.y_row_major ? a.y + (size_t)row * a.y_stride + tok : a.y + (size_t)tok * a.y_stride + row;
-                        *dst = a.accumulate ? *dst + acc[tt][r] : acc[tt][r];
-                    }
-                }
-            }
+        store_wave_tile<TTN, 1>(a, ksplit, split, row0 + wrow0 + l16, tok0 + 4 * kq, [&](int tt, int, int r) { return acc[tt][r]; });
     }
 }
 
