@@ -910,6 +910,7 @@ def main():
         # shipped LFM2 Q4_0 files keep the tied embedding / LM head in Q6_K (wick/src/model/metal_lfm2.rs:175-180)
         out["lm_head_q6_k_65536x1024"] = bench_single_gemv(ctx, W, O, W.Q6_K, 65536, 1024)
         out["lfm2_decode_step"] = bench_lfm2_step(ctx, W, O)
+        out["lfm2_decode_step_kv_f16"] = bench_lfm2_step(ctx, W, O, kernel_times=False, kv_f16=True)  # the same model on f16 K / V rows
     ctx.close()
     out["roofline"] = roofline  # (last, with cpu_baseline: the end of the line is what a truncated log still shows)
     if not args.skip_cpu:
