@@ -176,10 +176,13 @@ private:
 // conv state and scratch; the GGUF file may be closed once the constructor has returned.
 class RocmLfm2Model {
 public:
-    RocmLfm2Model(RocmContext& ctx, const GgufFile& gguf, uint32_t context_size) : ctx_(ctx) {
-        ctx_.check(wick_rocm_lfm2_load(ctx_.raw(), gguf.raw(), context_size, &m_));
+    // kv_f16: K / V rows kept in half like the reference's GPU model (wick/src/model/metal_lfm2.rs:4117-4247) instead of
+    // the CPU model's f32 rows.
+    RocmLfm2Model(RocmContext& ctx, const GgufFile& gguf, uint32_t context_size, bool kv_f16 = false) : ctx_(ctx) {
+        ctx_.check(wick_rocm_lfm2_load_kv(ctx_.raw(), gguf.raw(), context_size, kv_f16 ? WICK_ROCM_KV_F16 : WICK_ROCM_KV_F32, &m_));
         ctx_.check(wick_rocm_lfm2_get_config(m_, &cfg_));
     }
+    bool kv_f16() const { return wick_rocm_lfm2_kv_dtype(m_) == WICK_ROCM_KV_F16; }
     ~RocmLfm2Model() { wick_rocm_lfm2_free(ctx_.raw(), m_); }
     RocmLfm2Model(const RocmLfm2Model&) = delete;
     RocmLfm2Model& operator=(const RocmLfm2Model&) = delete;
