@@ -887,7 +887,7 @@ def main():
 
     gemm_profile = "gemm_q4_0_6912x2002x2048.txt"
     g = bench_gemm(ctx, W, O, W.Q4_0, 6912, 2002, 2048, samples=100)
-    g["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma_kernel<Q4_0>", "workload": "prefill GEMM Q4_0 m=6912, n=2002, k=2048 (2 m n k int8 ops per launch)",
+    g["roofline"] = {"bound": "mfma", "kernel": "gemm_mfma32_kernel<Q4_0>", "workload": "prefill GEMM Q4_0 m=6912, n=2002, k=2048 (2 m n k int8 ops per launch)",
                      "achieved": g["gemm_kernel_TOPS"], "peak": INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": g["gemm_kernel_TOPS"] / INT8_PEAK_TOPS, "frac_median": g["gemm_kernel_TOPS_median"] / INT8_PEAK_TOPS,
                      "frac_best": g["gemm_kernel_TOPS_best"] / INT8_PEAK_TOPS, "avg_launch_us": g["gemm_kernel_ms"] * 1e3,

@@ -195,6 +195,12 @@ int wick_rocm_set_gemm_min_n(wick_rocm_ctx *ctx, uint32_t min_n);
  * the one above; wick_rocm_matmul_f32_noalloc never splits. */
 int wick_rocm_set_gemm_max_k_splits(wick_rocm_ctx *ctx, uint32_t max_splits);
 
+/* Which matrix-core instruction the wide-tile GEMM's block loop is built on: 32 (the default, also 0) = two
+ * v_mfma_i32_32x32x32_i8 per block and wave, 16 = eight v_mfma_i32_16x16x32_i8 (what the gated feed-forward launch and the
+ * narrow tile always use).  Block dots are bit-identical either way, f32 sums agree to the last bit or two (the order in
+ * which a row's blocks are added is the same, the lanes that hold them differ).  A tuning knob like the ones above. */
+int wick_rocm_set_gemm_mfma_shape(wick_rocm_ctx *ctx, int shape);
+
 /* How the single-token GEMV fetches its weights, by bytes of weights in one launch: below
  * direct_max_bytes every lane loads its own block pair; from there on a wave loads whole
  * cache lines and redistributes them through LDS.  Negative = the built-in default (3 MiB

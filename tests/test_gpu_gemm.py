@@ -42,6 +42,56 @@ def test_gemm_parity(ctx, oracle, dtype, m, n, k):
         assert np.array_equal(dots, oracle.block_dots_i32(dtype, p.wb, p.q, m, n, k))
 
 
+# more than 256 wide tiles (fewer run on the narrow tile), ragged in rows and tokens; the last one is cut over K on the wide tile
+WIDE_SHAPES = [(2100, 2010, 128, True), (2100, 1990, 256, False), (4700, 1100, 384, False), (1024, 2002, 4608, False)]
+
+
+@pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
+@pytest.mark.parametrize("m,n,k,with_dots", WIDE_SHAPES)
+def test_wide_tile_on_either_mfma_shape(ctx, oracle, dtype, m, n, k, with_dots):
+    """The wide tile's two block loops (32x32x32, the default, and 16x16x32): each against the oracle (two row bands over all
+    tokens) in both layouts with ragged strides and with the accumulate flag, block dots bit-exact through either, and the
+    two within 1e-6 of each other everywhere."""
+    rb = (k // 32) * (18 if dtype == W.Q4_0 else 34)
+    bands = [(0, 96), (m - 70, m)]
+    with Problem(ctx, oracle, dtype, m, k, n, seed=3 * m + 7 * n + k + dtype) as p:
+        refs = [oracle.gemm_q8(dtype, p.wb[r0 * rb:r1 * rb], p.s, p.q, r1 - r0, n, k) for r0, r1 in bands]
+        outs = {}
+        try:
+            for shape in (32, 16):
+                ctx.set_gemm_mfma_shape(shape)
+                for layout, stride in ((W.LAYOUT_TOKEN_MAJOR, m), (W.LAYOUT_ROW_MAJOR, n + 3), (W.LAYOUT_TOKEN_MAJOR, m + 5)):
+                    rows = m if layout == W.LAYOUT_ROW_MAJOR else n
+                    d_y = ctx.to_device(np.full(rows * stride, -7.0, np.float32))
+                    ctx.gemm_preq(p.w, p.d_s, p.d_q, n, d_y, y_stride=stride, layout=layout)
+                    got = fetch_gemm(d_y, m, n, stride, layout)
+                    for (r0, r1), ref in zip(bands, refs):
+                        assert_f32_parity(got[r0:r1], ref, f"gemm {dtype} {m}x{n}x{k} layout {layout} mfma {shape} rows {r0}..{r1}")
+                    full = d_y.download(np.float32, rows * stride).reshape(rows, stride)
+                    assert np.all(full[:, (n if layout == W.LAYOUT_ROW_MAJOR else m):] == -7.0)
+                    if layout == W.LAYOUT_TOKEN_MAJOR and stride == m:
+                        outs[shape] = got
+                        ctx.gemm_preq(p.w, p.d_s, p.d_q, n, d_y, y_stride=stride, layout=layout, accumulate=True)  # y += W x
+                        twice = fetch_gemm(d_y, m, n, stride, layout)
+                        for (r0, r1), ref in zip(bands, refs):
+                            assert_f32_parity(twice[r0:r1], 2.0 * ref, f"accumulate, mfma {shape}")
+                    d_y.free()
+                if with_dots:
+                    d_d = p.alloc(n * m * (k // 32) * 4)
+                    ctx.block_dots_i32(p.w, p.d_q, n, d_d)
+                    dots = d_d.download(np.int32, n * m * (k // 32)).reshape(n, m, k // 32)
+                    assert np.array_equal(dots, oracle.block_dots_i32(dtype, p.wb, p.q, m, n, k))
+        finally:
+            ctx.set_gemm_mfma_shape(0)
+        assert rel_l2(outs[16], outs[32]) < 1e-6
+
+
+def test_mfma_shape_knob_rejects_other_values(ctx):
+    with pytest.raises(W.RocmError):
+        ctx.set_gemm_mfma_shape(8)
+    ctx.set_gemm_mfma_shape(0)
+
+
 @pytest.mark.parametrize("dtype,n", [(W.Q4_0, 7), (W.Q8_0, 5), (W.Q4_0, 8), (W.Q4_0, 11), (W.Q4_0, 16)])
 def test_reference_gemm_vs_gemv_inputs(ctx, oracle, dtype, n):
     """The reference's GEMM == sequential GEMV tests (simd.rs:1440-1623) on their own

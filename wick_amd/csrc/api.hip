@@ -277,6 +277,13 @@ int wick_rocm_set_gemm_packing(wick_rocm_ctx* ctx, int enabled) {
 
 size_t wick_rocm_weight_device_bytes(const wick_rocm_weight* w) { return w ? w->nbytes + w->gemm_bytes : 0; }
 
+int wick_rocm_set_gemm_mfma_shape(wick_rocm_ctx* ctx, int shape) {
+    WR_ENTER(ctx);
+    if (shape != 0 && shape != 16 && shape != 32) return fail(ctx, WICK_ROCM_ERR_INVALID_ARG, "set_gemm_mfma_shape: 0 (default), 16 or 32");
+    ctx->gemm_mfma16 = shape == 16;
+    return WICK_ROCM_OK;
+}
+
 int wick_rocm_set_gemm_min_n(wick_rocm_ctx* ctx, uint32_t min_n) {
     WR_ENTER(ctx);
     ctx->gemm_min_n = min_n;  // 0: back to the per-weight default

@@ -8,13 +8,16 @@
 // into f32 accumulators on the vector ALU.
 //
 // Workgroup = 512 threads = 8 waves, tile = 128 weight rows x 128 tokens, each wave
-// owns 64 rows x 32 tokens = 4 x 2 tiles of v_mfma_i32_16x16x32_i8.  The small MFMA
-// shape is chosen for its register footprint: 4 result registers per tile (16 for the
-// 32x32 shape), a 4-register bias and 4 token scales per tile keep the kernel under 128
-// VGPRs, so FOUR waves share a SIMD.  That matters more than the matrix rate (the 16x16x32
-// instruction runs at half the 32x32x32 rate, 1.9 vs 3.8 POP/s measured): a wave can issue
-// a vector-ALU instruction only every ~4.7 cycles while a SIMD retires one every ~2.2, and
-// the kernel is bound by the two scaling FMAs per result.
+// owns 64 rows x 32 tokens.  Two block loops exist for that wave tile:
+//   * gemm_mfma32_kernel (plain projections, the default): 2 x v_mfma_i32_32x32x32_i8 per block, one 16-register
+//     result buffer, 16-register bias tuple, 16 token scales and 2 row-scale pairs per block -- 125 VGPRs;
+//   * gemm_mfma_kernel (the gated feed-forward launch, and plain projections on request): 4 x 2 tiles of
+//     v_mfma_i32_16x16x32_i8, four 4-register result buffers, 4-register bias -- 109 VGPRs.
+// Both stay under 128 VGPRs so that FOUR waves share a SIMD, which matters more than anything else here: a wave can
+// issue a vector-ALU instruction only every ~4.7 cycles while a SIMD retires one every ~2.2, and the kernel is bound by
+// the two scaling FMAs per result plus the matrix instructions, which a SIMD does not overlap with them.  The small
+// shape runs the matrix unit at a third of the large one's rate (1.7 vs 4.9 POP/s measured), which is what the
+// 32x32x32 loop recovers part of (3 - 8 % of a launch).
 // One stage = 4 blocks (128 elements of K).  Both operands are copied global -> LDS directly
 // (global_load_lds_dwordx4: asynchronous, no registers, 1 KB per wave instruction):
 //   * weights from the GEMM's own copy of the matrix, made from the raw GGUF blocks when the
@@ -411,24 +414,25 @@ __device__ __forceinline__ void tile_of_block(uint32_t bid, uint32_t row_tiles, 
 }
 
 // Results of a wave's MFMA tiles into the output (or into a K share's partial sums): element (tt, rt, r) of the wave tile is
-// (row + 16 rt, tok + 16 tt + r), `row` / `tok` being this lane's first row and token.  One instantiation per output layout
+// (row + RSTEP rt, tok + TSTEP tt + r), `row` / `tok` being this lane's first row and token (16 / 16 for the 16x16 MFMA
+// layout: a lane holds 4 consecutive tokens of one row per tile; 8 / 32 for the 32x32 layout: 4 groups of 4 tokens, 8 apart).  One instantiation per output layout
 // so that the inner index is an immediate offset of the store; CHECK = false for wave tiles that lie inside the matrix (no
 // predicates at all), ACC adds onto what is there.  The mode is uniform per launch, the bounds are uniform per wave: the
 // callers branch once, not per element.
-template <int NTT, int NRT, bool ROW_MAJOR, bool CHECK, bool ACC, typename F>
+template <int NTT, int NRT, int TSTEP, int RSTEP, bool ROW_MAJOR, bool CHECK, bool ACC, typename F>
 __device__ __forceinline__ void store_results(float* __restrict__ base, size_t stride, uint32_t row, uint32_t tok, uint32_t m, uint32_t n,
                                               F&& value) {
     if constexpr (ROW_MAJOR) {
 #pragma unroll
         for (int rt = 0; rt < NRT; rt++) {
-            float* q = base + (size_t)(row + 16 * rt) * stride + tok;
+            float* q = base + (size_t)(row + RSTEP * rt) * stride + tok;
 #pragma unroll
             for (int tt = 0; tt < NTT; tt++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    if (CHECK && !(row + 16 * rt < m && tok + 16 * tt + r < n)) continue;
+                    if (CHECK && !(row + RSTEP * rt < m && tok + TSTEP * tt + r < n)) continue;
                     const float v = value(tt, rt, r);
-                    q[16 * tt + r] = ACC ? q[16 * tt + r] + v : v;
+                    q[TSTEP * tt + r] = ACC ? q[TSTEP * tt + r] + v : v;
                 }
         }
     } else {
@@ -436,35 +440,35 @@ __device__ __forceinline__ void store_results(float* __restrict__ base, size_t s
         for (int tt = 0; tt < NTT; tt++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                float* q = base + (size_t)(tok + 16 * tt + r) * stride + row;
+                float* q = base + (size_t)(tok + TSTEP * tt + r) * stride + row;
 #pragma unroll
                 for (int rt = 0; rt < NRT; rt++) {
-                    if (CHECK && !(row + 16 * rt < m && tok + 16 * tt + r < n)) continue;
+                    if (CHECK && !(row + RSTEP * rt < m && tok + TSTEP * tt + r < n)) continue;
                     const float v = value(tt, rt, r);
-                    q[16 * rt] = ACC ? q[16 * rt] + v : v;
+                    q[RSTEP * rt] = ACC ? q[RSTEP * rt] + v : v;
                 }
             }
     }
 }
 // The launch's output mode picked once per wave: a K share's partial sums [share][n][m], or y in either layout, plain or accumulating.
-template <int NTT, int NRT, typename F>
+template <int NTT, int NRT, int TSTEP = 16, int RSTEP = 16, typename F>
 __device__ __forceinline__ void store_wave_tile(const GemmArgs& a, uint32_t ksplit, uint32_t split, uint32_t row, uint32_t tok, F&& value) {
     // the wave tile's corner is the same for every lane: keep the test (and the branches on it) scalar
-    const uint32_t row_end = (uint32_t)__builtin_amdgcn_readfirstlane((int)(row - (row & 15u))) + 16u * NRT;
-    const uint32_t tok_end = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tok - (tok & 15u))) + 16u * NTT;
+    const uint32_t row_end = (uint32_t)__builtin_amdgcn_readfirstlane((int)(row - (row & (uint32_t)(RSTEP - 1)))) + (uint32_t)(RSTEP * NRT);
+    const uint32_t tok_end = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tok - (tok & (uint32_t)(TSTEP - 1)))) + (uint32_t)(TSTEP * NTT);
     const bool inside = row_end <= a.m && tok_end <= a.n;
     if (ksplit > 1) {  // this share's sums; the reduce launch (or the caller's next kernel) adds the shares up
         float* base = a.partial + (size_t)split * a.n * a.m;
-        if (inside) store_results<NTT, NRT, false, false, false>(base, a.m, row, tok, a.m, a.n, value);
-        else store_results<NTT, NRT, false, true, false>(base, a.m, row, tok, a.m, a.n, value);
+        if (inside) store_results<NTT, NRT, TSTEP, RSTEP, false, false, false>(base, a.m, row, tok, a.m, a.n, value);
+        else store_results<NTT, NRT, TSTEP, RSTEP, false, true, false>(base, a.m, row, tok, a.m, a.n, value);
     } else if (a.y_row_major) {
-        if (a.accumulate) store_results<NTT, NRT, true, true, true>(a.y, a.y_stride, row, tok, a.m, a.n, value);
-        else if (inside) store_results<NTT, NRT, true, false, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
-        else store_results<NTT, NRT, true, true, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        if (a.accumulate) store_results<NTT, NRT, TSTEP, RSTEP, true, true, true>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        else if (inside) store_results<NTT, NRT, TSTEP, RSTEP, true, false, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        else store_results<NTT, NRT, TSTEP, RSTEP, true, true, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
     } else {
-        if (a.accumulate) store_results<NTT, NRT, false, true, true>(a.y, a.y_stride, row, tok, a.m, a.n, value);
-        else if (inside) store_results<NTT, NRT, false, false, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
-        else store_results<NTT, NRT, false, true, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        if (a.accumulate) store_results<NTT, NRT, TSTEP, RSTEP, false, true, true>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        else if (inside) store_results<NTT, NRT, TSTEP, RSTEP, false, false, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
+        else store_results<NTT, NRT, TSTEP, RSTEP, false, true, false>(a.y, a.y_stride, row, tok, a.m, a.n, value);
     }
 }
 
@@ -628,6 +632,200 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_mfma_kernel(GemmArgs a) {
     } else if constexpr (!DUMP) {
         store_wave_tile<TT, RT>(a, ksplit, split, row0 + wrow0 + l16, tok0 + wtok0 + 4 * kq,
                                 [&](int tt, int rt, int r) { return acc[tt][rt][r]; });
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// The wide tile on the large MFMA shape: same workgroup tile (128 rows x 128 tokens), same stages, copies and LDS layouts
+// as gemm_mfma_kernel, but a wave's 64 rows x 32 tokens are TWO v_mfma_i32_32x32x32_i8 per block (rows 0..31 and 32..63 of
+// the wave against its 32 tokens) instead of eight 16x16x32: the small shape runs the matrix unit at a third of its rate and
+// its time adds to the scaling FMAs' (a SIMD does not overlap the two), so a block's matrix work drops from ~160 to ~57 cycles.
+// Layout of the 32x32 result: lane l holds weight row n = l % 32 (of its row half) and the 16 tokens
+// m = 8 g + 4 (l / 32) + r, g = 0..3, r = 0..3 -- one row-scale pair per MFMA and 16 token scales per block (four 16-byte LDS
+// reads, shared by both MFMAs).  ONE result buffer: MFMA -> its 32 FMAs -> MFMA -> its 32 FMAs; the other waves of the SIMD
+// cover the MFMA's latency (measured: faster than two buffers, and 16 registers cheaper, which is what lets the 16-register
+// bias tuple, 16 token scales and 32 accumulators fit four waves per SIMD).  Operands of block b+1 are requested as soon as
+// the second MFMA of block b has been issued, token scales group by group behind their last use.
+// Plain projections only (the gated launch keeps the 16x16 kernel, whose epilogue is written for that result layout).
+typedef int v16i __attribute__((ext_vector_type(16)));
+struct Mats32 {
+    v4i a, b0, b1;  // 16 K-bytes of this lane's token / of its row in the wave's first and second 32 rows
+};
+struct Scales32 {
+    float2 dw0, dw1;  // {dw, -12582912*dw} of this lane's two rows
+    v4f dx[4];        // token scales of its four token groups
+};
+template <int OFF>
+__device__ __forceinline__ void lds_read16(uint32_t addr, v4i& dst) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+__device__ __forceinline__ void load_mats(const LaneAddr& la, Mats32& m) {  // 3 reads
+    lds_read16<0>(la.xt, m.a);
+    lds_read16<0>(la.wt, m.b0);
+    lds_read16<kSlabWt>(la.wt, m.b1);  // the wave's second granule
+}
+template <int G>
+__device__ __forceinline__ void load_tok_scales32(const LaneAddr& la, Scales32& s) {  // 1 read
+    lds_read16<32 * G>(la.dxf, s.dx[G]);
+}
+// (the waits tie the registers that become valid, so nothing that uses them can be scheduled above)
+template <int N>
+__device__ __forceinline__ void lds_wait_a_b0(Mats32& m) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(m.a), "+v"(m.b0) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_phase_a(Mats32& m, Scales32& s) {
+    asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(m.b1), "+v"(s.dw0), "+v"(s.dx[0]), "+v"(s.dx[1]), "+v"(s.dx[2]), "+v"(s.dx[3]) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_dw1(Scales32& s) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(s.dw1) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_all(Mats32& m, Scales32& s) {
+    asm volatile("s_waitcnt lgkmcnt(%9)"
+                 : "+v"(m.a), "+v"(m.b0), "+v"(m.b1), "+v"(s.dw0), "+v"(s.dw1), "+v"(s.dx[0]), "+v"(s.dx[1]), "+v"(s.dx[2]), "+v"(s.dx[3])
+                 : "n"(N)
+                 : "memory");
+}
+
+template <int TYPE, bool DUMP>
+__global__ __launch_bounds__(THREADS, 4) void gemm_mfma32_kernel(GemmArgs a) {
+    __shared__ Smem sm;
+    uint32_t row_tile, tok_tile;
+    bool valid_tile;
+    const uint32_t ksplit = DUMP || a.ksplit < 2 ? 1u : a.ksplit;
+    const uint32_t split = ksplit > 1 ? blockIdx.x % ksplit : 0u;
+    tile_of_block(ksplit > 1 ? blockIdx.x / ksplit : blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
+    if (!valid_tile) return;  // whole workgroup leaves together
+    select_weight(a, row_tile);
+    const uint32_t row0 = row_tile * BM;
+    const uint32_t tok0 = tok_tile * BN;
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t l32 = lane & 31u;
+    const uint32_t kh = lane >> 5;            // which 16-byte half of the block this lane feeds
+    const uint32_t wrow0 = (wave >> 2) * 64;  // wave's rows within the tile
+    const uint32_t wtok0 = (wave & 3u) * 32;  // wave's tokens within the tile
+    const uint32_t nb = a.k >> 5;
+    const uint32_t all_stages = nb / KB;
+    const uint32_t first = split * all_stages / ksplit;  // shares differ by at most one stage, none is empty
+    const uint32_t stages = (split + 1u) * all_stages / ksplit - first;
+
+    float acc[2][16];  // [row half][4 g + r]
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[j][i] = 0.0f;
+
+    v16i cbias;
+#pragma unroll
+    for (int i = 0; i < 16; i++) cbias[i] = (int)kBiasBits;
+    asm volatile("" : "+v"(cbias));  // keep it in registers (left alone, the compiler rebuilds it before every MFMA)
+
+    StageRegs regs;
+    StagePtrs<BN> ptrs;
+    init_stage_ptrs<BN, false>(a, row_tile, tok0, first * KB, ptrs);
+    dma_stage(ptrs, sm.st[0]);
+    load_stage(ptrs, regs);
+    store_stage(sm.st[0], regs);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
+    __syncthreads();
+
+    LaneAddr la;
+    {
+        const Stage& s = sm.st[0];
+        // this lane's token row; K-chunk 2*block + kh sits at position chunk ^ swizzle
+        const uint32_t sw = xt_swizzle(wtok0 + l32);
+        la.xsh = sw >> 1;
+        la.xbase = lds_addr(&s.xt[wtok0 + l32][0]) + (((kh ^ sw) & 1u) << 4);
+        la.xt = la.xbase + (la.xsh << 5);
+        la.wt = lds_addr(&s.wt[wrow0 / GR][kh][0][l32]);  // the wave's 64 rows are two granules
+        la.dws = lds_addr(&s.dws[wrow0 / GR][0][l32]);
+        la.dxf = lds_addr(&s.dxf[0][wtok0 + 4 * kh]);
+    }
+
+    for (uint32_t st = 0; st < stages; st++) {
+        if (st + 1 < stages) {
+            dma_stage(ptrs, sm.st[(st + 1) & 1u]);
+            load_stage(ptrs, regs);
+        }
+
+        // Reads of a block, in issue order (LDS data returns in that order): a, b0, b1, dw0, dx0..dx3, dw1.
+        Mats32 mt;
+        Scales32 sc;
+        load_mats(la, mt);                  // 3
+        lds_read8<0>(la.dws, sc.dw0);       // 1
+        load_tok_scales32<0>(la, sc);       // 4
+        load_tok_scales32<1>(la, sc);
+        load_tok_scales32<2>(la, sc);
+        load_tok_scales32<3>(la, sc);
+        lds_read8<kSlabDws>(la.dws, sc.dw1);  // 1
+#pragma unroll 1
+        for (int b = 0; b < KB; b++) {
+            next_block(la, (uint32_t)b, b + 1 < KB);  // last iteration: harmless re-read of its own block
+            const uint32_t row = row0 + wrow0 + l32, tok = tok0 + wtok0 + 4 * kh, blk = (first + st) * KB + b;
+            auto consume = [&](const v16i& d, int j, const float2 dw) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    if constexpr (DUMP) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            if (row + 32 * j < a.m && tok + 8 * g + r < a.n) {
+                                int v = d[4 * g + r] - (int)kBiasBits;
+                                if (TYPE == 2) v >>= 4;  // weights were stored x16; exact
+                                a.dots[((size_t)(tok + 8 * g + r) * a.m + row + 32 * j) * nb + blk] = v;
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const float v = __builtin_fmaf(__int_as_float(d[4 * g + r]), dw.x, dw.y);
+                            acc[j][4 * g + r] = __builtin_fmaf(v, sc.dx[g][r], acc[j][4 * g + r]);
+                        }
+                    }
+                    if (j == 1) {  // this group's token scales are done with: request the next block's
+                        if (g == 0) load_tok_scales32<0>(la, sc);
+                        if (g == 1) load_tok_scales32<1>(la, sc);
+                        if (g == 2) load_tok_scales32<2>(la, sc);
+                        if (g == 3) load_tok_scales32<3>(la, sc);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            lds_wait_a_b0<7>(mt);  // the seven reads issued after a and b0 may still be in flight
+            v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.a, mt.b0, cbias, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);  // (the MFMA goes out before the wait for what only the FMAs need)
+            lds_wait_phase_a<1>(mt, sc);  // everything but dw1
+            __builtin_amdgcn_sched_barrier(0);
+            consume(d, 0, sc.dw0);
+            d = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.a, mt.b1, cbias, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_mats(la, mt);             // both MFMAs of this block have been issued
+            lds_read8<0>(la.dws, sc.dw0);  // the first row half is done
+            lds_wait_dw1<4>(sc);           // (the four reads just issued stay in flight)
+            __builtin_amdgcn_sched_barrier(0);
+            consume(d, 1, sc.dw1);
+            lds_read8<kSlabDws>(la.dws, sc.dw1);
+        }
+        lds_wait_all<0>(mt, sc);  // nothing of this stage's buffer is read past this point
+        {   // block 0 of the other buffer (the block loop left wt / dws / dxf at block KB - 1)
+            const uint32_t other = (st & 1u) ? 0u - (uint32_t)sizeof(Stage) : (uint32_t)sizeof(Stage);
+            la.xbase += other;
+            la.xt = la.xbase + (la.xsh << 5);
+            la.wt += other - (KB - 1) * kOffWt;
+            la.dws += other - (KB - 1) * kOffDws;
+            la.dxf += other - (KB - 1) * kOffDxf;
+        }
+        if (st + 1 < stages) store_stage(sm.st[(st + 1) & 1u], regs);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS copies of the next stage have landed
+        __syncthreads();
+    }
+
+    if constexpr (!DUMP) {
+        store_wave_tile<4, 2, 8, 32>(a, ksplit, split, row0 + wrow0 + l32, tok0 + wtok0 + 4 * kh,
+                                     [&](int g, int j, int r) { return acc[j][4 * g + r]; });
     }
 }
 
@@ -880,12 +1078,19 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0, boo
         return narrow_launch(blocks);
     }
     if (wide_split) {
-        hipError_t e = type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, DUMP>, dim3(blocks * a.ksplit), dim3(THREADS), a)
-                                         : launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, DUMP>, dim3(blocks * a.ksplit), dim3(THREADS), a);
+        hipError_t e = !L.gemm_mfma16
+                           ? (type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_mfma32_kernel<2, DUMP>, dim3(blocks * a.ksplit), dim3(THREADS), a)
+                                                : launch_kernel(L, kFamGemm, gemm_mfma32_kernel<8, DUMP>, dim3(blocks * a.ksplit), dim3(THREADS), a))
+                           : (type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, DUMP>, dim3(blocks * a.ksplit), dim3(THREADS), a)
+                                                : launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, DUMP>, dim3(blocks * a.ksplit), dim3(THREADS), a));
         if (e != hipSuccess || defer_reduce) return e;
         return launch_reduce(a, L);
     }
     a.ksplit = 1;  // an unsplit launch of the wide kernel
+    if (!L.gemm_mfma16) {
+        if (type == kTypeQ4_0) return launch_kernel(L, kFamGemm, gemm_mfma32_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
+        return launch_kernel(L, kFamGemm, gemm_mfma32_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);
+    }
     if (type == kTypeQ4_0)
         return launch_kernel(L, kFamGemm, gemm_mfma_kernel<2, DUMP>, dim3(blocks), dim3(THREADS), a);
     return launch_kernel(L, kFamGemm, gemm_mfma_kernel<8, DUMP>, dim3(blocks), dim3(THREADS), a);

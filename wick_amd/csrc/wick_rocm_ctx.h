@@ -42,8 +42,9 @@ struct wick_rocm_ctx {
     uint32_t gemm_max_splits = kGemmMaxSplits;  // K split of GEMM launches with few tiles (1: off)
     KernelTimer timer;
     int64_t gemv_direct_max_bytes = -1;
+    bool gemm_mfma16 = false;  // wick_rocm_set_gemm_mfma_shape(ctx, 16)
     unsigned long long* argmax_partial = nullptr;  // kArgmaxPartials keys for wick_rocm_argmax
-    Launch launch() { return Launch{stream, &timer, gemv_direct_max_bytes}; }
+    Launch launch() { return Launch{stream, &timer, gemv_direct_max_bytes, gemm_mfma16}; }
 };
 
 struct wick_rocm_weight {

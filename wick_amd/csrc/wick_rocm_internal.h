@@ -48,6 +48,7 @@ struct Launch {
     hipStream_t stream;
     KernelTimer* timer;  // may be null
     int64_t gemv_direct_max_bytes = -1;  // single-token GEMV: per-lane loads below, span loads from here on; < 0 = per-dtype default
+    bool gemm_mfma16 = false;            // plain wide GEMM launches: the 16x16x32 block loop instead of the 32x32x32 one
 };
 
 template <typename... KArgs, typename... Args>

@@ -73,6 +73,7 @@ _SIGNATURES = {
     "wick_rocm_download": (C.c_int, [_P, _P, _P, C.c_size_t]),
     "wick_rocm_sync": (C.c_int, [_P]),
     "wick_rocm_set_gemm_min_n": (C.c_int, [_P, C.c_uint32]),
+    "wick_rocm_set_gemm_mfma_shape": (C.c_int, [_P, C.c_int]),
     "wick_rocm_set_gemm_packing": (C.c_int, [_P, C.c_int]),
     "wick_rocm_weight_device_bytes": (C.c_size_t, [_P]),
     "wick_rocm_set_gemm_max_k_splits": (C.c_int, [_P, C.c_uint32]),
@@ -242,6 +243,10 @@ class RocmContext:
     def set_gemm_packing(self, enabled: bool) -> None:
         """Whether upload_weight also makes the prefill GEMM's own copy of a Q4_0 / Q8_0 weight (default: yes)."""
         self._check(self._lib.wick_rocm_set_gemm_packing(self._h, 1 if enabled else 0))
+
+    def set_gemm_mfma_shape(self, shape: int = 0) -> None:
+        """Block loop of the wide-tile GEMM: 32 (default, also 0) or 16 (the small MFMA shape)."""
+        self._check(self._lib.wick_rocm_set_gemm_mfma_shape(self._h, shape))
 
     def set_gemm_min_n(self, min_n: int) -> None:
         self._check(self._lib.wick_rocm_set_gemm_min_n(self._h, min_n))
