@@ -784,6 +784,7 @@ def main():
     ap.add_argument("--skip-extra", action="store_true", help="only the headline GEMV, the GEMM (+ CPU baseline)")
     ap.add_argument("--prompt-tokens", type=int, default=2002, help="lfm2_prefill_trace: tokens of the traced prompt pass")
     ap.add_argument("--graph-only", action="store_true", help="decode legs: graph replays only, no eager launches (for kernel tracers)")
+    ap.add_argument("--mfma-shape", type=int, default=0, help="block loop of the wide GEMM tile: 0 / 32 (default) or 16 (A/B runs)")
     ap.add_argument("--leg", default="all", help="all | c1 | gemm | decode | decode_q8 | gemv | prefill_sites | lm_head | lm_head_q6k | upload | lfm2_step | lfm2_step_q8 | lfm2_step_kv16 | lfm2_step_1p2b | lfm2_step_trace | lfm2_prefill_trace | copy | probe | cpu")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -798,6 +799,7 @@ def main():
         print(json.dumps({"cpu_baseline": cpu_baseline(O, W)}))
         return
     ctx = W.RocmContext(0)
+    ctx.set_gemm_mfma_shape(args.mfma_shape)
     if leg != "all":
         one = {
             # graph replays only (warm-up included): every gemv_pairs_kernel dispatch a kernel tracer sees belongs to the timed workload
