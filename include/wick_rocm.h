@@ -195,9 +195,9 @@ int wick_rocm_set_gemm_min_n(wick_rocm_ctx *ctx, uint32_t min_n);
  * the one above; wick_rocm_matmul_f32_noalloc never splits. */
 int wick_rocm_set_gemm_max_k_splits(wick_rocm_ctx *ctx, uint32_t max_splits);
 
-/* Which matrix-core instruction the wide-tile GEMM's block loop is built on: 32 (the default, also 0) = two
- * v_mfma_i32_32x32x32_i8 per block and wave, 16 = eight v_mfma_i32_16x16x32_i8 (what the gated feed-forward launch and the
- * narrow tile always use).  Block dots are bit-identical either way, f32 sums agree to the last bit or two (the order in
+/* Which matrix-core instruction the GEMM's block loops are built on: 32 (the default, also 0) = v_mfma_i32_32x32x32_i8
+ * (two per block and wave on the wide tile, one on the narrow tile when the launch has more than 48 tokens), 16 = eight / four
+ * v_mfma_i32_16x16x32_i8 (what the gated feed-forward launch and narrow launches of up to 48 tokens always use).  Block dots are bit-identical either way, f32 sums agree to the last bit or two (the order in
  * which a row's blocks are added is the same, the lanes that hold them differ).  A tuning knob like the ones above. */
 int wick_rocm_set_gemm_mfma_shape(wick_rocm_ctx *ctx, int shape);
 

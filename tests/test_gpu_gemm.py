@@ -42,14 +42,16 @@ def test_gemm_parity(ctx, oracle, dtype, m, n, k):
         assert np.array_equal(dots, oracle.block_dots_i32(dtype, p.wb, p.q, m, n, k))
 
 
-# more than 256 wide tiles (fewer run on the narrow tile), ragged in rows and tokens; the last one is cut over K on the wide tile
-WIDE_SHAPES = [(2100, 2010, 128, True), (2100, 1990, 256, False), (4700, 1100, 384, False), (1024, 2002, 4608, False)]
+# more than 256 wide tiles (fewer run on the narrow tile), ragged in rows and tokens; the fourth is cut over K on the wide tile;
+# the last two take the narrow tile (n > 48: both of its block loops exist), the very last one cut over K
+WIDE_SHAPES = [(2100, 2010, 128, True), (2100, 1990, 256, False), (4700, 1100, 384, False), (1024, 2002, 4608, False),
+               (300, 64, 512, True), (1000, 700, 1024, False)]
 
 
 @pytest.mark.parametrize("dtype", [W.Q4_0, W.Q8_0])
 @pytest.mark.parametrize("m,n,k,with_dots", WIDE_SHAPES)
 def test_wide_tile_on_either_mfma_shape(ctx, oracle, dtype, m, n, k, with_dots):
-    """The wide tile's two block loops (32x32x32, the default, and 16x16x32): each against the oracle (two row bands over all
+    """The two block loops of the wide tile and of the full narrow tile (32x32x32, the default, and 16x16x32): each against the oracle (two row bands over all
     tokens) in both layouts with ragged strides and with the accumulate flag, block dots bit-exact through either, and the
     two within 1e-6 of each other everywhere."""
     rb = (k // 32) * (18 if dtype == W.Q4_0 else 34)

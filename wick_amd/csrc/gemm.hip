@@ -10,7 +10,8 @@
 // Workgroup = 512 threads = 8 waves, tile = 128 weight rows x 128 tokens, each wave
 // owns 64 rows x 32 tokens.  Two block loops exist for that wave tile:
 //   * gemm_mfma32_kernel (plain projections, the default): 2 x v_mfma_i32_32x32x32_i8 per block, one 16-register
-//     result buffer, 16-register bias tuple, 16 token scales and 2 row-scale pairs per block -- 125 VGPRs;
+//     result buffer, 16-register bias tuple, 16 token scales and 2 row-scale pairs per block -- 125 VGPRs
+//     (gemm_narrow32_kernel is the same loop with one MFMA per block on the 128 x 64 tile);
 //   * gemm_mfma_kernel (the gated feed-forward launch, and plain projections on request): 4 x 2 tiles of
 //     v_mfma_i32_16x16x32_i8, four 4-register result buffers, 4-register bias -- 109 VGPRs.
 // Both stay under 128 VGPRs so that FOUR waves share a SIMD, which matters more than anything else here: a wave can
@@ -980,6 +981,159 @@ __global__ __launch_bounds__(THREADS, 4) void gemm_narrow_kernel(GemmArgs a) {
     }
 }
 
+// The narrow tile (128 rows x 64 tokens) on the large MFMA shape, for launches that have tokens for the whole tile
+// (n > 48; the shorter ones keep gemm_narrow_kernel's 16-token tiles): wave w owns rows 32 (w / 2) .. of the tile (one
+// granule) against tokens 32 (w % 2) .., ONE v_mfma_i32_32x32x32_i8 per block instead of four 16x16x32, the result layout,
+// scale reads and single result buffer of gemm_mfma32_kernel.  Same stages, copies and LDS layouts as gemm_narrow_kernel.
+struct NarrowMats32 {
+    v4i a, b;
+};
+struct NarrowScales32 {
+    float2 dw;
+    v4f dx[4];
+};
+template <int N>
+__device__ __forceinline__ void lds_wait(NarrowMats32& m) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(m.a), "+v"(m.b) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(NarrowScales32& s) {
+    asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(s.dw), "+v"(s.dx[0]), "+v"(s.dx[1]), "+v"(s.dx[2]), "+v"(s.dx[3]) : "n"(N) : "memory");
+}
+
+template <int TYPE, bool DUMP>
+__global__ __launch_bounds__(THREADS, 4) void gemm_narrow32_kernel(GemmArgs a) {
+    __shared__ SmemT<BN_NARROW> sm;
+    uint32_t row_tile, tok_tile;
+    bool valid_tile;
+    const uint32_t ksplit = DUMP || a.ksplit < 2 ? 1u : a.ksplit;
+    const uint32_t split = ksplit > 1 ? blockIdx.x % ksplit : 0u;
+    tile_of_block(ksplit > 1 ? blockIdx.x / ksplit : blockIdx.x, a.row_tiles, a.tok_tiles, row_tile, tok_tile, valid_tile);
+    if (!valid_tile) return;  // whole workgroup leaves together
+    select_weight(a, row_tile);
+    const uint32_t row0 = row_tile * BM;
+    const uint32_t tok0 = tok_tile * BN_NARROW;
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t l32 = lane & 31u;
+    const uint32_t kh = lane >> 5;             // which 16-byte half of the block this lane feeds
+    const uint32_t wrow0 = (wave >> 1) * 32;   // wave's rows within the tile: one granule
+    const uint32_t wtok0 = (wave & 1u) * 32;   // wave's tokens within the tile
+    const uint32_t nb = a.k >> 5;
+    const uint32_t all_stages = nb / KB;
+    const uint32_t first = split * all_stages / ksplit;
+    const uint32_t stages = (split + 1u) * all_stages / ksplit - first;
+
+    float acc[16];  // [4 g + r]
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.0f;
+    v16i cbias;
+#pragma unroll
+    for (int i = 0; i < 16; i++) cbias[i] = (int)kBiasBits;
+    asm volatile("" : "+v"(cbias));
+
+    StageRegs regs;
+    StagePtrs<BN_NARROW> ptrs;
+    init_stage_ptrs<BN_NARROW>(a, row_tile, tok0, first * KB, ptrs);
+    dma_stage(ptrs, sm.st[0]);
+    load_stage(ptrs, regs);
+    store_stage(sm.st[0], regs);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct-to-LDS copies have landed
+    __syncthreads();
+
+    LaneAddr la;  // block 0 of buffer 0; moved on as in the wide kernel
+    {
+        const StageT<BN_NARROW>& s = sm.st[0];
+        const uint32_t sw = xt_swizzle(wtok0 + l32);
+        la.xsh = sw >> 1;
+        la.xbase = lds_addr(&s.xt[wtok0 + l32][0]) + (((kh ^ sw) & 1u) << 4);
+        la.xt = la.xbase + (la.xsh << 5);
+        la.wt = lds_addr(&s.wt[wrow0 / GR][kh][0][l32]);
+        la.dws = lds_addr(&s.dws[wrow0 / GR][0][l32]);
+        la.dxf = lds_addr(&s.dxf[0][wtok0 + 4 * kh]);
+    }
+
+    for (uint32_t st = 0; st < stages; st++) {
+        if (st + 1 < stages) {
+            dma_stage(ptrs, sm.st[(st + 1) & 1u]);
+            load_stage(ptrs, regs);
+        }
+
+        // Reads of a block, in issue order: a, b, dx0..dx3, dw.
+        NarrowMats32 mt;
+        NarrowScales32 sc;
+        lds_read16<0>(la.xt, mt.a);
+        lds_read16<0>(la.wt, mt.b);
+        lds_read16<0>(la.dxf, sc.dx[0]);
+        lds_read16<32>(la.dxf, sc.dx[1]);
+        lds_read16<64>(la.dxf, sc.dx[2]);
+        lds_read16<96>(la.dxf, sc.dx[3]);
+        lds_read8<0>(la.dws, sc.dw);
+#pragma unroll 1
+        for (int b = 0; b < KB; b++) {
+            const bool adv = b + 1 < KB;  // last iteration: harmless re-read of its own block
+            la.xt = la.xbase + ((((uint32_t)(adv ? b + 1 : b)) ^ la.xsh) << 5);
+            la.wt += adv ? kOffWt : 0;
+            la.dws += adv ? kOffDws : 0;
+            la.dxf += adv ? kOffDxfNarrow : 0;
+            const uint32_t row = row0 + wrow0 + l32, tok = tok0 + wtok0 + 4 * kh, blk = (first + st) * KB + b;
+            lds_wait<5>(mt);  // the five scale reads issued after a and b may still be in flight
+            const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(mt.a, mt.b, cbias, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            lds_read16<0>(la.xt, mt.a);  // the MFMA that reads block b's operands has been issued
+            lds_read16<0>(la.wt, mt.b);
+            lds_wait<2>(sc);  // (the two reads just issued stay in flight)
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                if constexpr (DUMP) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        if (row < a.m && tok + 8 * g + r < a.n) {
+                            int v = d[4 * g + r] - (int)kBiasBits;
+                            if (TYPE == 2) v >>= 4;  // weights were stored x16; exact
+                            a.dots[((size_t)(tok + 8 * g + r) * a.m + row) * nb + blk] = v;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const float v = __builtin_fmaf(__int_as_float(d[4 * g + r]), sc.dw.x, sc.dw.y);
+                        acc[4 * g + r] = __builtin_fmaf(v, sc.dx[g][r], acc[4 * g + r]);
+                    }
+                }
+                // this group's token scales are done with: request the next block's
+                if (g == 0) lds_read16<0>(la.dxf, sc.dx[0]);
+                if (g == 1) lds_read16<32>(la.dxf, sc.dx[1]);
+                if (g == 2) lds_read16<64>(la.dxf, sc.dx[2]);
+                if (g == 3) lds_read16<96>(la.dxf, sc.dx[3]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            lds_read8<0>(la.dws, sc.dw);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(mt.a), "+v"(mt.b), "+v"(sc.dw), "+v"(sc.dx[0]), "+v"(sc.dx[1]), "+v"(sc.dx[2]), "+v"(sc.dx[3])
+                     :
+                     : "memory");  // nothing of this stage's buffer is read past this point
+        {
+            const uint32_t other = (st & 1u) ? 0u - (uint32_t)sizeof(StageT<BN_NARROW>) : (uint32_t)sizeof(StageT<BN_NARROW>);
+            la.xbase += other;
+            la.xt = la.xbase + (la.xsh << 5);
+            la.wt += other - (KB - 1) * kOffWt;
+            la.dws += other - (KB - 1) * kOffDws;
+            la.dxf += other - (KB - 1) * kOffDxfNarrow;
+        }
+        if (st + 1 < stages) store_stage(sm.st[(st + 1) & 1u], regs);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS copies of the next stage have landed
+        __syncthreads();
+    }
+
+    if constexpr (!DUMP) {
+        store_wave_tile<4, 1, 8, 32>(a, ksplit, split, row0 + wrow0 + l32, tok0 + wtok0 + 4 * kh, [&](int g, int, int r) { return acc[4 * g + r]; });
+    }
+}
+
 // y (+)= partial[0] + partial[1] + ... in that order, element by element (token-major partials [split][n][m]).
 // (S a template parameter: all of an element's loads are in flight together instead of one round trip per share.)
 template <int S>
@@ -1066,6 +1220,9 @@ hipError_t launch(int type, GemmArgs& a, const Launch& L, uint32_t more = 0, boo
                 if (a.n <= 48) return launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, false, 3>, dim3(grid), dim3(THREADS), a);
             }
             // (the product kernels do not depend on the weight type any more: the copy they read is the same for both)
+            if (!L.gemm_mfma16 && a.n > 48)
+                return type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_narrow32_kernel<2, DUMP>, dim3(grid), dim3(THREADS), a)
+                                         : launch_kernel(L, kFamGemm, gemm_narrow32_kernel<8, DUMP>, dim3(grid), dim3(THREADS), a);
             return type == kTypeQ4_0 ? launch_kernel(L, kFamGemm, gemm_narrow_kernel<2, DUMP>, dim3(grid), dim3(THREADS), a)
                                      : launch_kernel(L, kFamGemm, gemm_narrow_kernel<8, DUMP>, dim3(grid), dim3(THREADS), a);
         };
