@@ -313,3 +313,34 @@ def test_a_graph_that_used_the_scratch_goes_stale_when_it_regrows(oracle):
         b.free()
     w.free(), w2.free(), wide.free()
     ctx.close()
+
+
+def test_a_graph_that_only_quantizes_survives_a_larger_partial_sum_buffer(oracle):
+    """Every scratch buffer has a generation of its own: a graph whose launches hold the quantized-activation buffers stays
+    good when a later K-split projection grows the partial-sum buffer, which it never touched."""
+    ctx = W.RocmContext(0)
+    m, k = 64, 2080  # odd block count: the call quantizes into the context's scratch
+    wb = oracle.synth_weight(W.Q4_0, m, k, 9)
+    w = ctx.upload_weight(wb, W.Q4_0, m, k)
+    x = oracle.fill_normal(2, 1.0, k)
+    d_x, d_y = ctx.to_device(x), ctx.alloc(m * 4)
+    # quants / scales large enough for everything below (4 x 73728 = 64 x 4608 elements), no room for K shares (fewer tokens than
+    # the hand-off to the MFMA GEMM): only the partial sums will grow
+    ctx.reserve_scratch(4, 73728)
+    ctx.graph_begin()
+    ctx.encode_gemv(w, d_x, 0, d_y, 0)
+    g = ctx.graph_end()
+    # a short prompt's down projection: few tiles, long K -> cut over K, partial sums in context scratch (grown here)
+    n, m2, k2 = 64, 1024, 4608
+    w2 = ctx.upload_weight(oracle.synth_weight(W.Q4_0, m2, k2, 5), W.Q4_0, m2, k2)
+    d_x2, d_y2 = ctx.to_device(oracle.fill_normal(7, 1.0, n * k2)), ctx.alloc(n * m2 * 4)
+    ctx.encode_gemm(w2, d_x2, 0, d_y2, 0, n, k2, m2)
+    d_y.upload(np.zeros(m, np.float32))
+    ctx.graph_launch(g)
+    s, q = oracle.quantize_q8_0(x)
+    assert_f32_parity(d_y.download(np.float32, m), oracle.gemv_q8(W.Q4_0, wb, s, q, m, k), "graph after the partial sums grew")
+    ctx.graph_destroy(g)
+    for b in (d_x, d_y, d_x2, d_y2):
+        b.free()
+    w.free(), w2.free()
+    ctx.close()

@@ -56,12 +56,16 @@ int check_weight(wick_rocm_ctx* ctx, const wick_rocm_weight* w) {
 }
 
 int ensure_scratch(wick_rocm_ctx* ctx, size_t q_bytes, size_t s_floats, size_t f_floats = 0) {
-    if (ctx->capturing) ctx->capture_used_scratch = true;  // the graph being captured will hold these addresses
+    // the graph being captured will hold the addresses of the buffers this call asks for
+    if (ctx->capturing) ctx->capture_used_scratch |= (q_bytes ? 1u : 0u) | (s_floats ? 2u : 0u) | (f_floats ? 4u : 0u);
     if (q_bytes <= ctx->scratch_q_cap && s_floats <= ctx->scratch_s_cap && f_floats <= ctx->scratch_f_cap) return WICK_ROCM_OK;
     if (ctx->capturing)
         return fail(ctx, WICK_ROCM_ERR_STATE, "activation scratch too small during graph capture; call wick_rocm_reserve_scratch first");
     WR_HIP(ctx, hipStreamSynchronize(ctx->stream));  // earlier launches may still read the old scratch
-    ctx->scratch_gen++;  // graphs captured against the old buffers are stale from here on (wick_rocm_graph_launch refuses them)
+    // graphs captured against a buffer that moves are stale from here on (wick_rocm_graph_launch refuses them)
+    if (q_bytes > ctx->scratch_q_cap) ctx->scratch_gen[0]++;
+    if (s_floats > ctx->scratch_s_cap) ctx->scratch_gen[1]++;
+    if (f_floats > ctx->scratch_f_cap) ctx->scratch_gen[2]++;
     if (q_bytes > ctx->scratch_q_cap) {
         if (ctx->scratch_q) WR_HIP(ctx, hipFree(ctx->scratch_q));
         ctx->scratch_q = nullptr, ctx->scratch_q_cap = 0;
@@ -790,7 +794,7 @@ int wick_rocm_graph_begin(wick_rocm_ctx* ctx) {
     if (ctx->timer.enabled) return fail(ctx, WICK_ROCM_ERR_STATE, "graph_begin: kernel timing is on");
     WR_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     ctx->capturing = true;
-    ctx->capture_used_scratch = false;
+    ctx->capture_used_scratch = 0;
     ctx->capture_used_noalloc = false;
     return WICK_ROCM_OK;
 }
@@ -819,7 +823,7 @@ int wick_rocm_graph_end(wick_rocm_ctx* ctx, wick_rocm_graph** out) {
         return fail_hip(ctx, e, "graph_end");
     }
     g->uses_scratch = ctx->capture_used_scratch;
-    g->scratch_gen = ctx->scratch_gen;
+    for (int i = 0; i < 3; i++) g->scratch_gen[i] = ctx->scratch_gen[i];
     g->uses_noalloc = ctx->capture_used_noalloc;
     *out = g;
     return WICK_ROCM_OK;

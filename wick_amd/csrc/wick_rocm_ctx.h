@@ -30,8 +30,10 @@ struct wick_rocm_ctx {
     size_t scratch_f_cap = 0;  // floats
     // A captured graph has the scratch addresses baked in.  Every regrow bumps the generation; a graph that used the
     // scratch remembers the generation it was captured under and refuses to launch under another one.
-    uint64_t scratch_gen = 0;
-    bool capture_used_scratch = false;
+    // One generation per scratch buffer (quants, scales, K-split partial sums): a graph that only quantizes is not made stale
+    // by a larger partial-sum buffer.
+    uint64_t scratch_gen[3] = {0, 0, 0};
+    unsigned capture_used_scratch = 0;  // bit i: the capture in progress holds the address of scratch buffer i
     bool capture_used_noalloc = false;  // the capture in progress holds a wick_rocm_matmul_f32_noalloc call
     unsigned char* noalloc_scratch = nullptr;  // this device's address of the static scratch array of wick_rocm_matmul_f32_noalloc
     uint32_t gemm_min_n = 0;  // hand-off from the multi-token GEMV to the MFMA GEMM; 0: the per-weight default (min_n_for)
@@ -59,13 +61,17 @@ struct wick_rocm_weight {
 struct wick_rocm_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
-    bool uses_scratch = false;  // some captured launch reads or writes the context's scratch
-    uint64_t scratch_gen = 0;   // ... as it was laid out then
+    unsigned uses_scratch = 0;             // bit i: some captured launch reads or writes scratch buffer i of the context
+    uint64_t scratch_gen[3] = {0, 0, 0};   // ... as they were laid out then
     bool uses_noalloc = false;  // some captured launch uses the GPU's static scratch array (wick_rocm_matmul_f32_noalloc)
 };
 
 // True when the graph refers to scratch memory that has been freed and reallocated since its capture.
-inline bool graph_is_stale(const wick_rocm_ctx* ctx, const wick_rocm_graph* g) { return g->uses_scratch && g->scratch_gen != ctx->scratch_gen; }
+inline bool graph_is_stale(const wick_rocm_ctx* ctx, const wick_rocm_graph* g) {
+    for (int i = 0; i < 3; i++)
+        if ((g->uses_scratch >> i & 1u) && g->scratch_gen[i] != ctx->scratch_gen[i]) return true;
+    return false;
+}
 
 struct wick_rocm_event {
     hipEvent_t ev = nullptr;
